@@ -1,0 +1,67 @@
+"""Loader of the HIP library behind the C ABI (include/fbgemm_amd.h).
+
+The library is built in-tree by ``fbgemm_amd.build`` (hipcc, gfx950). There is
+no CPU fallback: if the shared object is missing or a symbol cannot be bound,
+importing the ops fails loudly.
+"""
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "lib", "libfbgemm_amd.so")
+
+# every symbol include/fbgemm_amd.h declares: name -> (restype, argtypes)
+_P, _I32, _I64 = C.c_void_p, C.c_int32, C.c_int64
+
+
+class SpmdmConfig(C.Structure):
+    """struct fbgemm_amd_spmdm_config."""
+    _fields_ = [
+        ("weight_ty", _I32), ("output_ty", _I32), ("index_bits", _I32), ("offset_bits", _I32),
+        ("block_size", _I64), ("output_stride", _I64), ("input_stride", _I64),
+        ("normalize_by_lengths", _I32), ("is_weight_positional", _I32),
+        ("use_offsets", _I32), ("scale_bias_last", _I32),
+    ]
+
+
+SYMBOLS = {
+    "fbgemm_amd_last_error": (C.c_char_p, []),
+    "fbgemm_amd_version": (C.c_char_p, []),
+    "fbgemm_amd_status_clear": (C.c_int, [_P, _P]),
+    "fbgemm_amd_status_read": (C.c_int, [_P, _P, C.POINTER(_I32), C.POINTER(_I64)]),
+    "fbgemm_amd_spmdm_launch": (C.c_int, [C.POINTER(SpmdmConfig), _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _P, _P]),
+    "fbgemm_amd_spmdm_run": (C.c_int, [C.POINTER(SpmdmConfig), _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _P]),
+    "fbgemm_amd_tbe_plan_create": (C.c_int, [C.POINTER(_P), _I32, _P, _P, _P, _P, _I64, _I64, _I64]),
+    "fbgemm_amd_tbe_plan_destroy": (None, [_P]),
+    "fbgemm_amd_tbe_forward": (C.c_int, [_P, _P, _P, _P, _P, _I32, _I64, _I64, _I32, _P, _I32, _P, _P, _P]),
+    "fbgemm_amd_tbe_plan_num_rows": (_I64, [_P, _I32]),
+    "fbgemm_amd_tbe_plan_row_bytes": (_I64, [_P, _I32]),
+    "fbgemm_amd_pruned_array_lookup": (C.c_int, [_P, _P, _I32, _I64, _P, _I32, _P, _I32, _P, _P]),
+    "fbgemm_amd_unpadded_row_size_in_bytes": (_I32, [_I32, _I32, _I32]),
+    "fbgemm_amd_padded_row_size_in_bytes": (_I32, [_I32, _I32, _I32, _I32]),
+}
+
+_lib = None
+
+
+def lib():
+    """The loaded library; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `python -m fbgemm_amd.build` "
+                "(hipcc --offload-arch=gfx950). There is no CPU fallback.")
+        handle = C.CDLL(LIB_PATH)
+        for name, (res, args) in SYMBOLS.items():
+            fn = getattr(handle, name)  # AttributeError if the symbol is absent
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def check(rc):
+    if rc < 0:
+        raise RuntimeError(f"fbgemm_amd error {rc}: {lib().fbgemm_amd_last_error().decode()}")
+    return rc

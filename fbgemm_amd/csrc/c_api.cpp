@@ -1,0 +1,490 @@
+// Host side of the C ABI declared in include/fbgemm_amd.h: argument checks,
+// per-table lane mapping, work lists, launches. No torch types here.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <vector>
+
+#include "../../include/fbgemm_amd.h"
+#include "lookup_common.h"
+
+namespace fbgemm_amd {
+hipError_t launch_lookup(const LookupArgs& a, bool idx64, hipStream_t stream);
+hipError_t launch_lengths_to_offsets(const void* lengths, bool is64, int64_t n, int64_t* offsets, hipStream_t stream);
+hipError_t launch_status_clear(Status* st, hipStream_t stream);
+hipError_t launch_pruned_array_lookup(const void* indices, const void* offsets, bool idx64, const void* remap,
+                                      bool remap64, const int64_t* remap_offsets, int32_t B, int32_t T,
+                                      void* dense, hipStream_t stream);
+} // namespace fbgemm_amd
+
+using namespace fbgemm_amd;
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+#define HIP_TRY(expr)                                                                   \
+  do {                                                                                  \
+    hipError_t e_ = (expr);                                                             \
+    if (e_ != hipSuccess) return fail(FBGEMM_AMD_E_HIP, "%s: %s", #expr, hipGetErrorString(e_)); \
+  } while (0)
+
+int type_bits(int ty) {
+  switch (ty) {
+    case ST_FP32: return 32;
+    case ST_FP16: case ST_BF16: return 16;
+    case ST_INT8: return 8;
+    case ST_INT4: return 4;
+    case ST_INT2: return 2;
+    default: return 0;
+  }
+}
+
+bool quantised(int ty) { return ty == ST_INT8 || ty == ST_INT4 || ty == ST_INT2; }
+
+int env_int(const char* name, int dflt) {
+  const char* v = getenv(name);
+  return v && *v ? atoi(v) : dflt;
+}
+
+// Tunables, read once per process (the reference reads its FBGEMM_* switches
+// the same way, src/Utils.cc:773-875).
+int xcd_swizzle_default() {
+  static int v = env_int("FBGEMM_AMD_XCD_SWIZZLE", 1);
+  return v;
+}
+
+// Choose how lanes split a row. Wide 16-byte lanes need every row's data and
+// scale/bias to sit on 4-byte boundaries; anything else falls back to 4-byte
+// lanes and finally to element-sized lanes, which accept any layout.
+void plan_lanes(TableDesc& d, uintptr_t base_addr, int64_t out_stride, bool has_sb) {
+  const int bits = type_bits(d.ty);
+  d.data_bytes = (int32_t)(((int64_t)d.D * bits + 7) / 8);
+  const bool a4 = base_addr % 4 == 0 && d.weights_offset % 4 == 0 && d.row_stride % 4 == 0 &&
+      d.data_off % 4 == 0 && (!has_sb || d.sb_off % 4 == 0);
+  const int min_vb = bits >= 16 ? bits / 8 : 1;
+  static const int force_vb = env_int("FBGEMM_AMD_FORCE_VB", 0);
+  int vb = min_vb;
+  if (a4 && d.data_bytes % 16 == 0 && d.ty != ST_INT2) vb = 16;
+  else if (a4 && d.data_bytes % 4 == 0) vb = 4;
+  if (force_vb == 4 && vb == 16) vb = 4;
+  if (force_vb == 1) vb = min_vb;
+  d.vb = vb;
+  const int chunks = (d.data_bytes + vb - 1) / vb;
+  d.lanes = std::max(1, std::min(64, chunks));
+  d.passes = (chunks + d.lanes - 1) / d.lanes;
+  // whole-run vector stores: each lane writes E = vb*8/bits consecutive
+  // elements; allowed when every run starts on a multiple of min(16, run bytes)
+  // and no run is cut by the end of the row.
+  const int E = vb * 8 / bits;
+  d.vec_store = 0;
+  if (d.D % E == 0) {
+    for (int k = 0; k < 2; ++k) {
+      const int esz = k == 0 ? 4 : 2;
+      const int run = E * esz;
+      const int al = std::min(16, run);
+      if ((run == 2 || run == 4 || run == 8 || run % 16 == 0) && (out_stride * esz) % al == 0 &&
+          ((int64_t)d.out_col * esz) % al == 0)
+        d.vec_store |= 1 << k;
+    }
+  }
+}
+
+struct DeviceScratch {
+  Status* status = nullptr;
+  int64_t* offsets = nullptr;
+  int64_t offsets_cap = 0;
+};
+
+std::mutex g_mu;
+std::map<int, DeviceScratch> g_scratch;
+
+int get_scratch(DeviceScratch** out) {
+  int dev = 0;
+  HIP_TRY(hipGetDevice(&dev));
+  DeviceScratch& s = g_scratch[dev];
+  if (!s.status) HIP_TRY(hipMalloc((void**)&s.status, sizeof(Status)));
+  *out = &s;
+  return 0;
+}
+
+int check_cfg(const fbgemm_amd_spmdm_config* c) {
+  if (!c) return fail(FBGEMM_AMD_E_ARG, "config is null");
+  if (type_bits(c->weight_ty) == 0) return fail(FBGEMM_AMD_E_ARG, "unsupported weight_ty %d", c->weight_ty);
+  if (c->output_ty != ST_FP32 && c->output_ty != ST_FP16 && c->output_ty != ST_BF16)
+    return fail(FBGEMM_AMD_E_ARG, "unsupported output_ty %d", c->output_ty);
+  if ((c->index_bits != 32 && c->index_bits != 64) || (c->offset_bits != 32 && c->offset_bits != 64))
+    return fail(FBGEMM_AMD_E_ARG, "index_bits/offset_bits must be 32 or 64");
+  if (c->block_size <= 0 || c->block_size > (1 << 24)) return fail(FBGEMM_AMD_E_ARG, "bad block_size");
+  return 0;
+}
+
+} // namespace
+
+extern "C" {
+
+const char* fbgemm_amd_last_error(void) { return g_err; }
+const char* fbgemm_amd_version(void) { return "0.1"; }
+
+int fbgemm_amd_status_clear(void* d_status, void* stream) {
+  if (!d_status) return fail(FBGEMM_AMD_E_ARG, "d_status is null");
+  HIP_TRY(launch_status_clear((Status*)d_status, (hipStream_t)stream));
+  return 0;
+}
+
+int fbgemm_amd_status_read(const void* d_status, void* stream, int32_t* bits, int64_t* first_bad_pos) {
+  if (!d_status) return fail(FBGEMM_AMD_E_ARG, "d_status is null");
+  Status h;
+  HIP_TRY(hipMemcpyAsync(&h, d_status, sizeof(h), hipMemcpyDeviceToHost, (hipStream_t)stream));
+  HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+  if (bits) *bits = h.bits;
+  if (first_bad_pos) *first_bad_pos = h.first_bad_pos == ~0ull ? -1 : (int64_t)h.first_bad_pos;
+  return 0;
+}
+
+int32_t fbgemm_amd_unpadded_row_size_in_bytes(int32_t dim, int32_t ty, int32_t sb) {
+  switch (ty) {
+    case ST_FP32: return dim * 4;
+    case ST_FP16: case ST_BF16: return dim * 2;
+    case ST_INT8: return dim + sb;
+    case ST_INT4: return dim / 2 + sb;
+    case ST_INT2: return dim / 4 + sb;
+    default: return 0;
+  }
+}
+
+int32_t fbgemm_amd_padded_row_size_in_bytes(int32_t dim, int32_t ty, int32_t row_alignment, int32_t sb) {
+  const uint64_t r = (uint64_t)fbgemm_amd_unpadded_row_size_in_bytes(dim, ty, sb);
+  const uint64_t a = (uint64_t)(row_alignment > 0 ? row_alignment : 1);
+  return (int32_t)((r + a - 1) / a * a);
+}
+
+int fbgemm_amd_spmdm_launch(
+    const fbgemm_amd_spmdm_config* cfg, int64_t output_size, int64_t index_size,
+    int64_t data_size, const void* d_input, const void* d_indices,
+    const void* d_offsets_or_lengths, const float* d_weights, void* d_out,
+    const int32_t* d_remap, void* d_status, void* stream_) {
+  if (int rc = check_cfg(cfg)) return rc;
+  if (!d_status) return fail(FBGEMM_AMD_E_ARG, "d_status is null");
+  if (output_size < 0 || index_size < 0 || data_size < 0) return fail(FBGEMM_AMD_E_ARG, "negative size");
+  if (output_size > 0x7fffffffLL) return fail(FBGEMM_AMD_E_ARG, "output_size exceeds 2^31-1");
+  hipStream_t stream = (hipStream_t)stream_;
+  if (output_size == 0) {
+    // the reference returns (0 == index_size) without touching anything
+    if (index_size != 0) {
+      Status h{ERR_LENGTH_MISMATCH, 0, ~0ull};
+      HIP_TRY(hipMemcpyAsync(d_status, &h, sizeof(h), hipMemcpyHostToDevice, stream));
+      HIP_TRY(hipStreamSynchronize(stream));
+    }
+    return 0;
+  }
+  if (!d_input || !d_out || !d_offsets_or_lengths || (index_size > 0 && !d_indices))
+    return fail(FBGEMM_AMD_E_ARG, "null data pointer");
+  if (d_remap && !cfg->scale_bias_last && quantised(cfg->weight_ty))
+    return fail(FBGEMM_AMD_E_ARG, "row-wise-sparse lookups use the scale_bias_last layout");
+  if (d_remap && cfg->output_ty != ST_FP32)
+    return fail(FBGEMM_AMD_E_ARG, "row-wise-sparse lookups write fp32");
+
+  const int ty = cfg->weight_ty;
+  const int bits = type_bits(ty);
+  const int64_t D = cfg->block_size;
+  const int64_t elem_bytes = bits >= 8 ? bits / 8 : 1; // storage element of input_stride
+  LookupArgs a;
+  memset(&a, 0, sizeof(a));
+  TableDesc& d = a.single;
+  d.ty = ty;
+  d.D = (int32_t)D;
+  d.out_col = 0;
+  d.num_rows = data_size;
+  d.placement = 0;
+  d.weights_offset = 0;
+  d.skip_minus_one = cfg->scale_bias_last ? 0 : 1;
+  bool has_sb = false;
+  if (quantised(ty)) {
+    has_sb = true;
+    const int64_t packed = (D * bits + 7) / 8;
+    const int64_t sb = (ty == ST_INT8 && cfg->scale_bias_last) ? 8 : 4;
+    d.sb_fp32 = sb == 8;
+    d.row_stride = cfg->input_stride == -1 ? packed + sb : cfg->input_stride;
+    if (cfg->scale_bias_last) {
+      d.data_off = 0;
+      d.sb_off = (int32_t)packed;
+    } else {
+      d.sb_off = 0;
+      d.data_off = (int32_t)sb;
+    }
+  } else {
+    d.row_stride = (cfg->input_stride == -1 ? D : cfg->input_stride) * elem_bytes;
+    d.data_off = 0;
+    d.sb_off = 0;
+  }
+  const int64_t out_stride = cfg->output_stride == -1 ? D : cfg->output_stride;
+  if ((ty == ST_FP16 || ty == ST_BF16) && (uintptr_t)d_input % 2) return fail(FBGEMM_AMD_E_ARG, "fp16 table must be 2-byte aligned");
+  if (ty == ST_FP32 && (uintptr_t)d_input % 4) return fail(FBGEMM_AMD_E_ARG, "fp32 table must be 4-byte aligned");
+  plan_lanes(d, (uintptr_t)d_input, out_stride, has_sb);
+
+  a.tables = nullptr;
+  a.weights[0] = (const uint8_t*)d_input;
+  a.weights[1] = nullptr;
+  a.indices = d_indices;
+  a.sample_weights = d_weights;
+  a.remap = d_remap;
+  a.remap_rows = data_size;
+  if (d_remap) {
+    d.num_rows = INT64_MAX; // the reference does not bound the physical id (RefImplementations.cc:1789-1791)
+    d.skip_minus_one = 0;
+  }
+  a.out = d_out;
+  a.out_stride = out_stride;
+  a.index_size = index_size;
+  a.work = nullptr;
+  a.B = (int32_t)output_size;
+  a.T = 1;
+  a.out_ty = cfg->output_ty;
+  a.normalize = cfg->normalize_by_lengths;
+  a.positional = cfg->is_weight_positional;
+  a.xcd_swizzle = 0;
+  a.check_total = 1;
+  a.out_aligned = (uintptr_t)d_out % 16 == 0;
+  a.status = (Status*)d_status;
+  const int G = 64 / d.lanes;
+  a.num_waves = (output_size + G - 1) / G;
+
+  if (cfg->use_offsets) {
+    a.offsets = d_offsets_or_lengths;
+    a.off64 = cfg->offset_bits == 64;
+  } else {
+    std::lock_guard<std::mutex> lk(g_mu);
+    DeviceScratch* s;
+    if (int rc = get_scratch(&s)) return rc;
+    if (s->offsets_cap < output_size + 1) {
+      // grow-only; the old buffer may still be read by an enqueued kernel
+      HIP_TRY(hipStreamSynchronize(stream));
+      if (s->offsets) HIP_TRY(hipFree(s->offsets));
+      s->offsets = nullptr;
+      s->offsets_cap = 0;
+      const int64_t cap = std::max<int64_t>(output_size + 1, 4096);
+      HIP_TRY(hipMalloc((void**)&s->offsets, sizeof(int64_t) * cap));
+      s->offsets_cap = cap;
+    }
+    HIP_TRY(launch_lengths_to_offsets(d_offsets_or_lengths, cfg->offset_bits == 64, output_size, s->offsets, stream));
+    a.offsets = s->offsets;
+    a.off64 = 1;
+  }
+  HIP_TRY(launch_lookup(a, cfg->index_bits == 64, stream));
+  return 0;
+}
+
+int fbgemm_amd_spmdm_run(
+    const fbgemm_amd_spmdm_config* cfg, int64_t output_size, int64_t index_size,
+    int64_t data_size, const void* d_input, const void* d_indices,
+    const void* d_offsets_or_lengths, const float* d_weights, void* d_out,
+    const int32_t* d_remap, void* stream) {
+  Status* st;
+  {
+    std::lock_guard<std::mutex> lk(g_mu);
+    DeviceScratch* s;
+    if (int rc = get_scratch(&s)) return rc;
+    st = s->status;
+  }
+  if (int rc = fbgemm_amd_status_clear(st, stream)) return rc;
+  if (int rc = fbgemm_amd_spmdm_launch(cfg, output_size, index_size, data_size, d_input, d_indices,
+                                      d_offsets_or_lengths, d_weights, d_out, d_remap, st, stream))
+    return rc;
+  int32_t bits = 0;
+  if (int rc = fbgemm_amd_status_read(st, stream, &bits, nullptr)) return rc;
+  return bits == 0 ? 1 : 0;
+}
+
+} // extern "C"
+
+// ---- table-batched forward ---------------------------------------------------
+
+struct fbgemm_amd_tbe_plan {
+  int32_t T = 0;
+  int64_t total_D = 0;
+  int64_t row_alignment = 16;
+  std::vector<TableDesc> tables; // host copy
+  TableDesc* d_tables = nullptr;
+  int device = 0;
+  // per-B work lists
+  struct Work {
+    WaveWork* d_work = nullptr;
+    int64_t num_waves = 0;
+  };
+  std::map<int32_t, Work> work;
+  std::mutex mu;
+};
+
+extern "C" {
+
+int fbgemm_amd_tbe_plan_create(
+    fbgemm_amd_tbe_plan** out, int32_t T, const int64_t* weights_offsets,
+    const uint8_t* weights_tys, const int32_t* D_offsets, const int32_t* placements,
+    int64_t dev_bytes, int64_t uvm_bytes, int64_t row_alignment) {
+  if (!out || T <= 0 || !weights_offsets || !weights_tys || !D_offsets)
+    return fail(FBGEMM_AMD_E_ARG, "bad plan arguments");
+  if (row_alignment <= 0) row_alignment = 1;
+  auto plan = new fbgemm_amd_tbe_plan();
+  plan->T = T;
+  plan->total_D = D_offsets[T];
+  plan->row_alignment = row_alignment;
+  plan->tables.resize(T);
+  HIP_TRY(hipGetDevice(&plan->device));
+
+  // Rows per table are inferred from the distance to the next distinct
+  // offset in the same buffer, the last table being bounded by the buffer
+  // (embedding_forward_quantized_cpu_template.cpp:330-341,372-380).
+  std::vector<int64_t> phys[2];
+  for (int t = 0; t < T; ++t) phys[(placements && placements[t] != 0) ? 1 : 0].push_back(weights_offsets[t]);
+  for (auto& p : phys) {
+    std::sort(p.begin(), p.end());
+    p.erase(std::unique(p.begin(), p.end()), p.end());
+  }
+  for (int t = 0; t < T; ++t) {
+    TableDesc& d = plan->tables[t];
+    memset(&d, 0, sizeof(d));
+    d.ty = weights_tys[t];
+    if (type_bits(d.ty) == 0) {
+      delete plan;
+      return fail(FBGEMM_AMD_E_UNSUPPORTED, "table %d: weight type %d is not supported", t, d.ty);
+    }
+    d.D = D_offsets[t + 1] - D_offsets[t];
+    if (d.D <= 0) {
+      delete plan;
+      return fail(FBGEMM_AMD_E_ARG, "table %d: D_offsets must increase", t);
+    }
+    d.out_col = D_offsets[t];
+    d.placement = (placements && placements[t] != 0) ? 1 : 0;
+    d.weights_offset = weights_offsets[t];
+    d.row_stride = fbgemm_amd_padded_row_size_in_bytes(d.D, d.ty, (int32_t)row_alignment, 4);
+    const auto& p = phys[d.placement];
+    auto it = std::upper_bound(p.begin(), p.end(), d.weights_offset);
+    const int64_t next = it != p.end() ? *it : (d.placement ? uvm_bytes : dev_bytes);
+    d.num_rows = std::max<int64_t>(0, (next - d.weights_offset) / d.row_stride);
+    d.skip_minus_one = 1;
+    const bool q = quantised(d.ty);
+    d.sb_fp32 = 0;
+    d.sb_off = 0;
+    d.data_off = q ? 4 : 0;
+    // weights buffers come from hipMalloc / torch: at least 256-byte aligned
+    plan_lanes(d, 0, plan->total_D, q);
+  }
+  HIP_TRY(hipMalloc((void**)&plan->d_tables, sizeof(TableDesc) * T));
+  HIP_TRY(hipMemcpy(plan->d_tables, plan->tables.data(), sizeof(TableDesc) * T, hipMemcpyHostToDevice));
+  *out = plan;
+  return 0;
+}
+
+void fbgemm_amd_tbe_plan_destroy(fbgemm_amd_tbe_plan* plan) {
+  if (!plan) return;
+  (void)hipDeviceSynchronize();
+  for (auto& kv : plan->work)
+    if (kv.second.d_work) (void)hipFree(kv.second.d_work);
+  if (plan->d_tables) (void)hipFree(plan->d_tables);
+  delete plan;
+}
+
+int64_t fbgemm_amd_tbe_plan_num_rows(const fbgemm_amd_tbe_plan* plan, int32_t t) {
+  return (plan && t >= 0 && t < plan->T) ? plan->tables[t].num_rows : -1;
+}
+int64_t fbgemm_amd_tbe_plan_row_bytes(const fbgemm_amd_tbe_plan* plan, int32_t t) {
+  return (plan && t >= 0 && t < plan->T) ? plan->tables[t].row_stride : -1;
+}
+
+int fbgemm_amd_tbe_forward(
+    fbgemm_amd_tbe_plan* plan, const void* d_dev_weights, const void* d_uvm_weights,
+    const void* d_indices, const void* d_offsets, int32_t index_bits,
+    int64_t indices_numel, int64_t offsets_numel, int32_t pooling_mode,
+    const float* d_indice_weights, int32_t output_ty, void* d_output, void* d_status,
+    void* stream_) {
+  if (!plan) return fail(FBGEMM_AMD_E_ARG, "plan is null");
+  if (index_bits != 32 && index_bits != 64) return fail(FBGEMM_AMD_E_ARG, "index_bits must be 32 or 64");
+  if (output_ty != ST_FP32 && output_ty != ST_FP16 && output_ty != ST_BF16)
+    return fail(FBGEMM_AMD_E_UNSUPPORTED, "output type %d is not supported", output_ty);
+  if (pooling_mode != FBGEMM_AMD_POOL_SUM && pooling_mode != FBGEMM_AMD_POOL_MEAN)
+    return fail(FBGEMM_AMD_E_UNSUPPORTED, "pooling mode %d is not supported", pooling_mode);
+  if (!d_status) return fail(FBGEMM_AMD_E_ARG, "d_status is null");
+  if (offsets_numel < 1 || (offsets_numel - 1) % plan->T != 0)
+    return fail(FBGEMM_AMD_E_ARG, "offsets must hold T*B+1 entries");
+  const int64_t B64 = (offsets_numel - 1) / plan->T;
+  if (B64 == 0) return 0;
+  if (B64 > 0x7fffffffLL) return fail(FBGEMM_AMD_E_ARG, "B exceeds 2^31-1");
+  const int32_t B = (int32_t)B64;
+  if (!d_offsets || !d_output || (indices_numel > 0 && !d_indices)) return fail(FBGEMM_AMD_E_ARG, "null data pointer");
+  hipStream_t stream = (hipStream_t)stream_;
+
+  fbgemm_amd_tbe_plan::Work w;
+  {
+    std::lock_guard<std::mutex> lk(plan->mu);
+    auto it = plan->work.find(B);
+    if (it == plan->work.end()) {
+      std::vector<WaveWork> list;
+      for (int t = 0; t < plan->T; ++t) {
+        const int G = 64 / plan->tables[t].lanes;
+        for (int32_t fb = 0; fb < B; fb += G) list.push_back(WaveWork{t, fb});
+      }
+      fbgemm_amd_tbe_plan::Work nw;
+      nw.num_waves = (int64_t)list.size();
+      HIP_TRY(hipMalloc((void**)&nw.d_work, sizeof(WaveWork) * list.size()));
+      HIP_TRY(hipMemcpy(nw.d_work, list.data(), sizeof(WaveWork) * list.size(), hipMemcpyHostToDevice));
+      it = plan->work.emplace(B, nw).first;
+    }
+    w = it->second;
+  }
+
+  LookupArgs a;
+  memset(&a, 0, sizeof(a));
+  a.tables = plan->d_tables;
+  a.weights[0] = (const uint8_t*)d_dev_weights;
+  a.weights[1] = (const uint8_t*)d_uvm_weights;
+  a.indices = d_indices;
+  a.offsets = d_offsets;
+  a.off64 = index_bits == 64;
+  a.sample_weights = d_indice_weights;
+  a.out = d_output;
+  a.out_stride = plan->total_D;
+  a.index_size = indices_numel;
+  a.work = w.d_work;
+  a.num_waves = w.num_waves;
+  a.B = B;
+  a.T = plan->T;
+  a.out_ty = output_ty;
+  a.normalize = pooling_mode == FBGEMM_AMD_POOL_MEAN;
+  a.xcd_swizzle = xcd_swizzle_default();
+  a.check_total = 0;
+  a.out_aligned = (uintptr_t)d_output % 16 == 0;
+  a.status = (Status*)d_status;
+  HIP_TRY(launch_lookup(a, index_bits == 64, stream));
+  return 0;
+}
+
+int fbgemm_amd_pruned_array_lookup(
+    const void* d_indices, const void* d_offsets, int32_t index_bits, int64_t offsets_numel,
+    const void* d_remap, int32_t remap_bits, const int64_t* d_remap_offsets, int32_t T,
+    void* d_dense, void* stream) {
+  if (T <= 0 || offsets_numel < 1 || (offsets_numel - 1) % T != 0) return fail(FBGEMM_AMD_E_ARG, "offsets must hold T*B+1 entries");
+  if ((index_bits != 32 && index_bits != 64) || (remap_bits != 32 && remap_bits != 64))
+    return fail(FBGEMM_AMD_E_ARG, "index_bits/remap_bits must be 32 or 64");
+  const int64_t B = (offsets_numel - 1) / T;
+  if (B == 0) return 0;
+  if (!d_indices || !d_offsets || !d_remap_offsets || !d_dense) return fail(FBGEMM_AMD_E_ARG, "null data pointer");
+  HIP_TRY(launch_pruned_array_lookup(d_indices, d_offsets, index_bits == 64, d_remap, remap_bits == 64,
+                                     d_remap_offsets, (int32_t)B, T, d_dense, (hipStream_t)stream));
+  return 0;
+}
+
+} // extern "C"

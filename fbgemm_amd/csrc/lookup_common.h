@@ -1,0 +1,92 @@
+// Shared between the host-side launch code and the gfx950 kernels.
+#pragma once
+#include <stdint.h>
+
+namespace fbgemm_amd {
+
+// Row element types, numbered like the reference's SparseType
+// (fbgemm_gpu/include/fbgemm_gpu/embedding_common.h:20-32).
+enum : int32_t {
+  ST_FP32 = 0,
+  ST_FP16 = 1,
+  ST_INT8 = 2,
+  ST_INT4 = 3,
+  ST_INT2 = 4,
+  ST_BF16 = 5,
+};
+
+// Bits of the status word a lookup ORs in when it meets an input the reference
+// would reject (src/RefImplementations.cc:1294-1306,1346).
+enum : int32_t {
+  ERR_INDEX_OUT_OF_RANGE = 1, // idx < 0 (and not a skipped -1) or idx >= rows
+  ERR_BAG_OVERRUN = 2,        // a bag ends past index_size / past the index array
+  ERR_LENGTH_MISMATCH = 4,    // sum of bag lengths != index_size
+  ERR_NEGATIVE_LENGTH = 8,    // offsets decrease (the reference's result is then undefined)
+};
+
+// Device status block: word 0 = OR of ERR_* bits, words 2..3 = the smallest
+// position (into the index array) of an out-of-range index, as an int64
+// minimum so that the first offender in index order wins deterministically.
+struct Status {
+  int32_t bits;
+  int32_t pad;
+  unsigned long long first_bad_pos;
+};
+
+// How a wave walks one table. Filled on the host from the table's element
+// type, dimension, stride and alignment.
+struct TableDesc {
+  int64_t weights_offset; // byte offset of row 0 inside the weights buffer
+  int64_t row_stride;     // bytes between consecutive rows
+  int64_t num_rows;       // exclusive bound for a valid physical row id
+  int32_t D;              // elements per row
+  int32_t out_col;        // first output column of this table's block
+  int32_t ty;             // ST_*
+  int32_t vb;             // bytes each lane loads per row and pass: 1, 2, 4 or 16
+  int32_t sb_off;         // byte offset of (scale, bias) inside a row
+  int32_t data_off;       // byte offset of the element data inside a row
+  int32_t sb_fp32;        // 1: scale/bias are two floats, 0: two halfs
+  int32_t lanes;          // lanes cooperating on one bag (1..64)
+  int32_t passes;         // column passes when a row exceeds lanes * vb bytes
+  int32_t placement;      // which of the two weights buffers holds the table
+  int32_t data_bytes;     // bytes of element data per row (unpadded)
+  int32_t skip_minus_one; // 1: an index of -1 is a pruned row and is skipped
+  int32_t vec_store;      // bit 0 / bit 1: every lane's output run is aligned for whole-run
+                          // vector stores with 4-byte / 2-byte output elements
+  int32_t reserved;
+};
+
+// One entry per workgroup wave slot: which table and which first bag.
+struct WaveWork {
+  int32_t table;
+  int32_t first_bag;
+};
+
+struct LookupArgs {
+  const TableDesc* tables;   // device array, or nullptr when `single` is used
+  TableDesc single;
+  const uint8_t* weights[2]; // buffers selected by TableDesc::placement
+  const void* indices;
+  const void* offsets;       // T*B+1 offsets ((table, bag) order)
+  const float* sample_weights; // nullptr: unweighted
+  const int32_t* remap;      // logical -> physical row table, or nullptr
+  int64_t remap_rows;        // bound for logical ids when remap != nullptr
+  void* out;
+  int64_t out_stride;        // elements between consecutive bags' outputs
+  int64_t index_size;        // entries the index array holds for this call
+  const WaveWork* work;      // per-wave work list, or nullptr: single table, dense mapping
+  int64_t num_waves;         // waves with work
+  int32_t B;                 // bags per table
+  int32_t T;
+  int32_t out_ty;            // ST_FP32, ST_FP16 or ST_BF16
+  int32_t off64;             // offsets are int64 (else int32)
+  int32_t normalize;         // mean pooling: scale by 1/len, len counting skipped rows
+  int32_t positional;        // weight of entry i of a bag is sample_weights[i]
+  int32_t xcd_swizzle;       // remap block ids so that each XCD walks contiguous work
+  int32_t check_total;       // single-table call: positions are relative to offsets[0] and
+                             // offsets[last] - offsets[0] must equal index_size
+  int32_t out_aligned;       // `out` is 16-byte aligned (vector stores allowed)
+  Status* status;
+};
+
+} // namespace fbgemm_amd

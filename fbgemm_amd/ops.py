@@ -1,0 +1,315 @@
+"""Python face of the C ABI, shaped like the reference's own entry points.
+
+* ``generate_embedding_spmdm*`` mirror the kernel factories of
+  include/fbgemm/FbgemmEmbedding.h:65-262: fix the configuration once, get back
+  a callable with the ``EmbeddingSpMDMKernelSignature`` argument list that
+  returns the reference's ``bool``.
+* ``int_nbit_split_embedding_codegen_lookup_function`` and
+  ``pruned_array_lookup`` mirror the operators registered in
+  fbgemm_gpu/codegen/inference/embedding_forward_quantized_host_cpu.cpp:310-347.
+
+All tensors are device tensors (torch is only the owner of HBM and streams).
+Everything runs in the HIP library; nothing here computes.
+"""
+import ctypes as C
+
+import torch
+
+from . import _lib
+from ._lib import SpmdmConfig, check
+
+FP32, FP16, INT8, INT4, INT2, BF16 = 0, 1, 2, 3, 4, 5
+POOL_SUM, POOL_MEAN, POOL_NONE = 0, 1, 2
+
+_OUT_TORCH = {FP32: torch.float32, FP16: torch.float16, BF16: torch.bfloat16}
+_TORCH_OUT = {v: k for k, v in _OUT_TORCH.items()}
+
+ERR_INDEX_OUT_OF_RANGE, ERR_BAG_OVERRUN, ERR_LENGTH_MISMATCH, ERR_NEGATIVE_LENGTH = 1, 2, 4, 8
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def _bits(t):
+    if t.dtype == torch.int64:
+        return 64
+    if t.dtype == torch.int32:
+        return 32
+    raise TypeError(f"indices/offsets must be int32 or int64, got {t.dtype}")
+
+
+def _require_cuda(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise ValueError("fbgemm_amd ops take device tensors; there is no CPU path")
+
+
+class Status:
+    """A device status block (see include/fbgemm_amd.h)."""
+
+    def __init__(self, device=None):
+        self.buf = torch.zeros(4, dtype=torch.int32, device=device or "cuda")
+        self.clear()
+
+    def clear(self):
+        check(_lib.lib().fbgemm_amd_status_clear(_ptr(self.buf), _stream()))
+
+    def read(self):
+        """Synchronizes. Returns (bits, first_bad_pos)."""
+        bits, pos = C.c_int32(0), C.c_int64(-1)
+        check(_lib.lib().fbgemm_amd_status_read(_ptr(self.buf), _stream(), C.byref(bits), C.byref(pos)))
+        return bits.value, pos.value
+
+
+def _make_kernel(weight_ty, block_size, normalize_by_lengths, is_weight_positional, use_offsets,
+                 output_stride, input_stride, scale_bias_last, output_ty, has_weight, sparse):
+    def kernel(output_size, index_size, data_size, input, indices, offsets_or_lengths, weights, out,
+               compressed_indices_table=None, status=None):
+        _require_cuda(input, indices, offsets_or_lengths, weights, out, compressed_indices_table)
+        if sparse and compressed_indices_table is None:
+            raise ValueError("row-wise-sparse kernels need compressed_indices_table")
+        if has_weight != (weights is not None):
+            # the reference's generated code is specialised on has_weight; a mismatch is a caller bug
+            raise ValueError("weights must be given exactly when has_weight was set")
+        if weights is not None and weights.dtype != torch.float32:
+            raise TypeError("weights must be float32")
+        if compressed_indices_table is not None and compressed_indices_table.dtype != torch.int32:
+            raise TypeError("compressed_indices_table must be int32")
+        cfg = SpmdmConfig(
+            weight_ty=weight_ty, output_ty=output_ty, index_bits=_bits(indices),
+            offset_bits=_bits(offsets_or_lengths), block_size=block_size,
+            output_stride=output_stride, input_stride=input_stride,
+            normalize_by_lengths=int(normalize_by_lengths),
+            is_weight_positional=int(is_weight_positional), use_offsets=int(use_offsets),
+            scale_bias_last=int(scale_bias_last))
+        lib = _lib.lib()
+        if status is not None:
+            check(lib.fbgemm_amd_spmdm_launch(
+                C.byref(cfg), output_size, index_size, data_size, _ptr(input), _ptr(indices),
+                _ptr(offsets_or_lengths), _ptr(weights), _ptr(out), _ptr(compressed_indices_table),
+                _ptr(status.buf), _stream()))
+            return None
+        rc = check(lib.fbgemm_amd_spmdm_run(
+            C.byref(cfg), output_size, index_size, data_size, _ptr(input), _ptr(indices),
+            _ptr(offsets_or_lengths), _ptr(weights), _ptr(out), _ptr(compressed_indices_table),
+            _stream()))
+        return rc == 1
+
+    return kernel
+
+
+def generate_embedding_spmdm_with_strides(
+        in_ty, block_size, has_weight, normalize_by_lengths, prefetch=16,
+        is_weight_positional=False, use_offsets=True, output_stride=-1, input_stride=-1,
+        scale_bias_last=True, no_bag=False, is_bf16_out=False, is_bf16_in=False, out_ty=FP32):
+    """GenerateEmbeddingSpMDMWithStrides (FbgemmEmbedding.h:94-117). ``in_ty`` is
+    INT8 (fused 8-bit rows), FP16 or FP32; ``out_ty`` FP32 or FP16 (BF16 via
+    ``is_bf16_out``). ``prefetch`` is accepted and ignored: the GPU hides
+    latency with loads in flight, not software prefetch."""
+    if no_bag:
+        raise NotImplementedError("no_bag (sequence output) is not on this path")
+    if in_ty == FP16 and is_bf16_in:
+        in_ty = BF16
+    if is_bf16_out:
+        out_ty = BF16
+    return _make_kernel(in_ty, block_size, normalize_by_lengths, is_weight_positional, use_offsets,
+                        output_stride, input_stride, scale_bias_last, out_ty, has_weight, False)
+
+
+def generate_embedding_spmdm(in_ty, block_size, has_weight, normalize_by_lengths, prefetch=16,
+                             is_weight_positional=False, use_offsets=True, is_bf16_out=False,
+                             is_bf16_in=False, out_ty=FP32):
+    """GenerateEmbeddingSpMDM (FbgemmEmbedding.h:65-84)."""
+    return generate_embedding_spmdm_with_strides(
+        in_ty, block_size, has_weight, normalize_by_lengths, prefetch, is_weight_positional,
+        use_offsets, -1, -1, True, False, is_bf16_out, is_bf16_in, out_ty)
+
+
+def generate_embedding_spmdm_nbit_with_strides(
+        input_bit_rate, block_size, has_weight, normalize_by_lengths, prefetch=16,
+        is_weight_positional=False, use_offsets=True, output_stride=-1, input_stride=-1,
+        scale_bias_last=True, is_bf16_out=False, no_bag=False, output_bit_rate=-1, out_ty=FP32):
+    """GenerateEmbeddingSpMDMNBitWithStrides (FbgemmEmbedding.h:151-174)."""
+    if input_bit_rate not in (2, 4):
+        raise ValueError("input_bit_rate must be 2 or 4")
+    if no_bag:
+        raise NotImplementedError("no_bag (sequence output) is not on this path")
+    if is_bf16_out:
+        out_ty = BF16
+    return _make_kernel(INT4 if input_bit_rate == 4 else INT2, block_size, normalize_by_lengths,
+                        is_weight_positional, use_offsets, output_stride, input_stride,
+                        scale_bias_last, out_ty, has_weight, False)
+
+
+def generate_embedding_spmdm_nbit(bit_rate, block_size, has_weight, normalize_by_lengths, prefetch=16,
+                                  is_weight_positional=False, use_offsets=True, out_ty=FP32):
+    """GenerateEmbeddingSpMDMNBit (FbgemmEmbedding.h:124-140)."""
+    return generate_embedding_spmdm_nbit_with_strides(
+        bit_rate, block_size, has_weight, normalize_by_lengths, prefetch, is_weight_positional,
+        use_offsets, out_ty=out_ty)
+
+
+def generate_embedding_spmdm_rowwise_sparse(in_ty, block_size, has_weight, normalize_by_lengths,
+                                            prefetch=16, is_weight_positional=False, use_offsets=True):
+    """GenerateEmbeddingSpMDMRowWiseSparse (FbgemmEmbedding.h:229-243): the kernel
+    takes ``compressed_indices_table`` as a trailing argument and writes fp32."""
+    return _make_kernel(in_ty, block_size, normalize_by_lengths, is_weight_positional, use_offsets,
+                        -1, -1, True, FP32, has_weight, True)
+
+
+def generate_embedding_spmdm_nbit_rowwise_sparse(bit_rate, block_size, has_weight, normalize_by_lengths,
+                                                 prefetch=16, is_weight_positional=False,
+                                                 use_offsets=True):
+    """GenerateEmbeddingSpMDMNBitRowWiseSparse (FbgemmEmbedding.h:250-262)."""
+    if bit_rate not in (2, 4):
+        raise ValueError("bit_rate must be 2 or 4")
+    return _make_kernel(INT4 if bit_rate == 4 else INT2, block_size, normalize_by_lengths,
+                        is_weight_positional, use_offsets, -1, -1, True, FP32, has_weight, True)
+
+
+# ---- table-batched forward -------------------------------------------------
+
+
+class TbePlan:
+    """Owner of a fbgemm_amd_tbe_plan handle."""
+
+    def __init__(self, weights_offsets, weights_tys, D_offsets, weights_placements,
+                 dev_weights_bytes, uvm_weights_bytes, row_alignment):
+        wo = weights_offsets.detach().to("cpu", torch.int64).contiguous()
+        wt = weights_tys.detach().to("cpu", torch.uint8).contiguous()
+        do = D_offsets.detach().to("cpu", torch.int32).contiguous()
+        wp = weights_placements.detach().to("cpu", torch.int32).contiguous()
+        self.T = do.numel() - 1
+        self.total_D = int(do[-1])
+        handle = C.c_void_p()
+        check(_lib.lib().fbgemm_amd_tbe_plan_create(
+            C.byref(handle), self.T, _ptr(wo), _ptr(wt), _ptr(do), _ptr(wp),
+            dev_weights_bytes, uvm_weights_bytes, row_alignment))
+        self.handle = handle
+
+    def num_rows(self, t):
+        return _lib.lib().fbgemm_amd_tbe_plan_num_rows(self.handle, t)
+
+    def row_bytes(self, t):
+        return _lib.lib().fbgemm_amd_tbe_plan_row_bytes(self.handle, t)
+
+    def __del__(self):
+        h, self.handle = getattr(self, "handle", None), None
+        if h:
+            try:
+                _lib.lib().fbgemm_amd_tbe_plan_destroy(h)
+            except Exception:
+                pass
+
+
+_plans = {}
+
+
+def _plan_for(dev_weights, uvm_weights, weights_placements, weights_offsets, weights_tys, D_offsets,
+              row_alignment):
+    # The operator receives its metadata as device tensors on every call; the
+    # host copy a plan needs is made once per distinct set of tensors.
+    key = (weights_offsets.data_ptr(), weights_tys.data_ptr(), D_offsets.data_ptr(),
+           weights_placements.data_ptr(), weights_offsets._version, D_offsets._version,
+           weights_tys._version, D_offsets.numel(), dev_weights.numel(), uvm_weights.numel(),
+           row_alignment)
+    plan = _plans.get(key)
+    if plan is None:
+        plan = TbePlan(weights_offsets, weights_tys, D_offsets, weights_placements,
+                       dev_weights.numel(), uvm_weights.numel(), row_alignment)
+        if len(_plans) > 64:
+            _plans.clear()
+        _plans[key] = plan
+    return plan
+
+
+def int_nbit_split_embedding_codegen_lookup_function(
+        dev_weights, uvm_weights, weights_placements, weights_offsets, weights_tys, D_offsets,
+        total_D, max_int2_D, max_int4_D, max_int8_D, max_float16_D, max_float32_D, indices,
+        offsets, pooling_mode, indice_weights=None, output_dtype=FP16, lxu_cache_weights=None,
+        lxu_cache_locations=None, row_alignment=None, max_float8_D=0, fp8_exponent_bits=-1,
+        fp8_exponent_bias=-1, status=None, plan=None):
+    """Same arguments, in the same order, as the reference operator
+    (embedding_forward_quantized_host_cpu.cpp:316-318). Returns [B, total_D].
+
+    Input errors raise like the CPU operator does, unless ``status`` is given:
+    then the call stays asynchronous and the caller reads the block later."""
+    _require_cuda(dev_weights, indices, offsets, indice_weights)
+    if pooling_mode == POOL_NONE:
+        raise NotImplementedError("PoolingMode.NONE (sequence output) is not on this path")
+    if max_float8_D:
+        raise NotImplementedError("FP8 tables are not on this path")
+    if lxu_cache_locations is not None and lxu_cache_locations.numel() > 0:
+        raise NotImplementedError("the LXU cache is not on this path: tables are resident in HBM")
+    if output_dtype not in _OUT_TORCH:
+        raise NotImplementedError(f"output_dtype {output_dtype} is not on this path")
+    if offsets.dtype != indices.dtype:
+        offsets = offsets.to(indices.dtype)  # as embedding_forward_quantized_host_cpu.cpp:111-113
+    if indice_weights is not None and indice_weights.numel() == 0:
+        indice_weights = None
+    if indice_weights is not None and indice_weights.dtype != torch.float32:
+        indice_weights = indice_weights.float()  # embedding_forward_quantized_host.cpp:345
+    if row_alignment is None:
+        row_alignment = 16  # the GPU operator's default (embedding_forward_quantized_host.cpp:310)
+    if plan is None:
+        plan = _plan_for(dev_weights, uvm_weights, weights_placements, weights_offsets, weights_tys,
+                         D_offsets, row_alignment)
+    T = plan.T
+    if total_D != plan.total_D:
+        raise ValueError(f"total_D {total_D} does not match D_offsets[-1] {plan.total_D}")
+    B = (offsets.numel() - 1) // T
+    out = torch.empty((B, total_D), dtype=_OUT_TORCH[output_dtype], device=dev_weights.device)
+    if B == 0:
+        return out
+    own = status is None
+    st = Status(dev_weights.device) if own else status
+    check(_lib.lib().fbgemm_amd_tbe_forward(
+        plan.handle, _ptr(dev_weights), _ptr(uvm_weights), _ptr(indices.contiguous()),
+        _ptr(offsets.contiguous()), _bits(indices), indices.numel(), offsets.numel(), pooling_mode,
+        _ptr(indice_weights), output_dtype, _ptr(out), _ptr(st.buf), _stream()))
+    if own:
+        bits, pos = st.read()
+        if bits:
+            _raise_embedding_error(bits, pos, indices, offsets, plan, B)
+    return out
+
+
+def _raise_embedding_error(bits, pos, indices, offsets, plan, B):
+    # wording follows report_embedding_error (fbgemm_gpu/include/fbgemm_gpu/utils/cpu_utils.h:25-52)
+    if bits & ERR_INDEX_OUT_OF_RANGE and pos >= 0:
+        idx = int(indices[pos])
+        off = offsets.cpu()
+        t = int(torch.searchsorted(off[::B].contiguous(), torch.tensor([pos], dtype=off.dtype), right=True)) - 1
+        t = max(0, min(plan.T - 1, t))
+        raise RuntimeError(
+            f"Index {pos} is out of bounds: {idx}, range 0 to {plan.num_rows(t)} (table {t})")
+    raise RuntimeError(f"embedding lookup rejected its inputs (status bits {bits:#x})")
+
+
+def pruned_array_lookup(indices, offsets, index_remappings, index_remappings_offsets):
+    """pruned_array_lookup (embedding_forward_quantized_host_cpu.cpp:343-346)."""
+    _require_cuda(indices, offsets, index_remappings, index_remappings_offsets)
+    if indices.dtype != offsets.dtype:
+        raise TypeError("indices and offsets must have the same dtype")
+    T = index_remappings_offsets.numel() - 1
+    dense = torch.empty_like(indices)
+    ro = index_remappings_offsets.to(torch.int64).contiguous()
+    check(_lib.lib().fbgemm_amd_pruned_array_lookup(
+        _ptr(indices.contiguous()), _ptr(offsets.contiguous()), _bits(indices), offsets.numel(),
+        _ptr(index_remappings), _bits(index_remappings), _ptr(ro), T, _ptr(dense), _stream()))
+    return dense
+
+
+def padded_row_size_in_bytes(dim, weight_ty, row_alignment, scale_bias_bytes=4):
+    """nbit::padded_row_size_in_bytes (embedding_common.h:217-225)."""
+    return _lib.lib().fbgemm_amd_padded_row_size_in_bytes(dim, weight_ty, row_alignment, scale_bias_bytes)
+
+
+def unpadded_row_size_in_bytes(dim, weight_ty, scale_bias_bytes=4):
+    """nbit::unpadded_row_size_in_bytes (embedding_common.h:189-215)."""
+    return _lib.lib().fbgemm_amd_unpadded_row_size_in_bytes(dim, weight_ty, scale_bias_bytes)

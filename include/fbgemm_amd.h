@@ -1,0 +1,182 @@
+/*
+ * fbgemm_amd -- C ABI of the MI355X (gfx950) quantized embedding-bag library.
+ *
+ * Every data pointer named d_* is a DEVICE pointer (HBM). `stream` is a
+ * hipStream_t passed as void* (NULL = the default stream). Launch calls are
+ * asynchronous: they enqueue on `stream` and return. Nothing is allocated per
+ * call except where a function says so.
+ *
+ * Return values: 0 = enqueued / done, < 0 = FBGEMM_AMD_E_* (bad argument or a
+ * HIP error). Input errors that the reference reports by returning false
+ * (index out of range, bag overrun, length mismatch) are detected ON THE
+ * DEVICE and recorded in a 16-byte status block the caller owns; read it back
+ * with fbgemm_amd_status_read (this is the only call that synchronizes).
+ */
+#ifndef FBGEMM_AMD_H_
+#define FBGEMM_AMD_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Element types; values follow the reference's SparseType
+ * (fbgemm_gpu/include/fbgemm_gpu/embedding_common.h:20-32). */
+enum {
+  FBGEMM_AMD_FP32 = 0,
+  FBGEMM_AMD_FP16 = 1,
+  FBGEMM_AMD_INT8 = 2,
+  FBGEMM_AMD_INT4 = 3,
+  FBGEMM_AMD_INT2 = 4,
+  FBGEMM_AMD_BF16 = 5
+};
+
+/* Pooling modes (embedding_common.h:34). NONE is not on this path. */
+enum { FBGEMM_AMD_POOL_SUM = 0, FBGEMM_AMD_POOL_MEAN = 1 };
+
+/* Error codes returned by the entry points. */
+enum {
+  FBGEMM_AMD_OK = 0,
+  FBGEMM_AMD_E_ARG = -1,      /* invalid argument combination */
+  FBGEMM_AMD_E_HIP = -2,      /* a HIP runtime call failed; see fbgemm_amd_last_error */
+  FBGEMM_AMD_E_UNSUPPORTED = -3
+};
+
+/* Bits of the device status word (what made the reference return false). */
+enum {
+  FBGEMM_AMD_ERR_INDEX_OUT_OF_RANGE = 1,
+  FBGEMM_AMD_ERR_BAG_OVERRUN = 2,
+  FBGEMM_AMD_ERR_LENGTH_MISMATCH = 4,
+  FBGEMM_AMD_ERR_NEGATIVE_LENGTH = 8
+};
+
+#define FBGEMM_AMD_STATUS_BYTES 16
+
+/* Human-readable text of the last FBGEMM_AMD_E_* on this thread. */
+const char* fbgemm_amd_last_error(void);
+
+/* Library version, "major.minor". */
+const char* fbgemm_amd_version(void);
+
+/* ---- status block ------------------------------------------------------- */
+
+/* Reset a status block (launches a one-thread fill kernel; capture-safe). */
+int fbgemm_amd_status_clear(void* d_status, void* stream);
+
+/* Synchronize `stream`, copy the block back. *bits = OR of FBGEMM_AMD_ERR_*;
+ * *first_bad_pos = smallest position in the index array holding an
+ * out-of-range index, or -1. Either out pointer may be NULL. */
+int fbgemm_amd_status_read(const void* d_status, void* stream, int32_t* bits, int64_t* first_bad_pos);
+
+/* ---- single-table pooled lookup ----------------------------------------- *
+ *
+ * Replaces the kernels returned by fbgemm::GenerateEmbeddingSpMDMWithStrides,
+ * GenerateEmbeddingSpMDMNBitWithStrides, GenerateEmbeddingSpMDMRowWiseSparse
+ * and GenerateEmbeddingSpMDMNBitRowWiseSparse
+ * (include/fbgemm/FbgemmEmbedding.h:94-117,151-174,229-262): the config holds
+ * what those factories fix at generation time, the launch takes what
+ * EmbeddingSpMDMKernelSignature::Type takes (FbgemmEmbedding.h:41-49,211-221).
+ */
+typedef struct fbgemm_amd_spmdm_config {
+  int32_t weight_ty;            /* FBGEMM_AMD_INT8/INT4/INT2/FP16/BF16/FP32 */
+  int32_t output_ty;            /* FBGEMM_AMD_FP32/FP16/BF16 */
+  int32_t index_bits;           /* 32 or 64 */
+  int32_t offset_bits;          /* 32 or 64 */
+  int64_t block_size;           /* elements per row (D) */
+  int64_t output_stride;        /* elements between output rows; -1 = block_size */
+  int64_t input_stride;         /* storage elements between table rows (bytes for the
+                                   integer formats, halfs for fp16/bf16, floats for
+                                   fp32); -1 = densely packed rows */
+  int32_t normalize_by_lengths; /* mean pooling */
+  int32_t is_weight_positional; /* weights[i] belongs to entry i of every bag */
+  int32_t use_offsets;          /* 1: offsets[output_size+1]; 0: lengths[output_size] */
+  int32_t scale_bias_last;      /* 1: scale/bias after the row data (fp32 pair for
+                                   INT8, fp16 pair for INT4/INT2); 0: fp16 pair in
+                                   front of the data, and index -1 is skipped */
+} fbgemm_amd_spmdm_config;
+
+/* Enqueue one pooled lookup. d_weights may be NULL (unweighted).
+ * d_compressed_indices_table, when non-NULL, selects the row-wise-sparse
+ * variant: data_size then bounds the LOGICAL ids and the table maps them to
+ * physical rows (-1 = pruned). d_status must be a cleared status block.
+ * With use_offsets == 0 the call makes a prefix sum of the lengths into a
+ * library-owned scratch buffer first (grown with hipMalloc when too small). */
+int fbgemm_amd_spmdm_launch(
+    const fbgemm_amd_spmdm_config* cfg, int64_t output_size, int64_t index_size,
+    int64_t data_size, const void* d_input, const void* d_indices,
+    const void* d_offsets_or_lengths, const float* d_weights, void* d_out,
+    const int32_t* d_compressed_indices_table, void* d_status, void* stream);
+
+/* Same, synchronous, with the reference's return convention: 1 = true,
+ * 0 = false (the inputs were rejected; output unspecified), < 0 = API error.
+ * Uses a library-owned status block. */
+int fbgemm_amd_spmdm_run(
+    const fbgemm_amd_spmdm_config* cfg, int64_t output_size, int64_t index_size,
+    int64_t data_size, const void* d_input, const void* d_indices,
+    const void* d_offsets_or_lengths, const float* d_weights, void* d_out,
+    const int32_t* d_compressed_indices_table, void* stream);
+
+/* ---- table-batched forward ----------------------------------------------- *
+ *
+ * Replaces int_nbit_split_embedding_codegen_lookup_function
+ * (fbgemm_gpu/codegen/inference/embedding_forward_quantized_host_cpu.cpp:84-227,
+ * embedding_forward_quantized_cpu_template.cpp:208-520; GPU dispatcher
+ * embedding_forward_quantized_host.cpp:259-370). A plan is made once from the
+ * operator's metadata tensors (HOST copies), then reused for every forward.
+ */
+typedef struct fbgemm_amd_tbe_plan fbgemm_amd_tbe_plan;
+
+/* weights_offsets[T] (bytes), weights_tys[T] (element types), D_offsets[T+1],
+ * weights_placements[T] (0 = dev_weights, anything else = uvm_weights) are the
+ * operator's tensors of the same names, on the host. *_weights_bytes are the
+ * sizes of the two weights buffers (they bound the last table's row count, as
+ * embedding_forward_quantized_cpu_template.cpp:372-380 does). row_alignment
+ * is the operator's argument (16 on GPU builds of the reference). */
+int fbgemm_amd_tbe_plan_create(
+    fbgemm_amd_tbe_plan** plan, int32_t T, const int64_t* weights_offsets,
+    const uint8_t* weights_tys, const int32_t* D_offsets,
+    const int32_t* weights_placements, int64_t dev_weights_bytes,
+    int64_t uvm_weights_bytes, int64_t row_alignment);
+
+void fbgemm_amd_tbe_plan_destroy(fbgemm_amd_tbe_plan* plan);
+
+/* Enqueue the forward of all T tables in ONE kernel launch.
+ * d_offsets holds T*B+1 entries in (table, bag) order with the width of the
+ * indices (index_bits). d_indice_weights NULL = unweighted. d_output is
+ * [B, total_D] of output_ty, row-major; columns of table t start at
+ * D_offsets[t]. The first forward with a new B uploads a per-wave work list
+ * (allocates); later ones reuse it. */
+int fbgemm_amd_tbe_forward(
+    fbgemm_amd_tbe_plan* plan, const void* d_dev_weights, const void* d_uvm_weights,
+    const void* d_indices, const void* d_offsets, int32_t index_bits,
+    int64_t indices_numel, int64_t offsets_numel, int32_t pooling_mode,
+    const float* d_indice_weights, int32_t output_ty, void* d_output,
+    void* d_status, void* stream);
+
+/* Rows the plan inferred for table t (what an index is checked against). */
+int64_t fbgemm_amd_tbe_plan_num_rows(const fbgemm_amd_tbe_plan* plan, int32_t t);
+/* Padded row bytes of table t. */
+int64_t fbgemm_amd_tbe_plan_row_bytes(const fbgemm_amd_tbe_plan* plan, int32_t t);
+
+/* ---- pruned-row remap ------------------------------------------------------ *
+ * Replaces pruned_array_lookup
+ * (embedding_forward_quantized_cpu_template.cpp:605-659,
+ * embedding_forward_quantized_split_lookup.cu:120-168): position-preserving,
+ * d_dense[i] = remap[remap_offsets[t] + indices[i]] for tables that own a
+ * mapping (remap_offsets[t+1] > remap_offsets[t]), a copy otherwise. */
+int fbgemm_amd_pruned_array_lookup(
+    const void* d_indices, const void* d_offsets, int32_t index_bits,
+    int64_t offsets_numel, const void* d_index_remappings, int32_t remap_bits,
+    const int64_t* d_index_remappings_offsets, int32_t T, void* d_dense,
+    void* stream);
+
+/* ---- row-size arithmetic (host, no GPU) ------------------------------------ *
+ * embedding_common.h:189-225. */
+int32_t fbgemm_amd_unpadded_row_size_in_bytes(int32_t dim, int32_t weight_ty, int32_t scale_bias_bytes);
+int32_t fbgemm_amd_padded_row_size_in_bytes(int32_t dim, int32_t weight_ty, int32_t row_alignment, int32_t scale_bias_bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FBGEMM_AMD_H_ */

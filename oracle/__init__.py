@@ -1,0 +1,216 @@
+"""TEST INFRASTRUCTURE ONLY: ctypes front-end of the CPU checkers.
+
+Only tests, the smoke check and the benchmark's CPU-baseline leg import this
+package; the shipped library never does.
+
+Two back-ends expose the same call:
+  * ``impl="oracle"``: our C restatement (oracle/embedding_oracle.c).
+  * ``impl="ref"``: the reference's own scalar code, compiled from its
+    sources by ``make -C oracle ref`` into oracle/_ref/ (present only where it
+    was built).
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ORACLE_SO = os.path.join(HERE, "_build", "libembedding_oracle.so")
+REF_SO = os.path.join(HERE, "_ref", "libfbgemm_ref.so")
+JIT_SO = os.path.join(HERE, "_build", "libfbgemm_jit_bridge.so")
+
+ST_FP32, ST_FP16, ST_INT8, ST_INT4, ST_INT2, ST_BF16 = 0, 1, 2, 3, 4, 5
+POOL_SUM, POOL_MEAN = 0, 1
+
+_c = ctypes
+_SPMDM_ARGS = [
+    _c.c_int, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_void_p, _c.c_void_p,
+    _c.c_int, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_int,
+    _c.c_int, _c.c_int, _c.c_int64, _c.c_int64, _c.c_int, _c.c_void_p,
+]
+_REMAP_ARGS = [
+    _c.c_int32, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_void_p,
+    _c.c_void_p, _c.c_void_p, _c.c_void_p,
+]
+
+
+def build(targets=("oracle",)):
+    """Compile the requested checker libraries (gcc/g++ only)."""
+    subprocess.check_call(["make", "-s", "-C", HERE, *targets])
+
+
+_libs = {}
+
+
+def _lib(impl):
+    if impl in _libs:
+        return _libs[impl]
+    if impl == "oracle":
+        if not os.path.exists(ORACLE_SO):
+            build(("oracle",))
+        lib = _c.CDLL(ORACLE_SO)
+        lib.oracle_embedding_spmdm.argtypes = _SPMDM_ARGS
+        lib.oracle_embedding_spmdm.restype = _c.c_int
+        lib.oracle_compressed_indices_remap.argtypes = _REMAP_ARGS
+        lib.oracle_compressed_indices_remap.restype = None
+        lib.oracle_pruned_array_lookup.argtypes = [
+            _c.c_int32, _c.c_int32, _c.c_void_p, _c.c_void_p, _c.c_int, _c.c_void_p,
+            _c.c_int, _c.c_void_p, _c.c_void_p]
+        lib.oracle_pruned_array_lookup.restype = None
+        lib.oracle_tbe_forward.argtypes = [
+            _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int32,
+            _c.c_int64, _c.c_void_p, _c.c_void_p, _c.c_int, _c.c_int64, _c.c_int,
+            _c.c_void_p, _c.c_int, _c.c_int64, _c.c_void_p]
+        lib.oracle_tbe_forward.restype = _c.c_int
+        lib.oracle_padded_row_bytes.argtypes = [_c.c_int32, _c.c_int, _c.c_int32, _c.c_int32]
+        lib.oracle_padded_row_bytes.restype = _c.c_int32
+    elif impl == "ref":
+        if not os.path.exists(REF_SO):
+            raise FileNotFoundError(REF_SO)
+        lib = _c.CDLL(REF_SO)
+        lib.ref_embedding_spmdm.argtypes = _SPMDM_ARGS
+        lib.ref_embedding_spmdm.restype = _c.c_int
+        lib.ref_compressed_indices_remap.argtypes = _REMAP_ARGS
+        lib.ref_compressed_indices_remap.restype = None
+    else:
+        raise ValueError(impl)
+    _libs[impl] = lib
+    return lib
+
+
+def have_ref():
+    return os.path.exists(REF_SO)
+
+
+def _ptr(a):
+    return None if a is None else a.ctypes.data_as(_c.c_void_p)
+
+
+def _is64(a):
+    if a.dtype == np.int64:
+        return 1
+    if a.dtype == np.int32:
+        return 0
+    raise TypeError(f"index arrays must be int32 or int64, got {a.dtype}")
+
+
+def out_dtype(out_ty):
+    return np.float32 if out_ty == ST_FP32 else np.uint16
+
+
+def spmdm(in_ty, block_size, table, indices, offsets_or_lengths, *, weights=None,
+          normalize=False, out_ty=ST_FP32, positional=False, use_offsets=True,
+          output_stride=-1, input_stride=-1, scale_bias_last=True, remap=None,
+          data_size, output_size=None, index_size=None, impl="oracle", out=None):
+    """Pooled lookup on the CPU. Returns (ok, out); fp16/bf16 outputs are the
+    raw 16-bit patterns (uint16). ``out`` may be passed in to observe which
+    positions the call leaves untouched."""
+    table = np.ascontiguousarray(table)
+    indices = np.ascontiguousarray(indices)
+    offsets_or_lengths = np.ascontiguousarray(offsets_or_lengths)
+    if output_size is None:
+        output_size = len(offsets_or_lengths) - (1 if use_offsets else 0)
+    if index_size is None:
+        index_size = len(indices)
+    stride = block_size if output_stride == -1 else output_stride
+    if out is None:
+        out = np.zeros(max(output_size, 0) * stride, dtype=out_dtype(out_ty))
+    if weights is not None:
+        weights = np.ascontiguousarray(weights, dtype=np.float32)
+    if remap is not None:
+        remap = np.ascontiguousarray(remap, dtype=np.int32)
+    lib = _lib(impl)
+    fn = lib.oracle_embedding_spmdm if impl == "oracle" else lib.ref_embedding_spmdm
+    ok = fn(in_ty, block_size, output_size, index_size, data_size, _ptr(table),
+            _ptr(indices), _is64(indices), _ptr(offsets_or_lengths),
+            _is64(offsets_or_lengths), _ptr(weights), int(normalize), _ptr(out), out_ty,
+            int(positional), int(use_offsets), output_stride, input_stride,
+            int(scale_bias_last), _ptr(remap))
+    return bool(ok), out
+
+
+def compressed_indices_remap(indices, mapping, offsets, weights=None, impl="oracle"):
+    """Compacting remap. Returns (out_indices[:n], out_offsets, out_weights[:n])."""
+    indices = np.ascontiguousarray(indices)
+    offsets = np.ascontiguousarray(offsets, dtype=indices.dtype)
+    mapping = np.ascontiguousarray(mapping, dtype=np.int32)
+    out_idx = np.zeros_like(indices)
+    out_off = np.zeros_like(offsets)
+    out_w = None
+    if weights is not None:
+        weights = np.ascontiguousarray(weights, dtype=np.float32)
+        out_w = np.zeros_like(weights)
+    lib = _lib(impl)
+    fn = (lib.oracle_compressed_indices_remap if impl == "oracle"
+          else lib.ref_compressed_indices_remap)
+    fn(len(offsets), _ptr(indices), _is64(indices), _ptr(mapping), _ptr(offsets),
+       _ptr(weights), _ptr(out_idx), _ptr(out_off), _ptr(out_w))
+    n = int(out_off[-1])
+    return out_idx[:n], out_off, (None if out_w is None else out_w[:n])
+
+
+def pruned_array_lookup(indices, offsets, remap, remap_offsets):
+    indices = np.ascontiguousarray(indices)
+    offsets = np.ascontiguousarray(offsets, dtype=indices.dtype)
+    remap = np.ascontiguousarray(remap)
+    remap_offsets = np.ascontiguousarray(remap_offsets, dtype=np.int64)
+    T = len(remap_offsets) - 1
+    B = (len(offsets) - 1) // T
+    dense = np.empty_like(indices)
+    _lib("oracle").oracle_pruned_array_lookup(
+        T, B, _ptr(indices), _ptr(offsets), _is64(indices), _ptr(remap), _is64(remap),
+        _ptr(remap_offsets), _ptr(dense))
+    return dense
+
+
+def tbe_forward(dev_weights, weights_offsets, weights_tys, D_offsets, total_D, indices,
+                offsets, pooling_mode, indice_weights, out_ty, row_alignment):
+    """Table-batched forward on the CPU. Returns (rc, out[B, total_D]); rc is 0
+    or 1 + the first failing table."""
+    dev_weights = np.ascontiguousarray(dev_weights, dtype=np.uint8)
+    weights_offsets = np.ascontiguousarray(weights_offsets, dtype=np.int64)
+    weights_tys = np.ascontiguousarray(weights_tys, dtype=np.uint8)
+    D_offsets = np.ascontiguousarray(D_offsets, dtype=np.int32)
+    indices = np.ascontiguousarray(indices)
+    offsets = np.ascontiguousarray(offsets, dtype=indices.dtype)
+    if indice_weights is not None:
+        indice_weights = np.ascontiguousarray(indice_weights, dtype=np.float32)
+    T = len(D_offsets) - 1
+    B = (len(offsets) - 1) // T
+    out = np.zeros((B, total_D), dtype=out_dtype(out_ty))
+    rc = _lib("oracle").oracle_tbe_forward(
+        _ptr(dev_weights), dev_weights.size, _ptr(weights_offsets), _ptr(weights_tys),
+        _ptr(D_offsets), T, total_D, _ptr(indices), _ptr(offsets), _is64(indices),
+        len(offsets), pooling_mode, _ptr(indice_weights), out_ty, row_alignment,
+        _ptr(out))
+    return rc, out
+
+
+def _conv(name, arr, in_dt, out_dt, impl):
+    arr = np.ascontiguousarray(arr, dtype=in_dt)
+    out = np.empty(arr.shape, dtype=out_dt)
+    fn = getattr(_lib(impl), ("oracle_" if impl == "oracle" else "ref_") + name + "_array")
+    fn.argtypes = [_c.c_void_p, _c.c_void_p, _c.c_int64]
+    fn.restype = None
+    fn(_ptr(arr), _ptr(out), arr.size)
+    return out
+
+
+def half2float(h, impl="oracle"):
+    """uint16 half patterns -> float32."""
+    return _conv("half2float", h, np.uint16, np.float32, impl)
+
+
+def float2half_rn(f, impl="oracle"):
+    """float32 -> uint16 half patterns, round to nearest even."""
+    return _conv("float2half_rn", f, np.float32, np.uint16, impl)
+
+
+def float2bf16(f, impl="oracle"):
+    """float32 -> uint16 bf16 patterns, the reference's add-0x8000-and-truncate rule."""
+    return _conv("float2bf16", f, np.float32, np.uint16, impl)
+
+
+def padded_row_bytes(dim, ty, row_alignment, scale_bias_bytes=4):
+    return _lib("oracle").oracle_padded_row_bytes(dim, ty, row_alignment, scale_bias_bytes)

@@ -1,0 +1,238 @@
+"""GPU parity of the single-table pooled lookup, through the C ABI, against the
+CPU oracle on the same seeded inputs. Integer/index behaviour and every output
+bit must match: the kernels consume rows in index order with one lane per
+output column, so fp32 results are bit-identical (tolerance 0; the path's
+stated bound is 1e-5 relative for fp32 and 1 ulp for fp16).
+
+Parameter space after test/EmbeddingSpMDMNBitTest.cc:92-418 and
+test/EmbeddingSpMDM8BitTest.cc:82-372: bit rates, weighted / positional,
+normalize, offsets vs lengths, index and offset widths, output types, odd
+dims, corner cases, and ten sentinel values after the output."""
+import itertools
+
+import numpy as np
+import pytest
+
+import helpers as H
+from helpers import BF16, FP16, FP32, INT2, INT4, INT8
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+SENTINELS = 10
+
+SHAPES = [
+    (10, 400, 2, 5), (10, 400, 4, 5), (10, 400, 7, 5), (10, 400, 8, 5), (10, 400, 16, 5),
+    (10, 400, 32, 5), (10, 400, 40, 5), (10, 400, 48, 5), (10, 400, 56, 5), (10, 400, 64, 5),
+    (3, 1000, 86, 20), (20, 1000, 128, 50), (10, 400, 164, 5), (40, 300, 256, 10),
+    (7, 200, 384, 12), (5, 100, 1024, 9), (3, 60, 2048, 7), (2, 40, 2600, 5),
+    (1, 50, 32, 100), (300, 5000, 128, 20), (0, 20, 32, 5),
+]
+
+
+def dev(a, torch_dtype=None):
+    t = torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    return t
+
+
+def run_gpu(ops, *, ty, D, table, idx, off_or_len, w, normalize, out_ty, positional, use_offsets,
+            output_stride, input_stride, sbl, remap, data_size, output_size, index_size=None):
+    stride = D if output_stride == -1 else output_stride
+    np_dt = np.float32 if out_ty == FP32 else np.uint16
+    sentinel = np.float32(-12345.5) if out_ty == FP32 else np.uint16(0xBEEF)
+    out_host = np.full(output_size * stride + SENTINELS, sentinel, dtype=np_dt)
+    t_out = dev(out_host.view(np.int16) if np_dt == np.uint16 else out_host)
+    t_table = dev(table)
+    if ty in (FP16, BF16):
+        assert t_table.data_ptr() % 2 == 0
+    t_idx, t_off = dev(idx), dev(off_or_len)
+    t_w = None if w is None else dev(w)
+    t_remap = None if remap is None else dev(remap)
+    if remap is not None:
+        kern = (ops.generate_embedding_spmdm_nbit_rowwise_sparse(
+                    4 if ty == INT4 else 2, D, w is not None, normalize, 16, positional, use_offsets)
+                if ty in (INT4, INT2) else
+                ops.generate_embedding_spmdm_rowwise_sparse(
+                    ty, D, w is not None, normalize, 16, positional, use_offsets))
+    elif ty in (INT4, INT2):
+        kern = ops.generate_embedding_spmdm_nbit_with_strides(
+            4 if ty == INT4 else 2, D, w is not None, normalize, 16, positional, use_offsets,
+            output_stride, input_stride, sbl, out_ty=out_ty)
+    else:
+        kern = ops.generate_embedding_spmdm_with_strides(
+            ty, D, w is not None, normalize, 16, positional, use_offsets, output_stride,
+            input_stride, sbl, out_ty=out_ty)
+    ok = kern(output_size, len(idx) if index_size is None else index_size, data_size, t_table,
+              t_idx, t_off, t_w, t_out, t_remap) if remap is not None else \
+        kern(output_size, len(idx) if index_size is None else index_size, data_size, t_table,
+             t_idx, t_off, t_w, t_out)
+    res = t_out.cpu().numpy()
+    res = res.view(np.uint16) if np_dt == np.uint16 else res
+    n = output_size * stride
+    assert (res[n:] == sentinel).all(), "wrote past the end of the output"
+    return ok, res[:n], sentinel
+
+
+def check_case(ops, oracle, *, ty, D, table, idx, off_or_len, w=None, normalize=False, out_ty=FP32,
+               positional=False, use_offsets=True, output_stride=-1, input_stride=-1, sbl=True,
+               remap=None, data_size, output_size, index_size=None, what=""):
+    stride = D if output_stride == -1 else output_stride
+    np_dt = np.float32 if out_ty == FP32 else np.uint16
+    ok_g, out_g, sentinel = run_gpu(
+        ops, ty=ty, D=D, table=table, idx=idx, off_or_len=off_or_len, w=w, normalize=normalize,
+        out_ty=out_ty, positional=positional, use_offsets=use_offsets, output_stride=output_stride,
+        input_stride=input_stride, sbl=sbl, remap=remap, data_size=data_size,
+        output_size=output_size, index_size=index_size)
+    pre = np.full(output_size * stride, sentinel, dtype=np_dt)
+    ok_o, out_o = oracle.spmdm(
+        ty, D, table, idx, off_or_len, weights=w, normalize=normalize, out_ty=out_ty,
+        positional=positional, use_offsets=use_offsets, output_stride=output_stride,
+        input_stride=input_stride, scale_bias_last=sbl, remap=remap, data_size=data_size,
+        output_size=output_size, index_size=index_size, out=pre)
+    assert ok_g == ok_o, f"{what}: gpu returned {ok_g}, oracle {ok_o}"
+    if ok_o:
+        H.assert_same_bits(out_g, out_o, what)
+    return ok_g
+
+
+@pytest.fixture(scope="module")
+def ops():
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    import fbgemm_amd.ops as o
+    return o
+
+
+@pytest.mark.parametrize("ty", [INT8, INT4, INT2, FP16, FP32, BF16])
+@pytest.mark.parametrize("shape", SHAPES)
+def test_parity_grid(ops, oracle, ty, shape):
+    nb, rows, D, avg = shape
+    if ty == INT2 and D % 4 and D > 4:
+        D = (D + 3) // 4 * 4
+    rng = np.random.default_rng(hash((ty, shape, 1)) % 2**32)
+    ran = 0
+    combos = list(itertools.product(
+        (True, False), (FP32, FP16, BF16), (0, 1, 2), (False, True),
+        (np.int32, np.int64), (np.int32, np.int64), (True, False)))
+    rng.shuffle(combos)
+    for sbl, out_ty, weighted, normalize, idx_dt, off_dt, use_offsets in combos[:6]:
+        table, stride = H.make_table(rng, ty, rows, D, sbl)
+        idx, off, lens = H.make_bags(rng, rows, nb, avg, idx_dt, off_dt, empty_frac=0.15)
+        if not sbl and len(idx):
+            idx[rng.random(len(idx)) < 0.2] = -1
+        w = None
+        if weighted == 1:
+            w = rng.normal(size=len(idx)).astype(np.float32)
+        elif weighted == 2:
+            w = rng.normal(size=max(1, int(lens.max()) if len(lens) else 1)).astype(np.float32)
+        what = f"ty={ty} shape={shape} sbl={sbl} out={out_ty} w={weighted} norm={normalize} " \
+               f"idx={np.dtype(idx_dt).name} off={np.dtype(off_dt).name} use_offsets={use_offsets}"
+        print(what, flush=True)
+        ok = check_case(ops, oracle, ty=ty, D=D, table=table, idx=idx,
+                        off_or_len=off if use_offsets else lens, w=w, normalize=normalize,
+                        out_ty=out_ty, positional=weighted == 2, use_offsets=use_offsets, sbl=sbl,
+                        data_size=rows, output_size=nb, what=what)
+        assert ok
+        ran += 1
+    assert ran
+
+
+@pytest.mark.parametrize("ty", [INT8, INT4, INT2, FP16, FP32])
+@pytest.mark.parametrize("align", [1, 4, 16])
+def test_tbe_row_layout_and_strides(ops, oracle, ty, align):
+    rng = np.random.default_rng(100 + ty * 7 + align)
+    for D in (8, 24, 64, 128, 200):
+        rows, nb = 300, 33
+        stride = oracle.padded_row_bytes(D, ty, align)
+        if ty == FP32:
+            stride = (stride + 3) // 4 * 4
+        table, stride = H.make_table(rng, ty, rows, D, False, stride_bytes=stride)
+        idx, off, _ = H.make_bags(rng, rows, nb, 9, empty_frac=0.1)
+        idx[::4] = -1
+        for out_ty, total_D in ((FP16, D + 24), (FP32, D + 3), (BF16, D)):
+            what = f"ty={ty} align={align} D={D} out={out_ty} total_D={total_D}"
+            print(what, flush=True)
+            assert check_case(ops, oracle, ty=ty, D=D, table=table, idx=idx, off_or_len=off,
+                              w=rng.uniform(size=len(idx)).astype(np.float32), out_ty=out_ty,
+                              output_stride=total_D, input_stride=H.input_stride_elems(ty, stride),
+                              sbl=False, data_size=rows, output_size=nb, what=what)
+
+
+@pytest.mark.parametrize("ty", [INT8, INT4, INT2, FP16])
+def test_rejections(ops, oracle, ty):
+    rng = np.random.default_rng(11 + ty)
+    rows, D, nb = 100, 32, 8
+    table, _ = H.make_table(rng, ty, rows, D, True)
+    idx, off, _ = H.make_bags(rng, rows, nb, 5)
+    kw = dict(ty=ty, D=D, table=table, data_size=rows, output_size=nb)
+    assert check_case(ops, oracle, idx=idx, off_or_len=off, what="valid", **kw)
+    bad = idx.copy(); bad[len(bad) // 2] = rows
+    assert not check_case(ops, oracle, idx=bad, off_or_len=off, what="idx == rows", **kw)
+    bad = idx.copy(); bad[1] = -1
+    assert not check_case(ops, oracle, idx=bad, off_or_len=off, what="-1 in trailer layout", **kw)
+    bad = idx.copy(); bad[-1] = -7
+    assert not check_case(ops, oracle, idx=bad, off_or_len=off, what="negative", **kw)
+    assert not check_case(ops, oracle, idx=idx, off_or_len=off, index_size=len(idx) - 1, what="short", **kw)
+    longer = np.concatenate([idx, idx[:1]])
+    assert not check_case(ops, oracle, idx=longer, off_or_len=off, index_size=len(idx) + 1, what="long", **kw)
+    zero_off = np.zeros_like(off)
+    assert check_case(ops, oracle, idx=idx[:0], off_or_len=zero_off, what="all bags empty", **kw)
+    one = np.zeros(1, idx.dtype)
+    assert not check_case(ops, oracle, idx=one, off_or_len=zero_off, index_size=1, what="unused index", **kw)
+
+
+@pytest.mark.parametrize("ty", [INT8, INT4, INT2, FP16, FP32])
+def test_rowwise_sparse(ops, oracle, ty):
+    rng = np.random.default_rng(23 + ty)
+    logical, nb = 500, 37
+    for D in (16, 48, 64, 128):
+        keep = rng.random(logical) >= 0.7
+        mapping = np.full(logical, -1, np.int32)
+        mapping[keep] = np.arange(int(keep.sum()), dtype=np.int32)
+        rows = max(1, int(keep.sum()))
+        table, _ = H.make_table(rng, ty, rows, D, True)
+        for weighted, normalize, idx_dt, use_offsets in itertools.product(
+                (0, 1, 2), (False, True), (np.int32, np.int64), (True, False)):
+            idx, off, lens = H.make_bags(rng, logical, nb, 8, idx_dt, np.int32)
+            w = None
+            if weighted == 1:
+                w = rng.normal(size=len(idx)).astype(np.float32)
+            elif weighted == 2:
+                w = rng.normal(size=int(lens.max())).astype(np.float32)
+            what = f"sparse ty={ty} D={D} w={weighted} norm={normalize} use_offsets={use_offsets}"
+            assert check_case(ops, oracle, ty=ty, D=D, table=table, idx=idx,
+                              off_or_len=off if use_offsets else lens, w=w, normalize=normalize,
+                              positional=weighted == 2, use_offsets=use_offsets, remap=mapping,
+                              data_size=logical, output_size=nb, what=what)
+        bad = idx.copy(); bad[0] = logical
+        assert not check_case(ops, oracle, ty=ty, D=D, table=table, idx=bad, off_or_len=off,
+                              remap=mapping, data_size=logical, output_size=nb, what="logical OOB")
+
+
+def test_closed_forms(ops, oracle):
+    """scale=1, bias=0 rows sum to exact integers ("should be exact",
+    test/EmbeddingSpMDMNBitTest.cc:490-507); rows of ones count the bag."""
+    rng = np.random.default_rng(1)
+    rows, D, nb = 64, 64, 50
+    for ty in (INT8, INT4, INT2):
+        table, stride = H.make_table(rng, ty, rows, D, True, scale_range=(1, 1), bias_range=(0, 0))
+        idx, off, lens = H.make_bags(rng, rows, nb, 10)
+        ok, out, _ = run_gpu(ops, ty=ty, D=D, table=table, idx=idx, off_or_len=off, w=None,
+                             normalize=False, out_ty=FP32, positional=False, use_offsets=True,
+                             output_stride=-1, input_stride=-1, sbl=True, remap=None,
+                             data_size=rows, output_size=nb)
+        assert ok
+        bits = H.BITS[ty]
+        pb = H.packed_bytes(ty, D)
+        q = table.reshape(rows, stride)[:, :pb]
+        epb = 8 // bits
+        vals = np.stack([(q >> (bits * k)) & ((1 << bits) - 1) for k in range(epb)], axis=2).reshape(rows, -1)[:, :D]
+        want = np.stack([vals[idx[off[b]:off[b + 1]]].sum(axis=0) for b in range(nb)]).astype(np.float32)
+        assert (out.reshape(nb, D) == want).all()
+        ones, _ = H.make_table(rng, ty, rows, D, True, ones=True)
+        ok, out, _ = run_gpu(ops, ty=ty, D=D, table=ones, idx=idx, off_or_len=off, w=None,
+                             normalize=False, out_ty=FP16, positional=False, use_offsets=True,
+                             output_stride=-1, input_stride=-1, sbl=True, remap=None,
+                             data_size=rows, output_size=nb)
+        assert ok
+        got = out.view(np.float16).reshape(nb, D).astype(np.float32)
+        assert (got == lens.astype(np.float32)[:, None]).all()
