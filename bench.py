@@ -1,0 +1,245 @@
+#!/usr/bin/env python3
+"""Benchmark of the table-batched int4/int8/fp16 embedding forward on one MI355X.
+
+    python bench.py [--steps K] [--warmup W] [--config 3|5|1|2|4] [--scale S]
+
+A step is one forward over one batch of synthetic, seeded input already
+resident in HBM (fbgemm_amd/bench_configs.py). The printed JSON line reports
+useful row bytes per second (unpadded row data + scale/bias of every lookup
+that reads a row; indices, offsets, weights, padding and output are not
+credited), the same figure as a fraction of the 8 TB/s HBM peak, pooled rows
+per second, and a CPU baseline timed on this machine's host cores.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", type=int, default=3, choices=[1, 2, 3, 4, 5])
+    ap.add_argument("--scale", type=float, default=1.0, help="shrink rows and batch (1.0 = the real configuration)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    ap.add_argument("--check", action="store_true", help="verify a sample of the output against the oracle first")
+    return ap.parse_args()
+
+
+def tbe_runner(p, torch):
+    """Returns (launch, out, status, plan) for a TbeProblem: launch() enqueues one forward."""
+    from fbgemm_amd import _lib, ops
+
+    lib = _lib.lib()
+    dev = p.dev_weights.device
+    plan = ops.TbePlan(torch.from_numpy(p.weights_offsets), torch.from_numpy(p.tys), torch.from_numpy(p.D_offsets),
+                       torch.zeros(p.T, dtype=torch.int32), p.dev_weights.numel(), 0, p.row_alignment)
+    out_dt = {0: torch.float32, 1: torch.float16, 5: torch.bfloat16}[p.output_dtype]
+    out = torch.empty((p.B, p.total_D), dtype=out_dt, device=dev)
+    st = ops.Status(dev)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    args = (plan.handle, C.c_void_p(p.dev_weights.data_ptr()), None, C.c_void_p(p.indices.data_ptr()),
+            C.c_void_p(p.offsets.data_ptr()), 64 if p.indices.dtype == torch.int64 else 32, p.indices.numel(),
+            p.offsets.numel(), p.pooling_mode,
+            None if p.indice_weights is None else C.c_void_p(p.indice_weights.data_ptr()),
+            p.output_dtype, C.c_void_p(out.data_ptr()), C.c_void_p(st.buf.data_ptr()), stream)
+
+    def launch():
+        rc = lib.fbgemm_amd_tbe_forward(*args)
+        if rc:
+            raise RuntimeError(lib.fbgemm_amd_last_error().decode())
+
+    return launch, out, st, plan
+
+
+def spmdm_runner(probs, torch):
+    """Single-table configurations: one launch per table."""
+    from fbgemm_amd import _lib, ops
+    from fbgemm_amd._lib import SpmdmConfig
+
+    lib = _lib.lib()
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    st = ops.Status(probs[0].table.device)
+    calls, outs = [], []
+    for p in probs:
+        out_dt = {0: torch.float32, 1: torch.float16, 5: torch.bfloat16}[p.out_ty]
+        out = torch.empty(p.num_bags * p.D, dtype=out_dt, device=p.table.device)
+        cfg = SpmdmConfig(weight_ty=p.ty, output_ty=p.out_ty, index_bits=64, offset_bits=32, block_size=p.D,
+                          output_stride=-1, input_stride=-1, normalize_by_lengths=int(p.normalize),
+                          is_weight_positional=0, use_offsets=1, scale_bias_last=1)
+        calls.append((cfg, (p.num_bags, p.lookups, p.data_size, C.c_void_p(p.table.data_ptr()),
+                            C.c_void_p(p.indices.data_ptr()), C.c_void_p(p.offsets.data_ptr()), None,
+                            C.c_void_p(out.data_ptr()),
+                            None if p.remap is None else C.c_void_p(p.remap.data_ptr()),
+                            C.c_void_p(st.buf.data_ptr()), stream)))
+        outs.append(out)
+
+    def launch():
+        for cfg, a in calls:
+            rc = lib.fbgemm_amd_spmdm_launch(C.byref(cfg), *a)
+            if rc:
+                raise RuntimeError(lib.fbgemm_amd_last_error().decode())
+
+    return launch, outs, st
+
+
+def cpu_baseline_tbe(p, seconds, torch):
+    """Time the CPU path on a bounded sample of the same workload: whole tables
+    of the problem, taken in order until about `seconds` of work is reached."""
+    import numpy as np
+    import oracle
+
+    kind, fn = "port", None
+    try:
+        from oracle import jit_baseline
+        fn = jit_baseline.tbe_table_runner()
+        kind = "reference"
+    except Exception:
+        fn = None
+    spent, rows_done, bytes_done, tables_done = 0.0, 0, 0, 0
+    from fbgemm_amd.bench_configs import unpadded_row_bytes
+    for t in range(p.T):
+        if spent >= seconds:
+            break
+        tbl = p.table_host_bytes(t)
+        s, e = int(p.host_offsets[t * p.B]), int(p.host_offsets[(t + 1) * p.B])
+        idx = np.ascontiguousarray(p.host_indices[s:e])
+        off = np.ascontiguousarray(p.host_offsets[t * p.B:(t + 1) * p.B + 1] - p.host_offsets[t * p.B])
+        w = None if p.host_weights is None else np.ascontiguousarray(p.host_weights[s:e])
+        D, ty, rb = int(p.Ds[t]), int(p.tys[t]), int(p.row_bytes[t])
+        elem = 4 if ty == 0 else 2 if ty == 1 else 1
+        t0 = time.perf_counter()
+        if fn is not None:
+            ok = fn(ty, D, tbl, idx, off, w, p.pooling_mode == 1, p.output_dtype, rb // elem, int(p.rows[t]), p.B)
+        else:
+            ok, _ = oracle.spmdm(ty, D, tbl, idx, off, weights=w, normalize=p.pooling_mode == 1,
+                                 out_ty=p.output_dtype, input_stride=rb // elem, scale_bias_last=False,
+                                 data_size=int(p.rows[t]), output_size=p.B,
+                                 impl="ref" if oracle.have_ref() else "oracle")
+        spent += time.perf_counter() - t0
+        assert ok
+        kept = int((idx != -1).sum())
+        rows_done += e - s
+        bytes_done += kept * unpadded_row_bytes(D, ty)
+        tables_done += 1
+    if fn is None and oracle.have_ref():
+        kind = "reference"
+    impl = ("fbgemm AVX2/AVX-512 JIT kernels exported by libtorch_cpu.so, THREAD_LOCAL, prefetch 16"
+            if fn is not None else
+            ("reference scalar EmbeddingSpMDM*_ref built from its sources (oracle/_ref)" if kind == "reference"
+             else "C restatement of the reference's scalar loop (oracle/)"))
+    return {
+        "value": round(bytes_done / spent / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": kind,
+        "pooled_rows_per_s": round(rows_done / spent, 1),
+        "sample": f"first {tables_done} of {p.T} tables of the same problem, all {p.B} bags each, one pass, "
+                  f"{spent:.1f} s; {impl}",
+    }
+
+
+def main():
+    a = parse()
+    if a.gpus != 1:
+        print("bench.py: this path is measured on ONE GPU (no sharding, no collectives); "
+              f"--gpus {a.gpus} is not supported", file=sys.stderr)
+        sys.exit(2)
+    import numpy as np
+    import torch
+
+    from fbgemm_amd import bench_configs as bc
+
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    torch.cuda.set_device(0)
+    t_build = time.time()
+    if a.config in (3, 5):
+        p = bc.config3("cuda", a.scale) if a.config == 3 else bc.config5("cuda", a.scale)
+        launch, out, st, plan = tbe_runner(p, torch)
+        lookups, useful = p.lookups, p.useful_row_bytes()
+        other = p.other_bytes()
+        name, dtype_out = p.name, {0: "fp32", 1: "fp16", 5: "bf16"}[p.output_dtype]
+        launches_per_step = 1
+    else:
+        probs = {1: lambda: [bc.config1("cuda", a.scale)], 2: lambda: [bc.config2("cuda", a.scale)],
+                 4: lambda: bc.config4("cuda", a.scale)}[a.config]()
+        launch, out, st = spmdm_runner(probs, torch)
+        lookups = sum(q.lookups for q in probs)
+        useful = sum(q.useful_row_bytes() for q in probs)
+        other = {}
+        name = probs[0].name.split("[")[0] if len(probs) > 1 else probs[0].name
+        dtype_out = {0: "fp32", 1: "fp16", 5: "bf16"}[probs[0].out_ty]
+        launches_per_step = len(probs)
+        p = None
+    torch.cuda.synchronize()
+    build_s = time.time() - t_build
+
+    if a.check and p is not None:
+        import oracle
+        launch()
+        torch.cuda.synchronize()
+        for t in list(range(min(3, p.T))) + [p.T - 1]:
+            s, e = int(p.host_offsets[t * p.B]), int(p.host_offsets[(t + 1) * p.B])
+            elem = 4 if int(p.tys[t]) == 0 else 2 if int(p.tys[t]) == 1 else 1
+            ok, want = oracle.spmdm(int(p.tys[t]), int(p.Ds[t]), p.table_host_bytes(t), p.host_indices[s:e],
+                                    p.host_offsets[t * p.B:(t + 1) * p.B + 1] - p.host_offsets[t * p.B],
+                                    weights=None if p.host_weights is None else p.host_weights[s:e],
+                                    normalize=p.pooling_mode == 1, out_ty=p.output_dtype,
+                                    input_stride=int(p.row_bytes[t]) // elem, scale_bias_last=False,
+                                    data_size=int(p.rows[t]), output_size=p.B)
+            got = out[:, int(p.D_offsets[t]):int(p.D_offsets[t + 1])].contiguous().cpu()
+            got = got.numpy() if p.output_dtype == 0 else got.view(torch.int16).numpy().view(np.uint16)
+            assert ok and (got.reshape(-1).view(want.dtype) == want).all(), f"table {t} differs from the oracle"
+        print(f"check: tables 0..2 and {p.T - 1} match the oracle bit for bit", file=sys.stderr)
+
+    for _ in range(a.warmup):
+        launch()
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record()
+    for _ in range(a.steps):
+        launch()
+    ev1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    bits, pos = st.read()
+    assert bits == 0, f"the lookup rejected its inputs: status {bits:#x} at {pos}"
+    ms_per_step = wall * 1e3 / a.steps
+    kernel_ms = ev0.elapsed_time(ev1) / a.steps  # events on the launch stream, back-to-back launches
+
+    gbps = useful / (ms_per_step * 1e-3) / 1e9
+    kern_gbps = useful / (kernel_ms * 1e-3) / 1e9
+    res = {
+        "metric": "achieved HBM GB/s (% peak) + pooled rows/s, int4 TBE fwd on 1 MI355X",
+        "value": round(gbps, 2), "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": name, "config_id": a.config, "scale": a.scale, "lookups_per_step": lookups,
+                   "useful_row_bytes_per_step": useful, "other_bytes_per_step": other,
+                   "output_dtype": dtype_out, "launches_per_step": launches_per_step},
+        "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
+        "pooled_rows_per_s": round(lookups / (ms_per_step * 1e-3), 1),
+        "roofline": {"bound": "hbm", "achieved": round(kern_gbps, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(kern_gbps / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel": "lookup_kernel", "kernel_ms": round(kernel_ms / launches_per_step, 5),
+                     "algorithmic_bytes_per_launch": useful // launches_per_step},
+        "setup_s": round(build_s, 1),
+    }
+    if not a.no_cpu and p is not None:
+        res["cpu_baseline"] = cpu_baseline_tbe(p, a.cpu_seconds, torch)
+    elif not a.no_cpu:
+        res["cpu_baseline"] = None
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,197 @@
+"""GPU parity of the table-batched forward and of pruned_array_lookup, through
+the C ABI, against the CPU oracle. Bit-exact (tolerance 0) for fp32, fp16 and
+bf16 outputs; the path's stated bound is 1e-5 relative / 1 ulp.
+
+Cases after fbgemm_gpu/test/tbe/inference/nbit_forward_test.py: the exact-count
+fixture (:577-659), an out-of-range index in one table (:661-688), mixed
+types / dims / pooling / index widths (:746-815)."""
+import numpy as np
+import pytest
+
+import helpers as H
+from helpers import BF16, FP16, FP32, INT2, INT4, INT8
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    import fbgemm_amd.ops as o
+    return o
+
+
+def cu(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def build_weights(rng, specs, row_alignment, ones=False):
+    """specs: (rows, D, ty). Returns (flat uint8 weights, weights_offsets, row_bytes)."""
+    import oracle
+    blobs, offs, rbs, cur = [], [], [], 0
+    for rows, D, ty in specs:
+        rb = oracle.padded_row_bytes(D, ty, row_alignment)
+        tbl, _ = H.make_table(rng, ty, rows, D, False, stride_bytes=rb, ones=ones)
+        offs.append(cur)
+        rbs.append(rb)
+        size = (tbl.size + 127) // 128 * 128
+        blobs.append(tbl)
+        blobs.append(rng.integers(0, 256, size=size - tbl.size, dtype=np.uint8))
+        cur += size
+    return np.concatenate(blobs), np.array(offs, np.int64), rbs
+
+
+def run_both(ops, oracle, weights, wo, specs, indices, offsets, pooling, psw, out_ty, row_alignment):
+    tys = np.array([s[2] for s in specs], np.uint8)
+    D_offsets = np.concatenate([[0], np.cumsum([s[1] for s in specs])]).astype(np.int32)
+    total_D = int(D_offsets[-1])
+    maxd = lambda ty: max([s[1] for s in specs if s[2] == ty], default=0)
+    got = ops.int_nbit_split_embedding_codegen_lookup_function(
+        cu(weights), torch.zeros(0, dtype=torch.uint8, device="cuda"),
+        cu(np.zeros(len(specs), np.int32)), cu(wo), cu(tys), cu(D_offsets), total_D,
+        maxd(INT2), maxd(INT4), maxd(INT8), maxd(FP16), maxd(FP32), cu(indices), cu(offsets),
+        pooling, None if psw is None else cu(psw), out_ty, row_alignment=row_alignment)
+    rc, want = oracle.tbe_forward(weights, wo, tys, D_offsets, total_D, indices, offsets, pooling,
+                                  psw, out_ty, row_alignment)
+    assert rc == 0
+    g = got.cpu()
+    g = g.numpy() if out_ty == FP32 else g.view(torch.int16).numpy().view(np.uint16)
+    return g, want
+
+
+def test_exact_count_fixture(ops, oracle):
+    """Rows of ones: every output column equals the number of kept indices of
+    its (table, bag); empty and fully pruned bags give exact zeros."""
+    E, Ds = 100, [16, 24, 40]
+    Ls = [[0, 2, 5, 0, 3, 4], [1, 0, 4, 2, 0, 6], [3, 3, 0, 1, 5, 0]]
+    fully_pruned = [4, 2, 3]
+    T, B = len(Ds), len(Ls[0])
+    rng = np.random.default_rng(0)
+    for ty in (FP16, INT8, INT4, INT2, FP32):
+        specs = [(E, d, ty) for d in Ds]
+        for align in (16, 1):
+            weights, wo, _ = build_weights(rng, specs, align, ones=True)
+            idx, off, running = [], [0], 0
+            expected = np.zeros((B, sum(Ds)), np.float32)
+            dpre = np.cumsum([0] + Ds)
+            for t in range(T):
+                for b in range(B):
+                    kept = 0
+                    for _ in range(Ls[t][b]):
+                        prune = b == fully_pruned[t] or running % 3 == 0
+                        idx.append(-1 if prune else running % E)
+                        kept += 0 if prune else 1
+                        running += 1
+                    off.append(len(idx))
+                    expected[b, dpre[t]:dpre[t + 1]] = kept
+            for out_ty in (FP32, FP16, BF16):
+                for dt in (np.int32, np.int64):
+                    got, want = run_both(ops, oracle, weights, wo, specs, np.array(idx, dt),
+                                         np.array(off, dt), 0, None, out_ty, align)
+                    H.assert_same_bits(got, want, f"ty={ty} out={out_ty}")
+                    if out_ty == FP32:
+                        val = got
+                    elif out_ty == FP16:
+                        val = got.view(np.float16).astype(np.float32)
+                    else:
+                        val = (got.astype(np.uint32) << 16).view(np.float32)
+                    assert (val == expected).all()
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_mixed_tables_random(ops, oracle, seed):
+    rng = np.random.default_rng(500 + seed)
+    T = int(rng.integers(1, 11))
+    B = int(rng.integers(1, 41))
+    dims = {INT8: [4, 8, 16, 32, 64, 100, 128, 256, 1024], INT4: [8, 16, 24, 32, 40, 64, 128, 160, 256, 1024],
+            INT2: [16, 32, 64, 128, 256], FP16: [4, 8, 16, 64, 128, 256, 2048], FP32: [4, 8, 32, 128]}
+    specs = []
+    for _ in range(T):
+        ty = int(rng.choice([INT8, INT4, INT2, FP16, FP32]))
+        specs.append((int(rng.integers(1, 300)), int(rng.choice(dims[ty])), ty))
+    align = int(rng.choice([1, 16]))
+    weights, wo, _ = build_weights(rng, specs, align)
+    lens = rng.integers(0, 25, size=T * B)
+    lens[rng.random(T * B) < 0.1] = 0
+    dt = rng.choice([np.int32, np.int64])
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(dt)
+    idx = np.concatenate([rng.integers(0, specs[t][0], size=int(lens[t * B:(t + 1) * B].sum()))
+                          for t in range(T)] + [np.zeros(0, np.int64)]).astype(dt)
+    idx[rng.random(len(idx)) < 0.15] = -1
+    for pooling in (0, 1):
+        for weighted in (False, True):
+            psw = rng.uniform(0, 1, size=len(idx)).astype(np.float32) if weighted else None
+            for out_ty in (FP32, FP16, BF16):
+                what = f"seed={seed} T={T} B={B} specs={specs} align={align} pool={pooling} w={weighted} out={out_ty}"
+                print(what, flush=True)
+                got, want = run_both(ops, oracle, weights, wo, specs, idx, off, pooling, psw, out_ty, align)
+                H.assert_same_bits(got, want, what)
+
+
+def test_out_of_range_index_raises(ops, oracle):
+    rng = np.random.default_rng(9)
+    E = 100
+    specs = [(E, 16, INT8), (E, 32, INT8)]
+    weights, wo, _ = build_weights(rng, specs, 16)
+    tys = np.array([INT8, INT8], np.uint8)
+    D_offsets = np.array([0, 16, 48], np.int32)
+    args = lambda idx, off: (cu(weights), torch.zeros(0, dtype=torch.uint8, device="cuda"),
+                            cu(np.zeros(2, np.int32)), cu(wo), cu(tys), cu(D_offsets), 48, 0, 0, 32, 0, 0,
+                            cu(idx), cu(off), 0, None, FP16)
+    idx = np.array([0, E + 500000, 3], np.int32)
+    off = np.array([0, 1, 1, 2, 3], np.int32)
+    with pytest.raises(RuntimeError, match="out of bounds"):
+        ops.int_nbit_split_embedding_codegen_lookup_function(*args(idx, off), row_alignment=16)
+    rc, _ = oracle.tbe_forward(weights, wo, tys, D_offsets, 48, idx, off, 0, None, FP16, 16)
+    assert rc == 2  # the oracle blames the second table too
+    # asynchronous form: the caller reads the status block
+    st = ops.Status()
+    out = ops.int_nbit_split_embedding_codegen_lookup_function(*args(idx, off), row_alignment=16, status=st)
+    bits, pos = st.read()
+    assert bits == ops.ERR_INDEX_OUT_OF_RANGE and pos == 1
+    assert torch.isfinite(out.float()).all()
+    # the inferred row bound includes the table's 128-byte padding, as in the reference
+    rb = oracle.padded_row_bytes(32, INT8, 16)
+    bound = (len(weights) - int(wo[1])) // rb
+    idx = np.array([0, bound - 1, 3], np.int32)
+    ops.int_nbit_split_embedding_codegen_lookup_function(*args(idx, off), row_alignment=16)
+    idx = np.array([0, bound, 3], np.int32)
+    with pytest.raises(RuntimeError):
+        ops.int_nbit_split_embedding_codegen_lookup_function(*args(idx, off), row_alignment=16)
+
+
+@pytest.mark.parametrize("dt,rdt", [(np.int32, np.int32), (np.int64, np.int32), (np.int64, np.int64), (np.int32, np.int64)])
+def test_pruned_array_lookup(ops, oracle, dt, rdt):
+    rng = np.random.default_rng(3)
+    T, B = 5, 17
+    caps = [200, 0, 1000, 50, 0]
+    remap_off = np.concatenate([[0], np.cumsum(caps)]).astype(np.int64)
+    remap = np.full(int(remap_off[-1]), -1, rdt)
+    for t in range(T):
+        s, e = remap_off[t], remap_off[t + 1]
+        keep = rng.random(e - s) < 0.5
+        remap[s:e][keep] = np.arange(int(keep.sum()), dtype=rdt)
+    lens = rng.integers(0, 12, size=T * B)
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(dt)
+    idx = np.concatenate([rng.integers(0, caps[t] if caps[t] else 10**6, size=int(lens[t * B:(t + 1) * B].sum()))
+                          for t in range(T)]).astype(dt)
+    got = ops.pruned_array_lookup(cu(idx), cu(off), cu(remap), cu(remap_off)).cpu().numpy()
+    want = oracle.pruned_array_lookup(idx, off, remap, remap_off)
+    assert got.dtype == want.dtype and (got == want).all()
+
+
+def test_config3_scaled(ops, oracle):
+    """The headline workload at 1/50 scale, checked in full against the oracle."""
+    from fbgemm_amd import bench_configs as bc
+    p = bc.config3("cuda", scale=0.02)
+    got = ops.int_nbit_split_embedding_codegen_lookup_function(
+        p.dev_weights, torch.zeros(0, dtype=torch.uint8, device="cuda"),
+        cu(np.zeros(p.T, np.int32)), cu(p.weights_offsets), cu(p.tys), cu(p.D_offsets), p.total_D,
+        0, 256, 256, 256, 0, p.indices, p.offsets, p.pooling_mode, p.indice_weights, p.output_dtype,
+        row_alignment=p.row_alignment)
+    rc, want = oracle.tbe_forward(p.dev_weights.cpu().numpy(), p.weights_offsets, p.tys, p.D_offsets,
+                                  p.total_D, p.host_indices, p.host_offsets, p.pooling_mode,
+                                  p.host_weights, p.output_dtype, p.row_alignment)
+    assert rc == 0
+    H.assert_same_bits(got.cpu().view(torch.int16).numpy().view(np.uint16), want, "config3 @ 0.02")
