@@ -33,6 +33,8 @@ def parse():
     ap.add_argument("--scale", type=float, default=1.0, help="shrink rows and batch (1.0 = the real configuration)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    ap.add_argument("--calibration-copy-mib", type=int, default=0,
+                    help="also run one plain copy of this many MiB (yardstick for hardware byte counters)")
     ap.add_argument("--check", action="store_true", help="verify a sample of the output against the oracle first")
     return ap.parse_args()
 
@@ -213,6 +215,15 @@ def main():
     wall = time.perf_counter() - t0
     bits, pos = st.read()
     assert bits == 0, f"the lookup rejected its inputs: status {bits:#x} at {pos}"
+    if a.calibration_copy_mib:
+        from fbgemm_amd import _lib
+        n = a.calibration_copy_mib << 20
+        src = torch.zeros(n, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        _lib.check(_lib.lib().fbgemm_amd_calibration_copy(
+            C.c_void_p(src.data_ptr()), C.c_void_p(dst.data_ptr()), n,
+            C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+        torch.cuda.synchronize()
     ms_per_step = wall * 1e3 / a.steps
     kernel_ms = ev0.elapsed_time(ev1) / a.steps  # events on the launch stream, back-to-back launches
 

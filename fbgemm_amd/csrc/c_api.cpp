@@ -17,6 +17,8 @@ namespace fbgemm_amd {
 hipError_t launch_lookup(const LookupArgs& a, bool idx64, hipStream_t stream);
 hipError_t launch_lengths_to_offsets(const void* lengths, bool is64, int64_t n, int64_t* offsets, hipStream_t stream);
 hipError_t launch_status_clear(Status* st, hipStream_t stream);
+hipError_t launch_bag_order(const void* offsets, bool off64, int32_t B, int32_t T, int32_t* order, hipStream_t stream);
+hipError_t launch_calibration_copy(const void* src, void* dst, int64_t bytes, hipStream_t stream);
 hipError_t launch_pruned_array_lookup(const void* indices, const void* offsets, bool idx64, const void* remap,
                                       bool remap64, const int64_t* remap_offsets, int32_t B, int32_t T,
                                       void* dense, hipStream_t stream);
@@ -63,7 +65,13 @@ int env_int(const char* name, int dflt) {
 // Tunables, read once per process (the reference reads its FBGEMM_* switches
 // the same way, src/Utils.cc:773-875).
 int xcd_swizzle_default() {
-  static int v = env_int("FBGEMM_AMD_XCD_SWIZZLE", 1);
+  static int v = env_int("FBGEMM_AMD_XCD_SWIZZLE", 0);
+  return v;
+}
+
+// 1: order each table's bags by length on the device before the lookup.
+int sort_bags_default() {
+  static int v = env_int("FBGEMM_AMD_SORT_BAGS", 1);
   return v;
 }
 
@@ -84,7 +92,7 @@ void plan_lanes(TableDesc& d, uintptr_t base_addr, int64_t out_stride, bool has_
   if (force_vb == 1) vb = min_vb;
   d.vb = vb;
   const int chunks = (d.data_bytes + vb - 1) / vb;
-  d.lanes = std::max(1, std::min(64, chunks));
+  d.lanes = std::max(2, std::min(64, chunks)); // >= 2: a wave stages at most 32 bags
   d.passes = (chunks + d.lanes - 1) / d.lanes;
   // whole-run vector stores: each lane writes E = vb*8/bits consecutive
   // elements; allowed when every run starts on a multiple of min(16, run bytes)
@@ -105,9 +113,15 @@ void plan_lanes(TableDesc& d, uintptr_t base_addr, int64_t out_stride, bool has_
 
 struct DeviceScratch {
   Status* status = nullptr;
-  int64_t* offsets = nullptr;
+  int64_t* offsets = nullptr; // lengths -> offsets
   int64_t offsets_cap = 0;
+  int32_t* order = nullptr;   // bag order of single-table calls
+  int64_t order_cap = 0;
 };
+
+// Grow-only device buffer; the old one may still be read by an enqueued kernel.
+template <typename T>
+int grow(T** buf, int64_t* cap, int64_t need, hipStream_t stream);
 
 std::mutex g_mu;
 std::map<int, DeviceScratch> g_scratch;
@@ -118,6 +132,20 @@ int get_scratch(DeviceScratch** out) {
   DeviceScratch& s = g_scratch[dev];
   if (!s.status) HIP_TRY(hipMalloc((void**)&s.status, sizeof(Status)));
   *out = &s;
+  return 0;
+}
+
+template <typename T>
+int grow(T** buf, int64_t* cap, int64_t need, hipStream_t stream) {
+  if (*cap >= need) return 0;
+  HIP_TRY(hipStreamSynchronize(stream));
+  HIP_TRY(hipDeviceSynchronize());
+  if (*buf) HIP_TRY(hipFree(*buf));
+  *buf = nullptr;
+  *cap = 0;
+  const int64_t n = std::max<int64_t>(need + need / 2, 4096);
+  HIP_TRY(hipMalloc((void**)buf, sizeof(T) * n));
+  *cap = n;
   return 0;
 }
 
@@ -152,6 +180,12 @@ int fbgemm_amd_status_read(const void* d_status, void* stream, int32_t* bits, in
   HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
   if (bits) *bits = h.bits;
   if (first_bad_pos) *first_bad_pos = h.first_bad_pos == ~0ull ? -1 : (int64_t)h.first_bad_pos;
+  return 0;
+}
+
+int fbgemm_amd_calibration_copy(const void* d_src, void* d_dst, int64_t bytes, void* stream) {
+  if (!d_src || !d_dst || bytes < 0 || bytes % 16) return fail(FBGEMM_AMD_E_ARG, "copy needs 16-byte multiples");
+  HIP_TRY(launch_calibration_copy(d_src, d_dst, bytes, (hipStream_t)stream));
   return 0;
 }
 
@@ -263,26 +297,28 @@ int fbgemm_amd_spmdm_launch(
   const int G = 64 / d.lanes;
   a.num_waves = (output_size + G - 1) / G;
 
+  // Ordering the bags pays once several waves' worth of bags exist.
+  const bool sort = sort_bags_default() && output_size > 2 * G;
   if (cfg->use_offsets) {
     a.offsets = d_offsets_or_lengths;
     a.off64 = cfg->offset_bits == 64;
-  } else {
+  }
+  if (!cfg->use_offsets || sort) {
+    // library-owned scratch: calls that use it must be ordered on one stream
     std::lock_guard<std::mutex> lk(g_mu);
     DeviceScratch* s;
     if (int rc = get_scratch(&s)) return rc;
-    if (s->offsets_cap < output_size + 1) {
-      // grow-only; the old buffer may still be read by an enqueued kernel
-      HIP_TRY(hipStreamSynchronize(stream));
-      if (s->offsets) HIP_TRY(hipFree(s->offsets));
-      s->offsets = nullptr;
-      s->offsets_cap = 0;
-      const int64_t cap = std::max<int64_t>(output_size + 1, 4096);
-      HIP_TRY(hipMalloc((void**)&s->offsets, sizeof(int64_t) * cap));
-      s->offsets_cap = cap;
+    if (!cfg->use_offsets) {
+      if (int rc = grow(&s->offsets, &s->offsets_cap, output_size + 1, stream)) return rc;
+      HIP_TRY(launch_lengths_to_offsets(d_offsets_or_lengths, cfg->offset_bits == 64, output_size, s->offsets, stream));
+      a.offsets = s->offsets;
+      a.off64 = 1;
     }
-    HIP_TRY(launch_lengths_to_offsets(d_offsets_or_lengths, cfg->offset_bits == 64, output_size, s->offsets, stream));
-    a.offsets = s->offsets;
-    a.off64 = 1;
+    if (sort) {
+      if (int rc = grow(&s->order, &s->order_cap, output_size, stream)) return rc;
+      HIP_TRY(launch_bag_order(a.offsets, a.off64, (int32_t)output_size, 1, s->order, stream));
+      a.order = s->order;
+    }
   }
   HIP_TRY(launch_lookup(a, cfg->index_bits == 64, stream));
   return 0;
@@ -323,6 +359,7 @@ struct fbgemm_amd_tbe_plan {
   // per-B work lists
   struct Work {
     WaveWork* d_work = nullptr;
+    int32_t* d_order = nullptr; // T*B bag ids, rewritten by every forward
     int64_t num_waves = 0;
   };
   std::map<int32_t, Work> work;
@@ -393,7 +430,10 @@ void fbgemm_amd_tbe_plan_destroy(fbgemm_amd_tbe_plan* plan) {
   if (!plan) return;
   (void)hipDeviceSynchronize();
   for (auto& kv : plan->work)
+  {
     if (kv.second.d_work) (void)hipFree(kv.second.d_work);
+    if (kv.second.d_order) (void)hipFree(kv.second.d_order);
+  }
   if (plan->d_tables) (void)hipFree(plan->d_tables);
   delete plan;
 }
@@ -441,6 +481,7 @@ int fbgemm_amd_tbe_forward(
       nw.num_waves = (int64_t)list.size();
       HIP_TRY(hipMalloc((void**)&nw.d_work, sizeof(WaveWork) * list.size()));
       HIP_TRY(hipMemcpy(nw.d_work, list.data(), sizeof(WaveWork) * list.size(), hipMemcpyHostToDevice));
+      HIP_TRY(hipMalloc((void**)&nw.d_order, sizeof(int32_t) * (size_t)plan->T * (size_t)B));
       it = plan->work.emplace(B, nw).first;
     }
     w = it->second;
@@ -468,6 +509,10 @@ int fbgemm_amd_tbe_forward(
   a.check_total = 0;
   a.out_aligned = (uintptr_t)d_output % 16 == 0;
   a.status = (Status*)d_status;
+  if (sort_bags_default()) {
+    HIP_TRY(launch_bag_order(d_offsets, index_bits == 64, B, plan->T, w.d_order, stream));
+    a.order = w.d_order;
+  }
   HIP_TRY(launch_lookup(a, index_bits == 64, stream));
   return 0;
 }

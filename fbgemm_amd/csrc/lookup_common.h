@@ -74,6 +74,8 @@ struct LookupArgs {
   void* out;
   int64_t out_stride;        // elements between consecutive bags' outputs
   int64_t index_size;        // entries the index array holds for this call
+  const int32_t* order;      // per table, its B bag ids in the order waves take them
+                             // (longest first), or nullptr: natural order
   const WaveWork* work;      // per-wave work list, or nullptr: single table, dense mapping
   int64_t num_waves;         // waves with work
   int32_t B;                 // bags per table

@@ -273,114 +273,226 @@ __device__ __forceinline__ int64_t read_offset(const void* p, bool is64, int64_t
   return is64 ? reinterpret_cast<const int64_t*>(p)[i] : (int64_t) reinterpret_cast<const int32_t*>(p)[i];
 }
 
-template <typename index_t, int TY, int VB, int U>
-__device__ __forceinline__ void pool_bags(const LookupArgs& a, const TableDesc& d, int table, int first_bag, int lane) {
+// What one staging lane leaves in LDS for the lanes that own the columns.
+struct __attribute__((aligned(16))) StageEntry {
+  int64_t off;  // byte offset of the row from the table's first row, or < 0: nothing to add
+  float scale;  // w * row scale (quantised rows) or w (fp16 / bf16 / fp32 rows)
+  float bias;   // w * row bias
+};
+
+constexpr int MAX_GROUPS = 32; // bags per wave at most; lanes per bag >= 2
+constexpr int MAX_ROUND = 8;
+constexpr int64_t NO_ENTRY = INT64_MIN;
+
+// One wave pools 64 / lanes bags of one table.
+//
+// Per-entry work (index load, per-sample weight, -1 / bounds / remap handling,
+// row offset, scale/bias fetch and the two products with the weight) is done
+// ONCE per entry by a staging lane and handed to the `lanes` column lanes of
+// the bag through LDS, instead of being repeated by each of them. Rounds of
+// ROUND entries per bag are software-pipelined: while round r is accumulated,
+// the scale/bias gathers of round r+1 (which also pull the row's first cache
+// line towards L2) and the index loads of round r+2 are in flight.
+template <typename index_t, int TY, int VB, int ROUND>
+__device__ __forceinline__ void pool_bags(const LookupArgs& a, const TableDesc& d, int table, int first_slot,
+                                          int lane, StageEntry* stage) {
   constexpr int BITS = type_bits(TY);
   constexpr int E = VB * 8 / BITS;
   constexpr int NW = (VB + 3) / 4;
   constexpr bool QUANT = TY == ST_INT8 || TY == ST_INT4 || TY == ST_INT2;
   constexpr bool ALIGNED = VB >= 4;
+  constexpr int MAXR = 2; // entries one staging lane handles per round, at most
 
   const int S = d.lanes;
   const int G = 64 / S;
   const int grp = lane / S;
   const int sub = lane - grp * S;
-  const int bag = first_bag + grp;
-  const bool bag_ok = grp < G && bag < a.B;
+  const int slot = first_slot + grp;
+  const bool bag_ok = grp < G && slot < a.B;
   const bool reporter = sub == 0;
+  // Entries staged per bag and round: ROUND, or half of it for bags that only
+  // have two or three lanes (each staging lane handles at most MAXR entries).
+  const int RN = S >= 4 ? ROUND : ROUND / 2;
+  const int SL = S >= RN ? RN : (S >= 4 ? 4 : 2); // staging lanes per bag (power of two, <= S)
+  const int R = RN / SL;                          // entries per staging lane per round
+  const bool stager = bag_ok && sub < SL;
+
+  // Bags are taken in the order the scheduler left them (longest first), so
+  // that the bags sharing a wave have nearly equal lengths.
+  int bag = slot;
+  if (bag_ok && a.order) bag = a.order[(int64_t)table * a.B + slot];
 
   // Positions are counted the way the reference counts `current`: relative to
   // the first offset of the table's slice.
-  int64_t pos0 = 0; // position of the bag's first entry in the index array
+  int64_t pos0 = 0;
   int64_t len = 0;
-  int64_t table_shift = 0; // what positions are relative to
   if (bag_ok) {
     const int64_t ob = (int64_t)table * a.B;
     const int64_t base = read_offset(a.offsets, a.off64, ob);
     const int64_t o0 = read_offset(a.offsets, a.off64, ob + bag);
     const int64_t o1 = read_offset(a.offsets, a.off64, ob + bag + 1);
-    table_shift = a.check_total ? 0 : base; // table-batched calls index the shared array
-    pos0 = o0 - base + table_shift;
+    pos0 = a.check_total ? o0 - base : o0; // table-batched calls index the shared array
     len = o1 - o0;
     if (len < 0) {
       if (reporter) report(a.status, ERR_NEGATIVE_LENGTH);
       len = 0;
     }
-    if (pos0 < 0 || pos0 + len > a.index_size) {
+    if (len > 0x7fffffffLL || pos0 < 0 || pos0 + len > a.index_size) {
       if (reporter) report(a.status, ERR_BAG_OVERRUN);
       len = 0;
     }
     if (a.check_total && bag == a.B - 1 && o1 - base != a.index_size && reporter)
       report(a.status, ERR_LENGTH_MISMATCH);
   }
+  const int n = (int)len; // same for every lane of the bag
 
   const index_t* idx = reinterpret_cast<const index_t*>(a.indices);
   const uint8_t* wbase = (d.placement ? a.weights[1] : a.weights[0]) + d.weights_offset;
+  const uint8_t* psb = wbase + d.sb_off;
+  StageEntry* my = stage + grp * RN;
   // the reference keeps the bag length in an int when it forms 1/len
-  const float inv_len = (a.normalize && len > 0) ? 1.0f / (float)(int)len : 1.0f;
+  const float inv_len = (a.normalize && n > 0) ? 1.0f / (float)n : 1.0f;
 
   for (int pass = 0; pass < d.passes; ++pass) {
     const int chunk = pass * S + sub;
     const int byte_off = chunk * VB;
     const bool lane_on = bag_ok && byte_off < d.data_bytes;
-    const int n = lane_on ? (int)len : 0;
     const uint8_t* pdata = wbase + d.data_off + byte_off;
-    const uint8_t* psb = wbase + d.sb_off;
 
     float acc[E];
 #pragma unroll
     for (int e = 0; e < E; ++e) acc[e] = 0.0f;
 
-    for (int i = 0; i < n; i += U) {
-      uint32_t raw[U][NW];
-      float s[U], b[U];
-      bool ok[U];
+    // registers of the staging pipeline
+    int64_t nrow[MAXR]; // raw index of the round whose loads are in flight
+    float nw[MAXR];
+    int64_t coff[MAXR]; // row offset / weight / raw scale+bias of the round being staged
+    float cw[MAXR];
+    uint32_t h0[MAXR], h1[MAXR];
+
+    auto load_idx = [&](int round) {
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
-        ok[u] = i + u < n;
-        int64_t row = 0;
-        if (ok[u]) {
-          const int64_t pos = pos0 + i + u;
-          row = (int64_t)idx[pos];
+      for (int rr = 0; rr < MAXR; ++rr) {
+        nrow[rr] = NO_ENTRY;
+        nw[rr] = 1.0f;
+        const int i = round * RN + sub + rr * SL;
+        if (rr < R && stager && i < n) {
+          nrow[rr] = (int64_t)idx[pos0 + i];
+          if (a.sample_weights) nw[rr] = a.sample_weights[a.positional ? (int64_t)i : pos0 + i];
+        }
+      }
+    };
+    // index -> row offset (or "nothing to add"), then fetch the row's scale/bias
+    auto stage_gather = [&](int round) {
+#pragma unroll
+      for (int rr = 0; rr < MAXR; ++rr) {
+        int64_t row = nrow[rr];
+        int64_t off = -1;
+        if (rr < R && row != NO_ENTRY) {
+          const int64_t pos = pos0 + round * RN + sub + rr * SL;
+          bool ok = true;
           if (a.remap) {
             if (row < 0 || row >= a.remap_rows) {
-              if (reporter && pass == 0) report_index(a.status, pos);
-              ok[u] = false;
+              if (pass == 0) report_index(a.status, pos);
+              ok = false;
             } else {
               row = (int64_t)a.remap[row];
-              if (row == -1) ok[u] = false;
+              ok = row != -1;
             }
           } else if (d.skip_minus_one && row == -1) {
-            ok[u] = false;
+            ok = false;
           } else if (row < 0 || row >= d.num_rows) {
-            if (reporter && pass == 0) report_index(a.status, pos);
-            ok[u] = false;
+            if (pass == 0) report_index(a.status, pos);
+            ok = false;
+          }
+          if (ok) {
+            off = row * d.row_stride;
+            if constexpr (QUANT) {
+              if (d.sb_fp32) {
+                if constexpr (ALIGNED) {
+                  const Dwordx2 v = *reinterpret_cast<const Dwordx2*>(psb + off);
+                  h0[rr] = v.v[0]; h1[rr] = v.v[1];
+                } else {
+                  const Bytes8 v = *reinterpret_cast<const Bytes8*>(psb + off);
+                  h0[rr] = v.v[0] | (v.v[1] << 8) | (v.v[2] << 16) | ((uint32_t)v.v[3] << 24);
+                  h1[rr] = v.v[4] | (v.v[5] << 8) | (v.v[6] << 16) | ((uint32_t)v.v[7] << 24);
+                }
+              } else {
+                if constexpr (ALIGNED) {
+                  h0[rr] = *reinterpret_cast<const uint32_t*>(psb + off);
+                } else {
+                  const Bytes4 v = *reinterpret_cast<const Bytes4*>(psb + off);
+                  h0[rr] = v.v[0] | (v.v[1] << 8) | (v.v[2] << 16) | ((uint32_t)v.v[3] << 24);
+                }
+              }
+            }
           }
         }
-        if (ok[u]) {
-          const int64_t roff = row * d.row_stride;
-          load_raw<VB>(raw[u], pdata + roff);
-          float w = 1.0f;
-          if (a.sample_weights) w = a.sample_weights[a.positional ? (i + u) : (pos0 + i + u)];
-          if constexpr (QUANT) {
-            float rs, rb;
-            load_scale_bias(psb + roff, d.sb_fp32, ALIGNED, rs, rb);
-            s[u] = w * rs;
-            b[u] = w * rb;
-          } else {
-            s[u] = w;
-            b[u] = 0.0f;
-          }
-        }
+        coff[rr] = off;
+        cw[rr] = nw[rr];
       }
+    };
+    auto stage_publish = [&]() {
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
-        if (ok[u]) Accum<TY, VB>::run(acc, raw[u], s[u], b[u]);
+      for (int rr = 0; rr < MAXR; ++rr) {
+        if (rr < R && stager) {
+          StageEntry ent;
+          ent.off = coff[rr];
+          ent.scale = cw[rr];
+          ent.bias = 0.0f;
+          if constexpr (QUANT) {
+            if (coff[rr] >= 0) {
+              const float rs = d.sb_fp32 ? bits_to_float(h0[rr]) : half_lo(h0[rr]);
+              const float rb = d.sb_fp32 ? bits_to_float(h1[rr]) : half_hi(h0[rr]);
+              ent.scale = cw[rr] * rs;
+              ent.bias = cw[rr] * rb;
+            }
+          }
+          my[sub + rr * SL] = ent;
+        }
       }
+    };
+
+    load_idx(0);
+    stage_gather(0);
+    load_idx(1);
+    stage_publish();
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+
+    for (int r = 0; r * RN < n; ++r) {
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      // this round's entries, then the row loads
+      float sc[ROUND], bi[ROUND];
+      uint32_t raw[ROUND][NW];
+      uint32_t valid = 0;
+      const int left = min(n - r * RN, RN);
+#pragma unroll
+      for (int e = 0; e < ROUND; ++e) {
+        if (e < left) {
+          const StageEntry ent = my[e];
+          sc[e] = ent.scale;
+          bi[e] = ent.bias;
+          if (lane_on && ent.off >= 0) {
+            valid |= 1u << e;
+            load_raw<VB>(raw[e], pdata + ent.off);
+          }
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
+      stage_gather(r + 1);
+      load_idx(r + 2);
+#pragma unroll
+      for (int e = 0; e < ROUND; ++e) {
+        if (valid & (1u << e)) Accum<TY, VB>::run(acc, raw[e], sc[e], bi[e]);
+      }
+      stage_publish();
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
     }
 
     if (lane_on) {
-      if (a.normalize && len > 0) {
+      if (a.normalize && n > 0) {
 #pragma unroll
         for (int e = 0; e < E; ++e) acc[e] *= inv_len;
       }
@@ -393,21 +505,23 @@ __device__ __forceinline__ void pool_bags(const LookupArgs& a, const TableDesc& 
 }
 
 template <typename index_t, int TY>
-__device__ __forceinline__ void pool_dispatch_vb(const LookupArgs& a, const TableDesc& d, int table, int first_bag, int lane) {
+__device__ __forceinline__ void pool_dispatch_vb(const LookupArgs& a, const TableDesc& d, int table, int first_slot,
+                                                 int lane, StageEntry* stage) {
   constexpr int BITS = type_bits(TY);
   constexpr int MINVB = BITS >= 16 ? BITS / 8 : 1;
   if (d.vb == 16) {
-    if constexpr (TY == ST_INT2) pool_bags<index_t, TY, 4, 8>(a, d, table, first_bag, lane); // not selected by the host
-    else pool_bags<index_t, TY, 16, 4>(a, d, table, first_bag, lane);
+    if constexpr (TY == ST_INT2) pool_bags<index_t, TY, 4, 8>(a, d, table, first_slot, lane, stage); // not selected by the host
+    else pool_bags<index_t, TY, 16, 8>(a, d, table, first_slot, lane, stage);
   } else if (d.vb == 4) {
-    pool_bags<index_t, TY, 4, 8>(a, d, table, first_bag, lane);
+    pool_bags<index_t, TY, 4, 8>(a, d, table, first_slot, lane, stage);
   } else {
-    pool_bags<index_t, TY, MINVB, 4>(a, d, table, first_bag, lane);
+    pool_bags<index_t, TY, MINVB, 8>(a, d, table, first_slot, lane, stage);
   }
 }
 
 template <typename index_t>
 __global__ __launch_bounds__(256) void lookup_kernel(const LookupArgs a) {
+  __shared__ StageEntry stage_all[4][MAX_GROUPS * MAX_ROUND];
   const int lane = threadIdx.x & 63;
   int64_t blk = blockIdx.x;
   if (a.xcd_swizzle) {
@@ -419,25 +533,71 @@ __global__ __launch_bounds__(256) void lookup_kernel(const LookupArgs a) {
     const int64_t x = blk & 7;
     blk = x * q + (x < r ? x : r) + (blk >> 3);
   }
-  const int64_t wave = blk * 4 + __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int wid = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int64_t wave = blk * 4 + wid;
   if (wave >= a.num_waves) return;
-  int table = 0, first_bag;
+  StageEntry* stage = stage_all[wid];
+  int table = 0, first_slot;
   if (a.work) {
     const WaveWork ww = a.work[wave];
     table = ww.table;
-    first_bag = ww.first_bag;
+    first_slot = ww.first_bag;
   } else {
-    first_bag = (int)(wave * (64 / a.single.lanes));
+    first_slot = (int)(wave * (64 / a.single.lanes));
   }
   const TableDesc d = a.tables ? a.tables[table] : a.single;
   switch (d.ty) {
-    case ST_INT4: pool_dispatch_vb<index_t, ST_INT4>(a, d, table, first_bag, lane); break;
-    case ST_INT8: pool_dispatch_vb<index_t, ST_INT8>(a, d, table, first_bag, lane); break;
-    case ST_FP16: pool_dispatch_vb<index_t, ST_FP16>(a, d, table, first_bag, lane); break;
-    case ST_INT2: pool_dispatch_vb<index_t, ST_INT2>(a, d, table, first_bag, lane); break;
-    case ST_FP32: pool_dispatch_vb<index_t, ST_FP32>(a, d, table, first_bag, lane); break;
-    case ST_BF16: pool_dispatch_vb<index_t, ST_BF16>(a, d, table, first_bag, lane); break;
+    case ST_INT4: pool_dispatch_vb<index_t, ST_INT4>(a, d, table, first_slot, lane, stage); break;
+    case ST_INT8: pool_dispatch_vb<index_t, ST_INT8>(a, d, table, first_slot, lane, stage); break;
+    case ST_FP16: pool_dispatch_vb<index_t, ST_FP16>(a, d, table, first_slot, lane, stage); break;
+    case ST_INT2: pool_dispatch_vb<index_t, ST_INT2>(a, d, table, first_slot, lane, stage); break;
+    case ST_FP32: pool_dispatch_vb<index_t, ST_FP32>(a, d, table, first_slot, lane, stage); break;
+    case ST_BF16: pool_dispatch_vb<index_t, ST_BF16>(a, d, table, first_slot, lane, stage); break;
     default: break;
+  }
+}
+
+// ---- bag scheduler -------------------------------------------------------------
+//
+// One workgroup per table orders the table's bags by length, longest first
+// (counting sort over lengths, lengths >= SORT_BINS - 1 share the first bin).
+// Waves then take consecutive runs of the order, so the bags a wave pools side
+// by side need the same number of rounds and no lane idles behind a long
+// neighbour. Ties are placed in arrival order of the LDS atomics: the order
+// may differ between runs, the results cannot (each bag is summed on its own).
+constexpr int SORT_BINS = 1024;
+
+__global__ __launch_bounds__(1024) void bag_order_kernel(const void* offsets, int off64, int32_t B, int32_t* order) {
+  __shared__ int bins[SORT_BINS];
+  __shared__ int partial[1024];
+  const int t = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int64_t ob = (int64_t)t * B;
+  for (int i = tid; i < SORT_BINS; i += 1024) bins[i] = 0;
+  __syncthreads();
+  auto bin_of = [&](int b) {
+    int64_t len = read_offset(offsets, off64, ob + b + 1) - read_offset(offsets, off64, ob + b);
+    if (len < 0) len = 0;
+    if (len > SORT_BINS - 1) len = SORT_BINS - 1;
+    return SORT_BINS - 1 - (int)len; // longest first
+  };
+  for (int b = tid; b < B; b += 1024) atomicAdd(&bins[bin_of(b)], 1);
+  __syncthreads();
+  // exclusive scan of the SORT_BINS (== blockDim) counters
+  const int mine = bins[tid];
+  partial[tid] = mine;
+  __syncthreads();
+  for (int step = 1; step < 1024; step <<= 1) {
+    const int v = tid >= step ? partial[tid - step] : 0;
+    __syncthreads();
+    partial[tid] += v;
+    __syncthreads();
+  }
+  bins[tid] = partial[tid] - mine;
+  __syncthreads();
+  for (int b = tid; b < B; b += 1024) {
+    const int p = atomicAdd(&bins[bin_of(b)], 1);
+    order[ob + p] = b;
   }
 }
 
@@ -493,7 +653,21 @@ __global__ __launch_bounds__(256) void pruned_array_lookup_kernel(
   }
 }
 
+// Plain 16-byte-per-lane copy of a known size: the yardstick hardware byte
+// counters are scaled against.
+__global__ __launch_bounds__(256) void calibration_copy_kernel(const uint4* src, uint4* dst, int64_t n16) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (int64_t)gridDim.x * blockDim.x)
+    dst[i] = src[i];
+}
+
 // ---- launchers (called from the C ABI) ---------------------------------------
+
+hipError_t launch_calibration_copy(const void* src, void* dst, int64_t bytes, hipStream_t stream) {
+  const int64_t n16 = bytes / 16;
+  if (n16 <= 0) return hipSuccess;
+  hipLaunchKernelGGL(calibration_copy_kernel, dim3(256 * 16), dim3(256), 0, stream, (const uint4*)src, (uint4*)dst, n16);
+  return hipGetLastError();
+}
 
 hipError_t launch_lookup(const LookupArgs& a, bool idx64, hipStream_t stream) {
   if (a.num_waves <= 0) return hipSuccess;
@@ -501,6 +675,12 @@ hipError_t launch_lookup(const LookupArgs& a, bool idx64, hipStream_t stream) {
   if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
   if (idx64) hipLaunchKernelGGL(lookup_kernel<int64_t>, dim3((unsigned)blocks), dim3(256), 0, stream, a);
   else hipLaunchKernelGGL(lookup_kernel<int32_t>, dim3((unsigned)blocks), dim3(256), 0, stream, a);
+  return hipGetLastError();
+}
+
+hipError_t launch_bag_order(const void* offsets, bool off64, int32_t B, int32_t T, int32_t* order, hipStream_t stream) {
+  if (T <= 0 || B <= 0) return hipSuccess;
+  hipLaunchKernelGGL(bag_order_kernel, dim3((unsigned)T), dim3(1024), 0, stream, offsets, off64 ? 1 : 0, B, order);
   return hipGetLastError();
 }
 

@@ -1,0 +1,61 @@
+"""Condense rocprofv3 CSV output into a few lines per kernel of this library.
+
+    python -m fbgemm_amd.profile_summary <rocprofv3 output dir> [more dirs...]
+
+Prints, for every kernel whose name contains ``lookup_kernel`` or
+``calibration_copy_kernel`` (and the totals row of --stats), the call count and
+average duration, and the per-dispatch average of every hardware counter
+collected. Raw CSVs hold every torch kernel of the run and are large; this is
+the part worth keeping.
+"""
+import csv
+import glob
+import os
+import sys
+from collections import defaultdict
+
+OURS = ("lookup_kernel", "calibration_copy_kernel", "lengths_to_offsets", "pruned_array_lookup")
+
+
+def short(name):
+    for k in OURS:
+        if k in name:
+            return k + ("<int64>" if "IlE" in name else "<int32>" if "IiE" in name else "")
+    return None
+
+
+def summarize(d):
+    lines = []
+    for f in sorted(glob.glob(os.path.join(d, "**", "*kernel_stats.csv"), recursive=True)):
+        with open(f) as fh:
+            for row in csv.DictReader(fh):
+                s = short(row.get("Name", ""))
+                if s:
+                    lines.append(f"stats  {s}: calls={row.get('Calls')} avg_ns={row.get('AverageNs')} "
+                                 f"min_ns={row.get('MinNs')} max_ns={row.get('MaxNs')} pct={row.get('Percentage')}")
+    for f in sorted(glob.glob(os.path.join(d, "**", "*counter_collection.csv"), recursive=True)):
+        acc = defaultdict(lambda: [0.0, 0])
+        grid = {}
+        with open(f) as fh:
+            for row in csv.DictReader(fh):
+                s = short(row.get("Kernel_Name", ""))
+                if not s:
+                    continue
+                key = (s, row.get("Counter_Name"))
+                acc[key][0] += float(row.get("Counter_Value", 0))
+                acc[key][1] += 1
+                grid[s] = (row.get("Grid_Size"), row.get("Workgroup_Size"), row.get("VGPR_Count"),
+                           row.get("Accum_VGPR_Count"), row.get("SGPR_Count"), row.get("LDS_Block_Size"),
+                           row.get("Scratch_Size"))
+        for (s, c), (tot, n) in sorted(acc.items()):
+            lines.append(f"pmc    {s}: {c} avg_per_dispatch={tot / n:.6g} dispatches={n}")
+        for s, g in sorted(grid.items()):
+            lines.append(f"launch {s}: grid={g[0]} wg={g[1]} vgpr={g[2]} agpr={g[3]} sgpr={g[4]} lds={g[5]} scratch={g[6]}")
+    return lines
+
+
+if __name__ == "__main__":
+    for d in sys.argv[1:]:
+        print(f"# {d}")
+        for l in summarize(d):
+            print(l)

@@ -171,6 +171,13 @@ int fbgemm_amd_pruned_array_lookup(
     const int64_t* d_index_remappings_offsets, int32_t T, void* d_dense,
     void* stream);
 
+/* ---- measurement aid -------------------------------------------------------- *
+ * No counterpart in the reference. A plain device-to-device copy of `bytes`
+ * (a multiple of 16) by a kernel named calibration_copy_kernel: profiles scale
+ * the hardware byte counters of the lookup kernel against what the same
+ * counters read for this copy of known size. */
+int fbgemm_amd_calibration_copy(const void* d_src, void* d_dst, int64_t bytes, void* stream);
+
 /* ---- row-size arithmetic (host, no GPU) ------------------------------------ *
  * embedding_common.h:189-225. */
 int32_t fbgemm_amd_unpadded_row_size_in_bytes(int32_t dim, int32_t weight_ty, int32_t scale_bias_bytes);
