@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <cmath>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -64,10 +65,6 @@ int env_int(const char* name, int dflt) {
 
 // Tunables, read once per process (the reference reads its FBGEMM_* switches
 // the same way, src/Utils.cc:773-875).
-int xcd_swizzle_default() {
-  static int v = env_int("FBGEMM_AMD_XCD_SWIZZLE", 0);
-  return v;
-}
 
 // 1: order each table's bags by length on the device before the lookup.
 int sort_bags_default() {
@@ -290,7 +287,6 @@ int fbgemm_amd_spmdm_launch(
   a.out_ty = cfg->output_ty;
   a.normalize = cfg->normalize_by_lengths;
   a.positional = cfg->is_weight_positional;
-  a.xcd_swizzle = 0;
   a.check_total = 1;
   a.out_aligned = (uintptr_t)d_out % 16 == 0;
   a.status = (Status*)d_status;
@@ -360,6 +356,7 @@ struct fbgemm_amd_tbe_plan {
   struct Work {
     WaveWork* d_work = nullptr;
     int32_t* d_order = nullptr; // T*B bag ids, rewritten by every forward
+    int64_t* d_xcd_start = nullptr;
     int64_t num_waves = 0;
   };
   std::map<int32_t, Work> work;
@@ -433,6 +430,7 @@ void fbgemm_amd_tbe_plan_destroy(fbgemm_amd_tbe_plan* plan) {
   {
     if (kv.second.d_work) (void)hipFree(kv.second.d_work);
     if (kv.second.d_order) (void)hipFree(kv.second.d_order);
+    if (kv.second.d_xcd_start) (void)hipFree(kv.second.d_xcd_start);
   }
   if (plan->d_tables) (void)hipFree(plan->d_tables);
   delete plan;
@@ -472,15 +470,69 @@ int fbgemm_amd_tbe_forward(
     std::lock_guard<std::mutex> lk(plan->mu);
     auto it = plan->work.find(B);
     if (it == plan->work.end()) {
-      std::vector<WaveWork> list;
+      // The work list is 8 runs, one per XCD (see lookup_kernel). Tables are
+      // cut into slices of waves, the slices are dealt to the XCDs so that
+      // every XCD gets the same number of 128-byte line requests (what the
+      // memory system charges for), and inside a run every slice advances
+      // through its bag order (longest first) at the same relative pace, so
+      // that tables of different row types share the CUs at all times.
+      static const int xcd_lists = env_int("FBGEMM_AMD_XCD_LISTS", 1);
+      struct Slice { int t, first, step, count; double cost; };
+      std::vector<Slice> slices;
+      double total_cost = 0;
+      std::vector<double> wave_cost(plan->T);
+      std::vector<int> nwaves(plan->T);
       for (int t = 0; t < plan->T; ++t) {
-        const int G = 64 / plan->tables[t].lanes;
-        for (int32_t fb = 0; fb < B; fb += G) list.push_back(WaveWork{t, fb});
+        const TableDesc& d = plan->tables[t];
+        const int G = 64 / d.lanes;
+        nwaves[t] = (B + G - 1) / G;
+        const double lines = 1.0 + (double)(d.row_stride - 1) / 128.0; // expected lines a row touches
+        wave_cost[t] = G * (lines + 0.25);
+        total_cost += wave_cost[t] * nwaves[t];
       }
+      const int nx = xcd_lists ? 8 : 1;
+      for (int t = 0; t < plan->T; ++t) {
+        // slices no larger than 1/4 of an XCD's share; slice p takes waves p, p + parts, ...
+        int parts = (int)std::ceil(wave_cost[t] * nwaves[t] / (total_cost / nx / 4.0 + 1e-9));
+        parts = std::max(1, std::min(parts, std::min(nwaves[t], nx)));
+        for (int p = 0; p < parts; ++p) {
+          const int count = (nwaves[t] - p + parts - 1) / parts;
+          slices.push_back(Slice{t, p, parts, count, wave_cost[t] * count});
+        }
+      }
+      std::stable_sort(slices.begin(), slices.end(), [](const Slice& x, const Slice& y) { return x.cost > y.cost; });
+      std::vector<std::vector<Slice>> per_x(nx);
+      std::vector<double> load(nx, 0.0);
+      for (const Slice& sl : slices) {
+        const int x = (int)(std::min_element(load.begin(), load.end()) - load.begin());
+        per_x[x].push_back(sl);
+        load[x] += sl.cost;
+      }
+      std::vector<WaveWork> list;
+      std::vector<int64_t> xcd_start(9, 0);
+      int64_t longest = 0;
+      for (int x = 0; x < nx; ++x) {
+        std::vector<std::pair<double, WaveWork>> keyed;
+        for (const Slice& sl : per_x[x]) {
+          const int G = 64 / plan->tables[sl.t].lanes;
+          for (int k = 0; k < sl.count; ++k)
+            keyed.push_back({(k + 0.5) / sl.count, WaveWork{sl.t, (sl.first + k * sl.step) * G}});
+        }
+        std::stable_sort(keyed.begin(), keyed.end(),
+                         [](const std::pair<double, WaveWork>& p, const std::pair<double, WaveWork>& q) { return p.first < q.first; });
+        for (auto& kv : keyed) list.push_back(kv.second);
+        xcd_start[x + 1] = (int64_t)list.size();
+        longest = std::max<int64_t>(longest, (int64_t)keyed.size());
+      }
+      for (int x = nx; x < 8; ++x) xcd_start[x + 1] = xcd_start[nx];
       fbgemm_amd_tbe_plan::Work nw;
-      nw.num_waves = (int64_t)list.size();
+      nw.num_waves = xcd_lists ? longest : (int64_t)list.size();
       HIP_TRY(hipMalloc((void**)&nw.d_work, sizeof(WaveWork) * list.size()));
       HIP_TRY(hipMemcpy(nw.d_work, list.data(), sizeof(WaveWork) * list.size(), hipMemcpyHostToDevice));
+      if (xcd_lists) {
+        HIP_TRY(hipMalloc((void**)&nw.d_xcd_start, sizeof(int64_t) * 9));
+        HIP_TRY(hipMemcpy(nw.d_xcd_start, xcd_start.data(), sizeof(int64_t) * 9, hipMemcpyHostToDevice));
+      }
       HIP_TRY(hipMalloc((void**)&nw.d_order, sizeof(int32_t) * (size_t)plan->T * (size_t)B));
       it = plan->work.emplace(B, nw).first;
     }
@@ -500,12 +552,12 @@ int fbgemm_amd_tbe_forward(
   a.out_stride = plan->total_D;
   a.index_size = indices_numel;
   a.work = w.d_work;
+  a.xcd_start = w.d_xcd_start;
   a.num_waves = w.num_waves;
   a.B = B;
   a.T = plan->T;
   a.out_ty = output_ty;
   a.normalize = pooling_mode == FBGEMM_AMD_POOL_MEAN;
-  a.xcd_swizzle = xcd_swizzle_default();
   a.check_total = 0;
   a.out_aligned = (uintptr_t)d_output % 16 == 0;
   a.status = (Status*)d_status;

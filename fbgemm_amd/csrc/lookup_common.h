@@ -77,14 +77,16 @@ struct LookupArgs {
   const int32_t* order;      // per table, its B bag ids in the order waves take them
                              // (longest first), or nullptr: natural order
   const WaveWork* work;      // per-wave work list, or nullptr: single table, dense mapping
-  int64_t num_waves;         // waves with work
+  const int64_t* xcd_start;  // 9 entries: the work list is 8 runs, run x = [xcd_start[x],
+                             // xcd_start[x+1]) is walked by the workgroups with id % 8 == x
+                             // (the workgroups one XCD receives); nullptr: one run
+  int64_t num_waves;         // waves with work (longest run when xcd_start is used)
   int32_t B;                 // bags per table
   int32_t T;
   int32_t out_ty;            // ST_FP32, ST_FP16 or ST_BF16
   int32_t off64;             // offsets are int64 (else int32)
   int32_t normalize;         // mean pooling: scale by 1/len, len counting skipped rows
   int32_t positional;        // weight of entry i of a bag is sample_weights[i]
-  int32_t xcd_swizzle;       // remap block ids so that each XCD walks contiguous work
   int32_t check_total;       // single-table call: positions are relative to offsets[0] and
                              // offsets[last] - offsets[0] must equal index_size
   int32_t out_aligned;       // `out` is 16-byte aligned (vector stores allowed)

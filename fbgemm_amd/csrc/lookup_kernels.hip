@@ -273,29 +273,36 @@ __device__ __forceinline__ int64_t read_offset(const void* p, bool is64, int64_t
   return is64 ? reinterpret_cast<const int64_t*>(p)[i] : (int64_t) reinterpret_cast<const int32_t*>(p)[i];
 }
 
-// What one staging lane leaves in LDS for the lanes that own the columns.
-struct __attribute__((aligned(16))) StageEntry {
-  int64_t off;  // byte offset of the row from the table's first row, or < 0: nothing to add
-  float scale;  // w * row scale (quantised rows) or w (fp16 / bf16 / fp32 rows)
-  float bias;   // w * row bias
+// What one staging lane leaves in LDS for the lanes that own the columns:
+// where the row is, and what to multiply it with.
+struct __attribute__((aligned(8))) StageRow {
+  int64_t off; // byte offset of the row from the table's first row, or < 0: nothing to add
+};
+struct __attribute__((aligned(8))) StageMul {
+  float scale; // w * row scale (quantised rows) or w (fp16 / bf16 / fp32 rows)
+  float bias;  // w * row bias
 };
 
 constexpr int MAX_GROUPS = 32; // bags per wave at most; lanes per bag >= 2
 constexpr int MAX_ROUND = 8;
 constexpr int64_t NO_ENTRY = INT64_MIN;
 
-// One wave pools 64 / lanes bags of one table.
+// One wave pools 64 / lanes bags of one table, `RN` entries of every bag per
+// round.
 //
 // Per-entry work (index load, per-sample weight, -1 / bounds / remap handling,
-// row offset, scale/bias fetch and the two products with the weight) is done
-// ONCE per entry by a staging lane and handed to the `lanes` column lanes of
-// the bag through LDS, instead of being repeated by each of them. Rounds of
-// ROUND entries per bag are software-pipelined: while round r is accumulated,
-// the scale/bias gathers of round r+1 (which also pull the row's first cache
-// line towards L2) and the index loads of round r+2 are in flight.
+// row offset, the scale/bias fetch and its two products with the weight) is
+// done ONCE per entry by a staging lane and handed to the `lanes` column lanes
+// of the bag through LDS, instead of being repeated by each of them.
+//
+// The memory system charges per 128-byte line request, so a row's scale/bias
+// must not cost a request of its own: the staging lane loads them in the same
+// round, immediately before the column lanes load the row's data, and the two
+// accesses to the row's first line merge in the L1. While the loads are in
+// flight the indices of the next round are fetched.
 template <typename index_t, int TY, int VB, int ROUND>
 __device__ __forceinline__ void pool_bags(const LookupArgs& a, const TableDesc& d, int table, int first_slot,
-                                          int lane, StageEntry* stage) {
+                                          int lane, StageRow* stage_row, StageMul* stage_mul) {
   constexpr int BITS = type_bits(TY);
   constexpr int E = VB * 8 / BITS;
   constexpr int NW = (VB + 3) / 4;
@@ -349,7 +356,8 @@ __device__ __forceinline__ void pool_bags(const LookupArgs& a, const TableDesc& 
   const index_t* idx = reinterpret_cast<const index_t*>(a.indices);
   const uint8_t* wbase = (d.placement ? a.weights[1] : a.weights[0]) + d.weights_offset;
   const uint8_t* psb = wbase + d.sb_off;
-  StageEntry* my = stage + grp * RN;
+  StageRow* my_row = stage_row + grp * RN;
+  StageMul* my_mul = stage_mul + grp * RN;
   // the reference keeps the bag length in an int when it forms 1/len
   const float inv_len = (a.normalize && n > 0) ? 1.0f / (float)n : 1.0f;
 
@@ -363,12 +371,11 @@ __device__ __forceinline__ void pool_bags(const LookupArgs& a, const TableDesc& 
 #pragma unroll
     for (int e = 0; e < E; ++e) acc[e] = 0.0f;
 
-    // registers of the staging pipeline
-    int64_t nrow[MAXR]; // raw index of the round whose loads are in flight
+    // registers of the staging lanes
+    int64_t nrow[MAXR]; // raw index of the next round (loads in flight)
     float nw[MAXR];
-    int64_t coff[MAXR]; // row offset / weight / raw scale+bias of the round being staged
+    int64_t coff[MAXR]; // row offset and weight of the round being pooled
     float cw[MAXR];
-    uint32_t h0[MAXR], h1[MAXR];
 
     auto load_idx = [&](int round) {
 #pragma unroll
@@ -382,8 +389,8 @@ __device__ __forceinline__ void pool_bags(const LookupArgs& a, const TableDesc& 
         }
       }
     };
-    // index -> row offset (or "nothing to add"), then fetch the row's scale/bias
-    auto stage_gather = [&](int round) {
+    // index -> row offset, or "nothing to add"; publish the offsets of `round`
+    auto stage_rows = [&](int round) {
 #pragma unroll
       for (int rr = 0; rr < MAXR; ++rr) {
         int64_t row = nrow[rr];
@@ -405,88 +412,103 @@ __device__ __forceinline__ void pool_bags(const LookupArgs& a, const TableDesc& 
             if (pass == 0) report_index(a.status, pos);
             ok = false;
           }
-          if (ok) {
-            off = row * d.row_stride;
-            if constexpr (QUANT) {
-              if (d.sb_fp32) {
-                if constexpr (ALIGNED) {
-                  const Dwordx2 v = *reinterpret_cast<const Dwordx2*>(psb + off);
-                  h0[rr] = v.v[0]; h1[rr] = v.v[1];
-                } else {
-                  const Bytes8 v = *reinterpret_cast<const Bytes8*>(psb + off);
-                  h0[rr] = v.v[0] | (v.v[1] << 8) | (v.v[2] << 16) | ((uint32_t)v.v[3] << 24);
-                  h1[rr] = v.v[4] | (v.v[5] << 8) | (v.v[6] << 16) | ((uint32_t)v.v[7] << 24);
-                }
-              } else {
-                if constexpr (ALIGNED) {
-                  h0[rr] = *reinterpret_cast<const uint32_t*>(psb + off);
-                } else {
-                  const Bytes4 v = *reinterpret_cast<const Bytes4*>(psb + off);
-                  h0[rr] = v.v[0] | (v.v[1] << 8) | (v.v[2] << 16) | ((uint32_t)v.v[3] << 24);
-                }
-              }
-            }
-          }
+          if (ok) off = row * d.row_stride;
         }
         coff[rr] = off;
         cw[rr] = nw[rr];
-      }
-    };
-    auto stage_publish = [&]() {
-#pragma unroll
-      for (int rr = 0; rr < MAXR; ++rr) {
         if (rr < R && stager) {
-          StageEntry ent;
-          ent.off = coff[rr];
-          ent.scale = cw[rr];
-          ent.bias = 0.0f;
-          if constexpr (QUANT) {
-            if (coff[rr] >= 0) {
-              const float rs = d.sb_fp32 ? bits_to_float(h0[rr]) : half_lo(h0[rr]);
-              const float rb = d.sb_fp32 ? bits_to_float(h1[rr]) : half_hi(h0[rr]);
-              ent.scale = cw[rr] * rs;
-              ent.bias = cw[rr] * rb;
-            }
+          my_row[sub + rr * SL].off = off;
+          if constexpr (!QUANT) {
+            StageMul m;
+            m.scale = nw[rr];
+            m.bias = 0.0f;
+            my_mul[sub + rr * SL] = m;
           }
-          my[sub + rr * SL] = ent;
         }
       }
     };
 
     load_idx(0);
-    stage_gather(0);
-    load_idx(1);
-    stage_publish();
+    stage_rows(0);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
 
     for (int r = 0; r * RN < n; ++r) {
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-      // this round's entries, then the row loads
-      float sc[ROUND], bi[ROUND];
       uint32_t raw[ROUND][NW];
+      uint32_t h0[MAXR], h1[MAXR];
       uint32_t valid = 0;
       const int left = min(n - r * RN, RN);
+      // scale/bias first, so that their wait does not cover the row loads
+      if constexpr (QUANT) {
 #pragma unroll
-      for (int e = 0; e < ROUND; ++e) {
-        if (e < left) {
-          const StageEntry ent = my[e];
-          sc[e] = ent.scale;
-          bi[e] = ent.bias;
-          if (lane_on && ent.off >= 0) {
-            valid |= 1u << e;
-            load_raw<VB>(raw[e], pdata + ent.off);
+        for (int rr = 0; rr < MAXR; ++rr) {
+          if (rr < R && stager && coff[rr] >= 0) {
+            const uint8_t* p = psb + coff[rr];
+            if (d.sb_fp32) {
+              if constexpr (ALIGNED) {
+                const Dwordx2 v = *reinterpret_cast<const Dwordx2*>(p);
+                h0[rr] = v.v[0]; h1[rr] = v.v[1];
+              } else {
+                const Bytes8 v = *reinterpret_cast<const Bytes8*>(p);
+                h0[rr] = v.v[0] | (v.v[1] << 8) | (v.v[2] << 16) | ((uint32_t)v.v[3] << 24);
+                h1[rr] = v.v[4] | (v.v[5] << 8) | (v.v[6] << 16) | ((uint32_t)v.v[7] << 24);
+              }
+            } else {
+              if constexpr (ALIGNED) {
+                h0[rr] = *reinterpret_cast<const uint32_t*>(p);
+              } else {
+                const Bytes4 v = *reinterpret_cast<const Bytes4*>(p);
+                h0[rr] = v.v[0] | (v.v[1] << 8) | (v.v[2] << 16) | ((uint32_t)v.v[3] << 24);
+              }
+            }
           }
         }
       }
+#pragma unroll
+      for (int e = 0; e < ROUND; ++e) {
+        if (e < left) {
+          const int64_t off = my_row[e].off;
+          if (lane_on && off >= 0) {
+            valid |= 1u << e;
+            load_raw<VB>(raw[e], pdata + off);
+          }
+        }
+      }
+      load_idx(r + 1);
+      if constexpr (QUANT) {
+#pragma unroll
+        for (int rr = 0; rr < MAXR; ++rr) {
+          if (rr < R && stager && coff[rr] >= 0) {
+            const float rs = d.sb_fp32 ? bits_to_float(h0[rr]) : half_lo(h0[rr]);
+            const float rb = d.sb_fp32 ? bits_to_float(h1[rr]) : half_hi(h0[rr]);
+            StageMul m;
+            m.scale = cw[rr] * rs;
+            m.bias = cw[rr] * rb;
+            my_mul[sub + rr * SL] = m;
+          }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      }
+      float sc[ROUND], bi[ROUND];
+#pragma unroll
+      for (int e = 0; e < ROUND; ++e) {
+        if (e < left) {
+          const StageMul m = my_mul[e];
+          sc[e] = m.scale;
+          bi[e] = m.bias;
+        }
+      }
       __builtin_amdgcn_wave_barrier();
-      stage_gather(r + 1);
-      load_idx(r + 2);
 #pragma unroll
       for (int e = 0; e < ROUND; ++e) {
         if (valid & (1u << e)) Accum<TY, VB>::run(acc, raw[e], sc[e], bi[e]);
       }
-      stage_publish();
+      // offsets (and plain weights) of the next round; the column lanes have
+      // read this round's entries by now
+      stage_rows(r + 1);
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
     }
@@ -506,37 +528,46 @@ __device__ __forceinline__ void pool_bags(const LookupArgs& a, const TableDesc& 
 
 template <typename index_t, int TY>
 __device__ __forceinline__ void pool_dispatch_vb(const LookupArgs& a, const TableDesc& d, int table, int first_slot,
-                                                 int lane, StageEntry* stage) {
+                                                 int lane, StageRow* stage_row, StageMul* stage_mul) {
   constexpr int BITS = type_bits(TY);
   constexpr int MINVB = BITS >= 16 ? BITS / 8 : 1;
+#ifdef FBGEMM_AMD_ONLY_VB
+  if (d.vb == FBGEMM_AMD_ONLY_VB) pool_bags<index_t, TY, FBGEMM_AMD_ONLY_VB, 8>(a, d, table, first_slot, lane, stage_row, stage_mul);
+#else
   if (d.vb == 16) {
-    if constexpr (TY == ST_INT2) pool_bags<index_t, TY, 4, 8>(a, d, table, first_slot, lane, stage); // not selected by the host
-    else pool_bags<index_t, TY, 16, 8>(a, d, table, first_slot, lane, stage);
+    if constexpr (TY == ST_INT2) pool_bags<index_t, TY, 4, 8>(a, d, table, first_slot, lane, stage_row, stage_mul); // not selected by the host
+    else pool_bags<index_t, TY, 16, (TY == ST_INT4 ? 4 : 8)>(a, d, table, first_slot, lane, stage_row, stage_mul);
   } else if (d.vb == 4) {
-    pool_bags<index_t, TY, 4, 8>(a, d, table, first_slot, lane, stage);
+    pool_bags<index_t, TY, 4, 8>(a, d, table, first_slot, lane, stage_row, stage_mul);
   } else {
-    pool_bags<index_t, TY, MINVB, 8>(a, d, table, first_slot, lane, stage);
+    pool_bags<index_t, TY, MINVB, 8>(a, d, table, first_slot, lane, stage_row, stage_mul);
   }
+#endif
 }
 
 template <typename index_t>
-__global__ __launch_bounds__(256) void lookup_kernel(const LookupArgs a) {
-  __shared__ StageEntry stage_all[4][MAX_GROUPS * MAX_ROUND];
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8))) void lookup_kernel(const LookupArgs a) {
+  __shared__ StageRow stage_rows_all[4][MAX_GROUPS * MAX_ROUND];
+  __shared__ StageMul stage_muls_all[4][MAX_GROUPS * MAX_ROUND];
   const int lane = threadIdx.x & 63;
-  int64_t blk = blockIdx.x;
-  if (a.xcd_swizzle) {
-    // Workgroups are handed to the 8 XCDs round-robin. Give each XCD one
-    // contiguous range of the work list, so that a table's hot rows are
-    // cached in one XCD's L2 rather than in all eight.
-    const int64_t nb = gridDim.x;
-    const int64_t q = nb >> 3, r = nb & 7;
-    const int64_t x = blk & 7;
-    blk = x * q + (x < r ? x : r) + (blk >> 3);
-  }
   const int wid = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-  const int64_t wave = blk * 4 + wid;
-  if (wave >= a.num_waves) return;
-  StageEntry* stage = stage_all[wid];
+  int64_t wave;
+  if (a.xcd_start) {
+    // Workgroups are handed to the 8 XCDs round-robin, so the workgroups with
+    // id % 8 == x all run on one XCD and share its L2. Each XCD walks its own
+    // run of the work list: whole tables (or slices of them) are pinned to
+    // one L2 instead of spreading their hot rows over all eight.
+    const int x = blockIdx.x & 7;
+    const int64_t w = (int64_t)(blockIdx.x >> 3) * 4 + wid;
+    const int64_t lo = a.xcd_start[x], hi = a.xcd_start[x + 1];
+    if (w >= hi - lo) return;
+    wave = lo + w;
+  } else {
+    wave = (int64_t)blockIdx.x * 4 + wid;
+    if (wave >= a.num_waves) return;
+  }
+  StageRow* stage_row = stage_rows_all[wid];
+  StageMul* stage_mul = stage_muls_all[wid];
   int table = 0, first_slot;
   if (a.work) {
     const WaveWork ww = a.work[wave];
@@ -546,15 +577,19 @@ __global__ __launch_bounds__(256) void lookup_kernel(const LookupArgs a) {
     first_slot = (int)(wave * (64 / a.single.lanes));
   }
   const TableDesc d = a.tables ? a.tables[table] : a.single;
+#ifdef FBGEMM_AMD_ONLY_TY // register-budget experiments: compile a single row type
+  if (d.ty == FBGEMM_AMD_ONLY_TY) pool_dispatch_vb<index_t, FBGEMM_AMD_ONLY_TY>(a, d, table, first_slot, lane, stage_row, stage_mul);
+#else
   switch (d.ty) {
-    case ST_INT4: pool_dispatch_vb<index_t, ST_INT4>(a, d, table, first_slot, lane, stage); break;
-    case ST_INT8: pool_dispatch_vb<index_t, ST_INT8>(a, d, table, first_slot, lane, stage); break;
-    case ST_FP16: pool_dispatch_vb<index_t, ST_FP16>(a, d, table, first_slot, lane, stage); break;
-    case ST_INT2: pool_dispatch_vb<index_t, ST_INT2>(a, d, table, first_slot, lane, stage); break;
-    case ST_FP32: pool_dispatch_vb<index_t, ST_FP32>(a, d, table, first_slot, lane, stage); break;
-    case ST_BF16: pool_dispatch_vb<index_t, ST_BF16>(a, d, table, first_slot, lane, stage); break;
+    case ST_INT4: pool_dispatch_vb<index_t, ST_INT4>(a, d, table, first_slot, lane, stage_row, stage_mul); break;
+    case ST_INT8: pool_dispatch_vb<index_t, ST_INT8>(a, d, table, first_slot, lane, stage_row, stage_mul); break;
+    case ST_FP16: pool_dispatch_vb<index_t, ST_FP16>(a, d, table, first_slot, lane, stage_row, stage_mul); break;
+    case ST_INT2: pool_dispatch_vb<index_t, ST_INT2>(a, d, table, first_slot, lane, stage_row, stage_mul); break;
+    case ST_FP32: pool_dispatch_vb<index_t, ST_FP32>(a, d, table, first_slot, lane, stage_row, stage_mul); break;
+    case ST_BF16: pool_dispatch_vb<index_t, ST_BF16>(a, d, table, first_slot, lane, stage_row, stage_mul); break;
     default: break;
   }
+#endif
 }
 
 // ---- bag scheduler -------------------------------------------------------------
@@ -671,7 +706,7 @@ hipError_t launch_calibration_copy(const void* src, void* dst, int64_t bytes, hi
 
 hipError_t launch_lookup(const LookupArgs& a, bool idx64, hipStream_t stream) {
   if (a.num_waves <= 0) return hipSuccess;
-  const int64_t blocks = (a.num_waves + 3) / 4;
+  const int64_t blocks = a.xcd_start ? 8 * ((a.num_waves + 3) / 4) : (a.num_waves + 3) / 4;
   if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
   if (idx64) hipLaunchKernelGGL(lookup_kernel<int64_t>, dim3((unsigned)blocks), dim3(256), 0, stream, a);
   else hipLaunchKernelGGL(lookup_kernel<int32_t>, dim3((unsigned)blocks), dim3(256), 0, stream, a);

@@ -14,7 +14,7 @@ import os
 import sys
 from collections import defaultdict
 
-OURS = ("lookup_kernel", "calibration_copy_kernel", "lengths_to_offsets", "pruned_array_lookup")
+OURS = ("lookup_kernel", "calibration_copy_kernel", "bag_order_kernel", "lengths_to_offsets", "pruned_array_lookup")
 
 
 def short(name):
