@@ -31,6 +31,8 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--config", type=int, default=3, choices=[1, 2, 3, 4, 5])
     ap.add_argument("--scale", type=float, default=1.0, help="shrink rows and batch (1.0 = the real configuration)")
+    ap.add_argument("--rows-scale", type=float, default=None,
+                    help="config 3 only: shrink the tables but not the batch (cache-resident experiment)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
@@ -164,7 +166,7 @@ def main():
     torch.cuda.set_device(0)
     t_build = time.time()
     if a.config in (3, 5):
-        p = bc.config3("cuda", a.scale) if a.config == 3 else bc.config5("cuda", a.scale)
+        p = bc.config3("cuda", a.scale, a.rows_scale) if a.config == 3 else bc.config5("cuda", a.scale)
         launch, out, st, plan = tbe_runner(p, torch)
         lookups, useful = p.lookups, p.useful_row_bytes()
         other = p.other_bytes()

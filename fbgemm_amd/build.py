@@ -19,6 +19,9 @@ SOURCES = ["lookup_kernels.hip", "c_api.cpp"]
 FLAGS = [
     "-x", "hip", "-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-shared",
     "-ffp-contract=off", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # error reporting uses a few atomics on one address; keep them as plain
+    # atomics instead of a wave-wide reduction loop in front of each
+    "-mllvm", "-amdgpu-atomic-optimizer-strategy=None",
 ]
 
 

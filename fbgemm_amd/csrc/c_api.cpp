@@ -18,7 +18,7 @@ namespace fbgemm_amd {
 hipError_t launch_lookup(const LookupArgs& a, bool idx64, hipStream_t stream);
 hipError_t launch_lengths_to_offsets(const void* lengths, bool is64, int64_t n, int64_t* offsets, hipStream_t stream);
 hipError_t launch_status_clear(Status* st, hipStream_t stream);
-hipError_t launch_bag_order(const void* offsets, bool off64, int32_t B, int32_t T, int32_t* order, hipStream_t stream);
+hipError_t launch_bag_order(const void* offsets, bool off64, int32_t B, int32_t T, BagEntry* order, hipStream_t stream);
 hipError_t launch_calibration_copy(const void* src, void* dst, int64_t bytes, hipStream_t stream);
 hipError_t launch_pruned_array_lookup(const void* indices, const void* offsets, bool idx64, const void* remap,
                                       bool remap64, const int64_t* remap_offsets, int32_t B, int32_t T,
@@ -89,8 +89,17 @@ void plan_lanes(TableDesc& d, uintptr_t base_addr, int64_t out_stride, bool has_
   if (force_vb == 1) vb = min_vb;
   d.vb = vb;
   const int chunks = (d.data_bytes + vb - 1) / vb;
-  d.lanes = std::max(2, std::min(64, chunks)); // >= 2: a wave stages at most 32 bags
-  d.passes = (chunks + d.lanes - 1) / d.lanes;
+  // Wide rows: give a lane several 16-byte chunks (up to 32 accumulators), so
+  // that the per-row bookkeeping is shared by more elements.
+  static const int max_chunks = env_int("FBGEMM_AMD_MAX_CHUNKS", 4);
+  const int type_c = bits >= 16 ? 4 : (bits == 8 ? 2 : 1);
+  int C = 1;
+  if (vb == 16)
+    for (int c = std::min(type_c, max_chunks); c > 1; c >>= 1)
+      if (chunks % c == 0 && chunks / c >= 2) { C = c; break; }
+  d.chunks = C;
+  d.lanes = std::max(2, std::min(64, chunks / C)); // >= 2: a wave stages at most 32 bags
+  d.passes = (chunks + d.lanes * C - 1) / (d.lanes * C);
   // whole-run vector stores: each lane writes E = vb*8/bits consecutive
   // elements; allowed when every run starts on a multiple of min(16, run bytes)
   // and no run is cut by the end of the row.
@@ -112,7 +121,7 @@ struct DeviceScratch {
   Status* status = nullptr;
   int64_t* offsets = nullptr; // lengths -> offsets
   int64_t offsets_cap = 0;
-  int32_t* order = nullptr;   // bag order of single-table calls
+  BagEntry* order = nullptr;  // bag order of single-table calls
   int64_t order_cap = 0;
 };
 
@@ -355,7 +364,7 @@ struct fbgemm_amd_tbe_plan {
   // per-B work lists
   struct Work {
     WaveWork* d_work = nullptr;
-    int32_t* d_order = nullptr; // T*B bag ids, rewritten by every forward
+    BagEntry* d_order = nullptr; // T*B bags, rewritten by every forward
     int64_t* d_xcd_start = nullptr;
     int64_t num_waves = 0;
   };
@@ -477,6 +486,7 @@ int fbgemm_amd_tbe_forward(
       // through its bag order (longest first) at the same relative pace, so
       // that tables of different row types share the CUs at all times.
       static const int xcd_lists = env_int("FBGEMM_AMD_XCD_LISTS", 1);
+      static const int interleave = env_int("FBGEMM_AMD_INTERLEAVE", 1);
       struct Slice { int t, first, step, count; double cost; };
       std::vector<Slice> slices;
       double total_cost = 0;
@@ -516,7 +526,8 @@ int fbgemm_amd_tbe_forward(
         for (const Slice& sl : per_x[x]) {
           const int G = 64 / plan->tables[sl.t].lanes;
           for (int k = 0; k < sl.count; ++k)
-            keyed.push_back({(k + 0.5) / sl.count, WaveWork{sl.t, (sl.first + k * sl.step) * G}});
+            keyed.push_back({interleave ? (k + 0.5) / sl.count : (double)keyed.size(),
+                             WaveWork{sl.t, (sl.first + k * sl.step) * G}});
         }
         std::stable_sort(keyed.begin(), keyed.end(),
                          [](const std::pair<double, WaveWork>& p, const std::pair<double, WaveWork>& q) { return p.first < q.first; });
@@ -533,7 +544,7 @@ int fbgemm_amd_tbe_forward(
         HIP_TRY(hipMalloc((void**)&nw.d_xcd_start, sizeof(int64_t) * 9));
         HIP_TRY(hipMemcpy(nw.d_xcd_start, xcd_start.data(), sizeof(int64_t) * 9, hipMemcpyHostToDevice));
       }
-      HIP_TRY(hipMalloc((void**)&nw.d_order, sizeof(int32_t) * (size_t)plan->T * (size_t)B));
+      HIP_TRY(hipMalloc((void**)&nw.d_order, sizeof(BagEntry) * (size_t)plan->T * (size_t)B));
       it = plan->work.emplace(B, nw).first;
     }
     w = it->second;

@@ -53,10 +53,19 @@ struct TableDesc {
   int32_t skip_minus_one; // 1: an index of -1 is a pruned row and is skipped
   int32_t vec_store;      // bit 0 / bit 1: every lane's output run is aligned for whole-run
                           // vector stores with 4-byte / 2-byte output elements
-  int32_t reserved;
+  int32_t chunks;         // 16-byte chunks per lane and pass (1, 2 or 4)
 };
 
-// One entry per workgroup wave slot: which table and which first bag.
+// What the bag scheduler leaves per bag, in the order waves take the bags.
+struct __attribute__((aligned(16))) BagEntry {
+  int64_t o0;  // offsets[bag]
+  int64_t o1;  // offsets[bag + 1]
+  int32_t bag; // bag id inside its table
+  int32_t pad0;
+  int64_t pad1;
+};
+
+// One entry per wave: which table and which first position of the bag order.
 struct WaveWork {
   int32_t table;
   int32_t first_bag;
@@ -74,7 +83,7 @@ struct LookupArgs {
   void* out;
   int64_t out_stride;        // elements between consecutive bags' outputs
   int64_t index_size;        // entries the index array holds for this call
-  const int32_t* order;      // per table, its B bag ids in the order waves take them
+  const BagEntry* order;     // per table, its B bags in the order waves take them
                              // (longest first), or nullptr: natural order
   const WaveWork* work;      // per-wave work list, or nullptr: single table, dense mapping
   const int64_t* xcd_start;  // 9 entries: the work list is 8 runs, run x = [xcd_start[x],

@@ -60,16 +60,38 @@ __device__ __forceinline__ void report_index(Status* st, int64_t pos) {
 // ---- per-row accumulate ---------------------------------------------------
 //
 // raw[] holds the VB bytes this lane loaded (VB < 4: in the low bits of raw[0]).
-// Products with |scale| >= 2^100 cannot take the pre-scaled route (scale * 2^24
-// would overflow); they use plain integer->float conversion instead.
+// fast() may pre-scale the row scale by 2^24, which is exact unless it
+// overflows: the caller uses it only when |scale| < 2^100 and slow() (plain
+// integer -> float conversion) otherwise. Both round identically.
 
 template <int TY, int VB>
 struct Accum;
 
+// 8-bit rows. Two bytes of a word are spread into the two halves of a register
+// with one byte permute; each half is then the half-precision denormal
+// q * 2^-24, which the fma widens exactly.
 template <int VB>
 struct Accum<ST_INT8, VB> {
   static constexpr int E = VB;
-  __device__ __forceinline__ static void run(float (&acc)[E], const uint32_t* raw, float scale, float bias) {
+  static constexpr bool kPrescaled = VB >= 4;
+  __device__ __forceinline__ static void fast(float (&acc)[E], const uint32_t* raw, float scale, float bias) {
+    if constexpr (kPrescaled) {
+      const float s24 = scale * 0x1p24f;
+#pragma unroll
+      for (int w = 0; w < VB / 4; ++w) {
+        const uint32_t lo = __builtin_amdgcn_perm(0u, raw[w], 0x0c010c00u); // bytes 0, 1
+        const uint32_t hi = __builtin_amdgcn_perm(0u, raw[w], 0x0c030c02u); // bytes 2, 3
+        float* c = acc + 4 * w;
+        c[0] = __builtin_fmaf(s24, half_lo(lo), c[0] + bias);
+        c[1] = __builtin_fmaf(s24, half_hi(lo), c[1] + bias);
+        c[2] = __builtin_fmaf(s24, half_lo(hi), c[2] + bias);
+        c[3] = __builtin_fmaf(s24, half_hi(hi), c[3] + bias);
+      }
+    } else {
+      slow(acc, raw, scale, bias);
+    }
+  }
+  __device__ __forceinline__ static void slow(float (&acc)[E], const uint32_t* raw, float scale, float bias) {
 #pragma unroll
     for (int e = 0; e < E; ++e) {
       const uint32_t q = (raw[e / 4] >> (8 * (e % 4))) & 0xffu;
@@ -78,35 +100,40 @@ struct Accum<ST_INT8, VB> {
   }
 };
 
+// 4-bit rows. Masks leave nibbles k and k + 4 of a word in the two halves of
+// a register as half-precision denormals (times 16 for the odd ones); the
+// powers of two are folded into two pre-scaled copies of the row scale.
 template <int VB>
 struct Accum<ST_INT4, VB> {
   static constexpr int E = VB * 2;
-  __device__ __forceinline__ static void run(float (&acc)[E], const uint32_t* raw, float scale, float bias) {
-    if constexpr (VB >= 4) {
-      if (__builtin_expect(__builtin_fabsf(scale) < 0x1p100f, 1)) {
-        const float s24 = scale * 0x1p24f;
-        const float s20 = scale * 0x1p20f;
+  static constexpr bool kPrescaled = VB >= 4;
+  __device__ __forceinline__ static void fast(float (&acc)[E], const uint32_t* raw, float scale, float bias) {
+    if constexpr (kPrescaled) {
+      const float s24 = scale * 0x1p24f;
+      const float s20 = scale * 0x1p20f;
 #pragma unroll
-        for (int w = 0; w < VB / 4; ++w) {
-          const uint32_t x = raw[w];
-          const uint32_t y = x >> 8;
-          const uint32_t a0 = x & 0x000f000fu; // nibbles 0, 4
-          const uint32_t a1 = x & 0x00f000f0u; // nibbles 1, 5 (times 16)
-          const uint32_t a2 = y & 0x000f000fu; // nibbles 2, 6
-          const uint32_t a3 = y & 0x00f000f0u; // nibbles 3, 7 (times 16)
-          float* c = acc + 8 * w;
-          c[0] = __builtin_fmaf(s24, half_lo(a0), c[0] + bias);
-          c[1] = __builtin_fmaf(s20, half_lo(a1), c[1] + bias);
-          c[2] = __builtin_fmaf(s24, half_lo(a2), c[2] + bias);
-          c[3] = __builtin_fmaf(s20, half_lo(a3), c[3] + bias);
-          c[4] = __builtin_fmaf(s24, half_hi(a0), c[4] + bias);
-          c[5] = __builtin_fmaf(s20, half_hi(a1), c[5] + bias);
-          c[6] = __builtin_fmaf(s24, half_hi(a2), c[6] + bias);
-          c[7] = __builtin_fmaf(s20, half_hi(a3), c[7] + bias);
-        }
-        return;
+      for (int w = 0; w < VB / 4; ++w) {
+        const uint32_t x = raw[w];
+        const uint32_t y = x >> 8;
+        const uint32_t a0 = x & 0x000f000fu; // nibbles 0, 4
+        const uint32_t a1 = x & 0x00f000f0u; // nibbles 1, 5 (times 16)
+        const uint32_t a2 = y & 0x000f000fu; // nibbles 2, 6
+        const uint32_t a3 = y & 0x00f000f0u; // nibbles 3, 7 (times 16)
+        float* c = acc + 8 * w;
+        c[0] = __builtin_fmaf(s24, half_lo(a0), c[0] + bias);
+        c[1] = __builtin_fmaf(s20, half_lo(a1), c[1] + bias);
+        c[2] = __builtin_fmaf(s24, half_lo(a2), c[2] + bias);
+        c[3] = __builtin_fmaf(s20, half_lo(a3), c[3] + bias);
+        c[4] = __builtin_fmaf(s24, half_hi(a0), c[4] + bias);
+        c[5] = __builtin_fmaf(s20, half_hi(a1), c[5] + bias);
+        c[6] = __builtin_fmaf(s24, half_hi(a2), c[6] + bias);
+        c[7] = __builtin_fmaf(s20, half_hi(a3), c[7] + bias);
       }
+    } else {
+      slow(acc, raw, scale, bias);
     }
+  }
+  __device__ __forceinline__ static void slow(float (&acc)[E], const uint32_t* raw, float scale, float bias) {
 #pragma unroll
     for (int e = 0; e < E; ++e) {
       const uint32_t q = (raw[e / 8] >> (4 * (e % 8))) & 0xfu;
@@ -118,46 +145,54 @@ struct Accum<ST_INT4, VB> {
 template <int VB>
 struct Accum<ST_INT2, VB> {
   static constexpr int E = VB * 4;
-  __device__ __forceinline__ static void run(float (&acc)[E], const uint32_t* raw, float scale, float bias) {
+  static constexpr bool kPrescaled = false;
+  __device__ __forceinline__ static void fast(float (&acc)[E], const uint32_t* raw, float scale, float bias) {
 #pragma unroll
     for (int e = 0; e < E; ++e) {
       const uint32_t q = (raw[e / 16] >> (2 * (e % 16))) & 0x3u;
       acc[e] = __builtin_fmaf(scale, (float)q, acc[e] + bias);
     }
   }
+  __device__ __forceinline__ static void slow(float (&acc)[E], const uint32_t* raw, float a, float b) { fast(acc, raw, a, b); }
 };
 
 template <int VB>
 struct Accum<ST_FP16, VB> {
   static constexpr int E = VB / 2;
-  __device__ __forceinline__ static void run(float (&acc)[E], const uint32_t* raw, float w, float) {
+  static constexpr bool kPrescaled = false;
+  __device__ __forceinline__ static void fast(float (&acc)[E], const uint32_t* raw, float w, float) {
 #pragma unroll
     for (int e = 0; e < E; ++e) {
       const float x = (e & 1) ? half_hi(raw[e / 2]) : half_lo(raw[e / 2]);
       acc[e] = __builtin_fmaf(w, x, acc[e]);
     }
   }
+  __device__ __forceinline__ static void slow(float (&acc)[E], const uint32_t* raw, float a, float b) { fast(acc, raw, a, b); }
 };
 
 template <int VB>
 struct Accum<ST_BF16, VB> {
   static constexpr int E = VB / 2;
-  __device__ __forceinline__ static void run(float (&acc)[E], const uint32_t* raw, float w, float) {
+  static constexpr bool kPrescaled = false;
+  __device__ __forceinline__ static void fast(float (&acc)[E], const uint32_t* raw, float w, float) {
 #pragma unroll
     for (int e = 0; e < E; ++e) {
       const uint32_t u = (e & 1) ? (raw[e / 2] & 0xffff0000u) : (raw[e / 2] << 16);
       acc[e] = __builtin_fmaf(w, bits_to_float(u), acc[e]);
     }
   }
+  __device__ __forceinline__ static void slow(float (&acc)[E], const uint32_t* raw, float a, float b) { fast(acc, raw, a, b); }
 };
 
 template <int VB>
 struct Accum<ST_FP32, VB> {
   static constexpr int E = VB / 4;
-  __device__ __forceinline__ static void run(float (&acc)[E], const uint32_t* raw, float w, float) {
+  static constexpr bool kPrescaled = false;
+  __device__ __forceinline__ static void fast(float (&acc)[E], const uint32_t* raw, float w, float) {
 #pragma unroll
     for (int e = 0; e < E; ++e) acc[e] = __builtin_fmaf(w, bits_to_float(raw[e]), acc[e]);
   }
+  __device__ __forceinline__ static void slow(float (&acc)[E], const uint32_t* raw, float a, float b) { fast(acc, raw, a, b); }
 };
 
 // ---- loads ----------------------------------------------------------------
@@ -288,7 +323,9 @@ constexpr int MAX_ROUND = 8;
 constexpr int64_t NO_ENTRY = INT64_MIN;
 
 // One wave pools 64 / lanes bags of one table, `RN` entries of every bag per
-// round.
+// round. Each lane owns C chunks of VB bytes of every row: chunk c of lane
+// `sub` starts at byte (c * lanes + sub) * VB of the row data, so every load
+// instruction of the wave reads contiguous bytes of each row.
 //
 // Per-entry work (index load, per-sample weight, -1 / bounds / remap handling,
 // row offset, the scale/bias fetch and its two products with the weight) is
@@ -300,8 +337,17 @@ constexpr int64_t NO_ENTRY = INT64_MIN;
 // round, immediately before the column lanes load the row's data, and the two
 // accesses to the row's first line merge in the L1. While the loads are in
 // flight the indices of the next round are fetched.
-template <typename index_t, int TY, int VB, int ROUND>
-__device__ __forceinline__ void pool_bags(const LookupArgs& a, const TableDesc& d, int table, int first_slot,
+//
+// A round in which every lane of the wave has RN rows to add (the normal case
+// once bags are ordered by length) runs without a single predicate.
+//
+// PRESCALE selects the arithmetic route of the 4- and 8-bit rows: the
+// pre-scaled one (scale * 2^24 times a half-precision denormal) is exact unless
+// scale * 2^24 overflows. A wave that meets |scale| >= 2^100 gives up, returns
+// false, and its work is redone from the start by the PRESCALE = false
+// instance, which converts integers to float the plain way.
+template <typename index_t, bool GENERAL, int TY, int VB, int C, int ROUND, bool PRESCALE>
+__device__ __forceinline__ bool pool_bags(const LookupArgs& a, const TableDesc& d, int table, int first_slot,
                                           int lane, StageRow* stage_row, StageMul* stage_mul) {
   constexpr int BITS = type_bits(TY);
   constexpr int E = VB * 8 / BITS;
@@ -309,6 +355,7 @@ __device__ __forceinline__ void pool_bags(const LookupArgs& a, const TableDesc& 
   constexpr bool QUANT = TY == ST_INT8 || TY == ST_INT4 || TY == ST_INT2;
   constexpr bool ALIGNED = VB >= 4;
   constexpr int MAXR = 2; // entries one staging lane handles per round, at most
+  using Acc = Accum<TY, VB>;
 
   const int S = d.lanes;
   const int G = 64 / S;
@@ -317,28 +364,36 @@ __device__ __forceinline__ void pool_bags(const LookupArgs& a, const TableDesc& 
   const int slot = first_slot + grp;
   const bool bag_ok = grp < G && slot < a.B;
   const bool reporter = sub == 0;
-  // Entries staged per bag and round: ROUND, or half of it for bags that only
-  // have two or three lanes (each staging lane handles at most MAXR entries).
-  const int RN = S >= 4 ? ROUND : ROUND / 2;
-  const int SL = S >= RN ? RN : (S >= 4 ? 4 : 2); // staging lanes per bag (power of two, <= S)
-  const int R = RN / SL;                          // entries per staging lane per round
+  // staging lanes per bag: a power of two <= lanes; entries per round: ROUND,
+  // or what MAXR entries per staging lane allow
+  const int SLmax = S >= 8 ? 8 : (S >= 4 ? 4 : 2);
+  const int RN = ROUND < SLmax * MAXR ? ROUND : SLmax * MAXR;
+  const int SL = SLmax < RN ? SLmax : RN;
+  const int R = RN / SL;
   const bool stager = bag_ok && sub < SL;
 
   // Bags are taken in the order the scheduler left them (longest first), so
-  // that the bags sharing a wave have nearly equal lengths.
+  // that the bags sharing a wave have nearly equal lengths. Positions are
+  // counted the way the reference counts `current`: relative to the first
+  // offset of the table's slice.
   int bag = slot;
-  if (bag_ok && a.order) bag = a.order[(int64_t)table * a.B + slot];
-
-  // Positions are counted the way the reference counts `current`: relative to
-  // the first offset of the table's slice.
   int64_t pos0 = 0;
   int64_t len = 0;
   if (bag_ok) {
     const int64_t ob = (int64_t)table * a.B;
-    const int64_t base = read_offset(a.offsets, a.off64, ob);
-    const int64_t o0 = read_offset(a.offsets, a.off64, ob + bag);
-    const int64_t o1 = read_offset(a.offsets, a.off64, ob + bag + 1);
-    pos0 = a.check_total ? o0 - base : o0; // table-batched calls index the shared array
+    int64_t o0, o1;
+    if (a.order) {
+      const BagEntry be = a.order[ob + slot];
+      bag = be.bag;
+      o0 = be.o0;
+      o1 = be.o1;
+    } else {
+      o0 = read_offset(a.offsets, a.off64, ob + bag);
+      o1 = read_offset(a.offsets, a.off64, ob + bag + 1);
+    }
+    int64_t base = 0;
+    if (GENERAL && a.check_total) base = read_offset(a.offsets, a.off64, ob);
+    pos0 = o0 - base; // table-batched calls index the shared array: base = 0
     len = o1 - o0;
     if (len < 0) {
       if (reporter) report(a.status, ERR_NEGATIVE_LENGTH);
@@ -348,7 +403,7 @@ __device__ __forceinline__ void pool_bags(const LookupArgs& a, const TableDesc& 
       if (reporter) report(a.status, ERR_BAG_OVERRUN);
       len = 0;
     }
-    if (a.check_total && bag == a.B - 1 && o1 - base != a.index_size && reporter)
+    if (GENERAL && a.check_total && bag == a.B - 1 && o1 - base != a.index_size && reporter)
       report(a.status, ERR_LENGTH_MISMATCH);
   }
   const int n = (int)len; // same for every lane of the bag
@@ -360,16 +415,24 @@ __device__ __forceinline__ void pool_bags(const LookupArgs& a, const TableDesc& 
   StageMul* my_mul = stage_mul + grp * RN;
   // the reference keeps the bag length in an int when it forms 1/len
   const float inv_len = (a.normalize && n > 0) ? 1.0f / (float)n : 1.0f;
+  const int chunk_stride = S * VB; // bytes between a lane's consecutive chunks
 
   for (int pass = 0; pass < d.passes; ++pass) {
-    const int chunk = pass * S + sub;
-    const int byte_off = chunk * VB;
-    const bool lane_on = bag_ok && byte_off < d.data_bytes;
-    const uint8_t* pdata = wbase + d.data_off + byte_off;
-
-    float acc[E];
+    const int chunk0 = pass * S * C + sub;
+    bool on[C];
+    bool all_on = bag_ok;
 #pragma unroll
-    for (int e = 0; e < E; ++e) acc[e] = 0.0f;
+    for (int c = 0; c < C; ++c) {
+      on[c] = bag_ok && (chunk0 + c * S) * VB < d.data_bytes;
+      all_on = all_on && on[c];
+    }
+    const uint8_t* pdata = wbase + d.data_off + chunk0 * VB;
+
+    float acc[C][E];
+#pragma unroll
+    for (int c = 0; c < C; ++c)
+#pragma unroll
+      for (int e = 0; e < E; ++e) acc[c][e] = 0.0f;
 
     // registers of the staging lanes
     int64_t nrow[MAXR]; // raw index of the next round (loads in flight)
@@ -385,12 +448,15 @@ __device__ __forceinline__ void pool_bags(const LookupArgs& a, const TableDesc& 
         const int i = round * RN + sub + rr * SL;
         if (rr < R && stager && i < n) {
           nrow[rr] = (int64_t)idx[pos0 + i];
-          if (a.sample_weights) nw[rr] = a.sample_weights[a.positional ? (int64_t)i : pos0 + i];
+          if (a.sample_weights) nw[rr] = a.sample_weights[(GENERAL && a.positional) ? (int64_t)i : pos0 + i];
         }
       }
     };
-    // index -> row offset, or "nothing to add"; publish the offsets of `round`
-    auto stage_rows = [&](int round) {
+    // index -> row offset, or "nothing to add"; publish the offsets of `round`.
+    // Returns true on a staging lane that leaves a hole (no entry, or a
+    // skipped / rejected one) in the round.
+    auto stage_rows = [&](int round) -> bool {
+      bool hole = false;
 #pragma unroll
       for (int rr = 0; rr < MAXR; ++rr) {
         int64_t row = nrow[rr];
@@ -398,7 +464,7 @@ __device__ __forceinline__ void pool_bags(const LookupArgs& a, const TableDesc& 
         if (rr < R && row != NO_ENTRY) {
           const int64_t pos = pos0 + round * RN + sub + rr * SL;
           bool ok = true;
-          if (a.remap) {
+          if (GENERAL && a.remap) {
             if (row < 0 || row >= a.remap_rows) {
               if (pass == 0) report_index(a.status, pos);
               ok = false;
@@ -417,27 +483,37 @@ __device__ __forceinline__ void pool_bags(const LookupArgs& a, const TableDesc& 
         coff[rr] = off;
         cw[rr] = nw[rr];
         if (rr < R && stager) {
+          hole = hole || off < 0;
           my_row[sub + rr * SL].off = off;
-          if constexpr (!QUANT) {
+          // Plain rows: the multiplier is the weight. A hole gets (-0, -0),
+          // which leaves every accumulator exactly as it is:
+          // fma(-0, q, acc + -0) == acc for any acc, +0 and -0 included.
+          if (!QUANT || off < 0) {
             StageMul m;
-            m.scale = nw[rr];
-            m.bias = 0.0f;
+            m.scale = off < 0 ? -0.0f : nw[rr];
+            m.bias = -0.0f;
             my_mul[sub + rr * SL] = m;
           }
         }
       }
+      return hole;
     };
 
+    // wave-uniform: every lane of the wave pools a bag and owns C live chunks
+    const bool wave_on = __builtin_amdgcn_ballot_w64(!all_on) == 0ull && __builtin_amdgcn_ballot_w64(true) == ~0ull;
     load_idx(0);
-    stage_rows(0);
+    // wave-uniform: the staged round has RN rows to add for every bag of the wave
+    // (the staging call comes first on its own line: it must run on every wave)
+    const bool hole0 = stage_rows(0);
+    bool fast = wave_on && __builtin_amdgcn_ballot_w64(hole0) == 0ull;
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
 
+    bool give_up = false;
     for (int r = 0; r * RN < n; ++r) {
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-      uint32_t raw[ROUND][NW];
+      uint32_t raw[ROUND][C][NW];
       uint32_t h0[MAXR], h1[MAXR];
-      uint32_t valid = 0;
       const int left = min(n - r * RN, RN);
       // scale/bias first, so that their wait does not cover the row loads
       if constexpr (QUANT) {
@@ -465,18 +541,39 @@ __device__ __forceinline__ void pool_bags(const LookupArgs& a, const TableDesc& 
           }
         }
       }
+      if (fast) {
 #pragma unroll
-      for (int e = 0; e < ROUND; ++e) {
-        if (e < left) {
-          const int64_t off = my_row[e].off;
-          if (lane_on && off >= 0) {
-            valid |= 1u << e;
-            load_raw<VB>(raw[e], pdata + off);
+        for (int e = 0; e < ROUND; ++e) {
+          if (e < RN) {
+            const uint8_t* p = pdata + my_row[e].off;
+#pragma unroll
+            for (int c = 0; c < C; ++c) load_raw<VB>(raw[e][c], p + c * chunk_stride);
+          }
+        }
+      } else {
+        // ragged round: rows that are not there read as zeros and are
+        // multiplied by -0 below
+#pragma unroll
+        for (int e = 0; e < ROUND; ++e) {
+          if (e < RN && __builtin_amdgcn_ballot_w64(e < left) != 0ull) {
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+#pragma unroll
+              for (int w = 0; w < NW; ++w) raw[e][c][w] = 0u;
+            if (e < left) {
+              const int64_t off = my_row[e].off;
+              if (off >= 0) {
+#pragma unroll
+                for (int c = 0; c < C; ++c)
+                  if (on[c]) load_raw<VB>(raw[e][c], pdata + off + c * chunk_stride);
+              }
+            }
           }
         }
       }
       load_idx(r + 1);
       if constexpr (QUANT) {
+        bool big = false;
 #pragma unroll
         for (int rr = 0; rr < MAXR; ++rr) {
           if (rr < R && stager && coff[rr] >= 0) {
@@ -485,72 +582,111 @@ __device__ __forceinline__ void pool_bags(const LookupArgs& a, const TableDesc& 
             StageMul m;
             m.scale = cw[rr] * rs;
             m.bias = cw[rr] * rb;
+            big = big || !(__builtin_fabsf(m.scale) < 0x1p100f);
             my_mul[sub + rr * SL] = m;
+          }
+        }
+        if constexpr (PRESCALE && Acc::kPrescaled) {
+          if (__builtin_amdgcn_ballot_w64(big) != 0ull) {
+            give_up = true;
+            break;
           }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
       }
-      float sc[ROUND], bi[ROUND];
+      // One straight-line accumulate for the whole wave; lanes past the end of
+      // their bag add holes.
 #pragma unroll
       for (int e = 0; e < ROUND; ++e) {
-        if (e < left) {
+        if (e < RN && (fast || __builtin_amdgcn_ballot_w64(e < left) != 0ull)) {
           const StageMul m = my_mul[e];
-          sc[e] = m.scale;
-          bi[e] = m.bias;
+#pragma unroll
+          for (int c = 0; c < C; ++c) {
+            if constexpr (PRESCALE) Acc::fast(acc[c], raw[e][c], m.scale, m.bias);
+            else Acc::slow(acc[c], raw[e][c], m.scale, m.bias);
+          }
         }
       }
       __builtin_amdgcn_wave_barrier();
-#pragma unroll
-      for (int e = 0; e < ROUND; ++e) {
-        if (valid & (1u << e)) Accum<TY, VB>::run(acc, raw[e], sc[e], bi[e]);
-      }
       // offsets (and plain weights) of the next round; the column lanes have
       // read this round's entries by now
-      stage_rows(r + 1);
+      const bool hole = stage_rows(r + 1);
+      fast = wave_on && __builtin_amdgcn_ballot_w64(hole) == 0ull;
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
     }
 
-    if (lane_on) {
-      if (a.normalize && n > 0) {
+    if (__builtin_amdgcn_ballot_w64(give_up) != 0ull) return false; // every lane of the wave is back here
+
+    const bool vec_ok = a.out_aligned && ((d.vec_store >> (a.out_ty == ST_FP32 ? 0 : 1)) & 1);
 #pragma unroll
-        for (int e = 0; e < E; ++e) acc[e] *= inv_len;
+    for (int c = 0; c < C; ++c) {
+      if (on[c]) {
+        if (a.normalize && n > 0) {
+#pragma unroll
+          for (int e = 0; e < E; ++e) acc[c][e] *= inv_len;
+        }
+        const int col0 = (chunk0 + c * S) * E;
+        const int64_t elem_pos = (int64_t)bag * a.out_stride + d.out_col + col0;
+        write_out<E>(a, acc[c], elem_pos, col0, d.D, vec_ok);
       }
-      const int col0 = chunk * E;
-      const int64_t elem_pos = (int64_t)bag * a.out_stride + d.out_col + col0;
-      const bool vec_ok = a.out_aligned && ((d.vec_store >> (a.out_ty == ST_FP32 ? 0 : 1)) & 1);
-      write_out<E>(a, acc, elem_pos, col0, d.D, vec_ok);
     }
+  }
+  return true;
+}
+
+template <typename index_t, bool GENERAL, int TY, int VB, int C, int ROUND>
+__device__ __forceinline__ void run_bags(const LookupArgs& a, const TableDesc& d, int table, int first_slot, int lane,
+                                         StageRow* stage_row, StageMul* stage_mul) {
+  if constexpr (Accum<TY, VB>::kPrescaled) {
+    if (!pool_bags<index_t, GENERAL, TY, VB, C, ROUND, true>(a, d, table, first_slot, lane, stage_row, stage_mul))
+      pool_bags<index_t, GENERAL, TY, VB, C, ROUND, false>(a, d, table, first_slot, lane, stage_row, stage_mul);
+  } else {
+    pool_bags<index_t, GENERAL, TY, VB, C, ROUND, true>(a, d, table, first_slot, lane, stage_row, stage_mul);
   }
 }
 
-template <typename index_t, int TY>
+// Row types and the lane shapes the host may pick for them (TableDesc::vb,
+// TableDesc::chunks): 16-byte chunks with up to 4 (fp16 / bf16 / fp32), 2
+// (int8) or 1 (int4) chunks per lane so that a lane holds at most 32
+// accumulators; 4-byte and element-sized chunks for everything else.
+template <typename index_t, bool GENERAL, int TY>
 __device__ __forceinline__ void pool_dispatch_vb(const LookupArgs& a, const TableDesc& d, int table, int first_slot,
                                                  int lane, StageRow* stage_row, StageMul* stage_mul) {
   constexpr int BITS = type_bits(TY);
   constexpr int MINVB = BITS >= 16 ? BITS / 8 : 1;
-#ifdef FBGEMM_AMD_ONLY_VB
-  if (d.vb == FBGEMM_AMD_ONLY_VB) pool_bags<index_t, TY, FBGEMM_AMD_ONLY_VB, 8>(a, d, table, first_slot, lane, stage_row, stage_mul);
-#else
+  constexpr int MAXC = BITS >= 16 ? 4 : (BITS == 8 ? 2 : 1);
+  // rows in flight per lane: ROUND * chunks = 8 loads of 16 bytes
   if (d.vb == 16) {
-    if constexpr (TY == ST_INT2) pool_bags<index_t, TY, 4, 8>(a, d, table, first_slot, lane, stage_row, stage_mul); // not selected by the host
-    else pool_bags<index_t, TY, 16, (TY == ST_INT4 ? 4 : 8)>(a, d, table, first_slot, lane, stage_row, stage_mul);
+    if constexpr (TY == ST_INT2) {
+      run_bags<index_t, GENERAL, TY, 4, 1, 8>(a, d, table, first_slot, lane, stage_row, stage_mul); // not selected by the host
+    } else {
+      if (d.chunks == 4 && MAXC >= 4) run_bags<index_t, GENERAL, TY, 16, (MAXC >= 4 ? 4 : 1), 2>(a, d, table, first_slot, lane, stage_row, stage_mul);
+      else if (d.chunks == 2 && MAXC >= 2) run_bags<index_t, GENERAL, TY, 16, (MAXC >= 2 ? 2 : 1), 4>(a, d, table, first_slot, lane, stage_row, stage_mul);
+      else run_bags<index_t, GENERAL, TY, 16, 1, 8>(a, d, table, first_slot, lane, stage_row, stage_mul);
+    }
   } else if (d.vb == 4) {
-    pool_bags<index_t, TY, 4, 8>(a, d, table, first_slot, lane, stage_row, stage_mul);
+    run_bags<index_t, GENERAL, TY, 4, 1, 8>(a, d, table, first_slot, lane, stage_row, stage_mul);
   } else {
-    pool_bags<index_t, TY, MINVB, 8>(a, d, table, first_slot, lane, stage_row, stage_mul);
+    run_bags<index_t, GENERAL, TY, MINVB, 1, 8>(a, d, table, first_slot, lane, stage_row, stage_mul);
   }
-#endif
 }
 
-template <typename index_t>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8))) void lookup_kernel(const LookupArgs a) {
-  __shared__ StageRow stage_rows_all[4][MAX_GROUPS * MAX_ROUND];
-  __shared__ StageMul stage_muls_all[4][MAX_GROUPS * MAX_ROUND];
-  const int lane = threadIdx.x & 63;
-  const int wid = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+#ifndef FBGEMM_AMD_MIN_WAVES
+#define FBGEMM_AMD_MIN_WAVES 3 // waves per SIMD the register allocation must leave room for
+#endif
+
+// One wave per workgroup: waves come and go independently, and a workgroup
+// needs no more than its own 4 KB of LDS.
+// GENERAL = false is the table-batched operator's subset (no logical->physical
+// remap, no positional weights, offsets indexing one shared index array).
+template <typename index_t, bool GENERAL>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(FBGEMM_AMD_MIN_WAVES, 8))) void lookup_kernel(const LookupArgs a) {
+  __shared__ StageRow stage_row[MAX_GROUPS * MAX_ROUND];
+  __shared__ StageMul stage_mul[MAX_GROUPS * MAX_ROUND];
+  const int lane = threadIdx.x;
   int64_t wave;
   if (a.xcd_start) {
     // Workgroups are handed to the 8 XCDs round-robin, so the workgroups with
@@ -558,16 +694,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8))) voi
     // run of the work list: whole tables (or slices of them) are pinned to
     // one L2 instead of spreading their hot rows over all eight.
     const int x = blockIdx.x & 7;
-    const int64_t w = (int64_t)(blockIdx.x >> 3) * 4 + wid;
+    const int64_t w = (int64_t)(blockIdx.x >> 3);
     const int64_t lo = a.xcd_start[x], hi = a.xcd_start[x + 1];
     if (w >= hi - lo) return;
     wave = lo + w;
   } else {
-    wave = (int64_t)blockIdx.x * 4 + wid;
+    wave = (int64_t)blockIdx.x;
     if (wave >= a.num_waves) return;
   }
-  StageRow* stage_row = stage_rows_all[wid];
-  StageMul* stage_mul = stage_muls_all[wid];
   int table = 0, first_slot;
   if (a.work) {
     const WaveWork ww = a.work[wave];
@@ -578,15 +712,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8))) voi
   }
   const TableDesc d = a.tables ? a.tables[table] : a.single;
 #ifdef FBGEMM_AMD_ONLY_TY // register-budget experiments: compile a single row type
-  if (d.ty == FBGEMM_AMD_ONLY_TY) pool_dispatch_vb<index_t, FBGEMM_AMD_ONLY_TY>(a, d, table, first_slot, lane, stage_row, stage_mul);
+  if (d.ty == FBGEMM_AMD_ONLY_TY) pool_dispatch_vb<index_t, GENERAL, FBGEMM_AMD_ONLY_TY>(a, d, table, first_slot, lane, stage_row, stage_mul);
 #else
   switch (d.ty) {
-    case ST_INT4: pool_dispatch_vb<index_t, ST_INT4>(a, d, table, first_slot, lane, stage_row, stage_mul); break;
-    case ST_INT8: pool_dispatch_vb<index_t, ST_INT8>(a, d, table, first_slot, lane, stage_row, stage_mul); break;
-    case ST_FP16: pool_dispatch_vb<index_t, ST_FP16>(a, d, table, first_slot, lane, stage_row, stage_mul); break;
-    case ST_INT2: pool_dispatch_vb<index_t, ST_INT2>(a, d, table, first_slot, lane, stage_row, stage_mul); break;
-    case ST_FP32: pool_dispatch_vb<index_t, ST_FP32>(a, d, table, first_slot, lane, stage_row, stage_mul); break;
-    case ST_BF16: pool_dispatch_vb<index_t, ST_BF16>(a, d, table, first_slot, lane, stage_row, stage_mul); break;
+    case ST_INT4: pool_dispatch_vb<index_t, GENERAL, ST_INT4>(a, d, table, first_slot, lane, stage_row, stage_mul); break;
+    case ST_INT8: pool_dispatch_vb<index_t, GENERAL, ST_INT8>(a, d, table, first_slot, lane, stage_row, stage_mul); break;
+    case ST_FP16: pool_dispatch_vb<index_t, GENERAL, ST_FP16>(a, d, table, first_slot, lane, stage_row, stage_mul); break;
+    case ST_INT2: pool_dispatch_vb<index_t, GENERAL, ST_INT2>(a, d, table, first_slot, lane, stage_row, stage_mul); break;
+    case ST_FP32: pool_dispatch_vb<index_t, GENERAL, ST_FP32>(a, d, table, first_slot, lane, stage_row, stage_mul); break;
+    case ST_BF16: pool_dispatch_vb<index_t, GENERAL, ST_BF16>(a, d, table, first_slot, lane, stage_row, stage_mul); break;
     default: break;
   }
 #endif
@@ -602,7 +736,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 8))) voi
 // may differ between runs, the results cannot (each bag is summed on its own).
 constexpr int SORT_BINS = 1024;
 
-__global__ __launch_bounds__(1024) void bag_order_kernel(const void* offsets, int off64, int32_t B, int32_t* order) {
+__global__ __launch_bounds__(1024) void bag_order_kernel(const void* offsets, int off64, int32_t B, BagEntry* order) {
   __shared__ int bins[SORT_BINS];
   __shared__ int partial[1024];
   const int t = blockIdx.x;
@@ -632,7 +766,13 @@ __global__ __launch_bounds__(1024) void bag_order_kernel(const void* offsets, in
   __syncthreads();
   for (int b = tid; b < B; b += 1024) {
     const int p = atomicAdd(&bins[bin_of(b)], 1);
-    order[ob + p] = b;
+    BagEntry be;
+    be.o0 = read_offset(offsets, off64, ob + b);
+    be.o1 = read_offset(offsets, off64, ob + b + 1);
+    be.bag = b;
+    be.pad0 = 0;
+    be.pad1 = 0;
+    order[ob + p] = be;
   }
 }
 
@@ -706,14 +846,21 @@ hipError_t launch_calibration_copy(const void* src, void* dst, int64_t bytes, hi
 
 hipError_t launch_lookup(const LookupArgs& a, bool idx64, hipStream_t stream) {
   if (a.num_waves <= 0) return hipSuccess;
-  const int64_t blocks = a.xcd_start ? 8 * ((a.num_waves + 3) / 4) : (a.num_waves + 3) / 4;
+  const int64_t blocks = a.xcd_start ? 8 * a.num_waves : a.num_waves;
   if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
-  if (idx64) hipLaunchKernelGGL(lookup_kernel<int64_t>, dim3((unsigned)blocks), dim3(256), 0, stream, a);
-  else hipLaunchKernelGGL(lookup_kernel<int32_t>, dim3((unsigned)blocks), dim3(256), 0, stream, a);
+  const bool general = a.remap || a.positional || a.check_total;
+  const dim3 grid((unsigned)blocks), block(64);
+  if (general) {
+    if (idx64) hipLaunchKernelGGL((lookup_kernel<int64_t, true>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((lookup_kernel<int32_t, true>), grid, block, 0, stream, a);
+  } else {
+    if (idx64) hipLaunchKernelGGL((lookup_kernel<int64_t, false>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((lookup_kernel<int32_t, false>), grid, block, 0, stream, a);
+  }
   return hipGetLastError();
 }
 
-hipError_t launch_bag_order(const void* offsets, bool off64, int32_t B, int32_t T, int32_t* order, hipStream_t stream) {
+hipError_t launch_bag_order(const void* offsets, bool off64, int32_t B, int32_t T, BagEntry* order, hipStream_t stream) {
   if (T <= 0 || B <= 0) return hipSuccess;
   hipLaunchKernelGGL(bag_order_kernel, dim3((unsigned)T), dim3(1024), 0, stream, offsets, off64 ? 1 : 0, B, order);
   return hipGetLastError();
