@@ -40,6 +40,49 @@ def build_library(verbose=False):
     return OUT
 
 
+TORCH_OP_OUT = os.path.join(HERE, "lib", "libfbgemm_amd_torch.so")
+CPP_TEST_OUT = os.path.join(os.path.dirname(HERE), "tests", "cpp", "_build", "test_factories")
+
+
+def _run(cmd, verbose):
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"{cmd[0]} failed:\n{proc.stdout}")
+
+
+def build_torch_op(verbose=False):
+    """The torch operator library (schema registration + CUDA-key kernels).
+    Host code only: g++ against the torch headers, linked to libfbgemm_amd.so."""
+    import torch
+
+    tdir = os.path.dirname(torch.__file__)
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch.compiled_with_cxx11_abi()),
+           f"-I{tdir}/include", f"-I{tdir}/include/torch/csrc/api/include", "-I/opt/rocm/include",
+           "-o", TORCH_OP_OUT, os.path.join(CSRC, "torch_op.cpp"),
+           f"-L{os.path.dirname(OUT)}", "-lfbgemm_amd", f"-L{tdir}/lib", "-ltorch_cpu", "-lc10", "-lc10_hip",
+           "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{tdir}/lib"]
+    _run(cmd, verbose)
+    return TORCH_OP_OUT
+
+
+def build_cpp_test(verbose=False):
+    """tests/cpp/test_factories: the C++ factory templates against the C oracle."""
+    root = os.path.dirname(HERE)
+    os.makedirs(os.path.dirname(CPP_TEST_OUT), exist_ok=True)
+    subprocess.check_call(["make", "-s", "-C", os.path.join(root, "oracle"), "oracle"])
+    obuild = os.path.join(root, "oracle", "_build")
+    cmd = ["hipcc", "-x", "hip", "-O2", "--offload-arch=gfx950", "-std=c++17", "-o", CPP_TEST_OUT,
+           os.path.join(root, "tests", "cpp", "test_factories.cpp"), f"-L{os.path.dirname(OUT)}", "-lfbgemm_amd",
+           f"-L{obuild}", "-lembedding_oracle", f"-Wl,-rpath,{os.path.dirname(OUT)}", f"-Wl,-rpath,{obuild}"]
+    _run(cmd, verbose)
+    return CPP_TEST_OUT
+
+
 if __name__ == "__main__":
     print(build_library(verbose=True))
+    print(build_torch_op(verbose=True))
+    print(build_cpp_test(verbose=True))
     sys.exit(0)

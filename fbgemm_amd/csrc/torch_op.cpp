@@ -1,0 +1,175 @@
+// torch operator registration: the reference's schema strings, verbatim, with
+// the HIP library behind the CUDA dispatch key (which is what HIP devices use
+// in PyTorch). Reference: TORCH_LIBRARY_FRAGMENT(fbgemm, ...) in
+// fbgemm_gpu/codegen/inference/embedding_forward_quantized_host_cpu.cpp:310-347
+// and the GPU dispatcher embedding_forward_quantized_host.cpp:259-370,574-583.
+//
+// torch is used for what it owns: tensors (HBM) and the current stream. All
+// work goes through the C ABI of include/fbgemm_amd.h.
+#include <ATen/ATen.h>
+#include <c10/hip/HIPStream.h>
+#include <torch/library.h>
+
+#include <map>
+#include <mutex>
+#include <tuple>
+
+#include "../../include/fbgemm_amd.h"
+
+namespace {
+
+using at::Tensor;
+
+void* current_stream(const Tensor& t) {
+  return (void*)c10::hip::getCurrentHIPStream(t.device().index()).stream();
+}
+
+// One plan per distinct set of metadata tensors (the operator receives them as
+// device tensors on every call; the host copy a plan needs is made once).
+struct PlanKey {
+  const void *wo, *wt, *dofs, *wp;
+  int64_t T, dev_bytes, uvm_bytes, row_alignment;
+  bool operator<(const PlanKey& o) const {
+    return std::tie(wo, wt, dofs, wp, T, dev_bytes, uvm_bytes, row_alignment) <
+        std::tie(o.wo, o.wt, o.dofs, o.wp, o.T, o.dev_bytes, o.uvm_bytes, o.row_alignment);
+  }
+};
+std::mutex g_mu;
+std::map<PlanKey, fbgemm_amd_tbe_plan*> g_plans;
+std::map<int, Tensor> g_status; // one status block per device, never freed
+
+Tensor& status_block(const Tensor& like) {
+  const int dev = like.device().index();
+  auto it = g_status.find(dev);
+  if (it == g_status.end()) {
+    Tensor st = at::zeros({4}, like.options().dtype(at::kInt));
+    TORCH_CHECK(fbgemm_amd_status_clear(st.data_ptr(), current_stream(like)) == 0, fbgemm_amd_last_error());
+    it = g_status.emplace(dev, st).first;
+  }
+  return it->second;
+}
+
+fbgemm_amd_tbe_plan* plan_for(const Tensor& dev_weights, const Tensor& uvm_weights, const Tensor& placements,
+                              const Tensor& weights_offsets, const Tensor& weights_tys, const Tensor& D_offsets,
+                              int64_t row_alignment) {
+  PlanKey key{weights_offsets.data_ptr(), weights_tys.data_ptr(), D_offsets.data_ptr(), placements.data_ptr(),
+              D_offsets.numel() - 1, dev_weights.numel(), uvm_weights.numel(), row_alignment};
+  auto it = g_plans.find(key);
+  if (it != g_plans.end()) return it->second;
+  const Tensor wo = weights_offsets.to(at::kCPU, at::kLong).contiguous();
+  const Tensor wt = weights_tys.to(at::kCPU, at::kByte).contiguous();
+  const Tensor dofs = D_offsets.to(at::kCPU, at::kInt).contiguous();
+  const Tensor wp = placements.to(at::kCPU, at::kInt).contiguous();
+  fbgemm_amd_tbe_plan* plan = nullptr;
+  const int rc = fbgemm_amd_tbe_plan_create(
+      &plan, (int32_t)(dofs.numel() - 1), wo.data_ptr<int64_t>(), wt.data_ptr<uint8_t>(), dofs.data_ptr<int32_t>(),
+      wp.data_ptr<int32_t>(), dev_weights.numel(), uvm_weights.numel(), row_alignment);
+  TORCH_CHECK(rc == 0, "fbgemm_amd: ", fbgemm_amd_last_error());
+  g_plans.emplace(key, plan);
+  return plan;
+}
+
+at::ScalarType out_scalar_type(int64_t output_dtype) {
+  switch (output_dtype) {
+    case FBGEMM_AMD_FP32: return at::kFloat;
+    case FBGEMM_AMD_FP16: return at::kHalf;
+    case FBGEMM_AMD_BF16: return at::kBFloat16;
+    default: TORCH_CHECK(false, "fbgemm_amd: output_dtype ", output_dtype, " (int8 / int4 outputs) is not on this path");
+  }
+}
+
+Tensor int_nbit_split_embedding_codegen_lookup_function_hip(
+    Tensor dev_weights, Tensor uvm_weights, Tensor weights_placements, Tensor weights_offsets, Tensor weights_tys,
+    Tensor D_offsets, int64_t total_D, int64_t /*max_int2_D*/, int64_t /*max_int4_D*/, int64_t /*max_int8_D*/,
+    int64_t /*max_float16_D*/, int64_t /*max_float32_D*/, Tensor indices, Tensor offsets, int64_t pooling_mode,
+    std::optional<Tensor> indice_weights, int64_t output_dtype, std::optional<Tensor> /*lxu_cache_weights*/,
+    std::optional<Tensor> lxu_cache_locations, std::optional<int64_t> row_alignment,
+    std::optional<int64_t> max_float8_D, std::optional<int64_t> /*fp8_exponent_bits*/,
+    std::optional<int64_t> /*fp8_exponent_bias*/) {
+  TORCH_CHECK(dev_weights.is_cuda() && indices.is_cuda() && offsets.is_cuda(), "fbgemm_amd: tensors must be on the GPU");
+  TORCH_CHECK(pooling_mode == FBGEMM_AMD_POOL_SUM || pooling_mode == FBGEMM_AMD_POOL_MEAN,
+              "fbgemm_amd: PoolingMode.NONE (sequence output) is not on this path");
+  TORCH_CHECK(!max_float8_D || *max_float8_D == 0, "fbgemm_amd: FP8 tables are not on this path");
+  TORCH_CHECK(!lxu_cache_locations || lxu_cache_locations->numel() == 0,
+              "fbgemm_amd: the LXU cache is not on this path (tables are resident in HBM)");
+  TORCH_CHECK(indices.scalar_type() == at::kInt || indices.scalar_type() == at::kLong, "indices must be int32 or int64");
+  // embedding_forward_quantized_host_cpu.cpp:111-113
+  if (offsets.scalar_type() != indices.scalar_type()) offsets = offsets.to(indices.scalar_type());
+  indices = indices.contiguous();
+  offsets = offsets.contiguous();
+  Tensor w;
+  if (indice_weights && indice_weights->numel() > 0) {
+    w = indice_weights->to(at::kFloat).contiguous(); // embedding_forward_quantized_host.cpp:345
+  }
+  const int64_t align = row_alignment ? *row_alignment : 16; // embedding_forward_quantized_host.cpp:310
+  std::lock_guard<std::mutex> lk(g_mu);
+  fbgemm_amd_tbe_plan* plan = plan_for(dev_weights, uvm_weights, weights_placements, weights_offsets, weights_tys,
+                                       D_offsets, align);
+  const int64_t T = D_offsets.numel() - 1;
+  TORCH_CHECK(T > 0 && total_D > 0);
+  const int64_t B = (offsets.numel() - 1) / T;
+  TORCH_CHECK(B >= 0);
+  Tensor out = at::empty({B, total_D}, dev_weights.options().dtype(out_scalar_type(output_dtype)));
+  if (B == 0) return out;
+  Tensor& st = status_block(dev_weights);
+  const int rc = fbgemm_amd_tbe_forward(
+      plan, dev_weights.data_ptr(), uvm_weights.numel() ? uvm_weights.data_ptr() : nullptr, indices.data_ptr(),
+      offsets.data_ptr(), indices.scalar_type() == at::kLong ? 64 : 32, indices.numel(), offsets.numel(),
+      (int32_t)pooling_mode, w.defined() ? w.data_ptr<float>() : nullptr, (int32_t)output_dtype, out.data_ptr(),
+      st.data_ptr(), current_stream(dev_weights));
+  TORCH_CHECK(rc == 0, "fbgemm_amd: ", fbgemm_amd_last_error());
+  return out;
+}
+
+// Out-of-range indices are recorded on the device and do not stop the stream
+// (the reference's GPU operator does not look at them at all; its CPU operator
+// raises). This reads the record: synchronizes, returns the FBGEMM_AMD_ERR_*
+// bits seen since the last call and clears them.
+int64_t lookup_status(Tensor like) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  Tensor& st = status_block(like);
+  int32_t bits = 0;
+  int64_t pos = -1;
+  TORCH_CHECK(fbgemm_amd_status_read(st.data_ptr(), current_stream(like), &bits, &pos) == 0, fbgemm_amd_last_error());
+  TORCH_CHECK(fbgemm_amd_status_clear(st.data_ptr(), current_stream(like)) == 0, fbgemm_amd_last_error());
+  return bits;
+}
+
+Tensor pruned_array_lookup_hip(Tensor indices, Tensor offsets, Tensor index_remappings, Tensor index_remappings_offsets) {
+  TORCH_CHECK(indices.is_cuda() && offsets.is_cuda() && index_remappings.is_cuda() && index_remappings_offsets.is_cuda());
+  TORCH_CHECK(indices.scalar_type() == offsets.scalar_type(), "indices and offsets must have the same dtype");
+  indices = indices.contiguous();
+  offsets = offsets.contiguous();
+  index_remappings = index_remappings.contiguous();
+  const Tensor ro = index_remappings_offsets.to(at::kLong).contiguous();
+  const int64_t T = ro.numel() - 1;
+  Tensor dense = at::empty_like(indices);
+  const int rc = fbgemm_amd_pruned_array_lookup(
+      indices.data_ptr(), offsets.data_ptr(), indices.scalar_type() == at::kLong ? 64 : 32, offsets.numel(),
+      index_remappings.data_ptr(), index_remappings.scalar_type() == at::kLong ? 64 : 32, ro.data_ptr<int64_t>(),
+      (int32_t)T, dense.data_ptr(), current_stream(indices));
+  TORCH_CHECK(rc == 0, "fbgemm_amd: ", fbgemm_amd_last_error());
+  return dense;
+}
+
+} // namespace
+
+// The schema strings are the reference's, character for character. When a real
+// fbgemm_gpu is loaded in the same process it has already defined them: build
+// with -DFBGEMM_AMD_IMPL_ONLY to register the implementations alone.
+TORCH_LIBRARY_FRAGMENT(fbgemm, m) {
+#ifndef FBGEMM_AMD_IMPL_ONLY
+  m.def(
+      "int_nbit_split_embedding_codegen_lookup_function(Tensor dev_weights, Tensor uvm_weights, Tensor weights_placements, Tensor weights_offsets, Tensor weights_tys, Tensor D_offsets, SymInt total_D, int max_int2_D, int max_int4_D, int max_int8_D, int max_float16_D, int max_float32_D, Tensor indices, Tensor offsets, int pooling_mode, Tensor? indice_weights, int output_dtype=1, Tensor? lxu_cache_weights=None, Tensor? lxu_cache_locations=None, int? row_alignment = None, int? max_float8_D=0, int? fp8_exponent_bits=-1, int? fp8_exponent_bias=-1) -> Tensor");
+  m.def(
+      "pruned_array_lookup(Tensor indices, Tensor offsets, Tensor index_remappings, Tensor index_remappings_offsets) -> Tensor");
+#endif
+  m.impl("int_nbit_split_embedding_codegen_lookup_function",
+         torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(int_nbit_split_embedding_codegen_lookup_function_hip)));
+  m.impl("pruned_array_lookup", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(pruned_array_lookup_hip)));
+}
+
+TORCH_LIBRARY_FRAGMENT(fbgemm_amd, m) {
+  m.def("lookup_status(Tensor like) -> int");
+  m.impl("lookup_status", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(lookup_status)));
+}

@@ -1,0 +1,230 @@
+// C++ face of the C ABI, shaped like include/fbgemm/FbgemmEmbedding.h of the
+// reference: the same factory templates with the same argument lists, returning
+// std::function objects with the EmbeddingSpMDMKernelSignature call signature.
+//
+// Differences a caller must know:
+//   * every pointer passed to a generated kernel is a DEVICE pointer;
+//   * the kernel runs on the stream set with fbgemm_amd::set_stream() (default
+//     stream otherwise) and, like the reference, returns only when done, with
+//     the reference's bool;
+//   * `prefetch` and THREAD_LOCAL are accepted and ignored (they tune the CPU
+//     code generator).
+// Header-only; link against libfbgemm_amd.so.
+#pragma once
+
+#include <cstdint>
+#include <functional>
+#include <stdexcept>
+#include <string>
+#include <type_traits>
+
+#include "fbgemm_amd.h"
+
+namespace fbgemm_amd {
+
+// 16-bit storage types, as in the reference's include/fbgemm/Types.h.
+struct float16 { std::uint16_t val; };
+struct bfloat16 { std::uint16_t val; };
+
+inline void*& stream_ref() {
+  static thread_local void* s = nullptr;
+  return s;
+}
+// Stream (hipStream_t) the kernels generated on this thread run on.
+inline void set_stream(void* hip_stream) { stream_ref() = hip_stream; }
+
+template <typename InType, typename IndexType, typename OffsetType = std::int32_t, typename OutType = float>
+class EmbeddingSpMDMKernelSignature {
+ public:
+  using Type = std::function<bool(
+      std::int64_t output_size, std::int64_t index_size, std::int64_t data_size, const InType* input,
+      const IndexType* indices, const OffsetType* offsets_or_lengths,
+      const float* weights, // optional, can be null for non-weighted sum
+      OutType* out)>;
+};
+
+template <typename InType, typename IndexType, typename OffsetType = std::int32_t>
+class EmbeddingSpMDMRowWiseSparseKernelSignature {
+ public:
+  using Type = std::function<bool(
+      std::int64_t output_size, std::int64_t index_size, std::int64_t uncompressed_data_size,
+      const InType* input, const IndexType* indices, const OffsetType* offsets_or_lengths,
+      const float* weights, float* out, const std::int32_t* compressed_indices_table)>;
+};
+
+namespace detail {
+
+template <typename T>
+constexpr int bits_of() {
+  static_assert(std::is_same_v<T, std::int32_t> || std::is_same_v<T, std::int64_t>, "index/offset type must be int32 or int64");
+  return sizeof(T) * 8;
+}
+
+template <typename InType>
+constexpr int weight_ty(bool is_bf16_in) {
+  if constexpr (std::is_same_v<InType, std::uint8_t>) return FBGEMM_AMD_INT8;
+  else if constexpr (std::is_same_v<InType, float>) return FBGEMM_AMD_FP32;
+  else if constexpr (std::is_same_v<InType, float16> || std::is_same_v<InType, std::uint16_t>)
+    return is_bf16_in ? FBGEMM_AMD_BF16 : FBGEMM_AMD_FP16;
+  else static_assert(sizeof(InType) == 0, "InType must be uint8_t, float16, uint16_t or float");
+}
+
+template <typename OutType>
+constexpr int output_ty(bool is_bf16_out) {
+  if constexpr (std::is_same_v<OutType, float>) return FBGEMM_AMD_FP32;
+  else if constexpr (std::is_same_v<OutType, float16> || std::is_same_v<OutType, std::uint16_t>)
+    return is_bf16_out ? FBGEMM_AMD_BF16 : FBGEMM_AMD_FP16;
+  else if constexpr (std::is_same_v<OutType, bfloat16>) return FBGEMM_AMD_BF16;
+  else static_assert(sizeof(OutType) == 0, "OutType must be float, float16, uint16_t or bfloat16");
+}
+
+inline bool run(const fbgemm_amd_spmdm_config& cfg, std::int64_t output_size, std::int64_t index_size,
+                std::int64_t data_size, const void* input, const void* indices, const void* offsets,
+                const float* weights, void* out, const std::int32_t* table, bool has_weight) {
+  if (has_weight != (weights != nullptr))
+    throw std::invalid_argument("fbgemm_amd: weights must be given exactly when has_weight was set");
+  const int rc = fbgemm_amd_spmdm_run(&cfg, output_size, index_size, data_size, input, indices, offsets, weights,
+                                      out, table, stream_ref());
+  if (rc < 0) throw std::runtime_error(std::string("fbgemm_amd: ") + fbgemm_amd_last_error());
+  return rc == 1;
+}
+
+} // namespace detail
+
+// GenerateEmbeddingSpMDMWithStrides (FbgemmEmbedding.h:94-117)
+template <typename InType, typename IndexType, typename OffsetType = std::int32_t, typename OutType = float,
+          bool THREAD_LOCAL = false>
+typename EmbeddingSpMDMKernelSignature<InType, IndexType, OffsetType, OutType>::Type
+GenerateEmbeddingSpMDMWithStrides(const std::int64_t block_size, bool has_weight, bool normalize_by_lengths,
+                                  int /*prefetch*/ = 16, bool is_weight_positional = false, bool use_offsets = true,
+                                  std::int64_t output_stride = -1, std::int64_t input_stride = -1,
+                                  bool scale_bias_last = true, bool no_bag = false, bool is_bf16_out = false,
+                                  bool is_bf16_in = false) {
+  if (no_bag) throw std::invalid_argument("fbgemm_amd: no_bag (sequence output) is not on this path");
+  fbgemm_amd_spmdm_config cfg{};
+  cfg.weight_ty = detail::weight_ty<InType>(is_bf16_in);
+  cfg.output_ty = detail::output_ty<OutType>(is_bf16_out);
+  cfg.index_bits = detail::bits_of<IndexType>();
+  cfg.offset_bits = detail::bits_of<OffsetType>();
+  cfg.block_size = block_size;
+  cfg.output_stride = output_stride;
+  cfg.input_stride = input_stride;
+  cfg.normalize_by_lengths = normalize_by_lengths;
+  cfg.is_weight_positional = is_weight_positional;
+  cfg.use_offsets = use_offsets;
+  cfg.scale_bias_last = scale_bias_last;
+  return [cfg, has_weight](std::int64_t output_size, std::int64_t index_size, std::int64_t data_size,
+                           const InType* input, const IndexType* indices, const OffsetType* offsets_or_lengths,
+                           const float* weights, OutType* out) {
+    return detail::run(cfg, output_size, index_size, data_size, input, indices, offsets_or_lengths, weights, out,
+                       nullptr, has_weight);
+  };
+}
+
+// GenerateEmbeddingSpMDM (FbgemmEmbedding.h:65-84)
+template <typename InType, typename IndexType, typename OffsetType = std::int32_t, typename OutType = float,
+          bool THREAD_LOCAL = false>
+typename EmbeddingSpMDMKernelSignature<InType, IndexType, OffsetType, OutType>::Type
+GenerateEmbeddingSpMDM(const std::int64_t block_size, bool has_weight, bool normalize_by_lengths, int prefetch = 16,
+                       bool is_weight_positional = false, bool use_offsets = true, bool is_bf16_out = false,
+                       bool is_bf16_in = false) {
+  return GenerateEmbeddingSpMDMWithStrides<InType, IndexType, OffsetType, OutType, THREAD_LOCAL>(
+      block_size, has_weight, normalize_by_lengths, prefetch, is_weight_positional, use_offsets, -1, -1, true, false,
+      is_bf16_out, is_bf16_in);
+}
+
+// GenerateEmbeddingSpMDMNBitWithStrides (FbgemmEmbedding.h:151-174)
+template <typename IndexType, typename OffsetType = std::int32_t, typename OutType = float, bool THREAD_LOCAL = false>
+typename EmbeddingSpMDMKernelSignature<std::uint8_t, IndexType, OffsetType, OutType>::Type
+GenerateEmbeddingSpMDMNBitWithStrides(const int input_bit_rate, const std::int64_t block_size, bool has_weight,
+                                      bool normalize_by_lengths, int /*prefetch*/ = 16,
+                                      bool is_weight_positional = false, bool use_offsets = true,
+                                      std::int64_t output_stride = -1, std::int64_t input_stride = -1,
+                                      bool scale_bias_last = true, const bool is_bf16_out = false,
+                                      const bool no_bag = false, int /*output_bit_rate*/ = -1) {
+  if (input_bit_rate != 2 && input_bit_rate != 4) throw std::invalid_argument("fbgemm_amd: input_bit_rate must be 2 or 4");
+  if (no_bag) throw std::invalid_argument("fbgemm_amd: no_bag (sequence output) is not on this path");
+  fbgemm_amd_spmdm_config cfg{};
+  cfg.weight_ty = input_bit_rate == 4 ? FBGEMM_AMD_INT4 : FBGEMM_AMD_INT2;
+  cfg.output_ty = detail::output_ty<OutType>(is_bf16_out);
+  cfg.index_bits = detail::bits_of<IndexType>();
+  cfg.offset_bits = detail::bits_of<OffsetType>();
+  cfg.block_size = block_size;
+  cfg.output_stride = output_stride;
+  cfg.input_stride = input_stride;
+  cfg.normalize_by_lengths = normalize_by_lengths;
+  cfg.is_weight_positional = is_weight_positional;
+  cfg.use_offsets = use_offsets;
+  cfg.scale_bias_last = scale_bias_last;
+  return [cfg, has_weight](std::int64_t output_size, std::int64_t index_size, std::int64_t data_size,
+                           const std::uint8_t* input, const IndexType* indices, const OffsetType* offsets_or_lengths,
+                           const float* weights, OutType* out) {
+    return detail::run(cfg, output_size, index_size, data_size, input, indices, offsets_or_lengths, weights, out,
+                       nullptr, has_weight);
+  };
+}
+
+// GenerateEmbeddingSpMDMNBit (FbgemmEmbedding.h:124-140)
+template <typename IndexType, typename OffsetType = std::int32_t, typename OutType = float>
+typename EmbeddingSpMDMKernelSignature<std::uint8_t, IndexType, OffsetType, OutType>::Type
+GenerateEmbeddingSpMDMNBit(int bit_rate, const std::int64_t block_size, bool has_weight, bool normalize_by_lengths,
+                           int prefetch = 16, bool is_weight_positional = false, bool use_offsets = true) {
+  return GenerateEmbeddingSpMDMNBitWithStrides<IndexType, OffsetType, OutType>(
+      bit_rate, block_size, has_weight, normalize_by_lengths, prefetch, is_weight_positional, use_offsets);
+}
+
+// GenerateEmbeddingSpMDMRowWiseSparse (FbgemmEmbedding.h:229-243)
+template <typename InType, typename IndexType, typename OffsetType = std::int32_t>
+typename EmbeddingSpMDMRowWiseSparseKernelSignature<InType, IndexType, OffsetType>::Type
+GenerateEmbeddingSpMDMRowWiseSparse(const std::int64_t block_size, bool has_weight, bool normalize_by_lengths,
+                                    int /*prefetch*/ = 16, bool is_weight_positional = false, bool use_offsets = true) {
+  fbgemm_amd_spmdm_config cfg{};
+  cfg.weight_ty = detail::weight_ty<InType>(false);
+  cfg.output_ty = FBGEMM_AMD_FP32;
+  cfg.index_bits = detail::bits_of<IndexType>();
+  cfg.offset_bits = detail::bits_of<OffsetType>();
+  cfg.block_size = block_size;
+  cfg.output_stride = -1;
+  cfg.input_stride = -1;
+  cfg.normalize_by_lengths = normalize_by_lengths;
+  cfg.is_weight_positional = is_weight_positional;
+  cfg.use_offsets = use_offsets;
+  cfg.scale_bias_last = true;
+  return [cfg, has_weight](std::int64_t output_size, std::int64_t index_size, std::int64_t uncompressed_data_size,
+                           const InType* input, const IndexType* indices, const OffsetType* offsets_or_lengths,
+                           const float* weights, float* out, const std::int32_t* compressed_indices_table) {
+    if (!compressed_indices_table) throw std::invalid_argument("fbgemm_amd: compressed_indices_table is null");
+    return detail::run(cfg, output_size, index_size, uncompressed_data_size, input, indices, offsets_or_lengths,
+                       weights, out, compressed_indices_table, has_weight);
+  };
+}
+
+// GenerateEmbeddingSpMDMNBitRowWiseSparse (FbgemmEmbedding.h:250-262)
+template <typename IndexType, typename OffsetType = std::int32_t>
+typename EmbeddingSpMDMRowWiseSparseKernelSignature<std::uint8_t, IndexType, OffsetType>::Type
+GenerateEmbeddingSpMDMNBitRowWiseSparse(int bit_rate, const std::int64_t block_size, bool has_weight,
+                                        bool normalize_by_lengths, int /*prefetch*/ = 16,
+                                        bool is_weight_positional = false, bool use_offsets = true) {
+  if (bit_rate != 2 && bit_rate != 4) throw std::invalid_argument("fbgemm_amd: bit_rate must be 2 or 4");
+  fbgemm_amd_spmdm_config cfg{};
+  cfg.weight_ty = bit_rate == 4 ? FBGEMM_AMD_INT4 : FBGEMM_AMD_INT2;
+  cfg.output_ty = FBGEMM_AMD_FP32;
+  cfg.index_bits = detail::bits_of<IndexType>();
+  cfg.offset_bits = detail::bits_of<OffsetType>();
+  cfg.block_size = block_size;
+  cfg.output_stride = -1;
+  cfg.input_stride = -1;
+  cfg.normalize_by_lengths = normalize_by_lengths;
+  cfg.is_weight_positional = is_weight_positional;
+  cfg.use_offsets = use_offsets;
+  cfg.scale_bias_last = true;
+  return [cfg, has_weight](std::int64_t output_size, std::int64_t index_size, std::int64_t uncompressed_data_size,
+                           const std::uint8_t* input, const IndexType* indices, const OffsetType* offsets_or_lengths,
+                           const float* weights, float* out, const std::int32_t* compressed_indices_table) {
+    if (!compressed_indices_table) throw std::invalid_argument("fbgemm_amd: compressed_indices_table is null");
+    return detail::run(cfg, output_size, index_size, uncompressed_data_size, input, indices, offsets_or_lengths,
+                       weights, out, compressed_indices_table, has_weight);
+  };
+}
+
+} // namespace fbgemm_amd

@@ -1,0 +1,163 @@
+// Drives the C++ factory templates of include/fbgemm_amd_embedding.hpp the way
+// the reference's gtests drive fbgemm::GenerateEmbeddingSpMDM*
+// (test/EmbeddingSpMDMNBitTest.cc:92-418, test/EmbeddingSpMDM8BitTest.cc:82-372):
+// random table, random bags, optimized kernel vs the scalar oracle, every
+// output bit equal, ten sentinel values after the output untouched, and the
+// corner cases (empty indices, out-of-range index, lengths-sum mismatch)
+// returning false. Exit code 0 = all cases passed.
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstring>
+#include <random>
+#include <vector>
+
+#include "../../include/fbgemm_amd_embedding.hpp"
+
+extern "C" int oracle_embedding_spmdm(
+    int in_ty, int64_t block_size, int64_t output_size, int64_t index_size, int64_t data_size, const void* input,
+    const void* indices, int idx64, const void* offsets_or_lengths, int off64, const float* weights,
+    int normalize_by_lengths, void* out, int out_ty, int is_weight_positional, int use_offsets,
+    int64_t output_stride, int64_t input_stride, int scale_bias_last, const int32_t* remap);
+extern "C" uint16_t oracle_float2half_rn(float f);
+
+#define HIP_OK(x) do { hipError_t e_ = (x); if (e_ != hipSuccess) { printf("%s: %s\n", #x, hipGetErrorString(e_)); return 2; } } while (0)
+
+template <typename T>
+struct Dev {
+  T* p = nullptr;
+  size_t n = 0;
+  explicit Dev(const std::vector<T>& h) : n(h.size()) {
+    (void)hipMalloc((void**)&p, std::max<size_t>(n, 1) * sizeof(T));
+    if (n) (void)hipMemcpy(p, h.data(), n * sizeof(T), hipMemcpyHostToDevice);
+  }
+  ~Dev() { (void)hipFree(p); }
+  std::vector<T> host() const {
+    std::vector<T> h(n);
+    if (n) (void)hipMemcpy(h.data(), p, n * sizeof(T), hipMemcpyDeviceToHost);
+    return h;
+  }
+};
+
+static int failures = 0;
+#define CHECK(cond, ...) do { if (!(cond)) { ++failures; printf("FAIL %s:%d: ", __FILE__, __LINE__); printf(__VA_ARGS__); printf("\n"); } } while (0)
+
+template <typename IndexType, typename OffsetType, typename OutType>
+void run_nbit(int bit_rate, int64_t D, int batch, int rows, int avg_len, bool weighted, bool normalize, bool use_offsets,
+              int corner /*0 none, 1 empty indices, 2 out-of-range, 3 unmatched lengths*/, unsigned seed) {
+  std::mt19937 rng(seed);
+  const int epb = 8 / bit_rate;
+  const int64_t stride = (D + epb - 1) / epb + 4;
+  std::vector<uint8_t> table(rows * stride);
+  for (auto& b : table) b = rng() & 0xff;
+  for (int r = 0; r < rows; ++r) {
+    uint16_t sb[2] = {oracle_float2half_rn(0.01f + 0.09f * (rng() % 1000) / 1000.f),
+                      oracle_float2half_rn(-1.f + 2.f * (rng() % 1000) / 1000.f)};
+    memcpy(&table[r * stride + stride - 4], sb, 4);
+  }
+  std::vector<OffsetType> lengths(batch), offsets(batch + 1, 0);
+  for (int b = 0; b < batch; ++b) {
+    lengths[b] = corner == 1 ? 0 : 1 + rng() % (2 * avg_len);
+    offsets[b + 1] = offsets[b] + lengths[b];
+  }
+  int64_t n = offsets[batch];
+  std::vector<IndexType> indices(n);
+  for (auto& i : indices) i = rng() % rows;
+  if (n) indices[0] = rows - 1;
+  if (corner == 2 && n) indices[n / 2] = rows;
+  int64_t index_size = n;
+  if (corner == 3) { index_size = n + 1; indices.push_back(0); }
+  std::vector<float> w(indices.size());
+  for (auto& x : w) x = (float)(rng() % 2000) / 1000.f - 1.f;
+
+  const int out_ty = std::is_same_v<OutType, float> ? FBGEMM_AMD_FP32 : FBGEMM_AMD_FP16;
+  constexpr int kSentinels = 10;
+  std::vector<OutType> out_ref(batch * D + kSentinels), out_init(batch * D + kSentinels);
+  OutType sentinel;
+  memset(&sentinel, 0xAB, sizeof(sentinel));
+  for (auto& o : out_init) o = sentinel;
+  out_ref = out_init;
+  const int ok_ref = oracle_embedding_spmdm(
+      bit_rate == 4 ? FBGEMM_AMD_INT4 : FBGEMM_AMD_INT2, D, batch, index_size, rows, table.data(), indices.data(),
+      sizeof(IndexType) == 8, use_offsets ? (const void*)offsets.data() : (const void*)lengths.data(),
+      sizeof(OffsetType) == 8, weighted ? w.data() : nullptr, normalize, out_ref.data(), out_ty, 0, use_offsets, -1, -1, 1,
+      nullptr);
+
+  Dev<uint8_t> d_table(table);
+  Dev<IndexType> d_idx(indices);
+  Dev<OffsetType> d_off(use_offsets ? offsets : lengths);
+  Dev<float> d_w(w);
+  Dev<OutType> d_out(out_init);
+  auto kernel = fbgemm_amd::GenerateEmbeddingSpMDMNBit<IndexType, OffsetType, OutType>(
+      bit_rate, D, weighted, normalize, 16, false, use_offsets);
+  const bool ok = kernel(batch, index_size, rows, d_table.p, d_idx.p, d_off.p, weighted ? d_w.p : nullptr, d_out.p);
+  CHECK(ok == (ok_ref != 0), "return value %d vs oracle %d (bit_rate %d D %ld corner %d)", (int)ok, ok_ref, bit_rate, (long)D, corner);
+  if (ok && ok_ref) {
+    auto got = d_out.host();
+    CHECK(memcmp(got.data(), out_ref.data(), got.size() * sizeof(OutType)) == 0,
+          "output differs (bit_rate %d D %ld batch %d weighted %d normalize %d use_offsets %d)", bit_rate, (long)D, batch,
+          weighted, normalize, use_offsets);
+  }
+}
+
+template <typename IndexType, typename OffsetType>
+void run_8bit(int64_t D, int batch, int rows, int avg_len, bool weighted, bool normalize, unsigned seed) {
+  std::mt19937 rng(seed);
+  const int64_t stride = D + 8;
+  std::vector<uint8_t> table(rows * stride);
+  for (auto& b : table) b = rng() & 0xff;
+  for (int r = 0; r < rows; ++r) {
+    float sb[2] = {0.001f + 0.009f * (rng() % 1000) / 1000.f, -1.f + 2.f * (rng() % 1000) / 1000.f};
+    memcpy(&table[r * stride + D], sb, 8);
+  }
+  std::vector<OffsetType> offsets(batch + 1, 0);
+  for (int b = 0; b < batch; ++b) offsets[b + 1] = offsets[b] + 1 + rng() % (2 * avg_len);
+  std::vector<IndexType> indices(offsets[batch]);
+  for (auto& i : indices) i = rng() % rows;
+  std::vector<float> w(indices.size());
+  for (auto& x : w) x = (float)(rng() % 2000) / 1000.f - 1.f;
+  std::vector<float> out_ref(batch * D, 0.f), out_init(batch * D, -7.f);
+  const int ok_ref = oracle_embedding_spmdm(FBGEMM_AMD_INT8, D, batch, indices.size(), rows, table.data(), indices.data(),
+                                            sizeof(IndexType) == 8, offsets.data(), sizeof(OffsetType) == 8,
+                                            weighted ? w.data() : nullptr, normalize, out_ref.data(), FBGEMM_AMD_FP32, 0, 1,
+                                            -1, -1, 1, nullptr);
+  Dev<uint8_t> d_table(table);
+  Dev<IndexType> d_idx(indices);
+  Dev<OffsetType> d_off(offsets);
+  Dev<float> d_w(w);
+  Dev<float> d_out(out_init);
+  auto kernel = fbgemm_amd::GenerateEmbeddingSpMDM<uint8_t, IndexType, OffsetType, float>(D, weighted, normalize);
+  const bool ok = kernel(batch, indices.size(), rows, d_table.p, d_idx.p, d_off.p, weighted ? d_w.p : nullptr, d_out.p);
+  CHECK(ok && ok_ref, "8-bit lookup rejected valid input");
+  auto got = d_out.host();
+  CHECK(memcmp(got.data(), out_ref.data(), got.size() * 4) == 0, "8-bit output differs (D %ld weighted %d normalize %d)",
+        (long)D, weighted, normalize);
+}
+
+int main() {
+  int ndev = 0;
+  HIP_OK(hipGetDeviceCount(&ndev));
+  if (ndev == 0) { printf("no GPU\n"); return 3; }
+  // shapes after test/EmbeddingSpMDMNBitTest.cc:21-46 (batch, rows, dim, average length)
+  const int shapes[][4] = {{10, 400, 2, 5}, {10, 400, 4, 5}, {10, 400, 8, 5}, {10, 400, 40, 5}, {10, 400, 48, 5},
+                           {10, 400, 56, 5}, {3, 1000, 86, 20}, {10, 400, 128, 5}, {10, 400, 164, 5}, {100, 4000, 256, 20}};
+  unsigned seed = 1;
+  for (auto& s : shapes)
+    for (int bit_rate : {2, 4})
+      for (int weighted = 0; weighted < 2; ++weighted)
+        for (int normalize = 0; normalize < 2; ++normalize)
+          for (int corner = 0; corner < 4; ++corner) {
+            if (bit_rate == 2 && s[2] % 4) continue;
+            run_nbit<int64_t, int32_t, float>(bit_rate, s[2], s[0], s[1], s[3], weighted, normalize, true, corner, ++seed);
+            run_nbit<int32_t, int64_t, fbgemm_amd::float16>(bit_rate, s[2], s[0], s[1], s[3], weighted, normalize,
+                                                            corner != 3 && (seed & 1), corner, ++seed);
+          }
+  for (auto& s : shapes)
+    for (int weighted = 0; weighted < 2; ++weighted)
+      for (int normalize = 0; normalize < 2; ++normalize) {
+        run_8bit<int64_t, int32_t>(s[2], s[0], s[1], s[3], weighted, normalize, ++seed);
+        run_8bit<int32_t, int32_t>(s[2], s[0], s[1], s[3], weighted, normalize, ++seed);
+      }
+  printf("%s: %d failure(s)\n", failures ? "FAILED" : "PASSED", failures);
+  return failures ? 1 : 0;
+}

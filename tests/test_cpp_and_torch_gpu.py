@@ -1,0 +1,101 @@
+"""The two compiled host faces of the library on the GPU: the C++ factory
+templates (include/fbgemm_amd_embedding.hpp, driven by tests/cpp/test_factories.cpp
+against the C oracle) and the torch operator library that registers the
+reference's schema."""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+import helpers as H
+from helpers import BF16, FP16, FP32, INT2, INT4, INT8
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_cpp_factories_against_oracle():
+    exe = os.path.join(ROOT, "tests", "cpp", "_build", "test_factories")
+    assert os.path.exists(exe), "build it with `python -m fbgemm_amd.build`"
+    proc = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+    print(proc.stdout[-3000:])
+    assert proc.returncode == 0 and "PASSED" in proc.stdout
+
+
+@pytest.fixture(scope="module")
+def torch_ops():
+    assert torch.cuda.is_available()
+    lib = os.path.join(ROOT, "fbgemm_amd", "lib", "libfbgemm_amd_torch.so")
+    assert os.path.exists(lib), "build it with `python -m fbgemm_amd.build`"
+    torch.ops.load_library(lib)
+    return torch.ops.fbgemm
+
+
+def cu(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def test_registered_schema_is_the_references(torch_ops):
+    schema = str(torch_ops.int_nbit_split_embedding_codegen_lookup_function.default._schema)
+    assert schema == (
+        "fbgemm::int_nbit_split_embedding_codegen_lookup_function(Tensor dev_weights, Tensor uvm_weights, "
+        "Tensor weights_placements, Tensor weights_offsets, Tensor weights_tys, Tensor D_offsets, SymInt total_D, "
+        "int max_int2_D, int max_int4_D, int max_int8_D, int max_float16_D, int max_float32_D, Tensor indices, "
+        "Tensor offsets, int pooling_mode, Tensor? indice_weights, int output_dtype=1, "
+        "Tensor? lxu_cache_weights=None, Tensor? lxu_cache_locations=None, int? row_alignment=None, "
+        "int? max_float8_D=0, int? fp8_exponent_bits=-1, int? fp8_exponent_bias=-1) -> Tensor")
+    assert str(torch_ops.pruned_array_lookup.default._schema) == (
+        "fbgemm::pruned_array_lookup(Tensor indices, Tensor offsets, Tensor index_remappings, "
+        "Tensor index_remappings_offsets) -> Tensor")
+
+
+def test_torch_operator_matches_oracle(torch_ops, oracle):
+    from test_tbe_gpu import build_weights
+    rng = np.random.default_rng(77)
+    specs = [(300, 64, INT4), (200, 128, INT8), (100, 32, FP16), (150, 256, INT4), (80, 32, INT2), (60, 16, FP32)]
+    T, B = len(specs), 29
+    weights, wo, _ = build_weights(rng, specs, 16)
+    tys = np.array([s[2] for s in specs], np.uint8)
+    D_offsets = np.concatenate([[0], np.cumsum([s[1] for s in specs])]).astype(np.int32)
+    total_D = int(D_offsets[-1])
+    lens = rng.integers(0, 30, size=T * B)
+    for dt in (np.int32, np.int64):
+        off = np.concatenate([[0], np.cumsum(lens)]).astype(dt)
+        idx = np.concatenate([rng.integers(0, specs[t][0], size=int(lens[t * B:(t + 1) * B].sum())) for t in range(T)]).astype(dt)
+        idx[rng.random(len(idx)) < 0.1] = -1
+        psw = rng.uniform(0, 1, len(idx)).astype(np.float32)
+        for pooling, w, out_ty, tdt in ((0, psw, FP16, torch.float16), (1, None, FP32, torch.float32), (0, None, BF16, torch.bfloat16)):
+            got = torch_ops.int_nbit_split_embedding_codegen_lookup_function(
+                cu(weights), torch.zeros(0, dtype=torch.uint8, device="cuda"), cu(np.zeros(T, np.int32)), cu(wo), cu(tys),
+                cu(D_offsets), total_D, 32, 256, 128, 32, 16, cu(idx), cu(off), pooling,
+                None if w is None else cu(w), out_ty, None, None, 16)
+            assert got.dtype == tdt and tuple(got.shape) == (B, total_D)
+            rc, want = oracle.tbe_forward(weights, wo, tys, D_offsets, total_D, idx, off, pooling, w, out_ty, 16)
+            assert rc == 0
+            g = got.cpu()
+            g = g.numpy() if out_ty == FP32 else g.view(torch.int16).numpy().view(np.uint16)
+            H.assert_same_bits(g, want, f"torch op dt={dt} pool={pooling} out={out_ty}")
+    assert torch.ops.fbgemm_amd.lookup_status(cu(weights)) == 0
+    # an out-of-range index is recorded, not fatal (the GPU operator of the reference does not check at all)
+    bad = idx.copy(); bad[5] = 10**6
+    out = torch_ops.int_nbit_split_embedding_codegen_lookup_function(
+        cu(weights), torch.zeros(0, dtype=torch.uint8, device="cuda"), cu(np.zeros(T, np.int32)), cu(wo), cu(tys),
+        cu(D_offsets), total_D, 32, 256, 128, 32, 16, cu(bad), cu(off), 0, None, FP16, None, None, 16)
+    assert torch.isfinite(out.float()).all()
+    assert torch.ops.fbgemm_amd.lookup_status(cu(weights)) == 1
+    assert torch.ops.fbgemm_amd.lookup_status(cu(weights)) == 0
+
+
+def test_torch_pruned_array_lookup(torch_ops, oracle):
+    rng = np.random.default_rng(5)
+    T, B = 3, 9
+    caps = [50, 0, 400]
+    ro = np.concatenate([[0], np.cumsum(caps)]).astype(np.int64)
+    remap = np.where(rng.random(int(ro[-1])) < 0.5, -1, rng.integers(0, 1000, int(ro[-1]))).astype(np.int32)
+    lens = rng.integers(0, 8, size=T * B)
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    idx = np.concatenate([rng.integers(0, caps[t] or 99, size=int(lens[t * B:(t + 1) * B].sum())) for t in range(T)]).astype(np.int64)
+    got = torch_ops.pruned_array_lookup(cu(idx), cu(off), cu(remap), cu(ro)).cpu().numpy()
+    assert (got == oracle.pruned_array_lookup(idx, off, remap, ro)).all()
