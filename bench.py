@@ -33,6 +33,8 @@ def parse():
     ap.add_argument("--scale", type=float, default=1.0, help="shrink rows and batch (1.0 = the real configuration)")
     ap.add_argument("--rows-scale", type=float, default=None,
                     help="config 3 only: shrink the tables but not the batch (cache-resident experiment)")
+    ap.add_argument("--only-type", type=int, default=None,
+                    help="config 3 only: give every table this row type (1 fp16, 2 int8, 3 int4); experiment")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
@@ -200,7 +202,7 @@ def main():
     torch.cuda.set_device(0)
     t_build = time.time()
     if a.config in (3, 5):
-        p = bc.config3("cuda", a.scale, a.rows_scale) if a.config == 3 else bc.config5("cuda", a.scale)
+        p = bc.config3("cuda", a.scale, a.rows_scale, a.only_type) if a.config == 3 else bc.config5("cuda", a.scale)
         launch, out, st, plan = tbe_runner(p, torch)
         lookups, useful = p.lookups, p.useful_row_bytes()
         other = p.other_bytes()

@@ -174,7 +174,7 @@ def build_tbe(name, seed, specs, B, lengths_fn, alpha, weighted, pooling_mode, o
         host_indices=indices, host_offsets=offsets, host_weights=w)
 
 
-def config3(device, scale=1.0, rows_scale=None):
+def config3(device, scale=1.0, rows_scale=None, only_type=None):
     """64 tables, int4/int8/fp16 = 50/25/25 %, rows 10**U[5,7], D in {64,128,256}, B = 2048 per
     table, L = min(Poisson(30), 200), Zipf(1.1), fp32 per-sample weights, weighted sum, fp16 out."""
     seed = 1003
@@ -183,6 +183,8 @@ def config3(device, scale=1.0, rows_scale=None):
     tys = rng.choice([INT4, INT8, FP16], size=T, p=[0.5, 0.25, 0.25])
     rows = np.round(10 ** rng.uniform(5, 7, size=T)).astype(np.int64)
     Ds = rng.choice([64, 128, 256], size=T)
+    if only_type is not None:  # experiment: same shapes, one row type
+        tys = np.full(T, only_type)
     rows_scale = scale if rows_scale is None else rows_scale
     if rows_scale != 1.0:
         rows = np.maximum(64, (rows * rows_scale).astype(np.int64))

@@ -1,0 +1,33 @@
+#!/bin/bash
+# Collect the rocprofv3 evidence for one benchmark configuration and condense it.
+#   bash fbgemm_amd/profile_run.sh <config id> <output summary file> [extra bench.py args]
+# Runs from the repository root on a machine with the GPU. One rocprofv3 run per
+# counter group (the hardware cannot collect them together); raw CSVs go to /tmp.
+set -o pipefail
+CFG=${1:-3}; OUT=${2:-profile_summary.txt}; shift; shift
+export TMPDIR=/tmp
+RAW=$(mktemp -d /tmp/fbgemm_amd_prof.XXXXXX)
+mkdir -p "$(dirname "$OUT")"
+BENCH="python3 bench.py --config $CFG --no-cpu --calibration-copy-mib 1024 $*"
+{
+  echo "# rocprofv3 summary, bench.py --config $CFG $*"
+  echo "# commands (each its own run):"
+  echo "#   rocprofv3 --kernel-trace --stats --output-format csv -d <dir> -o t -- $BENCH --steps 20 --warmup 3"
+  echo "#   rocprofv3 --pmc <counters> --output-format csv -d <dir> -o p -- $BENCH --steps 3 --warmup 1"
+  echo "# condensed with: python3 -m fbgemm_amd.profile_summary <dir>"
+} > "$OUT"
+echo "== kernel trace (--kernel-trace --stats), 23 launches" >> "$OUT"
+timeout -k 10 900 rocprofv3 --kernel-trace --stats --output-format csv -d $RAW/trace -o t -- $BENCH --steps 20 --warmup 3 > $RAW/trace.log 2>&1 || { echo "trace run failed" | tee -a "$OUT"; tail -5 $RAW/trace.log; exit 1; }
+grep '^{' $RAW/trace.log | tail -1 | cut -c1-1200 >> "$OUT"
+python3 -m fbgemm_amd.profile_summary $RAW/trace | grep -v '^#' >> "$OUT"
+for pass in "FETCH_SIZE" "WRITE_SIZE" "TCC_HIT_sum TCC_MISS_sum" "TCC_EA0_RDREQ_sum" \
+            "SQ_WAVES SQ_INSTS_VALU SQ_INSTS_VMEM_RD SQ_INSTS_LDS SQ_INSTS_SALU SQ_WAVE_CYCLES SQ_WAIT_INST_ANY SQ_ACTIVE_INST_VALU" \
+            "TCP_TCC_READ_REQ_sum TCP_TOTAL_CACHE_ACCESSES_sum TCP_TCC_READ_REQ_LATENCY_sum" "GRBM_GUI_ACTIVE"; do
+  n=$(echo $pass | tr ' ' '_' | cut -c1-40)
+  echo "== --pmc $pass" >> "$OUT"
+  timeout -s KILL 600 rocprofv3 --pmc $pass --output-format csv -d $RAW/pmc_$n -o p -- $BENCH --steps 3 --warmup 1 > $RAW/pmc_$n.log 2>&1 || { echo "pass failed: $pass" >> "$OUT"; tail -3 $RAW/pmc_$n.log >> "$OUT"; continue; }
+  python3 -m fbgemm_amd.profile_summary $RAW/pmc_$n | grep -v '^#\|^launch' >> "$OUT"
+done
+python3 -m fbgemm_amd.profile_summary $RAW/pmc_GRBM_GUI_ACTIVE | grep '^launch' >> "$OUT"
+rm -rf $RAW
+cat "$OUT"
