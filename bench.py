@@ -35,6 +35,9 @@ def parse():
                     help="config 3 only: shrink the tables but not the batch (cache-resident experiment)")
     ap.add_argument("--only-type", type=int, default=None,
                     help="config 3 only: give every table this row type (1 fp16, 2 int8, 3 int4); experiment")
+    ap.add_argument("--per-table", action="store_true",
+                    help="config 4 only: one row-wise-sparse kernel call per table (the reference's core-library "
+                         "API) instead of one table-batched forward with the remap fused in")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
@@ -59,10 +62,13 @@ def tbe_runner(p, torch):
             C.c_void_p(p.offsets.data_ptr()), 64 if p.indices.dtype == torch.int64 else 32, p.indices.numel(),
             p.offsets.numel(), p.pooling_mode,
             None if p.indice_weights is None else C.c_void_p(p.indice_weights.data_ptr()),
-            p.output_dtype, C.c_void_p(out.data_ptr()), C.c_void_p(st.buf.data_ptr()), stream)
+            p.output_dtype, C.c_void_p(out.data_ptr()),
+            C.c_void_p(p.extra["remap"].data_ptr()) if "remap" in p.extra else None, 32,
+            C.c_void_p(p.extra["remap_offsets"].data_ptr()) if "remap" in p.extra else None,
+            C.c_void_p(st.buf.data_ptr()), stream)
 
     def launch():
-        rc = lib.fbgemm_amd_tbe_forward(*args)
+        rc = lib.fbgemm_amd_tbe_forward_pruned(*args)
         if rc:
             raise RuntimeError(lib.fbgemm_amd_last_error().decode())
 
@@ -119,7 +125,7 @@ def cpu_baseline_tbe(p, seconds, torch):
     nt = max(nt, 1)
     end = int(p.weights_offsets[nt - 1] + p.rows[nt - 1] * p.row_bytes[nt - 1])
     host_w = p.dev_weights[:end].cpu().numpy()
-    idx = np.ascontiguousarray(p.host_indices, dtype=np.int64)
+    idx = np.ascontiguousarray(p.physical_indices, dtype=np.int64)  # after the remap, where there is one
     off = np.ascontiguousarray(p.host_offsets, dtype=np.int64)
     kept = p.kept_per_table()[:nt]
     sample_bytes = int(sum(int(k) * unpadded_row_bytes(int(D), int(ty)) for k, D, ty in zip(kept, p.Ds[:nt], p.tys[:nt])))
@@ -201,8 +207,9 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs the GPU"
     torch.cuda.set_device(0)
     t_build = time.time()
-    if a.config in (3, 5):
-        p = bc.config3("cuda", a.scale, a.rows_scale, a.only_type) if a.config == 3 else bc.config5("cuda", a.scale)
+    if a.config in (3, 5) or (a.config == 4 and not a.per_table):
+        p = (bc.config3("cuda", a.scale, a.rows_scale, a.only_type) if a.config == 3 else
+             bc.config5("cuda", a.scale) if a.config == 5 else bc.config4_batched("cuda", a.scale))
         launch, out, st, plan = tbe_runner(p, torch)
         lookups, useful = p.lookups, p.useful_row_bytes()
         other = p.other_bytes()
@@ -229,7 +236,7 @@ def main():
         for t in list(range(min(3, p.T))) + [p.T - 1]:
             s, e = int(p.host_offsets[t * p.B]), int(p.host_offsets[(t + 1) * p.B])
             elem = 4 if int(p.tys[t]) == 0 else 2 if int(p.tys[t]) == 1 else 1
-            ok, want = oracle.spmdm(int(p.tys[t]), int(p.Ds[t]), p.table_host_bytes(t), p.host_indices[s:e],
+            ok, want = oracle.spmdm(int(p.tys[t]), int(p.Ds[t]), p.table_host_bytes(t), p.physical_indices[s:e],
                                     p.host_offsets[t * p.B:(t + 1) * p.B + 1] - p.host_offsets[t * p.B],
                                     weights=None if p.host_weights is None else p.host_weights[s:e],
                                     normalize=p.pooling_mode == 1, out_ty=p.output_dtype,
@@ -243,6 +250,9 @@ def main():
     for _ in range(a.warmup):
         launch()
     torch.cuda.synchronize()
+    if p is not None:  # HIP events around every lookup_kernel launch of the timed region, on its stream
+        from fbgemm_amd import _lib
+        _lib.check(_lib.lib().fbgemm_amd_tbe_plan_profile(plan.handle, a.steps))
     ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     ev0.record()
@@ -263,7 +273,14 @@ def main():
             C.c_void_p(torch.cuda.current_stream().cuda_stream)))
         torch.cuda.synchronize()
     ms_per_step = wall * 1e3 / a.steps
-    kernel_ms = ev0.elapsed_time(ev1) / a.steps  # events on the launch stream, back-to-back launches
+    forward_ms = ev0.elapsed_time(ev1) / a.steps  # events on the launch stream, back-to-back forwards
+    kernel_ms, kernel_name = forward_ms, "lookup_kernel (+ bag_order_kernel), per forward"
+    if p is not None:
+        ms = (C.c_float * a.steps)()
+        n = C.c_int32(0)
+        _lib.check(_lib.lib().fbgemm_amd_tbe_plan_profile_read(plan.handle, ms, a.steps, C.byref(n)))
+        assert n.value == a.steps
+        kernel_ms, kernel_name = sum(ms[:n.value]) / n.value, "lookup_kernel"
 
     gbps = useful / (ms_per_step * 1e-3) / 1e9
     kern_gbps = useful / (kernel_ms * 1e-3) / 1e9
@@ -279,7 +296,8 @@ def main():
         "pooled_rows_per_s": round(lookups / (ms_per_step * 1e-3), 1),
         "roofline": {"bound": "hbm", "achieved": round(kern_gbps, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(kern_gbps / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel": "lookup_kernel", "kernel_ms": round(kernel_ms / launches_per_step, 5),
+                     "kernel": kernel_name, "kernel_ms": round(kernel_ms / launches_per_step, 5),
+                     "forward_ms": round(forward_ms, 5),
                      "algorithmic_bytes_per_launch": useful // launches_per_step},
         "setup_s": round(build_s, 1),
     }

@@ -34,6 +34,9 @@ SYMBOLS = {
     "fbgemm_amd_tbe_plan_create": (C.c_int, [C.POINTER(_P), _I32, _P, _P, _P, _P, _I64, _I64, _I64]),
     "fbgemm_amd_tbe_plan_destroy": (None, [_P]),
     "fbgemm_amd_tbe_forward": (C.c_int, [_P, _P, _P, _P, _P, _I32, _I64, _I64, _I32, _P, _I32, _P, _P, _P]),
+    "fbgemm_amd_tbe_forward_pruned": (C.c_int, [_P, _P, _P, _P, _P, _I32, _I64, _I64, _I32, _P, _I32, _P, _P, _I32, _P, _P, _P]),
+    "fbgemm_amd_tbe_plan_profile": (C.c_int, [_P, _I32]),
+    "fbgemm_amd_tbe_plan_profile_read": (C.c_int, [_P, _P, _I32, _P]),
     "fbgemm_amd_tbe_plan_num_rows": (_I64, [_P, _I32]),
     "fbgemm_amd_tbe_plan_row_bytes": (_I64, [_P, _I32]),
     "fbgemm_amd_pruned_array_lookup": (C.c_int, [_P, _P, _I32, _I64, _P, _I32, _P, _I32, _P, _P]),

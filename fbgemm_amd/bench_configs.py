@@ -70,12 +70,18 @@ class TbeProblem:
     def lookups(self):
         return int(self.host_offsets[-1])
 
+    @property
+    def physical_indices(self):
+        """Row ids after the pruned-row remap (the indices themselves when no table is pruned)."""
+        return self.extra.get("host_dense", self.host_indices)
+
     def kept_per_table(self):
-        """Lookups that actually read a row (index != -1), per table."""
+        """Lookups that actually read a row (physical index != -1), per table."""
         kept = np.zeros(self.T, np.int64)
+        phys = self.physical_indices
         for t in range(self.T):
             s, e = self.host_offsets[t * self.B], self.host_offsets[(t + 1) * self.B]
-            kept[t] = int((self.host_indices[s:e] != -1).sum())
+            kept[t] = int((phys[s:e] != -1).sum())
         return kept
 
     def useful_row_bytes(self):
@@ -93,6 +99,7 @@ class TbeProblem:
             "offsets": (self.T * self.B + 1) * isz,
             "per_sample_weights": self.lookups * 4 if self.indice_weights is not None else 0,
             "output": self.B * self.total_D * out_sz,
+            "remap_entries": self.lookups * 4 if "remap" in self.extra else 0,
         }
 
     def table_host_bytes(self, t):
@@ -128,11 +135,24 @@ def _fill_table(buf, rows, row_bytes, D, ty, gen, scale_range, chunk_rows=1 << 2
 
 
 def build_tbe(name, seed, specs, B, lengths_fn, alpha, weighted, pooling_mode, output_dtype,
-              device, row_alignment=16, index_dtype=np.int64, scale_ranges=None, prune_frac=0.0):
-    """specs: list of (rows, D, ty). lengths_fn(rng, n) -> bag lengths."""
+              device, row_alignment=16, index_dtype=np.int64, scale_ranges=None, prune_frac=0.0,
+              pruned_keep=None):
+    """specs: list of (rows, D, ty). lengths_fn(rng, n) -> bag lengths. With
+    ``pruned_keep`` = p, rows are LOGICAL rows: each table keeps a row with
+    probability p, stores only the kept rows, and indices are logical ids that
+    an int32 mapping (-1 = pruned) turns into physical rows."""
     rng = np.random.default_rng(np.random.PCG64(seed))
     T = len(specs)
     rows = np.array([s[0] for s in specs], np.int64)
+    logical = rows.copy()
+    mappings = []
+    if pruned_keep is not None:
+        for t in range(T):
+            keep = rng.random(int(logical[t])) < pruned_keep
+            m = np.full(int(logical[t]), -1, np.int32)
+            m[keep] = np.arange(int(keep.sum()), dtype=np.int32)
+            mappings.append(m)
+            rows[t] = max(1, int(keep.sum()))
     Ds = np.array([s[1] for s in specs], np.int32)
     tys = np.array([s[2] for s in specs], np.uint8)
     row_bytes = np.array([padded_row_bytes(int(D), int(ty), row_alignment) for D, ty in zip(Ds, tys)], np.int64)
@@ -146,7 +166,7 @@ def build_tbe(name, seed, specs, B, lengths_fn, alpha, weighted, pooling_mode, o
     idx_parts = []
     for t in range(T):
         n = int(offsets[(t + 1) * B] - offsets[t * B])
-        part = zipf_indices(rng, alpha, int(rows[t]), n)
+        part = zipf_indices(rng, alpha, int(logical[t]), n)
         if prune_frac > 0:
             part[rng.random(n) < prune_frac] = -1
         idx_parts.append(part)
@@ -164,7 +184,19 @@ def build_tbe(name, seed, specs, B, lengths_fn, alpha, weighted, pooling_mode, o
             sr = scale_ranges.get(int(tys[t]), sr)
         _fill_table(dev_weights[s:s + n], int(rows[t]), int(row_bytes[t]), int(Ds[t]), int(tys[t]), gen, sr)
 
+    extra = {}
+    if mappings:
+        remap_offsets = np.concatenate([[0], np.cumsum(logical)]).astype(np.int64)
+        remap = np.concatenate(mappings)
+        dense = indices.copy()
+        for t in range(T):
+            s, e = int(offsets[t * B]), int(offsets[(t + 1) * B])
+            dense[s:e] = mappings[t][indices[s:e]]
+        extra = {"remap": torch.from_numpy(remap).to(device), "remap_offsets": torch.from_numpy(remap_offsets).to(device),
+                 "host_remap": remap, "host_remap_offsets": remap_offsets, "host_dense": dense}
+
     return TbeProblem(
+        extra=extra,
         name=name, T=T, B=B, Ds=Ds, tys=tys, rows=rows, row_bytes=row_bytes,
         row_alignment=row_alignment, weights_offsets=weights_offsets, D_offsets=D_offsets,
         dev_weights=dev_weights, indices=torch.from_numpy(indices).to(device),
@@ -204,6 +236,19 @@ def config5(device, scale=1.0, tables_int4=400, tables_int2=32):
     B = max(4, int(round(16384 * scale)))
     return build_tbe("config5: HBM-sized int4 + int2 TBE forward", seed, specs, B,
                      lambda g, n: g.poisson(15, size=n), 1.2, False, POOL_SUM, BF16, device)
+
+
+def config4_batched(device, scale=1.0, tables=32):
+    """Config 4 as ONE table-batched call: 32 pruned int4 tables (2,000,000 logical rows x 64,
+    half of them pruned) in the operator's layout with 4-byte row alignment (36-byte rows), B =
+    4096, L = U{5..50}, Zipf(1.05) over logical ids, mean pooling, fp32 out; the int32 mappings of
+    all tables concatenated as pruned_array_lookup takes them."""
+    seed = 1004
+    logical = max(64, int(2_000_000 * scale))
+    B = max(4, int(round(4096 * scale)))
+    return build_tbe("config4: 32 pruned int4 tables, remap fused into one table-batched forward", seed,
+                     [(logical, 64, INT4)] * tables, B, lambda g, n: g.integers(5, 51, size=n), 1.05, False,
+                     POOL_MEAN, FP32, device, row_alignment=4, pruned_keep=0.5)
 
 
 @dataclass

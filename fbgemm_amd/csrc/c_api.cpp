@@ -370,6 +370,9 @@ struct fbgemm_amd_tbe_plan {
   };
   std::map<int32_t, Work> work;
   std::mutex mu;
+  // optional timing of the lookup kernel alone: a ring of (start, stop) event pairs
+  std::vector<hipEvent_t> prof_ev;
+  int64_t prof_count = 0;
 };
 
 extern "C" {
@@ -442,6 +445,7 @@ void fbgemm_amd_tbe_plan_destroy(fbgemm_amd_tbe_plan* plan) {
     if (kv.second.d_xcd_start) (void)hipFree(kv.second.d_xcd_start);
   }
   if (plan->d_tables) (void)hipFree(plan->d_tables);
+  for (hipEvent_t e : plan->prof_ev) (void)hipEventDestroy(e);
   delete plan;
 }
 
@@ -458,7 +462,21 @@ int fbgemm_amd_tbe_forward(
     int64_t indices_numel, int64_t offsets_numel, int32_t pooling_mode,
     const float* d_indice_weights, int32_t output_ty, void* d_output, void* d_status,
     void* stream_) {
+  return fbgemm_amd_tbe_forward_pruned(plan, d_dev_weights, d_uvm_weights, d_indices, d_offsets, index_bits,
+                                       indices_numel, offsets_numel, pooling_mode, d_indice_weights, output_ty,
+                                       d_output, nullptr, 32, nullptr, d_status, stream_);
+}
+
+int fbgemm_amd_tbe_forward_pruned(
+    fbgemm_amd_tbe_plan* plan, const void* d_dev_weights, const void* d_uvm_weights,
+    const void* d_indices, const void* d_offsets, int32_t index_bits,
+    int64_t indices_numel, int64_t offsets_numel, int32_t pooling_mode,
+    const float* d_indice_weights, int32_t output_ty, void* d_output,
+    const void* d_index_remappings, int32_t remap_bits, const int64_t* d_index_remappings_offsets,
+    void* d_status, void* stream_) {
   if (!plan) return fail(FBGEMM_AMD_E_ARG, "plan is null");
+  if (d_index_remappings && (!d_index_remappings_offsets || (remap_bits != 32 && remap_bits != 64)))
+    return fail(FBGEMM_AMD_E_ARG, "a remap array needs its T+1 offsets and 32- or 64-bit entries");
   if (index_bits != 32 && index_bits != 64) return fail(FBGEMM_AMD_E_ARG, "index_bits must be 32 or 64");
   if (output_ty != ST_FP32 && output_ty != ST_FP16 && output_ty != ST_BF16)
     return fail(FBGEMM_AMD_E_UNSUPPORTED, "output type %d is not supported", output_ty);
@@ -559,6 +577,9 @@ int fbgemm_amd_tbe_forward(
   a.offsets = d_offsets;
   a.off64 = index_bits == 64;
   a.sample_weights = d_indice_weights;
+  a.remap = d_index_remappings;
+  a.remap_offsets = d_index_remappings ? d_index_remappings_offsets : nullptr;
+  a.remap64 = remap_bits == 64;
   a.out = d_output;
   a.out_stride = plan->total_D;
   a.index_size = indices_numel;
@@ -576,7 +597,42 @@ int fbgemm_amd_tbe_forward(
     HIP_TRY(launch_bag_order(d_offsets, index_bits == 64, B, plan->T, w.d_order, stream));
     a.order = w.d_order;
   }
+  const size_t slots = plan->prof_ev.size() / 2;
+  const size_t slot = slots ? (size_t)(plan->prof_count % (int64_t)slots) : 0;
+  if (slots) HIP_TRY(hipEventRecord(plan->prof_ev[2 * slot], stream));
   HIP_TRY(launch_lookup(a, index_bits == 64, stream));
+  if (slots) {
+    HIP_TRY(hipEventRecord(plan->prof_ev[2 * slot + 1], stream));
+    ++plan->prof_count;
+  }
+  return 0;
+}
+
+int fbgemm_amd_tbe_plan_profile(fbgemm_amd_tbe_plan* plan, int32_t slots) {
+  if (!plan || slots < 0) return fail(FBGEMM_AMD_E_ARG, "bad profile arguments");
+  std::lock_guard<std::mutex> lk(plan->mu);
+  for (hipEvent_t e : plan->prof_ev) (void)hipEventDestroy(e);
+  plan->prof_ev.clear();
+  plan->prof_count = 0;
+  for (int i = 0; i < 2 * slots; ++i) {
+    hipEvent_t e;
+    HIP_TRY(hipEventCreate(&e));
+    plan->prof_ev.push_back(e);
+  }
+  return 0;
+}
+
+int fbgemm_amd_tbe_plan_profile_read(fbgemm_amd_tbe_plan* plan, float* ms, int32_t cap, int32_t* n) {
+  if (!plan || !ms || !n || cap < 0) return fail(FBGEMM_AMD_E_ARG, "bad profile arguments");
+  std::lock_guard<std::mutex> lk(plan->mu);
+  const int64_t slots = (int64_t)plan->prof_ev.size() / 2;
+  const int64_t have = std::min<int64_t>(std::min<int64_t>(plan->prof_count, slots), cap);
+  for (int64_t i = 0; i < have; ++i) {
+    HIP_TRY(hipEventSynchronize(plan->prof_ev[2 * i + 1]));
+    HIP_TRY(hipEventElapsedTime(&ms[i], plan->prof_ev[2 * i], plan->prof_ev[2 * i + 1]));
+  }
+  *n = (int32_t)have;
+  plan->prof_count = 0;
   return 0;
 }
 

@@ -78,8 +78,11 @@ struct LookupArgs {
   const void* indices;
   const void* offsets;       // T*B+1 offsets ((table, bag) order)
   const float* sample_weights; // nullptr: unweighted
-  const int32_t* remap;      // logical -> physical row table, or nullptr
-  int64_t remap_rows;        // bound for logical ids when remap != nullptr
+  const void* remap;         // logical -> physical row table(s), int32 or int64, or nullptr
+  const int64_t* remap_offsets; // nullptr: one table of remap_rows entries; else T+1 offsets
+                             // into `remap`, an empty range meaning "this table is not pruned"
+  int64_t remap_rows;        // bound for logical ids when remap_offsets == nullptr
+  int32_t remap64;           // remap entries are int64 (else int32)
   void* out;
   int64_t out_stride;        // elements between consecutive bags' outputs
   int64_t index_size;        // entries the index array holds for this call

@@ -408,6 +408,19 @@ __device__ __forceinline__ bool pool_bags(const LookupArgs& a, const TableDesc& 
   }
   const int n = (int)len; // same for every lane of the bag
 
+  // pruned tables: logical ids go through the table's slice of the remap array
+  int64_t remap_base = 0, remap_cap = 0;
+  bool remapped = false;
+  if (GENERAL && a.remap) {
+    remapped = true;
+    remap_cap = a.remap_rows;
+    if (a.remap_offsets) {
+      remap_base = a.remap_offsets[table];
+      remap_cap = a.remap_offsets[table + 1] - remap_base;
+      remapped = remap_cap > 0;
+    }
+  }
+
   const index_t* idx = reinterpret_cast<const index_t*>(a.indices);
   const uint8_t* wbase = (d.placement ? a.weights[1] : a.weights[0]) + d.weights_offset;
   const uint8_t* psb = wbase + d.sb_off;
@@ -464,13 +477,18 @@ __device__ __forceinline__ bool pool_bags(const LookupArgs& a, const TableDesc& 
         if (rr < R && row != NO_ENTRY) {
           const int64_t pos = pos0 + round * RN + sub + rr * SL;
           bool ok = true;
-          if (GENERAL && a.remap) {
-            if (row < 0 || row >= a.remap_rows) {
+          if (GENERAL && remapped) {
+            if (row < 0 || row >= remap_cap) {
               if (pass == 0) report_index(a.status, pos);
               ok = false;
             } else {
-              row = (int64_t)a.remap[row];
+              row = a.remap64 ? reinterpret_cast<const int64_t*>(a.remap)[remap_base + row]
+                              : (int64_t) reinterpret_cast<const int32_t*>(a.remap)[remap_base + row];
               ok = row != -1;
+              if (ok && (row < 0 || row >= d.num_rows)) {
+                if (pass == 0) report_index(a.status, pos);
+                ok = false;
+              }
             }
           } else if (d.skip_minus_one && row == -1) {
             ok = false;
@@ -823,7 +841,8 @@ __global__ __launch_bounds__(256) void pruned_array_lookup_kernel(
   const bool mapped = re - rs > 0;
   for (int64_t i = is + (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < ie; i += (int64_t)gridDim.x * blockDim.x) {
     index_t v = indices[i];
-    if (mapped) v = (index_t)remap[rs + v];
+    // an id outside the mapping reads nothing (the reference reads out of bounds there)
+    if (mapped) v = (v >= 0 && (int64_t)v < re - rs) ? (index_t)remap[rs + v] : (index_t)-1;
     dense[i] = v;
   }
 }

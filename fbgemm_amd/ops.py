@@ -233,12 +233,17 @@ def int_nbit_split_embedding_codegen_lookup_function(
         total_D, max_int2_D, max_int4_D, max_int8_D, max_float16_D, max_float32_D, indices,
         offsets, pooling_mode, indice_weights=None, output_dtype=FP16, lxu_cache_weights=None,
         lxu_cache_locations=None, row_alignment=None, max_float8_D=0, fp8_exponent_bits=-1,
-        fp8_exponent_bias=-1, status=None, plan=None):
+        fp8_exponent_bias=-1, status=None, plan=None, index_remappings=None,
+        index_remappings_offsets=None):
     """Same arguments, in the same order, as the reference operator
     (embedding_forward_quantized_host_cpu.cpp:316-318). Returns [B, total_D].
 
     Input errors raise like the CPU operator does, unless ``status`` is given:
-    then the call stays asynchronous and the caller reads the block later."""
+    then the call stays asynchronous and the caller reads the block later.
+
+    ``index_remappings`` / ``index_remappings_offsets`` (the arguments of
+    ``pruned_array_lookup``) fuse the pruned-row remap into the forward:
+    ``indices`` are then logical ids."""
     _require_cuda(dev_weights, indices, offsets, indice_weights)
     if pooling_mode == POOL_NONE:
         raise NotImplementedError("PoolingMode.NONE (sequence output) is not on this path")
@@ -268,10 +273,15 @@ def int_nbit_split_embedding_codegen_lookup_function(
         return out
     own = status is None
     st = Status(dev_weights.device) if own else status
-    check(_lib.lib().fbgemm_amd_tbe_forward(
+    ro = None
+    if index_remappings is not None:
+        _require_cuda(index_remappings, index_remappings_offsets)
+        ro = index_remappings_offsets.to(torch.int64).contiguous()
+    check(_lib.lib().fbgemm_amd_tbe_forward_pruned(
         plan.handle, _ptr(dev_weights), _ptr(uvm_weights), _ptr(indices.contiguous()),
         _ptr(offsets.contiguous()), _bits(indices), indices.numel(), offsets.numel(), pooling_mode,
-        _ptr(indice_weights), output_dtype, _ptr(out), _ptr(st.buf), _stream()))
+        _ptr(indice_weights), output_dtype, _ptr(out), _ptr(index_remappings),
+        32 if index_remappings is None else _bits(index_remappings), _ptr(ro), _ptr(st.buf), _stream()))
     if own:
         bits, pos = st.read()
         if bits:

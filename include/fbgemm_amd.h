@@ -154,6 +154,34 @@ int fbgemm_amd_tbe_forward(
     const float* d_indice_weights, int32_t output_ty, void* d_output,
     void* d_status, void* stream);
 
+/* The same forward with the pruned-row remap fused in: d_indices hold LOGICAL
+ * ids; for a table with a mapping (index_remappings_offsets[t+1] >
+ * index_remappings_offsets[t], both as in pruned_array_lookup) the physical
+ * row is index_remappings[offsets[t] + id], -1 = pruned = skipped; tables
+ * without a mapping take their ids as they are. Equal, bit for bit, to
+ * fbgemm_amd_pruned_array_lookup followed by fbgemm_amd_tbe_forward (the order
+ * of split_table_batched_embeddings_ops_inference.py:1067-1152) without the
+ * round trip of the dense indices through HBM. A logical id outside its
+ * mapping is reported as out of range. No counterpart as one call in the
+ * reference. */
+int fbgemm_amd_tbe_forward_pruned(
+    fbgemm_amd_tbe_plan* plan, const void* d_dev_weights, const void* d_uvm_weights,
+    const void* d_indices, const void* d_offsets, int32_t index_bits,
+    int64_t indices_numel, int64_t offsets_numel, int32_t pooling_mode,
+    const float* d_indice_weights, int32_t output_ty, void* d_output,
+    const void* d_index_remappings, int32_t remap_bits,
+    const int64_t* d_index_remappings_offsets, void* d_status, void* stream);
+
+/* Timing of the lookup kernel alone (without the bag scheduler that runs
+ * before it), for benchmarks: after fbgemm_amd_tbe_plan_profile(plan, slots)
+ * every forward of the plan records a HIP event on its stream before and
+ * after the lookup kernel, into a ring of `slots` pairs (0 switches it off).
+ * fbgemm_amd_tbe_plan_profile_read waits for the recorded forwards, writes
+ * their durations in milliseconds (at most `cap`, at most `slots`) and
+ * restarts the ring. No counterpart in the reference. */
+int fbgemm_amd_tbe_plan_profile(fbgemm_amd_tbe_plan* plan, int32_t slots);
+int fbgemm_amd_tbe_plan_profile_read(fbgemm_amd_tbe_plan* plan, float* ms, int32_t cap, int32_t* n);
+
 /* Rows the plan inferred for table t (what an index is checked against). */
 int64_t fbgemm_amd_tbe_plan_num_rows(const fbgemm_amd_tbe_plan* plan, int32_t t);
 /* Padded row bytes of table t. */
@@ -164,7 +192,8 @@ int64_t fbgemm_amd_tbe_plan_row_bytes(const fbgemm_amd_tbe_plan* plan, int32_t t
  * (embedding_forward_quantized_cpu_template.cpp:605-659,
  * embedding_forward_quantized_split_lookup.cu:120-168): position-preserving,
  * d_dense[i] = remap[remap_offsets[t] + indices[i]] for tables that own a
- * mapping (remap_offsets[t+1] > remap_offsets[t]), a copy otherwise. */
+ * mapping (remap_offsets[t+1] > remap_offsets[t]), a copy otherwise. An id
+ * outside its table's mapping yields -1 (the reference reads out of bounds). */
 int fbgemm_amd_pruned_array_lookup(
     const void* d_indices, const void* d_offsets, int32_t index_bits,
     int64_t offsets_numel, const void* d_index_remappings, int32_t remap_bits,

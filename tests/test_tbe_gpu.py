@@ -195,3 +195,84 @@ def test_config3_scaled(ops, oracle):
                                   p.host_weights, p.output_dtype, p.row_alignment)
     assert rc == 0
     H.assert_same_bits(got.cpu().view(torch.int16).numpy().view(np.uint16), want, "config3 @ 0.02")
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_forward_with_fused_remap(ops, oracle, seed):
+    """Logical ids + per-table mappings in one call == pruned_array_lookup (oracle)
+    followed by the forward (oracle), bit for bit; tables with an empty mapping
+    take their ids as they are; MEAN divides by the full bag length."""
+    rng = np.random.default_rng(900 + seed)
+    T = int(rng.integers(1, 8))
+    B = int(rng.integers(1, 50))
+    specs, caps = [], []
+    for _ in range(T):
+        ty = int(rng.choice([INT8, INT4, INT2, FP16, FP32]))
+        D = int(rng.choice({INT8: [8, 64, 128], INT4: [8, 64, 128, 256], INT2: [16, 64], FP16: [8, 64, 256], FP32: [4, 32]}[ty]))
+        specs.append((int(rng.integers(1, 200)), D, ty))
+        caps.append(0 if rng.random() < 0.3 else int(rng.integers(1, 600)))
+    align = int(rng.choice([1, 4, 16]))
+    weights, wo, _ = build_weights(rng, specs, align)
+    rdt = rng.choice([np.int32, np.int64])
+    dt = rng.choice([np.int32, np.int64])
+    remap_off = np.concatenate([[0], np.cumsum(caps)]).astype(np.int64)
+    remap = np.full(int(remap_off[-1]), -1, rdt)
+    for t in range(T):
+        s, e = int(remap_off[t]), int(remap_off[t + 1])
+        keep = rng.random(e - s) < 0.5
+        remap[s:e][keep] = rng.integers(0, specs[t][0], size=int(keep.sum()))
+    lens = rng.integers(0, 30, size=T * B)
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(dt)
+    idx = np.concatenate([rng.integers(0, caps[t] if caps[t] else specs[t][0], size=int(lens[t * B:(t + 1) * B].sum()))
+                          for t in range(T)] + [np.zeros(0, np.int64)]).astype(dt)
+    dense = oracle.pruned_array_lookup(idx, off, remap, remap_off)
+    tys = np.array([s[2] for s in specs], np.uint8)
+    D_offsets = np.concatenate([[0], np.cumsum([s[1] for s in specs])]).astype(np.int32)
+    total_D = int(D_offsets[-1])
+    for pooling in (0, 1):
+        for weighted in (False, True):
+            psw = rng.uniform(0, 1, size=len(idx)).astype(np.float32) if weighted else None
+            for out_ty in (FP32, FP16):
+                what = f"seed={seed} T={T} B={B} specs={specs} caps={caps} align={align} pool={pooling} w={weighted} out={out_ty}"
+                print(what, flush=True)
+                got = ops.int_nbit_split_embedding_codegen_lookup_function(
+                    cu(weights), torch.zeros(0, dtype=torch.uint8, device="cuda"), cu(np.zeros(T, np.int32)),
+                    cu(wo), cu(tys), cu(D_offsets), total_D, 0, 0, 0, 0, 0, cu(idx), cu(off), pooling,
+                    None if psw is None else cu(psw), out_ty, row_alignment=align,
+                    index_remappings=cu(remap), index_remappings_offsets=cu(remap_off)).cpu()
+                rc, want = oracle.tbe_forward(weights, wo, tys, D_offsets, total_D, dense, off, pooling, psw, out_ty, align)
+                assert rc == 0
+                g = got.numpy() if out_ty == FP32 else got.view(torch.int16).numpy().view(np.uint16)
+                H.assert_same_bits(g, want, what)
+
+
+def test_fused_remap_rejects_ids_outside_the_mapping(ops):
+    rng = np.random.default_rng(5)
+    specs = [(50, 16, INT4)]
+    weights, wo, _ = build_weights(rng, specs, 16)
+    remap = np.arange(20, dtype=np.int32)
+    args = lambda idx: (cu(weights), torch.zeros(0, dtype=torch.uint8, device="cuda"), cu(np.zeros(1, np.int32)),
+                        cu(wo), cu(np.array([INT4], np.uint8)), cu(np.array([0, 16], np.int32)), 16, 0, 16, 0, 0, 0,
+                        cu(idx), cu(np.array([0, len(idx)], np.int32)), 0, None, FP32)
+    kw = dict(row_alignment=16, index_remappings=cu(remap), index_remappings_offsets=cu(np.array([0, 20], np.int64)))
+    ops.int_nbit_split_embedding_codegen_lookup_function(*args(np.array([0, 19], np.int32)), **kw)
+    with pytest.raises(RuntimeError, match="out of bounds"):
+        ops.int_nbit_split_embedding_codegen_lookup_function(*args(np.array([0, 20], np.int32)), **kw)
+
+
+def test_config4_batched_scaled(ops, oracle):
+    """Config 4 as one table-batched call with the remap fused in, at 1/50 scale, in full."""
+    from fbgemm_amd import bench_configs as bc
+    p = bc.config4_batched("cuda", scale=0.02)
+    got = ops.int_nbit_split_embedding_codegen_lookup_function(
+        p.dev_weights, torch.zeros(0, dtype=torch.uint8, device="cuda"),
+        cu(np.zeros(p.T, np.int32)), cu(p.weights_offsets), cu(p.tys), cu(p.D_offsets), p.total_D,
+        0, 64, 0, 0, 0, p.indices, p.offsets, p.pooling_mode, None, p.output_dtype,
+        row_alignment=p.row_alignment, index_remappings=p.extra["remap"],
+        index_remappings_offsets=p.extra["remap_offsets"])
+    dense = oracle.pruned_array_lookup(p.host_indices, p.host_offsets, p.extra["host_remap"], p.extra["host_remap_offsets"])
+    assert (dense == p.extra["host_dense"]).all()
+    rc, want = oracle.tbe_forward(p.dev_weights.cpu().numpy(), p.weights_offsets, p.tys, p.D_offsets,
+                                  p.total_D, dense, p.host_offsets, p.pooling_mode, None, p.output_dtype, p.row_alignment)
+    assert rc == 0
+    H.assert_same_bits(got.cpu().numpy(), want, "config4 batched @ 0.02")
