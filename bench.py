@@ -46,6 +46,32 @@ def parse():
     return ap.parse_args()
 
 
+def traffic_from_profile(config_id):
+    """HBM bytes one lookup_kernel launch moves, from the committed hardware-counter
+    summary of this configuration (profiles/lookup_kernel_config<N>.txt): FETCH_SIZE
+    and WRITE_SIZE (KiB per dispatch), each scaled by what the same counter read
+    for the plain copy of known size that ran in the same process. None when the
+    summary is not there."""
+    import re
+    path = os.path.join(ROOT, "profiles", f"lookup_kernel_config{config_id}.txt")
+    if not os.path.exists(path):
+        return None
+    text = open(path).read()
+    m = re.search(r"--calibration-copy-mib (\d+)", text)
+    vals = {}
+    for kern, ctr, v in re.findall(r"pmc\s+(\w+)(?:<\w+>)?: (FETCH_SIZE|WRITE_SIZE) avg_per_dispatch=([0-9.e+]+)", text):
+        vals[(kern, ctr)] = float(v)
+    try:
+        copy_bytes = int(m.group(1)) << 20
+        total = 0.0
+        for ctr in ("FETCH_SIZE", "WRITE_SIZE"):
+            factor = copy_bytes / (vals[("calibration_copy_kernel", ctr)] * 1024.0)
+            total += vals[("lookup_kernel", ctr)] * 1024.0 * factor
+        return int(total)
+    except (AttributeError, KeyError, ZeroDivisionError):
+        return None
+
+
 def tbe_runner(p, torch):
     """Returns (launch, out, status, plan) for a TbeProblem: launch() enqueues one forward."""
     from fbgemm_amd import _lib, ops
@@ -295,7 +321,9 @@ def main():
         "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
         "pooled_rows_per_s": round(lookups / (ms_per_step * 1e-3), 1),
         "roofline": {"bound": "hbm", "achieved": round(kern_gbps, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(kern_gbps / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "frac": round(kern_gbps / HBM_PEAK_GBPS, 4),
+                     "traffic": traffic_from_profile(a.config) if (a.scale == 1.0 and p is not None and not a.rows_scale
+                                                                   and a.only_type is None) else None,
                      "kernel": kernel_name, "kernel_ms": round(kernel_ms / launches_per_step, 5),
                      "forward_ms": round(forward_ms, 5),
                      "algorithmic_bytes_per_launch": useful // launches_per_step},

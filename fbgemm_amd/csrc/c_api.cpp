@@ -505,6 +505,7 @@ int fbgemm_amd_tbe_forward_pruned(
       // that tables of different row types share the CUs at all times.
       static const int xcd_lists = env_int("FBGEMM_AMD_XCD_LISTS", 1);
       static const int interleave = env_int("FBGEMM_AMD_INTERLEAVE", 1);
+      static const int max_parts = env_int("FBGEMM_AMD_MAX_PARTS", 8);
       struct Slice { int t, first, step, count; double cost; };
       std::vector<Slice> slices;
       double total_cost = 0;
@@ -522,7 +523,7 @@ int fbgemm_amd_tbe_forward_pruned(
       for (int t = 0; t < plan->T; ++t) {
         // slices no larger than 1/4 of an XCD's share; slice p takes waves p, p + parts, ...
         int parts = (int)std::ceil(wave_cost[t] * nwaves[t] / (total_cost / nx / 4.0 + 1e-9));
-        parts = std::max(1, std::min(parts, std::min(nwaves[t], nx)));
+        parts = std::max(1, std::min(parts, std::min(nwaves[t], std::min(nx, max_parts))));
         for (int p = 0; p < parts; ++p) {
           const int count = (nwaves[t] - p + parts - 1) / parts;
           slices.push_back(Slice{t, p, parts, count, wave_cost[t] * count});

@@ -20,14 +20,20 @@ echo "== kernel trace (--kernel-trace --stats), 23 launches" >> "$OUT"
 timeout -k 10 900 rocprofv3 --kernel-trace --stats --output-format csv -d $RAW/trace -o t -- $BENCH --steps 20 --warmup 3 > $RAW/trace.log 2>&1 || { echo "trace run failed" | tee -a "$OUT"; tail -5 $RAW/trace.log; exit 1; }
 grep '^{' $RAW/trace.log | tail -1 | cut -c1-1200 >> "$OUT"
 python3 -m fbgemm_amd.profile_summary $RAW/trace | grep -v '^#' >> "$OUT"
-for pass in "FETCH_SIZE" "WRITE_SIZE" "TCC_HIT_sum TCC_MISS_sum" "TCC_EA0_RDREQ_sum" \
-            "SQ_WAVES SQ_INSTS_VALU SQ_INSTS_VMEM_RD SQ_INSTS_LDS SQ_INSTS_SALU SQ_WAVE_CYCLES SQ_WAIT_INST_ANY SQ_ACTIVE_INST_VALU" \
-            "TCP_TCC_READ_REQ_sum TCP_TOTAL_CACHE_ACCESSES_sum TCP_TCC_READ_REQ_LATENCY_sum" "GRBM_GUI_ACTIVE"; do
+# PROFILE_SHORT=1 keeps the byte counters only (for workloads whose set-up takes minutes)
+if [ -n "$PROFILE_SHORT" ]; then
+  PASSES=("FETCH_SIZE" "WRITE_SIZE" "TCC_HIT_sum TCC_MISS_sum" "GRBM_GUI_ACTIVE")
+else
+  PASSES=("FETCH_SIZE" "WRITE_SIZE" "TCC_HIT_sum TCC_MISS_sum" "TCC_EA0_RDREQ_sum"
+          "SQ_WAVES SQ_INSTS_VALU SQ_INSTS_VMEM_RD SQ_INSTS_LDS SQ_INSTS_SALU SQ_WAVE_CYCLES SQ_WAIT_INST_ANY SQ_ACTIVE_INST_VALU"
+          "TCP_TCC_READ_REQ_sum TCP_TOTAL_CACHE_ACCESSES_sum TCP_TCC_READ_REQ_LATENCY_sum" "GRBM_GUI_ACTIVE")
+fi
+for pass in "${PASSES[@]}"; do
   n=$(echo $pass | tr ' ' '_' | cut -c1-40)
   echo "== --pmc $pass" >> "$OUT"
-  timeout -s KILL 600 rocprofv3 --pmc $pass --output-format csv -d $RAW/pmc_$n -o p -- $BENCH --steps 3 --warmup 1 > $RAW/pmc_$n.log 2>&1 || { echo "pass failed: $pass" >> "$OUT"; tail -3 $RAW/pmc_$n.log >> "$OUT"; continue; }
+  timeout -s KILL 600 rocprofv3 --pmc $pass --output-format csv -d $RAW/pmc_$n -o p -- $BENCH --steps 3 --warmup 1 > $RAW/pmc_$n.log 2>&1 || { echo "pass failed: $pass" >> "$OUT"; tail -3 $RAW/pmc_$n.log >> "$OUT"; exit 1; }
   python3 -m fbgemm_amd.profile_summary $RAW/pmc_$n | grep -v '^#\|^launch' >> "$OUT"
 done
 python3 -m fbgemm_amd.profile_summary $RAW/pmc_GRBM_GUI_ACTIVE | grep '^launch' >> "$OUT"
 rm -rf $RAW
-cat "$OUT"
+echo "summary written to $OUT"
