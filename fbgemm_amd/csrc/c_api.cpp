@@ -100,6 +100,34 @@ void plan_lanes(TableDesc& d, uintptr_t base_addr, int64_t out_stride, bool has_
   d.chunks = C;
   d.lanes = std::max(2, std::min(64, chunks / C)); // >= 2: a wave stages at most 32 bags
   d.passes = (chunks + d.lanes * C - 1) / (d.lanes * C);
+  // Whole-row chunks for 4- and 8-bit rows with the fp16 header first and a
+  // stride that is a multiple of 16: the header rides in chunk 0 and costs no
+  // memory request of its own. Needs every 16-byte load of a row to stay
+  // inside the row's stride and a single pass.
+  static const int inline_hdr = env_int("FBGEMM_AMD_INLINE_HDR", 1);
+  d.inline_hdr = 0;
+  if (inline_hdr && has_sb && (d.ty == ST_INT4 || d.ty == ST_INT8) && !d.sb_fp32 && d.sb_off == 0 && d.data_off == 4 &&
+      base_addr % 16 == 0 && d.weights_offset % 16 == 0 && d.row_stride % 16 == 0 && force_vb == 0) {
+    const int nchunks = (d.data_bytes + 4 + 15) / 16;
+    const int Ci = (d.ty == ST_INT8 && max_chunks >= 2 && nchunks >= 4) ? 2 : 1;
+    const int lanes = std::max(2, (nchunks + Ci - 1) / Ci);
+    if (lanes <= 32 && (int64_t)nchunks * 16 <= d.row_stride) {
+      d.inline_hdr = 1;
+      d.vb = 16;
+      d.chunks = Ci;
+      d.lanes = lanes;
+      d.passes = 1;
+      // runs of E / 4 columns, each stored whole when aligned
+      const int GE = (16 * 8 / bits) / 4;
+      d.vec_store = 0;
+      for (int k = 0; k < 2; ++k) {
+        const int esz = k == 0 ? 4 : 2;
+        const int al = std::min(16, GE * esz);
+        if ((out_stride * esz) % al == 0 && ((int64_t)d.out_col * esz) % al == 0) d.vec_store |= 1 << k;
+      }
+      return;
+    }
+  }
   // whole-run vector stores: each lane writes E = vb*8/bits consecutive
   // elements; allowed when every run starts on a multiple of min(16, run bytes)
   // and no run is cut by the end of the row.
@@ -490,6 +518,10 @@ int fbgemm_amd_tbe_forward_pruned(
   if (B64 > 0x7fffffffLL) return fail(FBGEMM_AMD_E_ARG, "B exceeds 2^31-1");
   const int32_t B = (int32_t)B64;
   if (!d_offsets || !d_output || (indices_numel > 0 && !d_indices)) return fail(FBGEMM_AMD_E_ARG, "null data pointer");
+  // the lane shapes of the plan assume what every device allocator gives (the
+  // reference's kernels load uint4 from the same buffers)
+  if ((uintptr_t)d_dev_weights % 16 || (uintptr_t)d_uvm_weights % 16)
+    return fail(FBGEMM_AMD_E_ARG, "weights buffers must be 16-byte aligned");
   hipStream_t stream = (hipStream_t)stream_;
 
   fbgemm_amd_tbe_plan::Work w;

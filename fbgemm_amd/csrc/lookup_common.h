@@ -54,6 +54,9 @@ struct TableDesc {
   int32_t vec_store;      // bit 0 / bit 1: every lane's output run is aligned for whole-run
                           // vector stores with 4-byte / 2-byte output elements
   int32_t chunks;         // 16-byte chunks per lane and pass (1, 2 or 4)
+  int32_t inline_hdr;     // 1: lanes own 16-byte chunks of the WHOLE row (fp16 scale/bias
+                          // header first, then data), so the header arrives with the data
+                          // and costs no request of its own; `lanes` need not divide 64
 };
 
 // What the bag scheduler leaves per bag, in the order waves take the bags.

@@ -302,6 +302,50 @@ __device__ __forceinline__ void write_out(const LookupArgs& a, const float (&acc
   }
 }
 
+// Writer of the whole-row chunk layout: the 16-byte chunk a lane holds starts
+// one dword (the row header) before a 16-byte boundary of the element data, so
+// its E accumulators are 4 runs of E / 4 columns, the first of them at col0
+// (negative for the chunk that holds the header: that run is not output).
+template <int E>
+__device__ __forceinline__ void write_out_runs(const LookupArgs& a, const float (&acc)[E], int64_t row_pos, int col0, int D, bool vec_ok) {
+  constexpr int GE = E / 4;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int cj = col0 + j * GE;
+    const bool whole = cj >= 0 && cj + GE <= D;
+    if (a.out_ty == ST_FP32) {
+      float* o = reinterpret_cast<float*>(a.out) + row_pos + cj;
+      if (whole && vec_ok) {
+        uint32_t w[GE];
+#pragma unroll
+        for (int e = 0; e < GE; ++e) w[e] = float_to_bits(acc[j * GE + e]);
+        store_words<GE * 4>(o, w);
+      } else {
+#pragma unroll
+        for (int e = 0; e < GE; ++e)
+          if (cj + e >= 0 && cj + e < D) o[e] = acc[j * GE + e];
+      }
+    } else {
+      uint16_t* o = reinterpret_cast<uint16_t*>(a.out) + row_pos + cj;
+      const bool bf = a.out_ty == ST_BF16;
+      if (whole && vec_ok) {
+        uint32_t w[GE / 2];
+#pragma unroll
+        for (int e = 0; e < GE; e += 2) {
+          const uint32_t lo = bf ? to_bf16_bits(acc[j * GE + e]) : to_half_bits(acc[j * GE + e]);
+          const uint32_t hi = bf ? to_bf16_bits(acc[j * GE + e + 1]) : to_half_bits(acc[j * GE + e + 1]);
+          w[e / 2] = lo | (hi << 16);
+        }
+        store_words<GE * 2>(o, w);
+      } else {
+#pragma unroll
+        for (int e = 0; e < GE; ++e)
+          if (cj + e >= 0 && cj + e < D) o[e] = (uint16_t)(bf ? to_bf16_bits(acc[j * GE + e]) : to_half_bits(acc[j * GE + e]));
+      }
+    }
+  }
+}
+
 // ---- one wave, one table ----------------------------------------------------
 
 __device__ __forceinline__ int64_t read_offset(const void* p, bool is64, int64_t i) {
@@ -346,7 +390,15 @@ constexpr int64_t NO_ENTRY = INT64_MIN;
 // scale * 2^24 overflows. A wave that meets |scale| >= 2^100 gives up, returns
 // false, and its work is redone from the start by the PRESCALE = false
 // instance, which converts integers to float the plain way.
-template <typename index_t, bool GENERAL, int TY, int VB, int C, int ROUND, bool PRESCALE>
+//
+// INHDR (4- and 8-bit rows whose fp16 scale/bias pair comes first and whose
+// stride is a multiple of 16): the lanes of a bag own the 16-byte chunks of the
+// whole row, header included, so that the header costs no memory request of
+// its own: the lane that holds chunk 0 hands it to the others through a lane
+// permute. `lanes` then need not divide 64; the lanes left over shadow the last
+// bag of the wave (same addresses, nothing written), and so do chunk slots past
+// the end of the row.
+template <typename index_t, bool GENERAL, int TY, int VB, int C, int ROUND, bool PRESCALE, bool INHDR = false>
 __device__ __forceinline__ bool pool_bags(const LookupArgs& a, const TableDesc& d, int table, int first_slot,
                                           int lane, StageRow* stage_row, StageMul* stage_mul) {
   constexpr int BITS = type_bits(TY);
@@ -357,12 +409,15 @@ __device__ __forceinline__ bool pool_bags(const LookupArgs& a, const TableDesc& 
   constexpr int MAXR = 2; // entries one staging lane handles per round, at most
   using Acc = Accum<TY, VB>;
 
+  static_assert(!INHDR || (VB == 16 && QUANT), "whole-row chunks are 16 bytes of a quantised row");
   const int S = d.lanes;
   const int G = 64 / S;
   const int grp = lane / S;
   const int sub = lane - grp * S;
   const int slot = first_slot + grp;
-  const bool bag_ok = grp < G && slot < a.B;
+  const bool idle = grp >= G;           // lanes left over when lanes does not divide 64
+  const int lgrp = idle ? G - 1 : grp;  // ... read what the last group reads
+  const bool bag_ok = !idle && slot < a.B;
   const bool reporter = sub == 0;
   // staging lanes per bag: a power of two <= lanes; entries per round: ROUND,
   // or what MAXR entries per staging lane allow
@@ -424,8 +479,8 @@ __device__ __forceinline__ bool pool_bags(const LookupArgs& a, const TableDesc& 
   const index_t* idx = reinterpret_cast<const index_t*>(a.indices);
   const uint8_t* wbase = (d.placement ? a.weights[1] : a.weights[0]) + d.weights_offset;
   const uint8_t* psb = wbase + d.sb_off;
-  StageRow* my_row = stage_row + grp * RN;
-  StageMul* my_mul = stage_mul + grp * RN;
+  StageRow* my_row = stage_row + lgrp * RN;
+  StageMul* my_mul = stage_mul + lgrp * RN;
   // the reference keeps the bag length in an int when it forms 1/len
   const float inv_len = (a.normalize && n > 0) ? 1.0f / (float)n : 1.0f;
   const int chunk_stride = S * VB; // bytes between a lane's consecutive chunks
@@ -434,12 +489,24 @@ __device__ __forceinline__ bool pool_bags(const LookupArgs& a, const TableDesc& 
     const int chunk0 = pass * S * C + sub;
     bool on[C];
     bool all_on = bag_ok;
+    int rowb[C]; // INHDR: byte offset of the lane's chunks inside the row
+    if constexpr (INHDR) {
+      const int nchunks = (d.data_bytes + 4 + VB - 1) / VB;
 #pragma unroll
-    for (int c = 0; c < C; ++c) {
-      on[c] = bag_ok && (chunk0 + c * S) * VB < d.data_bytes;
-      all_on = all_on && on[c];
+      for (int c = 0; c < C; ++c) {
+        const int k = chunk0 + c * S;
+        on[c] = bag_ok && k < nchunks;
+        rowb[c] = (k < nchunks ? k : nchunks - 1) * VB; // a slot past the row shadows the last chunk
+      }
+    } else {
+#pragma unroll
+      for (int c = 0; c < C; ++c) {
+        on[c] = bag_ok && (chunk0 + c * S) * VB < d.data_bytes;
+        all_on = all_on && on[c];
+        rowb[c] = 0;
+      }
     }
-    const uint8_t* pdata = wbase + d.data_off + chunk0 * VB;
+    const uint8_t* pdata = INHDR ? wbase : wbase + d.data_off + chunk0 * VB;
 
     float acc[C][E];
 #pragma unroll
@@ -501,12 +568,12 @@ __device__ __forceinline__ bool pool_bags(const LookupArgs& a, const TableDesc& 
         coff[rr] = off;
         cw[rr] = nw[rr];
         if (rr < R && stager) {
-          hole = hole || off < 0;
+          hole = hole || (off < 0 && round * RN < n); // a bag that has ended leaves the loop instead
           my_row[sub + rr * SL].off = off;
           // Plain rows: the multiplier is the weight. A hole gets (-0, -0),
           // which leaves every accumulator exactly as it is:
           // fma(-0, q, acc + -0) == acc for any acc, +0 and -0 included.
-          if (!QUANT || off < 0) {
+          if (!QUANT || INHDR || off < 0) {
             StageMul m;
             m.scale = off < 0 ? -0.0f : nw[rr];
             m.bias = -0.0f;
@@ -518,7 +585,8 @@ __device__ __forceinline__ bool pool_bags(const LookupArgs& a, const TableDesc& 
     };
 
     // wave-uniform: every lane of the wave pools a bag and owns C live chunks
-    const bool wave_on = __builtin_amdgcn_ballot_w64(!all_on) == 0ull && __builtin_amdgcn_ballot_w64(true) == ~0ull;
+    // (whole-row chunks: slots past the row are clamped, lanes without a bag never enter the loop)
+    const bool wave_on = INHDR || (__builtin_amdgcn_ballot_w64(!all_on) == 0ull && __builtin_amdgcn_ballot_w64(true) == ~0ull);
     load_idx(0);
     // wave-uniform: the staged round has RN rows to add for every bag of the wave
     // (the staging call comes first on its own line: it must run on every wave)
@@ -534,7 +602,7 @@ __device__ __forceinline__ bool pool_bags(const LookupArgs& a, const TableDesc& 
       uint32_t h0[MAXR], h1[MAXR];
       const int left = min(n - r * RN, RN);
       // scale/bias first, so that their wait does not cover the row loads
-      if constexpr (QUANT) {
+      if constexpr (QUANT && !INHDR) {
 #pragma unroll
         for (int rr = 0; rr < MAXR; ++rr) {
           if (rr < R && stager && coff[rr] >= 0) {
@@ -565,7 +633,7 @@ __device__ __forceinline__ bool pool_bags(const LookupArgs& a, const TableDesc& 
           if (e < RN) {
             const uint8_t* p = pdata + my_row[e].off;
 #pragma unroll
-            for (int c = 0; c < C; ++c) load_raw<VB>(raw[e][c], p + c * chunk_stride);
+            for (int c = 0; c < C; ++c) load_raw<VB>(raw[e][c], INHDR ? p + rowb[c] : p + c * chunk_stride);
           }
         }
       } else {
@@ -582,15 +650,17 @@ __device__ __forceinline__ bool pool_bags(const LookupArgs& a, const TableDesc& 
               const int64_t off = my_row[e].off;
               if (off >= 0) {
 #pragma unroll
-                for (int c = 0; c < C; ++c)
-                  if (on[c]) load_raw<VB>(raw[e][c], pdata + off + c * chunk_stride);
+                for (int c = 0; c < C; ++c) {
+                  if constexpr (INHDR) load_raw<VB>(raw[e][c], pdata + off + rowb[c]);
+                  else if (on[c]) load_raw<VB>(raw[e][c], pdata + off + c * chunk_stride);
+                }
               }
             }
           }
         }
       }
       load_idx(r + 1);
-      if constexpr (QUANT) {
+      if constexpr (QUANT && !INHDR) {
         bool big = false;
 #pragma unroll
         for (int rr = 0; rr < MAXR; ++rr) {
@@ -616,15 +686,30 @@ __device__ __forceinline__ bool pool_bags(const LookupArgs& a, const TableDesc& 
       }
       // One straight-line accumulate for the whole wave; lanes past the end of
       // their bag add holes.
+      bool big = false;
 #pragma unroll
       for (int e = 0; e < ROUND; ++e) {
         if (e < RN && (fast || __builtin_amdgcn_ballot_w64(e < left) != 0ull)) {
-          const StageMul m = my_mul[e];
+          StageMul m = my_mul[e];
+          if constexpr (INHDR) {
+            // the row header sits in the first dword of chunk 0, which the first
+            // lane of the group holds (zeros for a row that is not there)
+            const uint32_t h = (uint32_t)__builtin_amdgcn_ds_bpermute(lgrp * S * 4, (int)raw[e][0][0]);
+            m.bias = m.scale * half_hi(h);
+            m.scale = m.scale * half_lo(h);
+            big = big || !(__builtin_fabsf(m.scale) < 0x1p100f);
+          }
 #pragma unroll
           for (int c = 0; c < C; ++c) {
             if constexpr (PRESCALE) Acc::fast(acc[c], raw[e][c], m.scale, m.bias);
             else Acc::slow(acc[c], raw[e][c], m.scale, m.bias);
           }
+        }
+      }
+      if constexpr (INHDR && PRESCALE && Acc::kPrescaled) {
+        if (__builtin_amdgcn_ballot_w64(big) != 0ull) {
+          give_up = true;
+          break;
         }
       }
       __builtin_amdgcn_wave_barrier();
@@ -646,23 +731,28 @@ __device__ __forceinline__ bool pool_bags(const LookupArgs& a, const TableDesc& 
 #pragma unroll
           for (int e = 0; e < E; ++e) acc[c][e] *= inv_len;
         }
-        const int col0 = (chunk0 + c * S) * E;
-        const int64_t elem_pos = (int64_t)bag * a.out_stride + d.out_col + col0;
-        write_out<E>(a, acc[c], elem_pos, col0, d.D, vec_ok);
+        if constexpr (INHDR) {
+          const int col0 = (chunk0 + c * S) * E - E / 4;
+          write_out_runs<E>(a, acc[c], (int64_t)bag * a.out_stride + d.out_col, col0, d.D, vec_ok);
+        } else {
+          const int col0 = (chunk0 + c * S) * E;
+          const int64_t elem_pos = (int64_t)bag * a.out_stride + d.out_col + col0;
+          write_out<E>(a, acc[c], elem_pos, col0, d.D, vec_ok);
+        }
       }
     }
   }
   return true;
 }
 
-template <typename index_t, bool GENERAL, int TY, int VB, int C, int ROUND>
+template <typename index_t, bool GENERAL, int TY, int VB, int C, int ROUND, bool INHDR = false>
 __device__ __forceinline__ void run_bags(const LookupArgs& a, const TableDesc& d, int table, int first_slot, int lane,
                                          StageRow* stage_row, StageMul* stage_mul) {
   if constexpr (Accum<TY, VB>::kPrescaled) {
-    if (!pool_bags<index_t, GENERAL, TY, VB, C, ROUND, true>(a, d, table, first_slot, lane, stage_row, stage_mul))
-      pool_bags<index_t, GENERAL, TY, VB, C, ROUND, false>(a, d, table, first_slot, lane, stage_row, stage_mul);
+    if (!pool_bags<index_t, GENERAL, TY, VB, C, ROUND, true, INHDR>(a, d, table, first_slot, lane, stage_row, stage_mul))
+      pool_bags<index_t, GENERAL, TY, VB, C, ROUND, false, INHDR>(a, d, table, first_slot, lane, stage_row, stage_mul);
   } else {
-    pool_bags<index_t, GENERAL, TY, VB, C, ROUND, true>(a, d, table, first_slot, lane, stage_row, stage_mul);
+    pool_bags<index_t, GENERAL, TY, VB, C, ROUND, true, INHDR>(a, d, table, first_slot, lane, stage_row, stage_mul);
   }
 }
 
@@ -677,6 +767,13 @@ __device__ __forceinline__ void pool_dispatch_vb(const LookupArgs& a, const Tabl
   constexpr int MINVB = BITS >= 16 ? BITS / 8 : 1;
   constexpr int MAXC = BITS >= 16 ? 4 : (BITS == 8 ? 2 : 1);
   // rows in flight per lane: ROUND * chunks = 8 loads of 16 bytes
+  if constexpr (TY == ST_INT4 || TY == ST_INT8) {
+    if (d.inline_hdr) {
+      if (d.chunks == 2 && MAXC >= 2) run_bags<index_t, GENERAL, TY, 16, (MAXC >= 2 ? 2 : 1), 4, true>(a, d, table, first_slot, lane, stage_row, stage_mul);
+      else run_bags<index_t, GENERAL, TY, 16, 1, 8, true>(a, d, table, first_slot, lane, stage_row, stage_mul);
+      return;
+    }
+  }
   if (d.vb == 16) {
     if constexpr (TY == ST_INT2) {
       run_bags<index_t, GENERAL, TY, 4, 1, 8>(a, d, table, first_slot, lane, stage_row, stage_mul); // not selected by the host
