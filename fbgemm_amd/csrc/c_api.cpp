@@ -111,7 +111,9 @@ void plan_lanes(TableDesc& d, uintptr_t base_addr, int64_t out_stride, bool has_
     const int nchunks = (d.data_bytes + 4 + 15) / 16;
     const int Ci = (d.ty == ST_INT8 && max_chunks >= 2 && nchunks >= 4) ? 2 : 1;
     const int lanes = std::max(2, (nchunks + Ci - 1) / Ci);
-    if (lanes <= 32 && (int64_t)nchunks * 16 <= d.row_stride) {
+    // lanes that would idle because a bag may not straddle a quarter of the wave
+    const int used = lanes <= 16 ? (16 / lanes) * lanes : 16;
+    if (lanes <= 32 && (int64_t)nchunks * 16 <= d.row_stride && used >= 14) {
       d.inline_hdr = 1;
       d.vb = 16;
       d.chunks = Ci;
@@ -327,7 +329,7 @@ int fbgemm_amd_spmdm_launch(
   a.check_total = 1;
   a.out_aligned = (uintptr_t)d_out % 16 == 0;
   a.status = (Status*)d_status;
-  const int G = 64 / d.lanes;
+  const int G = bags_per_wave(d.lanes);
   a.num_waves = (output_size + G - 1) / G;
 
   // Ordering the bags pays once several waves' worth of bags exist.
@@ -545,7 +547,7 @@ int fbgemm_amd_tbe_forward_pruned(
       std::vector<int> nwaves(plan->T);
       for (int t = 0; t < plan->T; ++t) {
         const TableDesc& d = plan->tables[t];
-        const int G = 64 / d.lanes;
+        const int G = bags_per_wave(d.lanes);
         nwaves[t] = (B + G - 1) / G;
         const double lines = 1.0 + (double)(d.row_stride - 1) / 128.0; // expected lines a row touches
         wave_cost[t] = G * (lines + 0.25);
@@ -572,13 +574,34 @@ int fbgemm_amd_tbe_forward_pruned(
       std::vector<WaveWork> list;
       std::vector<int64_t> xcd_start(9, 0);
       int64_t longest = 0;
+      // Inside a run the slices are walked in groups that hold one slice of every
+      // row shape (type, D) the run has; the slices of a group advance together,
+      // each through its bag order at the same relative pace, and the groups
+      // follow one another. Mixing shapes keeps waves of different cost on the
+      // CUs at all times; taking few tables at a time keeps the working set of
+      // the XCD's L2 small (hot rows of a table are reused while they are there).
+      static const int by_shape = env_int("FBGEMM_AMD_GROUP_BY_SHAPE", 1);
       for (int x = 0; x < nx; ++x) {
         std::vector<std::pair<double, WaveWork>> keyed;
+        std::map<std::pair<int, int>, std::vector<Slice>> shapes; // slices of a shape, largest first (per_x order)
         for (const Slice& sl : per_x[x]) {
-          const int G = 64 / plan->tables[sl.t].lanes;
-          for (int k = 0; k < sl.count; ++k)
-            keyed.push_back({interleave ? (k + 0.5) / sl.count : (double)keyed.size(),
-                             WaveWork{sl.t, (sl.first + k * sl.step) * G}});
+          const TableDesc& d = plan->tables[sl.t];
+          shapes[(interleave && by_shape) ? std::make_pair((int)d.ty, (int)d.D) : std::make_pair(0, 0)].push_back(sl);
+        }
+        size_t depth = 0;
+        for (auto& kv : shapes) depth = std::max(depth, kv.second.size());
+        int gidx = 0;
+        for (size_t i = 0; i < depth; ++i) {
+          for (auto& kv : shapes) {
+            if (i >= kv.second.size()) continue;
+            const Slice& sl = kv.second[i];
+            const int G = bags_per_wave(plan->tables[sl.t].lanes);
+            // one shape only (or no interleaving asked for): slice after slice
+            const double base = (interleave && by_shape) ? (double)gidx : (interleave ? 0.0 : (double)gidx++);
+            for (int k = 0; k < sl.count; ++k)
+              keyed.push_back({base + (k + 0.5) / sl.count, WaveWork{sl.t, (sl.first + k * sl.step) * G}});
+          }
+          if (interleave && by_shape) ++gidx;
         }
         std::stable_sort(keyed.begin(), keyed.end(),
                          [](const std::pair<double, WaveWork>& p, const std::pair<double, WaveWork>& q) { return p.first < q.first; });

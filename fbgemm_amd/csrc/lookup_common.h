@@ -59,6 +59,16 @@ struct TableDesc {
                           // and costs no request of its own; `lanes` need not divide 64
 };
 
+// Bags a wave pools side by side when `lanes` lanes share a bag. The memory
+// pipeline merges the addresses of a 16-byte-per-lane load 16 lanes at a time,
+// so a bag's lanes must not straddle a multiple of 16: each quarter of the wave
+// holds 16 / lanes whole bags and leaves the rest of its lanes idle. (For the
+// powers of two this is 64 / lanes.)
+#if defined(__HIPCC__)
+__host__ __device__
+#endif
+inline int bags_per_wave(int lanes) { return lanes <= 16 ? 4 * (16 / lanes) : 64 / lanes; }
+
 // What the bag scheduler leaves per bag, in the order waves take the bags.
 struct __attribute__((aligned(16))) BagEntry {
   int64_t o0;  // offsets[bag]

@@ -15,7 +15,7 @@
 // Lane mapping: `lanes` consecutive lanes of a wave share one bag; lane `sub`
 // of the group owns the `vb` bytes of every row that start at
 // (pass * lanes + sub) * vb, i.e. vb * 8 / bits consecutive output columns. A
-// wave therefore pools 64 / lanes bags at once and each row is fetched with
+// wave therefore pools bags_per_wave(lanes) bags at once and each row is fetched with
 // one coalesced run of 16-byte loads.
 #include <hip/hip_runtime.h>
 
@@ -366,7 +366,7 @@ constexpr int MAX_GROUPS = 32; // bags per wave at most; lanes per bag >= 2
 constexpr int MAX_ROUND = 8;
 constexpr int64_t NO_ENTRY = INT64_MIN;
 
-// One wave pools 64 / lanes bags of one table, `RN` entries of every bag per
+// One wave pools bags_per_wave(lanes) bags of one table, `RN` entries of every bag per
 // round. Each lane owns C chunks of VB bytes of every row: chunk c of lane
 // `sub` starts at byte (c * lanes + sub) * VB of the row data, so every load
 // instruction of the wave reads contiguous bytes of each row.
@@ -411,12 +411,24 @@ __device__ __forceinline__ bool pool_bags(const LookupArgs& a, const TableDesc& 
 
   static_assert(!INHDR || (VB == 16 && QUANT), "whole-row chunks are 16 bytes of a quantised row");
   const int S = d.lanes;
-  const int G = 64 / S;
-  const int grp = lane / S;
-  const int sub = lane - grp * S;
+  const int G = bags_per_wave(S);
+  // quarter q of the wave holds bags q * (16 / S) ...; its last 16 % S lanes idle
+  int grp, sub;
+  bool idle;
+  if (S <= 16) {
+    const int per_q = 16 / S;
+    const int j = lane & 15;
+    const int gq = j / S;
+    idle = gq >= per_q;
+    grp = (lane >> 4) * per_q + (idle ? per_q - 1 : gq);
+    sub = j - gq * S;
+  } else {
+    grp = lane / S;
+    sub = lane - grp * S;
+    idle = grp >= G;
+  }
   const int slot = first_slot + grp;
-  const bool idle = grp >= G;           // lanes left over when lanes does not divide 64
-  const int lgrp = idle ? G - 1 : grp;  // ... read what the last group reads
+  const int lgrp = idle ? G - 1 : grp;  // idle lanes never enter the loops; any valid staging slot will do
   const bool bag_ok = !idle && slot < a.B;
   const bool reporter = sub == 0;
   // staging lanes per bag: a power of two <= lanes; entries per round: ROUND,
@@ -694,7 +706,7 @@ __device__ __forceinline__ bool pool_bags(const LookupArgs& a, const TableDesc& 
           if constexpr (INHDR) {
             // the row header sits in the first dword of chunk 0, which the first
             // lane of the group holds (zeros for a row that is not there)
-            const uint32_t h = (uint32_t)__builtin_amdgcn_ds_bpermute(lgrp * S * 4, (int)raw[e][0][0]);
+            const uint32_t h = (uint32_t)__builtin_amdgcn_ds_bpermute((lane - sub) * 4, (int)raw[e][0][0]);
             m.bias = m.scale * half_hi(h);
             m.scale = m.scale * half_lo(h);
             big = big || !(__builtin_fabsf(m.scale) < 0x1p100f);
@@ -823,7 +835,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(FBGEMM_AMD_M
     table = ww.table;
     first_slot = ww.first_bag;
   } else {
-    first_slot = (int)(wave * (64 / a.single.lanes));
+    first_slot = (int)(wave * bags_per_wave(a.single.lanes));
   }
   const TableDesc d = a.tables ? a.tables[table] : a.single;
 #ifdef FBGEMM_AMD_ONLY_TY // register-budget experiments: compile a single row type
