@@ -37,6 +37,10 @@ SYMBOLS = {
     "fbgemm_amd_tbe_forward_pruned": (C.c_int, [_P, _P, _P, _P, _P, _I32, _I64, _I64, _I32, _P, _I32, _P, _P, _I32, _P, _P, _P]),
     "fbgemm_amd_tbe_plan_profile": (C.c_int, [_P, _I32]),
     "fbgemm_amd_tbe_plan_profile_read": (C.c_int, [_P, _P, _I32, _P]),
+    "fbgemm_amd_bounds_check_indices": (C.c_int, [_P, _I32, _P, _P, _I32, _I64, _I64, _I32, _P, _P, _P, _P]),
+    "fbgemm_amd_pruned_hashmap_lookup": (C.c_int, [_P, _P, _I32, _I64, _P, _I32, _P, _I32, _P, _P]),
+    "fbgemm_amd_quantize_rowwise": (C.c_int, [_P, _I32, _I64, _I32, _I32, _I32, _I32, _I64, _P, _P]),
+    "fbgemm_amd_dequantize_rowwise": (C.c_int, [_P, _I64, _I64, _I32, _I32, _I32, _I32, _I32, _P, _P]),
     "fbgemm_amd_tbe_plan_num_rows": (_I64, [_P, _I32]),
     "fbgemm_amd_tbe_plan_row_bytes": (_I64, [_P, _I32]),
     "fbgemm_amd_pruned_array_lookup": (C.c_int, [_P, _P, _I32, _I64, _P, _I32, _P, _I32, _P, _P]),

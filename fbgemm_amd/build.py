@@ -11,13 +11,14 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "lib", "libfbgemm_amd.so")
 
-SOURCES = ["lookup_kernels.hip", "c_api.cpp"]
+SOURCES = ["lookup_kernels.hip", "index_ops_kernels.hip", "quantize_kernels.hip", "c_api.cpp"]
+HEADERS = ["lookup_common.h", os.path.join("..", "..", "include", "fbgemm_amd.h")]
 
 # -ffp-contract=off: the kernels spell out every fma; nothing else may be fused,
 #   or the fp32 rounding sequence would differ from the reference's.
 # -packed-fp32-ops off: keep the compiler from forming packed fp32 instructions.
 FLAGS = [
-    "-x", "hip", "-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-shared",
+    "-x", "hip", "-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC",
     "-ffp-contract=off", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     # error reporting uses a few atomics on one address; keep them as plain
     # atomics instead of a wave-wide reduction loop in front of each
@@ -25,18 +26,42 @@ FLAGS = [
 ]
 
 
-def build_library(verbose=False):
-    os.makedirs(os.path.dirname(OUT), exist_ok=True)
-    cmd = ["hipcc", *FLAGS, "-o", OUT, *[os.path.join(CSRC, s) for s in SOURCES]]
-    if verbose:
-        print(" ".join(cmd), flush=True)
+def _hipcc(cmd):
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     # hipcc's host pass does not know the device-only target feature; that warning is noise
     out = "\n".join(l for l in proc.stdout.splitlines() if "packed-fp32-ops" not in l)
     if proc.returncode != 0:
         raise RuntimeError(f"hipcc failed:\n{out}")
-    if verbose and out.strip():
-        print(out)
+    return out
+
+
+def build_library(verbose=False, force=True):
+    """Compile every source to an object (side by side) and link them.
+    ``force=False`` keeps objects that are newer than their source and the
+    shared headers (for edit-compile loops); the default compiles everything."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    objdir = os.path.join(HERE, "lib", "obj")
+    os.makedirs(objdir, exist_ok=True)
+    newest_header = max(os.path.getmtime(os.path.join(CSRC, h)) for h in HEADERS)
+    jobs = []
+    for src in SOURCES:
+        path = os.path.join(CSRC, src)
+        obj = os.path.join(objdir, os.path.splitext(src)[0] + ".o")
+        stale = force or not os.path.exists(obj) or os.path.getmtime(obj) < max(os.path.getmtime(path), newest_header)
+        if stale:
+            jobs.append(["hipcc", *FLAGS, "-c", "-o", obj, path])
+    if verbose:
+        for j in jobs:
+            print(" ".join(j), flush=True)
+    with ThreadPoolExecutor(max_workers=4) as pool:
+        outs = list(pool.map(_hipcc, jobs))
+    objs = [os.path.join(objdir, os.path.splitext(s)[0] + ".o") for s in SOURCES]
+    outs.append(_hipcc(["hipcc", "--offload-arch=gfx950", "-fPIC", "-shared", "-o", OUT, *objs]))
+    if verbose:
+        for o in outs:
+            if o.strip():
+                print(o)
     return OUT
 
 
@@ -82,7 +107,7 @@ def build_cpp_test(verbose=False):
 
 
 if __name__ == "__main__":
-    print(build_library(verbose=True))
+    print(build_library(verbose=True, force="--incremental" not in sys.argv))
     print(build_torch_op(verbose=True))
     print(build_cpp_test(verbose=True))
     sys.exit(0)

@@ -20,6 +20,19 @@ hipError_t launch_lengths_to_offsets(const void* lengths, bool is64, int64_t n, 
 hipError_t launch_status_clear(Status* st, hipStream_t stream);
 hipError_t launch_bag_order(const void* offsets, bool off64, int32_t B, int32_t T, BagEntry* order, hipStream_t stream);
 hipError_t launch_calibration_copy(const void* src, void* dst, int64_t bytes, hipStream_t stream);
+hipError_t launch_bounds_check(const int64_t* rows_per_table, int32_t T, void* indices, void* offsets, bool is64,
+                               int64_t num_indices, int64_t total_B, int64_t B, const int32_t* B_offsets, int mode,
+                               int64_t* warning, int64_t* fixed, int64_t* partial, Status* status, hipStream_t stream);
+int64_t bounds_check_partials(int64_t total_B);
+hipError_t launch_quantize_rowwise(const void* input, bool half_in, int64_t rows, int32_t cols, int32_t bits,
+                                   int32_t sb_float, int32_t layout, int64_t out_stride, void* output,
+                                   hipStream_t stream);
+hipError_t launch_dequantize_rowwise(const void* input, int64_t rows, int64_t in_stride, int32_t cols, int32_t bits,
+                                     int32_t sb_float, int32_t layout, int32_t output_ty, void* output,
+                                     hipStream_t stream);
+hipError_t launch_pruned_hashmap_lookup(const void* indices, const void* offsets, bool idx64, const void* hash_table,
+                                        bool hash64, const int64_t* hash_table_offsets, int32_t B, int32_t T,
+                                        void* dense, hipStream_t stream);
 hipError_t launch_pruned_array_lookup(const void* indices, const void* offsets, bool idx64, const void* remap,
                                       bool remap64, const int64_t* remap_offsets, int32_t B, int32_t T,
                                       void* dense, hipStream_t stream);
@@ -153,6 +166,10 @@ struct DeviceScratch {
   int64_t offsets_cap = 0;
   BagEntry* order = nullptr;  // bag order of single-table calls
   int64_t order_cap = 0;
+  int64_t* fixed = nullptr;   // bounds check: repaired offsets before they are written back
+  int64_t fixed_cap = 0;
+  int64_t* partial = nullptr; // bounds check: per-block maxima of the offset scan
+  int64_t partial_cap = 0;
 };
 
 // Grow-only device buffer; the old one may still be read by an enqueued kernel.
@@ -689,6 +706,89 @@ int fbgemm_amd_tbe_plan_profile_read(fbgemm_amd_tbe_plan* plan, float* ms, int32
   }
   *n = (int32_t)have;
   plan->prof_count = 0;
+  return 0;
+}
+
+namespace {
+int check_quant_format(int32_t bit_rate, int32_t sb_float, int32_t layout, int32_t cols, int64_t row_stride) {
+  if (bit_rate != 2 && bit_rate != 4 && bit_rate != 8) return fail(FBGEMM_AMD_E_ARG, "bit_rate must be 2, 4 or 8");
+  if (sb_float && bit_rate != 8) return fail(FBGEMM_AMD_E_ARG, "fp32 scale/bias go with 8-bit rows only");
+  if (layout != FBGEMM_AMD_QLAYOUT_TRAILER && layout != FBGEMM_AMD_QLAYOUT_TBE) return fail(FBGEMM_AMD_E_ARG, "unknown row layout");
+  if (cols <= 0) return fail(FBGEMM_AMD_E_ARG, "cols must be positive");
+  const int epb = 8 / bit_rate;
+  const int64_t need = (cols + epb - 1) / epb + ((sb_float && layout == FBGEMM_AMD_QLAYOUT_TRAILER) ? 8 : 4);
+  if (row_stride < need) return fail(FBGEMM_AMD_E_ARG, "row stride %lld is below the %lld bytes a row takes", (long long)row_stride, (long long)need);
+  return 0;
+}
+} // namespace
+
+int fbgemm_amd_quantize_rowwise(
+    const void* d_input, int32_t input_ty, int64_t rows, int32_t cols, int32_t bit_rate, int32_t sb_float,
+    int32_t layout, int64_t out_row_stride, void* d_output, void* stream) {
+  if (input_ty != ST_FP32 && input_ty != ST_FP16) return fail(FBGEMM_AMD_E_ARG, "input must be fp32 or fp16");
+  if (rows < 0) return fail(FBGEMM_AMD_E_ARG, "rows must not be negative");
+  if (int rc = check_quant_format(bit_rate, sb_float, layout, cols, out_row_stride)) return rc;
+  if (rows == 0) return 0;
+  if (!d_input || !d_output) return fail(FBGEMM_AMD_E_ARG, "null data pointer");
+  HIP_TRY(launch_quantize_rowwise(d_input, input_ty == ST_FP16, rows, cols, bit_rate, sb_float, layout, out_row_stride,
+                                  d_output, (hipStream_t)stream));
+  return 0;
+}
+
+int fbgemm_amd_dequantize_rowwise(
+    const void* d_input, int64_t rows, int64_t in_row_stride, int32_t cols, int32_t bit_rate, int32_t sb_float,
+    int32_t layout, int32_t output_ty, void* d_output, void* stream) {
+  if (output_ty != ST_FP32 && output_ty != ST_FP16 && output_ty != ST_BF16) return fail(FBGEMM_AMD_E_ARG, "output must be fp32, fp16 or bf16");
+  if (rows < 0) return fail(FBGEMM_AMD_E_ARG, "rows must not be negative");
+  if (layout == FBGEMM_AMD_QLAYOUT_TBE && sb_float) return fail(FBGEMM_AMD_E_ARG, "TBE rows carry an fp16 scale/bias pair");
+  if (int rc = check_quant_format(bit_rate, sb_float, layout, cols, in_row_stride)) return rc;
+  if (rows == 0) return 0;
+  if (!d_input || !d_output) return fail(FBGEMM_AMD_E_ARG, "null data pointer");
+  HIP_TRY(launch_dequantize_rowwise(d_input, rows, in_row_stride, cols, bit_rate, sb_float, layout, output_ty, d_output,
+                                    (hipStream_t)stream));
+  return 0;
+}
+
+int fbgemm_amd_bounds_check_indices(
+    const int64_t* d_rows_per_table, int32_t T, void* d_indices, void* d_offsets, int32_t index_bits,
+    int64_t indices_numel, int64_t offsets_numel, int32_t bounds_check_mode, int64_t* d_warning,
+    const int32_t* d_B_offsets, void* d_status, void* stream_) {
+  if (T <= 0 || !d_rows_per_table) return fail(FBGEMM_AMD_E_ARG, "rows_per_table must hold T >= 1 entries");
+  if (index_bits != 32 && index_bits != 64) return fail(FBGEMM_AMD_E_ARG, "index_bits must be 32 or 64");
+  if (bounds_check_mode < 0 || bounds_check_mode > 2) return fail(FBGEMM_AMD_E_ARG, "bounds_check_mode must be 0 (FATAL), 1 (WARNING) or 2 (IGNORE)");
+  if (offsets_numel < 1 || !d_offsets) return fail(FBGEMM_AMD_E_ARG, "offsets must hold at least one entry");
+  const int64_t total_B = offsets_numel - 1;
+  // embedding_bounds_check_host_cpu.cpp:126-131
+  if (!d_B_offsets && total_B % T != 0)
+    return fail(FBGEMM_AMD_E_ARG, "offsets size %lld is not equal to B (%lld) * T (%d) + 1", (long long)offsets_numel,
+                (long long)(total_B / T), T);
+  if (indices_numel > 0 && !d_indices) return fail(FBGEMM_AMD_E_ARG, "null data pointer");
+  if (bounds_check_mode == 1 && !d_warning) return fail(FBGEMM_AMD_E_ARG, "WARNING mode needs the warning counter");
+  if (bounds_check_mode == 0 && !d_status) return fail(FBGEMM_AMD_E_ARG, "FATAL mode reports through d_status");
+  hipStream_t stream = (hipStream_t)stream_;
+  std::lock_guard<std::mutex> lk(g_mu);
+  DeviceScratch* s;
+  if (int rc = get_scratch(&s)) return rc;
+  if (int rc = grow(&s->fixed, &s->fixed_cap, total_B + 1, stream)) return rc;
+  if (int rc = grow(&s->partial, &s->partial_cap, bounds_check_partials(total_B), stream)) return rc;
+  HIP_TRY(launch_bounds_check(d_rows_per_table, T, d_indices, d_offsets, index_bits == 64, indices_numel, total_B,
+                              d_B_offsets ? 0 : total_B / T, d_B_offsets, bounds_check_mode, d_warning, s->fixed,
+                              s->partial, (Status*)d_status, stream));
+  return 0;
+}
+
+int fbgemm_amd_pruned_hashmap_lookup(
+    const void* d_indices, const void* d_offsets, int32_t index_bits, int64_t offsets_numel,
+    const void* d_hash_table, int32_t hash_bits, const int64_t* d_hash_table_offsets, int32_t T,
+    void* d_dense, void* stream) {
+  if (T <= 0 || offsets_numel < 1 || (offsets_numel - 1) % T != 0) return fail(FBGEMM_AMD_E_ARG, "offsets must hold T*B+1 entries");
+  if ((index_bits != 32 && index_bits != 64) || (hash_bits != 32 && hash_bits != 64))
+    return fail(FBGEMM_AMD_E_ARG, "index_bits/hash_bits must be 32 or 64");
+  const int64_t B = (offsets_numel - 1) / T;
+  if (B == 0) return 0;
+  if (!d_indices || !d_offsets || !d_hash_table_offsets || !d_dense) return fail(FBGEMM_AMD_E_ARG, "null data pointer");
+  HIP_TRY(launch_pruned_hashmap_lookup(d_indices, d_offsets, index_bits == 64, d_hash_table, hash_bits == 64,
+                                       d_hash_table_offsets, (int32_t)B, T, d_dense, (hipStream_t)stream));
   return 0;
 }
 

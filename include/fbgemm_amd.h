@@ -200,6 +200,71 @@ int fbgemm_amd_pruned_array_lookup(
     const int64_t* d_index_remappings_offsets, int32_t T, void* d_dense,
     void* stream);
 
+/* ---- index operators that run before the lookup ---------------------------- *
+ *
+ * bounds_check_indices (fbgemm_gpu/codegen/utils/embedding_bounds_check_host_cpu.cpp:76-219,
+ * schema :240-256; the step before the lookup in
+ * split_table_batched_embeddings_ops_inference.py:1067-1124). In place on
+ * d_indices / d_offsets (same width). bounds_check_mode: 0 FATAL, 1 WARNING,
+ * 2 IGNORE (embedding_common.h:44-48).
+ *   WARNING / IGNORE: offsets[last] becomes indices_numel; every offset is
+ *     clamped to [0, indices_numel] and raised to the largest offset before it
+ *     (what the reference's sequential loop leaves); an index other than -1
+ *     outside [0, rows_per_table[t]) becomes 0. WARNING zeroes d_warning[0]
+ *     first and counts one per repaired last offset, per bad bag and per bad
+ *     index, like the reference's counter.
+ *   FATAL: nothing is modified; the conditions the reference raises on are
+ *     ORed into d_status (FBGEMM_AMD_ERR_LENGTH_MISMATCH: last offset !=
+ *     indices_numel; FBGEMM_AMD_ERR_BAG_OVERRUN: offsets negative, decreasing
+ *     or beyond indices_numel; FBGEMM_AMD_ERR_INDEX_OUT_OF_RANGE, with the
+ *     first offending position). The reference's GPU kernel asserts on the
+ *     device instead, which takes the process down.
+ * d_B_offsets: NULL, or int32[T+1] first bag of every table (variable batch
+ * sizes). Uses library-owned scratch: calls must be ordered on one stream. */
+int fbgemm_amd_bounds_check_indices(
+    const int64_t* d_rows_per_table, int32_t T, void* d_indices, void* d_offsets, int32_t index_bits,
+    int64_t indices_numel, int64_t offsets_numel, int32_t bounds_check_mode, int64_t* d_warning,
+    const int32_t* d_B_offsets, void* d_status, void* stream);
+
+/* pruned_hashmap_lookup (embedding_forward_quantized_cpu_template.cpp:524-603; GPU
+ * embedding_forward_quantized_split_lookup.cu:19-118): d_hash_table holds
+ * [slots][2] (sparse id, dense id) pairs of hash_bits each, -1 = empty, built by
+ * the reference's pruned_hashmap_insert (linear probing from MurmurHash3's
+ * finalizer of the id, 32- or 64-bit after the index width, modulo the table's
+ * capacity). d_dense[i] = the dense id of d_indices[i], -1 when absent, a copy
+ * for tables with an empty slot range. */
+int fbgemm_amd_pruned_hashmap_lookup(
+    const void* d_indices, const void* d_offsets, int32_t index_bits, int64_t offsets_numel,
+    const void* d_hash_table, int32_t hash_bits, const int64_t* d_hash_table_offsets, int32_t T,
+    void* d_dense, void* stream);
+
+/* ---- row-wise quantizers: producers and readers of the row formats ---------- *
+ *
+ * fp32 / fp16 rows [rows][cols] -> fused quantized rows, bit for bit what the
+ * reference's CPU routines write:
+ *   bit_rate 2 / 4 / 8, sb_float 0: FloatOrHalfToFusedNBitRowwiseQuantizedSBHalf
+ *     (src/QuantUtils.cc:534-611): packed elements, then fp16 scale, fp16 bias;
+ *   bit_rate 8, sb_float 1: FloatOrHalfToFused8BitRowwiseQuantizedSBFloat
+ *     (src/QuantUtils.cc:677-718): bytes, then fp32 scale, fp32 bias.
+ * layout FBGEMM_AMD_QLAYOUT_TRAILER keeps that order; FBGEMM_AMD_QLAYOUT_TBE
+ * writes the table-batched operator's rows, fp16 scale and bias FIRST, then
+ * the elements, as quantize_embs rearranges them
+ * (fbgemm_gpu/fbgemm_gpu/tbe/utils/quantize.py:47-70; with sb_float 1 the fp32
+ * pair is rounded to fp16, as there). out_row_stride is in bytes (>= the row's
+ * size: padding bytes are left alone). */
+enum { FBGEMM_AMD_QLAYOUT_TRAILER = 0, FBGEMM_AMD_QLAYOUT_TBE = 1 };
+int fbgemm_amd_quantize_rowwise(
+    const void* d_input, int32_t input_ty, int64_t rows, int32_t cols, int32_t bit_rate, int32_t sb_float,
+    int32_t layout, int64_t out_row_stride, void* d_output, void* stream);
+
+/* The inverses (src/QuantUtils.cc:743-789 FusedNBitRowwiseQuantizedSBHalfToFloatOrHalf,
+ * :847-892 Fused8BitRowwiseQuantizedSBFloatToFloatOrHalf): element =
+ * float(double(scale) * q + double(bias)), written as fp32, fp16 (round to
+ * nearest even) or bf16 ((bits + 0x8000) >> 16); output [rows][cols], dense. */
+int fbgemm_amd_dequantize_rowwise(
+    const void* d_input, int64_t rows, int64_t in_row_stride, int32_t cols, int32_t bit_rate, int32_t sb_float,
+    int32_t layout, int32_t output_ty, void* d_output, void* stream);
+
 /* ---- measurement aid -------------------------------------------------------- *
  * No counterpart in the reference. A plain device-to-device copy of `bytes`
  * (a multiple of 16) by a kernel named calibration_copy_kernel: profiles scale

@@ -18,6 +18,7 @@ import numpy as np
 HERE = os.path.dirname(os.path.abspath(__file__))
 ORACLE_SO = os.path.join(HERE, "_build", "libembedding_oracle.so")
 REF_SO = os.path.join(HERE, "_ref", "libfbgemm_ref.so")
+REF_QUANT_SO = os.path.join(HERE, "_ref", "libfbgemm_ref_quant.so")
 JIT_SO = os.path.join(HERE, "_build", "libfbgemm_jit_bridge.so")
 
 ST_FP32, ST_FP16, ST_INT8, ST_INT4, ST_INT2, ST_BF16 = 0, 1, 2, 3, 4, 5
@@ -65,6 +66,28 @@ def _lib(impl):
         lib.oracle_tbe_forward.restype = _c.c_int
         lib.oracle_padded_row_bytes.argtypes = [_c.c_int32, _c.c_int, _c.c_int32, _c.c_int32]
         lib.oracle_padded_row_bytes.restype = _c.c_int32
+        lib.oracle_bounds_check_indices.argtypes = [
+            _c.c_void_p, _c.c_int32, _c.c_void_p, _c.c_void_p, _c.c_int, _c.c_int64, _c.c_int64,
+            _c.c_int, _c.c_void_p, _c.c_void_p]
+        lib.oracle_bounds_check_indices.restype = _c.c_int
+        lib.oracle_pruned_hash32.argtypes = [_c.c_uint32]
+        lib.oracle_pruned_hash32.restype = _c.c_uint32
+        lib.oracle_pruned_hash64.argtypes = [_c.c_uint64]
+        lib.oracle_pruned_hash64.restype = _c.c_uint64
+        lib.oracle_pruned_hashmap_insert.argtypes = [
+            _c.c_int32, _c.c_int32, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int, _c.c_void_p,
+            _c.c_int, _c.c_void_p]
+        lib.oracle_pruned_hashmap_insert.restype = _c.c_int
+        lib.oracle_pruned_hashmap_lookup.argtypes = [
+            _c.c_int32, _c.c_int32, _c.c_void_p, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_int,
+            _c.c_void_p, _c.c_void_p]
+        lib.oracle_pruned_hashmap_lookup.restype = None
+        lib.oracle_quantize_rowwise.argtypes = [
+            _c.c_void_p, _c.c_int, _c.c_int64, _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int64, _c.c_void_p]
+        lib.oracle_quantize_rowwise.restype = None
+        lib.oracle_dequantize_rowwise.argtypes = [
+            _c.c_void_p, _c.c_int64, _c.c_int64, _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32, _c.c_void_p]
+        lib.oracle_dequantize_rowwise.restype = None
     elif impl == "ref":
         if not os.path.exists(REF_SO):
             raise FileNotFoundError(REF_SO)
@@ -73,10 +96,26 @@ def _lib(impl):
         lib.ref_embedding_spmdm.restype = _c.c_int
         lib.ref_compressed_indices_remap.argtypes = _REMAP_ARGS
         lib.ref_compressed_indices_remap.restype = None
+    elif impl == "refquant":
+        if not os.path.exists(REF_QUANT_SO):
+            raise FileNotFoundError(REF_QUANT_SO)
+        # lazy binding: the reference's vector translation units are not part of
+        # this build, and nothing that is called here reaches them
+        lib = _c.CDLL(REF_QUANT_SO, mode=os.RTLD_LAZY)
+        lib.ref_quantize_nbit.argtypes = [_c.c_int, _c.c_void_p, _c.c_int, _c.c_int64, _c.c_int, _c.c_void_p]
+        lib.ref_quantize_8bit.argtypes = [_c.c_void_p, _c.c_int, _c.c_int64, _c.c_int, _c.c_void_p]
+        lib.ref_dequantize_nbit.argtypes = [_c.c_int, _c.c_void_p, _c.c_int64, _c.c_int, _c.c_int, _c.c_void_p]
+        lib.ref_dequantize_8bit.argtypes = [_c.c_void_p, _c.c_int64, _c.c_int, _c.c_int, _c.c_void_p]
+        for f in (lib.ref_quantize_nbit, lib.ref_quantize_8bit, lib.ref_dequantize_nbit, lib.ref_dequantize_8bit):
+            f.restype = None
     else:
         raise ValueError(impl)
     _libs[impl] = lib
     return lib
+
+
+def have_ref_quant():
+    return os.path.exists(REF_QUANT_SO)
 
 
 def have_ref():
@@ -162,6 +201,108 @@ def pruned_array_lookup(indices, offsets, remap, remap_offsets):
         T, B, _ptr(indices), _ptr(offsets), _is64(indices), _ptr(remap), _is64(remap),
         _ptr(remap_offsets), _ptr(dense))
     return dense
+
+
+BOUNDS_FATAL, BOUNDS_WARNING, BOUNDS_IGNORE = 0, 1, 2
+
+
+def bounds_check_indices(rows_per_table, indices, offsets, mode, warning, B_offsets=None):
+    """In place on ``indices`` / ``offsets`` / ``warning`` (numpy arrays, index
+    arrays of one dtype). Returns 0, or the condition a FATAL run stops at."""
+    rows_per_table = np.ascontiguousarray(rows_per_table, dtype=np.int64)
+    assert indices.flags.c_contiguous and offsets.flags.c_contiguous and offsets.dtype == indices.dtype
+    assert warning.dtype == np.int64
+    bo = None if B_offsets is None else np.ascontiguousarray(B_offsets, dtype=np.int32)
+    return _lib("oracle").oracle_bounds_check_indices(
+        _ptr(rows_per_table), len(rows_per_table), _ptr(indices), _ptr(offsets), _is64(indices),
+        indices.size, offsets.size, int(mode), _ptr(warning), _ptr(bo))
+
+
+def pruned_hash(x, bits):
+    lib = _lib("oracle")
+    return lib.oracle_pruned_hash64(x) if bits == 64 else lib.oracle_pruned_hash32(x)
+
+
+def pruned_hashmap_insert(indices, dense_indices, offsets, hash_table, hash_table_offsets):
+    """In place on ``hash_table`` ([slots, 2] int32 or int64, -1 = empty)."""
+    indices = np.ascontiguousarray(indices)
+    dense_indices = np.ascontiguousarray(dense_indices, dtype=indices.dtype)
+    offsets = np.ascontiguousarray(offsets, dtype=indices.dtype)
+    hto = np.ascontiguousarray(hash_table_offsets, dtype=np.int64)
+    assert hash_table.flags.c_contiguous and hash_table.ndim == 2 and hash_table.shape[1] == 2
+    T = len(hto) - 1
+    B = (len(offsets) - 1) // T
+    rc = _lib("oracle").oracle_pruned_hashmap_insert(
+        T, B, _ptr(indices), _ptr(dense_indices), _ptr(offsets), _is64(indices), _ptr(hash_table),
+        _is64(hash_table), _ptr(hto))
+    if rc:
+        raise RuntimeError("hash table full")
+
+
+def pruned_hashmap_lookup(indices, offsets, hash_table, hash_table_offsets):
+    indices = np.ascontiguousarray(indices)
+    offsets = np.ascontiguousarray(offsets, dtype=indices.dtype)
+    hto = np.ascontiguousarray(hash_table_offsets, dtype=np.int64)
+    hash_table = np.ascontiguousarray(hash_table)
+    T = len(hto) - 1
+    B = (len(offsets) - 1) // T
+    dense = np.empty_like(indices)
+    _lib("oracle").oracle_pruned_hashmap_lookup(
+        T, B, _ptr(indices), _ptr(offsets), _is64(indices), _ptr(hash_table), _is64(hash_table),
+        _ptr(hto), _ptr(dense))
+    return dense
+
+
+LAYOUT_TRAILER, LAYOUT_TBE = 0, 1
+
+
+def quantized_row_bytes(cols, bit_rate, sb_float, layout):
+    epb = 8 // bit_rate
+    return (cols + epb - 1) // epb + (8 if (sb_float and layout == LAYOUT_TRAILER) else 4)
+
+
+def quantize_rowwise(x, bit_rate, sb_float=False, layout=LAYOUT_TRAILER, out_stride=None, impl="oracle", fill=0):
+    """x: [rows, cols] float32 or float16 (numpy). Returns uint8 [rows, out_stride].
+    impl: "oracle" or "ref" (the reference's scalar routine, trailer layout only)."""
+    x = np.ascontiguousarray(x)
+    assert x.ndim == 2 and x.dtype in (np.float32, np.float16)
+    rows, cols = x.shape
+    need = quantized_row_bytes(cols, bit_rate, sb_float, layout)
+    out_stride = need if out_stride is None else out_stride
+    out = np.full((rows, out_stride), fill, np.uint8)
+    half = int(x.dtype == np.float16)
+    if impl == "oracle":
+        _lib("oracle").oracle_quantize_rowwise(_ptr(x), half, rows, cols, bit_rate, int(sb_float), layout,
+                                               out_stride, _ptr(out))
+    else:
+        assert layout == LAYOUT_TRAILER and out_stride == need
+        if sb_float:
+            _lib("refquant").ref_quantize_8bit(_ptr(x), half, rows, cols, _ptr(out))
+        else:
+            _lib("refquant").ref_quantize_nbit(bit_rate, _ptr(x), half, rows, cols, _ptr(out))
+    return out
+
+
+def dequantize_rowwise(q, cols, bit_rate, sb_float=False, layout=LAYOUT_TRAILER, out_ty=ST_FP32, impl="oracle"):
+    """q: uint8 [rows, stride]. Returns [rows, cols] float32, or uint16 patterns (fp16 / bf16)."""
+    q = np.ascontiguousarray(q)
+    rows, stride = q.shape
+    out = np.zeros((rows, cols), out_dtype(out_ty))
+    if impl == "oracle":
+        _lib("oracle").oracle_dequantize_rowwise(_ptr(q), rows, stride, cols, bit_rate, int(sb_float), layout,
+                                                 out_ty, _ptr(out))
+    else:
+        assert layout == LAYOUT_TRAILER and stride == quantized_row_bytes(cols, bit_rate, sb_float, layout)
+        # the reference derives the column count from the row's bytes: every
+        # element slot of the last byte is written (src/QuantUtils.cc:758-760)
+        ref_cols = (stride - (8 if sb_float else 4)) * (8 // bit_rate)
+        full = np.zeros((rows, ref_cols), out_dtype(out_ty))
+        if sb_float:
+            _lib("refquant").ref_dequantize_8bit(_ptr(q), rows, stride, out_ty, _ptr(full))
+        else:
+            _lib("refquant").ref_dequantize_nbit(bit_rate, _ptr(q), rows, stride, out_ty, _ptr(full))
+        out = np.ascontiguousarray(full[:, :cols])
+    return out
 
 
 def tbe_forward(dev_weights, weights_offsets, weights_tys, D_offsets, total_D, indices,
