@@ -323,3 +323,100 @@ def padded_row_size_in_bytes(dim, weight_ty, row_alignment, scale_bias_bytes=4):
 def unpadded_row_size_in_bytes(dim, weight_ty, scale_bias_bytes=4):
     """nbit::unpadded_row_size_in_bytes (embedding_common.h:189-215)."""
     return _lib.lib().fbgemm_amd_unpadded_row_size_in_bytes(dim, weight_ty, scale_bias_bytes)
+
+
+BOUNDS_FATAL, BOUNDS_WARNING, BOUNDS_IGNORE = 0, 1, 2
+
+
+def bounds_check_indices(rows_per_table, indices, offsets, bounds_check_mode, warning, weights=None,
+                         B_offsets=None, max_B=-1):
+    """bounds_check_indices (fbgemm_gpu/codegen/utils/embedding_bounds_check_host_cpu.cpp:76-219,
+    schema :240-256): in place on ``indices`` / ``offsets`` / ``warning``.
+
+    FATAL raises where the reference's CPU operator raises (after a
+    synchronization); WARNING and IGNORE repair and stay asynchronous."""
+    _require_cuda(rows_per_table, indices, offsets, warning, weights, B_offsets)
+    if indices.dtype != offsets.dtype:
+        raise TypeError("indices and offsets must have the same dtype")
+    if not (indices.is_contiguous() and offsets.is_contiguous()):
+        raise ValueError("indices and offsets are modified in place and must be contiguous")
+    if weights is not None and weights.numel() != 0 and weights.size(0) != indices.numel():
+        raise RuntimeError(f"weights size {weights.size(0)} is not equal to indices size {indices.numel()}")
+    if B_offsets is not None and max_B < 0:
+        raise RuntimeError("max_B must not be negative with B_offsets")
+    rpt = rows_per_table.to(torch.int64).contiguous()
+    bo = None if B_offsets is None else B_offsets.to(torch.int32).contiguous()
+    status = Status(indices.device) if bounds_check_mode == BOUNDS_FATAL else None
+    check(_lib.lib().fbgemm_amd_bounds_check_indices(
+        _ptr(rpt), rpt.numel(), _ptr(indices), _ptr(offsets), _bits(indices), indices.numel(), offsets.numel(),
+        int(bounds_check_mode), _ptr(warning), _ptr(bo), None if status is None else _ptr(status.buf), _stream()))
+    if status is not None:
+        bits, pos = status.read()
+        if bits & ERR_LENGTH_MISMATCH:
+            raise RuntimeError(f"the last offset is not the number of indices ({indices.numel()})")
+        if bits & ERR_BAG_OVERRUN:
+            raise RuntimeError("offsets are negative, decreasing or beyond the number of indices")
+        if bits & ERR_INDEX_OUT_OF_RANGE:
+            raise RuntimeError(f"Index {pos} is out of bounds: {int(indices[pos])}")
+
+
+def pruned_hashmap_lookup(indices, offsets, hash_table, hash_table_offsets):
+    """pruned_hashmap_lookup (embedding_forward_quantized_host_cpu.cpp:338-341;
+    embedding_forward_quantized_cpu_template.cpp:524-603)."""
+    _require_cuda(indices, offsets, hash_table, hash_table_offsets)
+    if indices.dtype != offsets.dtype:
+        raise TypeError("indices and offsets must have the same dtype")
+    T = hash_table_offsets.numel() - 1
+    if T <= 0 or (offsets.numel() - 1) // T <= 0:
+        raise RuntimeError("pruned_hashmap_lookup needs B > 0")  # TORCH_CHECK(B > 0), :537
+    dense = torch.empty_like(indices)
+    hto = hash_table_offsets.to(torch.int64).contiguous()
+    check(_lib.lib().fbgemm_amd_pruned_hashmap_lookup(
+        _ptr(indices.contiguous()), _ptr(offsets.contiguous()), _bits(indices), offsets.numel(),
+        _ptr(hash_table.contiguous()), _bits(hash_table), _ptr(hto), T, _ptr(dense), _stream()))
+    return dense
+
+
+QLAYOUT_TRAILER, QLAYOUT_TBE = 0, 1
+
+
+def quantized_row_bytes(cols, bit_rate, sb_float=False, layout=QLAYOUT_TRAILER):
+    epb = 8 // bit_rate
+    return (cols + epb - 1) // epb + (8 if (sb_float and layout == QLAYOUT_TRAILER) else 4)
+
+
+def quantize_rowwise(input, bit_rate, sb_float=False, layout=QLAYOUT_TRAILER, out=None):
+    """fp32 / fp16 ``[rows, cols]`` -> fused quantized rows, uint8 ``[rows, stride]``
+    (FloatOrHalfToFusedNBitRowwiseQuantizedSBHalf, src/QuantUtils.cc:534-611;
+    FloatOrHalfToFused8BitRowwiseQuantizedSBFloat, :677-718; TBE re-layout as
+    fbgemm_gpu/fbgemm_gpu/tbe/utils/quantize.py:47-70). ``out`` may be a wider
+    (padded) row buffer; bytes beyond the row's own are left alone."""
+    _require_cuda(input, out)
+    if input.dim() != 2 or input.dtype not in (torch.float32, torch.float16):
+        raise TypeError("input must be a 2-D fp32 or fp16 tensor")
+    input = input.contiguous()
+    rows, cols = input.shape
+    if out is None:
+        out = torch.empty((rows, quantized_row_bytes(cols, bit_rate, sb_float, layout)), dtype=torch.uint8,
+                          device=input.device)
+    if out.dtype != torch.uint8 or out.dim() != 2 or out.size(0) != rows or out.stride(1) != 1:
+        raise ValueError("out must be uint8 [rows, stride] with unit column stride")
+    check(_lib.lib().fbgemm_amd_quantize_rowwise(
+        _ptr(input), _TORCH_OUT[input.dtype], rows, cols, bit_rate, int(sb_float), layout,
+        out.stride(0) if rows > 1 else out.size(1), _ptr(out), _stream()))
+    return out
+
+
+def dequantize_rowwise(input, cols, bit_rate, sb_float=False, layout=QLAYOUT_TRAILER, output_dtype=torch.float32):
+    """Fused quantized rows uint8 ``[rows, stride]`` -> ``[rows, cols]`` fp32 / fp16 / bf16
+    (FusedNBitRowwiseQuantizedSBHalfToFloatOrHalf, src/QuantUtils.cc:743-789;
+    Fused8BitRowwiseQuantizedSBFloatToFloatOrHalf, :847-892)."""
+    _require_cuda(input)
+    if input.dtype != torch.uint8 or input.dim() != 2 or input.stride(1) != 1:
+        raise ValueError("input must be uint8 [rows, stride] with unit column stride")
+    rows = input.size(0)
+    out = torch.empty((rows, cols), dtype=output_dtype, device=input.device)
+    check(_lib.lib().fbgemm_amd_dequantize_rowwise(
+        _ptr(input), rows, input.stride(0) if rows > 1 else input.size(1), cols, bit_rate, int(sb_float), layout,
+        _TORCH_OUT[output_dtype], _ptr(out), _stream()))
+    return out
