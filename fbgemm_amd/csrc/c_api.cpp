@@ -160,6 +160,38 @@ void plan_lanes(TableDesc& d, uintptr_t base_addr, int64_t out_stride, bool has_
   }
 }
 
+// What fetching one row costs, in 128-byte line requests (what the memory
+// system charges for): the lines the loaded bytes of a row touch, averaged over
+// the alignments rows of this stride take, plus a request for a scale/bias pair
+// that is fetched apart from the data, plus the row's share of the index,
+// weight and bookkeeping traffic (fitted to measured run times: about a third
+// of a line).
+double row_cost(const TableDesc& d) {
+  const bool q = quantised(d.ty);
+  int64_t first = 0, last; // bytes of the row that are loaded: [first, last)
+  if (d.inline_hdr) {
+    last = ((int64_t)d.data_bytes + 4 + 15) / 16 * 16;
+  } else {
+    first = d.data_off;
+    last = (int64_t)d.data_off + d.data_bytes;
+    if (q) {
+      first = std::min<int64_t>(first, d.sb_off);
+      last = std::max<int64_t>(last, (int64_t)d.sb_off + (d.sb_fp32 ? 8 : 4));
+    }
+  }
+  // rows start at (offset of row 0 + k * gcd(stride, 128)) mod 128
+  int64_t g = 128, b = d.row_stride % 128;
+  while (b) { const int64_t r = g % b; g = b; b = r; }
+  double lines = 0;
+  for (int64_t k = 0; k < 128 / g; ++k) {
+    const int64_t o = (d.weights_offset % 128 + k * g) % 128;
+    lines += (double)((o + last - 1) / 128 - (o + first) / 128 + 1);
+  }
+  lines /= (double)(128 / g);
+  if (q && !d.inline_hdr) lines += 0.5;
+  return lines + 0.35;
+}
+
 struct DeviceScratch {
   Status* status = nullptr;
   int64_t* offsets = nullptr; // lengths -> offsets
@@ -566,8 +598,7 @@ int fbgemm_amd_tbe_forward_pruned(
         const TableDesc& d = plan->tables[t];
         const int G = bags_per_wave(d.lanes);
         nwaves[t] = (B + G - 1) / G;
-        const double lines = 1.0 + (double)(d.row_stride - 1) / 128.0; // expected lines a row touches
-        wave_cost[t] = G * (lines + 0.25);
+        wave_cost[t] = G * row_cost(d);
         total_cost += wave_cost[t] * nwaves[t];
       }
       const int nx = xcd_lists ? 8 : 1;
@@ -670,6 +701,18 @@ int fbgemm_amd_tbe_forward_pruned(
     HIP_TRY(launch_bag_order(d_offsets, index_bits == 64, B, plan->T, w.d_order, stream));
     a.order = w.d_order;
   }
+#ifdef FBGEMM_AMD_WAVE_TRACE
+  static unsigned long long* trace_buf = nullptr;
+  static size_t trace_cap = 0;
+  const size_t trace_words = (size_t)(w.d_xcd_start ? 8 * w.num_waves : w.num_waves) * 4; // >= items
+  if (trace_cap < trace_words) {
+    if (trace_buf) (void)hipFree(trace_buf);
+    HIP_TRY(hipMalloc((void**)&trace_buf, trace_words * 8));
+    trace_cap = trace_words;
+  }
+  HIP_TRY(hipMemsetAsync(trace_buf, 0, trace_words * 8, stream));
+  a.trace = trace_buf;
+#endif
   const size_t slots = plan->prof_ev.size() / 2;
   const size_t slot = slots ? (size_t)(plan->prof_count % (int64_t)slots) : 0;
   if (slots) HIP_TRY(hipEventRecord(plan->prof_ev[2 * slot], stream));
@@ -678,6 +721,17 @@ int fbgemm_amd_tbe_forward_pruned(
     HIP_TRY(hipEventRecord(plan->prof_ev[2 * slot + 1], stream));
     ++plan->prof_count;
   }
+#ifdef FBGEMM_AMD_WAVE_TRACE
+  if (const char* path = getenv("FBGEMM_AMD_TRACE_FILE")) {
+    std::vector<unsigned long long> h(trace_words);
+    HIP_TRY(hipStreamSynchronize(stream));
+    HIP_TRY(hipMemcpy(h.data(), trace_buf, trace_words * 8, hipMemcpyDeviceToHost));
+    if (FILE* f = fopen(path, "wb")) {
+      fwrite(h.data(), 8, h.size(), f);
+      fclose(f);
+    }
+  }
+#endif
   return 0;
 }
 

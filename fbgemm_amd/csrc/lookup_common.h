@@ -116,6 +116,11 @@ struct LookupArgs {
                              // offsets[last] - offsets[0] must equal index_size
   int32_t out_aligned;       // `out` is 16-byte aligned (vector stores allowed)
   Status* status;
+#ifdef FBGEMM_AMD_WAVE_TRACE
+  // diagnostic build only: 4 words per workgroup (start, end of the wave on the
+  // 100 MHz wall clock; hardware id | XCC id << 32; work-list position)
+  unsigned long long* trace;
+#endif
 };
 
 } // namespace fbgemm_amd

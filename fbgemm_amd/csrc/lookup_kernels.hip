@@ -805,30 +805,10 @@ __device__ __forceinline__ void pool_dispatch_vb(const LookupArgs& a, const Tabl
 #define FBGEMM_AMD_MIN_WAVES 3 // waves per SIMD the register allocation must leave room for
 #endif
 
-// One wave per workgroup: waves come and go independently, and a workgroup
-// needs no more than its own 4 KB of LDS.
-// GENERAL = false is the table-batched operator's subset (no logical->physical
-// remap, no positional weights, offsets indexing one shared index array).
+// One item of the work list: `wave` is the position in the list (or the wave's
+// number for a single-table call).
 template <typename index_t, bool GENERAL>
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(FBGEMM_AMD_MIN_WAVES, 8))) void lookup_kernel(const LookupArgs a) {
-  __shared__ StageRow stage_row[MAX_GROUPS * MAX_ROUND];
-  __shared__ StageMul stage_mul[MAX_GROUPS * MAX_ROUND];
-  const int lane = threadIdx.x;
-  int64_t wave;
-  if (a.xcd_start) {
-    // Workgroups are handed to the 8 XCDs round-robin, so the workgroups with
-    // id % 8 == x all run on one XCD and share its L2. Each XCD walks its own
-    // run of the work list: whole tables (or slices of them) are pinned to
-    // one L2 instead of spreading their hot rows over all eight.
-    const int x = blockIdx.x & 7;
-    const int64_t w = (int64_t)(blockIdx.x >> 3);
-    const int64_t lo = a.xcd_start[x], hi = a.xcd_start[x + 1];
-    if (w >= hi - lo) return;
-    wave = lo + w;
-  } else {
-    wave = (int64_t)blockIdx.x;
-    if (wave >= a.num_waves) return;
-  }
+__device__ __forceinline__ void run_item(const LookupArgs& a, int64_t wave, int lane, StageRow* stage_row, StageMul* stage_mul) {
   int table = 0, first_slot;
   if (a.work) {
     const WaveWork ww = a.work[wave];
@@ -850,6 +830,54 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(FBGEMM_AMD_M
     case ST_BF16: pool_dispatch_vb<index_t, GENERAL, ST_BF16>(a, d, table, first_slot, lane, stage_row, stage_mul); break;
     default: break;
   }
+#endif
+}
+
+#ifdef FBGEMM_AMD_WAVE_TRACE
+__device__ __forceinline__ void trace_item(const LookupArgs& a, int64_t wave, int lane, unsigned long long t0) {
+  if (a.trace && lane == 0) {
+    unsigned long long* t = a.trace + (size_t)wave * 4;
+    const unsigned hw = __builtin_amdgcn_s_getreg((31 << 11) | 4);   // HW_ID
+    const unsigned xcc = __builtin_amdgcn_s_getreg((3 << 11) | 20);  // XCC_ID
+    t[0] = t0;
+    t[1] = wall_clock64();
+    t[2] = (unsigned long long)hw | ((unsigned long long)xcc << 32);
+    t[3] = (unsigned long long)blockIdx.x | ((unsigned long long)(a.work ? a.work[wave].table : 0) << 32);
+  }
+}
+#endif
+
+// One wave per workgroup: waves come and go independently, and a workgroup
+// needs no more than its own 4 KB of LDS.
+// GENERAL = false is the table-batched operator's subset (no logical->physical
+// remap, no positional weights, offsets indexing one shared index array).
+//
+// The work list of a table-batched call is 8 runs, one per XCD: whole tables
+// (or slices of them) are pinned to one XCD's L2 instead of spreading their hot
+// rows over all eight. Workgroup i takes item i >> 3 of run i & 7 (workgroups
+// are handed to the XCDs round-robin).
+template <typename index_t, bool GENERAL>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(FBGEMM_AMD_MIN_WAVES, 8))) void lookup_kernel(const LookupArgs a) {
+  __shared__ StageRow stage_row[MAX_GROUPS * MAX_ROUND];
+  __shared__ StageMul stage_mul[MAX_GROUPS * MAX_ROUND];
+  const int lane = threadIdx.x;
+  int64_t wave;
+  if (a.xcd_start) {
+    const int xb = blockIdx.x & 7;
+    const int64_t w = (int64_t)(blockIdx.x >> 3);
+    const int64_t lo = a.xcd_start[xb], hi = a.xcd_start[xb + 1];
+    if (w >= hi - lo) return;
+    wave = lo + w;
+  } else {
+    wave = (int64_t)blockIdx.x;
+    if (wave >= a.num_waves) return;
+  }
+#ifdef FBGEMM_AMD_WAVE_TRACE
+  const unsigned long long trace_t0 = wall_clock64();
+#endif
+  run_item<index_t, GENERAL>(a, wave, lane, stage_row, stage_mul);
+#ifdef FBGEMM_AMD_WAVE_TRACE
+  trace_item(a, wave, lane, trace_t0);
 #endif
 }
 
