@@ -152,6 +152,138 @@ Tensor pruned_array_lookup_hip(Tensor indices, Tensor offsets, Tensor index_rema
   return dense;
 }
 
+// bounds_check_indices (fbgemm_gpu/codegen/utils/embedding_bounds_check_host_cpu.cpp:76-219):
+// in place on indices / offsets / warning. WARNING and IGNORE repair on the
+// device without a synchronization. FATAL raises where the reference's CPU
+// operator raises, which costs a synchronization (the reference's GPU kernel
+// asserts on the device instead).
+void bounds_check_indices_hip(
+    Tensor& rows_per_table, Tensor& indices, Tensor& offsets, int64_t bounds_check_mode, Tensor& warning,
+    const std::optional<Tensor>& weights, const std::optional<Tensor>& B_offsets, int64_t max_B,
+    const std::optional<Tensor>& /*b_t_map*/, int64_t /*info_B_num_bits*/, int64_t /*info_B_mask*/,
+    int64_t /*bounds_check_version*/, bool /*prefetch_pipeline*/) {
+  TORCH_CHECK(rows_per_table.is_cuda() && indices.is_cuda() && offsets.is_cuda() && warning.is_cuda(),
+              "fbgemm_amd: tensors must be on the GPU");
+  TORCH_CHECK(indices.scalar_type() == at::kInt || indices.scalar_type() == at::kLong, "indices must be int32 or int64");
+  TORCH_CHECK(offsets.scalar_type() == indices.scalar_type(), "indices and offsets must have the same dtype");
+  TORCH_CHECK(indices.is_contiguous() && offsets.is_contiguous(), "indices and offsets are modified in place and must be contiguous");
+  TORCH_CHECK(warning.scalar_type() == at::kLong && warning.numel() >= 1);
+  if (weights && weights->numel() != 0)
+    TORCH_CHECK(weights->size(0) == indices.numel(), "weights size ", weights->size(0), " is not equal to indices size ", indices.numel());
+  if (B_offsets) TORCH_CHECK(max_B >= 0);
+  const Tensor rpt = rows_per_table.to(at::kLong).contiguous();
+  Tensor bo;
+  if (B_offsets) bo = B_offsets->to(at::kInt).contiguous();
+  Tensor st;
+  if (bounds_check_mode == 0) {
+    st = at::zeros({4}, indices.options().dtype(at::kInt));
+    TORCH_CHECK(fbgemm_amd_status_clear(st.data_ptr(), current_stream(indices)) == 0, fbgemm_amd_last_error());
+  }
+  const int rc = fbgemm_amd_bounds_check_indices(
+      rpt.data_ptr<int64_t>(), (int32_t)rpt.numel(), indices.data_ptr(), offsets.data_ptr(),
+      indices.scalar_type() == at::kLong ? 64 : 32, indices.numel(), offsets.numel(), (int32_t)bounds_check_mode,
+      warning.data_ptr<int64_t>(), bo.defined() ? bo.data_ptr<int32_t>() : nullptr, st.defined() ? st.data_ptr() : nullptr,
+      current_stream(indices));
+  TORCH_CHECK(rc == 0, "fbgemm_amd: ", fbgemm_amd_last_error());
+  if (bounds_check_mode == 0) {
+    int32_t bits = 0;
+    int64_t pos = -1;
+    TORCH_CHECK(fbgemm_amd_status_read(st.data_ptr(), current_stream(indices), &bits, &pos) == 0, fbgemm_amd_last_error());
+    TORCH_CHECK(!(bits & FBGEMM_AMD_ERR_LENGTH_MISMATCH), "bounds_check_indices: the last offset is not the number of indices");
+    TORCH_CHECK(!(bits & FBGEMM_AMD_ERR_BAG_OVERRUN), "bounds_check_indices: offsets are negative, decreasing or beyond the number of indices");
+    TORCH_CHECK(!(bits & FBGEMM_AMD_ERR_INDEX_OUT_OF_RANGE), "bounds_check_indices: index at position ", pos, " is out of bounds");
+  }
+}
+
+Tensor pruned_hashmap_lookup_hip(Tensor indices, Tensor offsets, Tensor hash_table, Tensor hash_table_offsets) {
+  TORCH_CHECK(indices.is_cuda() && offsets.is_cuda() && hash_table.is_cuda() && hash_table_offsets.is_cuda());
+  TORCH_CHECK(indices.scalar_type() == offsets.scalar_type(), "indices and offsets must have the same dtype");
+  indices = indices.contiguous();
+  offsets = offsets.contiguous();
+  hash_table = hash_table.contiguous();
+  const Tensor hto = hash_table_offsets.to(at::kLong).contiguous();
+  const int64_t T = hto.numel() - 1;
+  TORCH_CHECK(T > 0 && (offsets.numel() - 1) / T > 0); // embedding_forward_quantized_cpu_template.cpp:537
+  Tensor dense = at::empty_like(indices);
+  const int rc = fbgemm_amd_pruned_hashmap_lookup(
+      indices.data_ptr(), offsets.data_ptr(), indices.scalar_type() == at::kLong ? 64 : 32, offsets.numel(),
+      hash_table.data_ptr(), hash_table.scalar_type() == at::kLong ? 64 : 32, hto.data_ptr<int64_t>(), (int32_t)T,
+      dense.data_ptr(), current_stream(indices));
+  TORCH_CHECK(rc == 0, "fbgemm_amd: ", fbgemm_amd_last_error());
+  return dense;
+}
+
+// Row-wise quantizers (fbgemm_gpu/src/quantize_ops/quantize_ops_cpu.cpp:44-330):
+// shapes and checks as the CPU operators have them.
+Tensor quantize_rows(const Tensor& input, int64_t bit_rate, bool sb_float) {
+  TORCH_CHECK(input.is_cuda(), "fbgemm_amd: tensors must be on the GPU");
+  TORCH_CHECK(input.dim() >= 2, "Tensor 'input' must have >= 2 dimension(s). Found ", input.dim());
+  TORCH_CHECK(input.scalar_type() == at::kFloat || input.scalar_type() == at::kHalf, "input must be float or half");
+  const Tensor in = input.contiguous();
+  const int64_t ncols = in.size(-1);
+  const int64_t nrows = ncols ? in.numel() / ncols : 0;
+  const int64_t epb = 8 / bit_rate;
+  const int64_t out_cols = (ncols + epb - 1) / epb + (sb_float ? 8 : 4);
+  auto dims = in.sizes().vec();
+  dims.back() = out_cols;
+  Tensor out = at::empty(dims, in.options().dtype(at::kByte));
+  if (nrows == 0 || ncols == 0) return out;
+  const int rc = fbgemm_amd_quantize_rowwise(
+      in.data_ptr(), in.scalar_type() == at::kHalf ? FBGEMM_AMD_FP16 : FBGEMM_AMD_FP32, nrows, (int32_t)ncols,
+      (int32_t)bit_rate, sb_float ? 1 : 0, FBGEMM_AMD_QLAYOUT_TRAILER, out_cols, out.data_ptr(), current_stream(in));
+  TORCH_CHECK(rc == 0, "fbgemm_amd: ", fbgemm_amd_last_error());
+  return out;
+}
+
+Tensor dequantize_rows(const Tensor& input, int64_t bit_rate, bool sb_float, bool scale_bias_last, int64_t output_dtype) {
+  TORCH_CHECK(input.is_cuda(), "fbgemm_amd: tensors must be on the GPU");
+  TORCH_CHECK(input.dim() >= 2, "Tensor 'input' must have >= 2 dimension(s). Found ", input.dim());
+  TORCH_CHECK(input.scalar_type() == at::kByte, "input must be uint8");
+  const Tensor in = input.contiguous();
+  const int64_t in_cols = in.size(-1);
+  const int64_t nrows = in_cols ? in.numel() / in_cols : 0;
+  // the column count follows from the bytes of a row (src/QuantUtils.cc:758-760, :855-856)
+  const int64_t cols = (in_cols - (sb_float ? 8 : 4)) * (8 / bit_rate);
+  TORCH_CHECK(cols >= 0, "rows are shorter than their scale and bias");
+  auto dims = in.sizes().vec();
+  dims.back() = cols;
+  Tensor out = at::empty(dims, in.options().dtype(out_scalar_type(output_dtype)));
+  if (nrows == 0 || cols == 0) return out;
+  const int rc = fbgemm_amd_dequantize_rowwise(
+      in.data_ptr(), nrows, in_cols, (int32_t)cols, (int32_t)bit_rate, sb_float ? 1 : 0,
+      scale_bias_last ? FBGEMM_AMD_QLAYOUT_TRAILER : FBGEMM_AMD_QLAYOUT_TBE, (int32_t)output_dtype, out.data_ptr(),
+      current_stream(in));
+  TORCH_CHECK(rc == 0, "fbgemm_amd: ", fbgemm_amd_last_error());
+  return out;
+}
+
+Tensor float_to_fused8bit(const Tensor& t) { return quantize_rows(t, 8, true); }
+Tensor fused8bit_to_float(const Tensor& t) { return dequantize_rows(t, 8, true, true, FBGEMM_AMD_FP32); }
+Tensor fused8bit_to_half(const Tensor& t) { return dequantize_rows(t, 8, true, true, FBGEMM_AMD_FP16); }
+Tensor fused8bit_to_bfloat16(const Tensor& t) { return dequantize_rows(t, 8, true, true, FBGEMM_AMD_BF16); }
+Tensor fused8bit_to_float_or_half(const Tensor& t, int64_t output_dtype, bool scale_bias_last, bool quant_padding_float_type) {
+  TORCH_CHECK(quant_padding_float_type || !scale_bias_last,
+              "2-byte padding (quant_padding_float_type=false) only works with scale_bias_last=false");
+  TORCH_CHECK(quant_padding_float_type == scale_bias_last,
+              "fbgemm_amd: rows are (data, fp32 scale, fp32 bias) or (fp16 scale, fp16 bias, data)");
+  return dequantize_rows(t, 8, quant_padding_float_type, scale_bias_last, output_dtype);
+}
+Tensor float_to_fusednbit(const Tensor& t, int64_t bit_rate) {
+  TORCH_CHECK(t.dim() == 2, "Tensor 'input' must have 2 dimension(s). Found ", t.dim());
+  TORCH_CHECK(bit_rate == 2 || bit_rate == 4 || bit_rate == 8, "bit_rate must be 2, 4 or 8");
+  TORCH_CHECK(t.size(1) % (2 * (8 / bit_rate)) == 0,
+              "ncols needs to be multiple of 2 Bytes (half type size) to make the address aligned");
+  return quantize_rows(t, bit_rate, false);
+}
+Tensor fusednbit_to_float(const Tensor& t, int64_t bit_rate) { return dequantize_rows(t, bit_rate, false, true, FBGEMM_AMD_FP32); }
+Tensor fusednbit_to_half(const Tensor& t, int64_t bit_rate) { return dequantize_rows(t, bit_rate, false, true, FBGEMM_AMD_FP16); }
+Tensor fusednbit_to_float_or_half(const Tensor& t, int64_t bit_rate, int64_t output_dtype, bool scale_bias_last) {
+  return dequantize_rows(t, bit_rate, false, scale_bias_last, output_dtype);
+}
+Tensor fusednbit_sbfront_to_float_or_half(const Tensor& t, int64_t bit_rate, int64_t output_dtype) {
+  return dequantize_rows(t, bit_rate, false, false, output_dtype);
+}
+
 } // namespace
 
 // The schema strings are the reference's, character for character. When a real
@@ -167,6 +299,67 @@ TORCH_LIBRARY_FRAGMENT(fbgemm, m) {
   m.impl("int_nbit_split_embedding_codegen_lookup_function",
          torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(int_nbit_split_embedding_codegen_lookup_function_hip)));
   m.impl("pruned_array_lookup", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(pruned_array_lookup_hip)));
+#ifndef FBGEMM_AMD_IMPL_ONLY
+  // embedding_forward_quantized_host_cpu.cpp:338-341
+  m.def(
+      "pruned_hashmap_lookup(Tensor indices, Tensor offsets, Tensor hash_table, Tensor hash_table_offsets) -> Tensor");
+  // fbgemm_gpu/codegen/utils/embedding_bounds_check_host_cpu.cpp:255-270
+  m.def(
+      "bounds_check_indices("
+      "    Tensor rows_per_table, "
+      "    Tensor(a!) indices, "
+      "    Tensor(b!) offsets, "
+      "    int bounds_check_mode, "
+      "    Tensor(c!) warning, "
+      "    Tensor(d!)? weights=None, "
+      "    Tensor? B_offsets=None, "
+      "    SymInt max_B=-1, "
+      "    Tensor? b_t_map=None, "
+      "    int info_B_num_bits=-1, "
+      "    int info_B_mask=-1, "
+      "    int bounds_check_version=1, "
+      "    bool prefetch_pipeline=False"
+      ") -> ()");
+  // fbgemm_gpu/src/quantize_ops/quantize_ops_cpu.cpp:632-666
+  m.def("FloatToFused8BitRowwiseQuantized(Tensor t) -> Tensor");
+  m.def("HalfToFused8BitRowwiseQuantized(Tensor t) -> Tensor");
+  m.def("FloatOrHalfToFused8BitRowwiseQuantized(Tensor t) -> Tensor");
+  m.def("Fused8BitRowwiseQuantizedToFloat(Tensor input) -> Tensor");
+  m.def("Fused8BitRowwiseQuantizedToHalf(Tensor input) -> Tensor");
+  m.def("Fused8BitRowwiseQuantizedToBfloat16(Tensor input) -> Tensor");
+  m.def(
+      "Fused8BitRowwiseQuantizedToFloatOrHalf(Tensor input, int output_dtype=0, bool scale_bias_last=True, bool quant_padding_float_type=True) -> Tensor");
+  m.def(
+      "FloatToFusedNBitRowwiseQuantizedSBHalf(Tensor input, int bit_rate) -> Tensor");
+  m.def(
+      "HalfToFusedNBitRowwiseQuantizedSBHalf(Tensor input, int bit_rate) -> Tensor");
+  m.def(
+      "FloatOrHalfToFusedNBitRowwiseQuantizedSBHalf(Tensor input, int bit_rate) -> Tensor");
+  m.def(
+      "FusedNBitRowwiseQuantizedSBHalfToFloat(Tensor input, int bit_rate) -> Tensor");
+  m.def(
+      "FusedNBitRowwiseQuantizedSBHalfFrontToFloatOrHalf(Tensor input, int bit_rate, int output_dtype) -> Tensor");
+  m.def(
+      "FusedNBitRowwiseQuantizedSBHalfToHalf(Tensor input, int bit_rate) -> Tensor");
+  m.def(
+      "FusedNBitRowwiseQuantizedSBHalfToFloatOrHalf(Tensor input, int bit_rate, int output_dtype=0, bool scale_bias_last=True) -> Tensor");
+#endif
+  m.impl("pruned_hashmap_lookup", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(pruned_hashmap_lookup_hip)));
+  m.impl("bounds_check_indices", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(bounds_check_indices_hip)));
+  m.impl("FloatToFused8BitRowwiseQuantized", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(float_to_fused8bit)));
+  m.impl("HalfToFused8BitRowwiseQuantized", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(float_to_fused8bit)));
+  m.impl("FloatOrHalfToFused8BitRowwiseQuantized", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(float_to_fused8bit)));
+  m.impl("Fused8BitRowwiseQuantizedToFloat", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(fused8bit_to_float)));
+  m.impl("Fused8BitRowwiseQuantizedToHalf", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(fused8bit_to_half)));
+  m.impl("Fused8BitRowwiseQuantizedToBfloat16", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(fused8bit_to_bfloat16)));
+  m.impl("Fused8BitRowwiseQuantizedToFloatOrHalf", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(fused8bit_to_float_or_half)));
+  m.impl("FloatToFusedNBitRowwiseQuantizedSBHalf", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(float_to_fusednbit)));
+  m.impl("HalfToFusedNBitRowwiseQuantizedSBHalf", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(float_to_fusednbit)));
+  m.impl("FloatOrHalfToFusedNBitRowwiseQuantizedSBHalf", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(float_to_fusednbit)));
+  m.impl("FusedNBitRowwiseQuantizedSBHalfToFloat", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(fusednbit_to_float)));
+  m.impl("FusedNBitRowwiseQuantizedSBHalfToHalf", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(fusednbit_to_half)));
+  m.impl("FusedNBitRowwiseQuantizedSBHalfToFloatOrHalf", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(fusednbit_to_float_or_half)));
+  m.impl("FusedNBitRowwiseQuantizedSBHalfFrontToFloatOrHalf", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(fusednbit_sbfront_to_float_or_half)));
 }
 
 TORCH_LIBRARY_FRAGMENT(fbgemm_amd, m) {

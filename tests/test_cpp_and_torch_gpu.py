@@ -99,3 +99,62 @@ def test_torch_pruned_array_lookup(torch_ops, oracle):
     idx = np.concatenate([rng.integers(0, caps[t] or 99, size=int(lens[t * B:(t + 1) * B].sum())) for t in range(T)]).astype(np.int64)
     got = torch_ops.pruned_array_lookup(cu(idx), cu(off), cu(remap), cu(ro)).cpu().numpy()
     assert (got == oracle.pruned_array_lookup(idx, off, remap, ro)).all()
+
+
+def test_torch_bounds_check_and_hashmap(torch_ops, oracle):
+    rng = np.random.default_rng(6)
+    T, B = 5, 21
+    rows = rng.integers(1, 500, size=T).astype(np.int64)
+    lens = rng.integers(0, 9, size=T * B)
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    idx = rng.integers(-2, 600, size=int(off[-1])).astype(np.int64)
+    off[7] = off[6] - 1 if off[6] > 0 else off[7]
+    off[-1] += 3
+    for mode in (1, 2):
+        d_idx, d_off = cu(idx), cu(off)
+        warning = torch.full((1,), 5, dtype=torch.int64, device="cuda")
+        torch_ops.bounds_check_indices(cu(rows), d_idx, d_off, mode, warning)
+        o_idx, o_off, o_warn = idx.copy(), off.copy(), np.full(1, 5, np.int64)
+        assert oracle.bounds_check_indices(rows, o_idx, o_off, mode, o_warn) == 0
+        assert (d_idx.cpu().numpy() == o_idx).all() and (d_off.cpu().numpy() == o_off).all()
+        assert int(warning.item()) == int(o_warn[0])
+    with pytest.raises(RuntimeError):
+        torch_ops.bounds_check_indices(cu(rows), cu(idx), cu(off), 0, torch.zeros(1, dtype=torch.int64, device="cuda"))
+    # hash map
+    keys = rng.choice(3000, size=200, replace=False).astype(np.int64)
+    hto = np.asarray([0, 401], np.int64)
+    table = np.full((401, 2), -1, np.int64)
+    oracle.pruned_hashmap_insert(keys, np.arange(200, dtype=np.int64), np.asarray([0, 200], np.int64), table, hto)
+    q = rng.integers(0, 3000, size=300).astype(np.int64)
+    qoff = np.asarray([0, 100, 300], np.int64)
+    got = torch_ops.pruned_hashmap_lookup(cu(q), cu(qoff), cu(table), cu(hto)).cpu().numpy()
+    assert (got == oracle.pruned_hashmap_lookup(q, qoff, table, hto)).all()
+
+
+def test_torch_rowwise_quantize_ops(torch_ops, oracle):
+    rng = np.random.default_rng(7)
+    x = rng.normal(0, 1, size=(37, 128)).astype(np.float32)
+    # 8-bit, fp32 scale/bias trailer
+    q8 = torch_ops.FloatToFused8BitRowwiseQuantized(cu(x))
+    want8 = oracle.quantize_rowwise(x, 8, True)
+    assert tuple(q8.shape) == (37, 136) and (q8.cpu().numpy() == want8).all()
+    qh = torch_ops.FloatOrHalfToFused8BitRowwiseQuantized(cu(x.astype(np.float16)))
+    assert (qh.cpu().numpy() == oracle.quantize_rowwise(x.astype(np.float16), 8, True)).all()
+    back = torch_ops.Fused8BitRowwiseQuantizedToFloat(q8)
+    assert (back.cpu().numpy().view(np.uint32) == oracle.dequantize_rowwise(want8, 128, 8, True).view(np.uint32)).all()
+    back16 = torch_ops.Fused8BitRowwiseQuantizedToHalf(q8)
+    assert (back16.cpu().view(torch.int16).numpy().view(np.uint16) ==
+            oracle.dequantize_rowwise(want8, 128, 8, True, out_ty=oracle.ST_FP16)).all()
+    # 4- and 2-bit, fp16 scale/bias
+    for bit_rate in (4, 2):
+        qn = torch_ops.FloatToFusedNBitRowwiseQuantizedSBHalf(cu(x), bit_rate)
+        wantn = oracle.quantize_rowwise(x, bit_rate)
+        assert (qn.cpu().numpy() == wantn).all()
+        for out_ty, tdt in ((oracle.ST_FP32, torch.float32), (oracle.ST_FP16, torch.float16), (oracle.ST_BF16, torch.bfloat16)):
+            got = torch_ops.FusedNBitRowwiseQuantizedSBHalfToFloatOrHalf(qn, bit_rate, out_ty)
+            assert got.dtype == tdt
+            want = oracle.dequantize_rowwise(wantn, 128, bit_rate, out_ty=out_ty)
+            g = got.cpu().view(torch.int32 if out_ty == oracle.ST_FP32 else torch.int16).numpy()
+            assert (g == want.view(g.dtype)).all()
+    with pytest.raises(RuntimeError):
+        torch_ops.FloatToFusedNBitRowwiseQuantizedSBHalf(cu(x[:, :3]), 4)
