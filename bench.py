@@ -43,6 +43,11 @@ def parse():
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="also run one plain copy of this many MiB (yardstick for hardware byte counters)")
     ap.add_argument("--check", action="store_true", help="verify a sample of the output against the oracle first")
+    ap.add_argument("--op", default="lookup",
+                    choices=["lookup", "quantize", "dequantize", "bounds_check", "pruned_array_lookup",
+                             "pruned_hashmap_lookup"],
+                    help="lookup = the table-batched forward (the metric); the others time one operator beside "
+                         "the path at the shape config 4 / config 3 gives it and print the same kind of line")
     return ap.parse_args()
 
 
@@ -219,12 +224,114 @@ def cpu_baseline_tbe(p, seconds, torch):
     }
 
 
+def side_op(a):
+    """One operator beside the lookup, timed with events on the launch stream.
+
+    Shapes: the index operators see config 4's batch (32 tables x 4096 bags,
+    3.6 M int64 indices, 2 M-row mappings); the quantizers see 1 M rows x 128
+    columns (a table of config 2's shape), 4-bit rows in the table-batched layout."""
+    import numpy as np
+    import torch
+
+    from fbgemm_amd import ops
+
+    torch.cuda.set_device(0)
+    rng = np.random.default_rng(4242)
+    cu = lambda x: torch.from_numpy(np.ascontiguousarray(x)).cuda()
+    cpu = None
+    if a.op in ("quantize", "dequantize"):
+        rows, cols = int((1 << 20) * a.scale), 128
+        x = torch.randn(rows, cols, device="cuda", dtype=torch.float32)
+        stride = ops.padded_row_size_in_bytes(cols, ops.INT4, 16)
+        q = torch.zeros(rows, stride, dtype=torch.uint8, device="cuda")
+        ops.quantize_rowwise(x, 4, False, ops.QLAYOUT_TBE, out=q)
+        row_bytes = cols * 4 + cols // 2 + 4
+        if a.op == "quantize":
+            launch = lambda: ops.quantize_rowwise(x, 4, False, ops.QLAYOUT_TBE, out=q)
+            kernel, workload = "quantize_rowwise_kernel", f"fp32 [{rows}, {cols}] -> 4-bit rows, fp16 scale/bias first"
+        else:
+            launch = lambda: ops.dequantize_rowwise(q, cols, 4, False, ops.QLAYOUT_TBE, torch.float32)
+            kernel, workload = "dequantize_rowwise_kernel", f"4-bit rows, fp16 scale/bias first [{rows}, {cols}] -> fp32"
+        alg_bytes, units = rows * row_bytes, rows
+
+        def cpu():  # the oracle's scalar restatement on a sample, one core
+            import oracle
+            n = min(rows, 200_000)
+            xs = x[:n].cpu().numpy()
+            qs = q[:n].cpu().numpy()
+            t0 = time.perf_counter()
+            if a.op == "quantize":
+                oracle.quantize_rowwise(xs, 4, False, oracle.LAYOUT_TBE, out_stride=stride)
+            else:
+                oracle.dequantize_rowwise(qs, cols, 4, False, oracle.LAYOUT_TBE)
+            dt = time.perf_counter() - t0
+            return {"value": round(n * row_bytes / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+                    "sample": f"first {n} rows, one pass"}
+    else:
+        T, B = 32, max(1, int(4096 * a.scale))
+        E = max(1000, int(2_000_000 * a.scale))
+        lens = rng.integers(5, 51, size=T * B)
+        off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+        n = int(off[-1])
+        idx = rng.integers(0, E, size=n).astype(np.int64)
+        d_idx, d_off = cu(idx), cu(off)
+        units = n
+        if a.op == "bounds_check":
+            rows_per_table = cu(np.full(T, E, np.int64))
+            warning = torch.zeros(1, dtype=torch.int64, device="cuda")
+            launch = lambda: ops.bounds_check_indices(rows_per_table, d_idx, d_off, ops.BOUNDS_WARNING, warning)
+            alg_bytes = 8 * n + 8 * (T * B + 1)
+            kernel, workload = "bounds_check_bags_kernel", f"WARNING mode, {T} tables x {B} bags, {n} int64 indices in range"
+        elif a.op == "pruned_array_lookup":
+            remap = cu(np.where(rng.random(T * E) < 0.5, -1, 1).astype(np.int32))
+            ro = cu(np.arange(T + 1, dtype=np.int64) * E)
+            launch = lambda: ops.pruned_array_lookup(d_idx, d_off, remap, ro)
+            alg_bytes = 8 * n + 4 * n + 8 * n
+            kernel, workload = "pruned_array_lookup_kernel", f"{T} mappings x {E} int32 entries, {n} int64 indices"
+        else:
+            import oracle  # building the map is set-up (the reference builds it on the CPU as well)
+            cap = int(E * 0.5 / 0.6) + 1
+            hto = np.arange(T + 1, dtype=np.int64) * cap
+            table = np.full((T * cap, 2), -1, np.int64)
+            keys = np.concatenate([rng.choice(E, size=E // 2, replace=False) for _ in range(T)]).astype(np.int64)
+            dense = np.concatenate([np.arange(E // 2) for _ in range(T)]).astype(np.int64)
+            oracle.pruned_hashmap_insert(keys, dense, (np.arange(T + 1) * (E // 2)).astype(np.int64), table, hto)
+            d_table, d_hto = cu(table), cu(hto)
+            launch = lambda: ops.pruned_hashmap_lookup(d_idx, d_off, d_table, d_hto)
+            alg_bytes = 8 * n + 16 * n + 8 * n
+            kernel, workload = "pruned_hashmap_lookup_kernel", f"{T} maps x {cap} slots (load 0.6), {n} int64 indices"
+    for _ in range(a.warmup):
+        launch()
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record()
+    for _ in range(a.steps):
+        launch()
+    ev1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / a.steps
+    ms = ev0.elapsed_time(ev1) / a.steps
+    gbps = alg_bytes / (ms * 1e-3) / 1e9
+    res = {"metric": f"achieved HBM GB/s, {a.op} on 1 MI355X", "value": round(gbps, 2), "unit": "GB/s", "n_gpus": 1,
+           "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(wall_ms, 5), "higher_is_better": True,
+           "scaling": "weak", "vs_baseline": None, "dtype": "f32" if "quant" in a.op else "int64", "data": "synthetic",
+           "config": {"workload": workload, "units_per_step": units},
+           "roofline": {"bound": "hbm", "achieved": round(gbps, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                        "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None, "kernel": kernel,
+                        "kernel_ms": round(ms, 5), "algorithmic_bytes_per_launch": alg_bytes},
+           "cpu_baseline": cpu() if (cpu is not None and not a.no_cpu) else None}
+    print(json.dumps(res))
+
+
 def main():
     a = parse()
     if a.gpus != 1:
         print("bench.py: this path is measured on ONE GPU (no sharding, no collectives); "
               f"--gpus {a.gpus} is not supported", file=sys.stderr)
         sys.exit(2)
+    if a.op != "lookup":
+        return side_op(a)
     import numpy as np
     import torch
 

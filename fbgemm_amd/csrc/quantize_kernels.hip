@@ -17,7 +17,11 @@
 // std::min_element / std::max_element return them (this decides the sign of a
 // zero bias or scale).
 //
-// One wave per row; a lane owns runs of 8 consecutive elements.
+// `lpr` lanes (a power of two, chosen by the host from the row length) share a
+// row and a lane owns runs of 8 consecutive elements, so a wave works on
+// 64 / lpr rows at once: 16-byte loads, one store per run, and the row's
+// elements stay in registers between the min/max pass and the rounding pass
+// when one run per lane covers the row.
 #include <hip/hip_runtime.h>
 
 #include "lookup_common.h"
@@ -91,33 +95,86 @@ __device__ __forceinline__ Extreme shuffle_xor(Extreme e, int mask) {
   return r;
 }
 
+// stores the nbytes (1, 2, 4 or 8) of one run of quantized elements
+__device__ __forceinline__ void store_run(uint8_t* p, uint64_t v, int nbytes) {
+  const uintptr_t a = reinterpret_cast<uintptr_t>(p);
+  if (nbytes == 8 && (a & 3) == 0) {
+    reinterpret_cast<uint32_t*>(p)[0] = (uint32_t)v;
+    reinterpret_cast<uint32_t*>(p)[1] = (uint32_t)(v >> 32);
+  } else if (nbytes == 4 && (a & 3) == 0) {
+    *reinterpret_cast<uint32_t*>(p) = (uint32_t)v;
+  } else if (nbytes == 2 && (a & 1) == 0) {
+    *reinterpret_cast<uint16_t*>(p) = (uint16_t)v;
+  } else {
+    for (int b = 0; b < nbytes; ++b) p[b] = (uint8_t)(v >> (8 * b));
+  }
+}
+
 // layout: 0 = data then (scale, bias) trailer; 1 = fp16 (scale, bias) header then data
-template <bool HALF_IN>
+template <bool HALF_IN, int BITS>
 __global__ __launch_bounds__(256) void quantize_rowwise_kernel(
-    const void* input, int64_t rows, int32_t cols, int32_t bits, int32_t sb_float, int32_t layout,
-    int64_t out_stride, uint8_t* output) {
+    const void* input, int64_t rows, int32_t cols, int32_t sb_float, int32_t layout,
+    int64_t out_stride, uint8_t* output, int32_t lpr) {
+  constexpr int bits = BITS;
   const int lane = threadIdx.x & 63;
-  const int64_t row = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-  if (row >= rows) return;
+  const int sub = lane & (lpr - 1);
+  const int rows_per_wave = 64 / lpr;
+  const int64_t nwaves = (int64_t)gridDim.x * (blockDim.x >> 6);
+  const int64_t ngroups = (rows + rows_per_wave - 1) / rows_per_wave;
+  // every wave walks row groups wave, wave + nwaves, ...: the loop bound is the same for all lanes of a wave
+  for (int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6); wave < ngroups; wave += nwaves) {
+  const int64_t row_raw = wave * rows_per_wave + lane / lpr;
+  const bool live = row_raw < rows;
+  const int64_t row = live ? row_raw : rows - 1; // lanes past the end shadow the last row and store nothing
   const void* in_row = reinterpret_cast<const uint8_t*>(input) + row * (int64_t)cols * (HALF_IN ? 2 : 4);
   uint8_t* out_row = output + row * out_stride;
+  const bool single = cols <= lpr * RUN; // one run per lane covers the row
 
-  Extreme mn{0.0f, 0x7fffffff}, mx{0.0f, 0x7fffffff};
-  for (int j0 = lane * RUN; j0 < cols; j0 += 64 * RUN) {
+  // Fast pass: plain minimum / maximum. Which of several equal extremes is
+  // taken only shows when the extreme is a zero and zeros of both signs are in
+  // the row (the sign of the stored bias / of max - min); a wave that meets a
+  // zero extreme redoes the search with positions (the first extreme wins, as
+  // std::min_element / std::max_element choose).
+  float lo = __builtin_inff(), hi = -__builtin_inff();
+  float keep[RUN];
+  int keep_n = 0;
+  for (int j0 = sub * RUN; j0 < cols; j0 += lpr * RUN) {
     float x[RUN];
     const int n = load_run<HALF_IN>(in_row, j0, cols, x);
     for (int k = 0; k < RUN; ++k) {
+      keep[k] = x[k];
       if (k < n) {
-        const Extreme e{x[k], j0 + k};
-        mn = mn.idx == 0x7fffffff ? e : first_min(mn, e);
-        mx = mx.idx == 0x7fffffff ? e : first_max(mx, e);
+        lo = x[k] < lo ? x[k] : lo;
+        hi = hi < x[k] ? x[k] : hi;
       }
     }
+    keep_n = n;
   }
-  for (int m = 1; m < 64; m <<= 1) {
-    const Extreme on = shuffle_xor(mn, m), ox = shuffle_xor(mx, m);
-    if (on.idx != 0x7fffffff) mn = mn.idx == 0x7fffffff ? on : first_min(mn, on);
-    if (ox.idx != 0x7fffffff) mx = mx.idx == 0x7fffffff ? ox : first_max(mx, ox);
+  for (int m = 1; m < lpr; m <<= 1) {
+    const float ol = __shfl_xor(lo, m, 64), oh = __shfl_xor(hi, m, 64);
+    lo = ol < lo ? ol : lo;
+    hi = hi < oh ? oh : hi;
+  }
+  Extreme mn{lo, 0}, mx{hi, 0};
+  if (__builtin_amdgcn_ballot_w64(lo == 0.0f || hi == 0.0f) != 0ull) {
+    mn = Extreme{0.0f, 0x7fffffff};
+    mx = Extreme{0.0f, 0x7fffffff};
+    for (int j0 = sub * RUN; j0 < cols; j0 += lpr * RUN) {
+      float x[RUN];
+      const int n = load_run<HALF_IN>(in_row, j0, cols, x);
+      for (int k = 0; k < RUN; ++k) {
+        if (k < n) {
+          const Extreme e{x[k], j0 + k};
+          mn = mn.idx == 0x7fffffff ? e : first_min(mn, e);
+          mx = mx.idx == 0x7fffffff ? e : first_max(mx, e);
+        }
+      }
+    }
+    for (int m = 1; m < lpr; m <<= 1) {
+      const Extreme on = shuffle_xor(mn, m), ox = shuffle_xor(mx, m);
+      if (on.idx != 0x7fffffff) mn = mn.idx == 0x7fffffff ? on : first_min(mn, on);
+      if (ox.idx != 0x7fffffff) mx = mx.idx == 0x7fffffff ? ox : first_max(mx, ox);
+    }
   }
   float minimum = mn.v;
   const float maximum = mx.v;
@@ -162,47 +219,51 @@ __global__ __launch_bounds__(256) void quantize_rowwise_kernel(
   }
   uint8_t* data = layout == 1 ? out_row + 4 : out_row;
   uint8_t* sb = layout == 1 ? out_row : out_row + data_bytes;
-  if (lane == 0) {
-    if (sb_bytes == 8) {
-      for (int i = 0; i < 4; ++i) sb[i] = (uint8_t)(sb0 >> (8 * i));
-      for (int i = 0; i < 4; ++i) sb[4 + i] = (uint8_t)(sb1 >> (8 * i));
-    } else {
-      sb[0] = (uint8_t)sb0; sb[1] = (uint8_t)(sb0 >> 8);
-      sb[2] = (uint8_t)sb1; sb[3] = (uint8_t)(sb1 >> 8);
-    }
+  if (live && sub == 0) {
+    if (sb_bytes == 8) store_run(sb, (uint64_t)sb0 | ((uint64_t)sb1 << 32), 8);
+    else store_run(sb, (uint64_t)(sb0 & 0xffffu) | ((uint64_t)(sb1 & 0xffffu) << 16), 4);
   }
-  for (int j0 = lane * RUN; j0 < cols; j0 += 64 * RUN) {
-    uint32_t q[RUN];
+  const int run_bytes = RUN / epb;
+  for (int j0 = sub * RUN; j0 < cols; j0 += lpr * RUN) {
     float xs[RUN];
-    const int n = load_run<HALF_IN>(in_row, j0, cols, xs);
+    int n;
+    if (single) {
+      for (int k = 0; k < RUN; ++k) xs[k] = keep[k];
+      n = keep_n;
+    } else {
+      n = load_run<HALF_IN>(in_row, j0, cols, xs);
+    }
+    uint32_t w0 = 0, w1 = 0; // the run's bytes: RUN * bits <= 32 bits fill w0; 8-bit runs use both
     for (int k = 0; k < RUN; ++k) {
-      q[k] = 0;
       if (k < n) {
-        const float x = xs[k];
-        float r = __builtin_rintf((x - minimum) * inverse_scale); // lrintf: to nearest, ties to even
+        float r = __builtin_rintf((xs[k] - minimum) * inverse_scale); // lrintf: to nearest, ties to even
         if (clamp) r = r < 0.0f ? 0.0f : (r > (float)maxq ? (float)maxq : r);
-        q[k] = (uint32_t)(int)r & 0xffu;
+        const uint32_t q = (uint32_t)(int)r & 0xffu;
+        if (bits == 8 && k >= 4) w1 |= q << ((k - 4) * 8);
+        else w0 |= q << (k * bits);
       }
     }
+    const uint64_t packed = (uint64_t)w0 | ((uint64_t)w1 << 32);
     // RUN elements = RUN * bits / 8 bytes, starting at a whole byte
     const int first_byte = j0 / epb;
-    const int nbytes = RUN / epb;
-    for (int b = 0; b < nbytes; ++b) {
-      if (first_byte + b < data_bytes) {
-        uint32_t byte = 0;
-        for (int k = 0; k < epb; ++k) byte |= q[b * epb + k] << (k * bits);
-        data[first_byte + b] = (uint8_t)byte;
-      }
-    }
+    const int nb = data_bytes - first_byte < run_bytes ? data_bytes - first_byte : run_bytes;
+    if (live) store_run(data + first_byte, packed, nb);
+  }
   }
 }
 
-// output_ty: ST_FP32, ST_FP16, ST_BF16
+// output_ty: ST_FP32, ST_FP16, ST_BF16. `lpr` lanes share a row; a lane turns
+// runs of 8 packed elements into 8 outputs.
+template <int BITS>
 __global__ __launch_bounds__(256) void dequantize_rowwise_kernel(
-    const uint8_t* input, int64_t rows, int64_t in_stride, int32_t cols, int32_t bits, int32_t sb_float,
-    int32_t layout, int32_t output_ty, void* output) {
+    const uint8_t* input, int64_t rows, int64_t in_stride, int32_t cols, int32_t sb_float,
+    int32_t layout, int32_t output_ty, void* output, int32_t lpr) {
+  constexpr int bits = BITS;
   const int lane = threadIdx.x & 63;
-  const int64_t row = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int sub = lane & (lpr - 1);
+  const int64_t nwaves = (int64_t)gridDim.x * (blockDim.x >> 6);
+  for (int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);; wave += nwaves) {
+  const int64_t row = wave * (64 / lpr) + lane / lpr;
   if (row >= rows) return;
   const uint8_t* in_row = input + row * in_stride;
   const int epb = 8 / bits;
@@ -212,25 +273,76 @@ __global__ __launch_bounds__(256) void dequantize_rowwise_kernel(
   float scale, bias;
   if (sb_float) {
     uint32_t u0 = 0, u1 = 0;
-    for (int i = 0; i < 4; ++i) {
-      u0 |= (uint32_t)sb[i] << (8 * i);
-      u1 |= (uint32_t)sb[4 + i] << (8 * i);
+    if ((reinterpret_cast<uintptr_t>(sb) & 3) == 0) {
+      u0 = reinterpret_cast<const uint32_t*>(sb)[0];
+      u1 = reinterpret_cast<const uint32_t*>(sb)[1];
+    } else {
+      for (int i = 0; i < 4; ++i) {
+        u0 |= (uint32_t)sb[i] << (8 * i);
+        u1 |= (uint32_t)sb[4 + i] << (8 * i);
+      }
     }
     scale = q_bits_to_float(u0);
     bias = q_bits_to_float(u1);
   } else {
-    scale = half_bits_to_float((uint16_t)(sb[0] | (sb[1] << 8)));
-    bias = half_bits_to_float((uint16_t)(sb[2] | (sb[3] << 8)));
+    uint32_t u;
+    if ((reinterpret_cast<uintptr_t>(sb) & 3) == 0) u = *reinterpret_cast<const uint32_t*>(sb);
+    else u = sb[0] | (sb[1] << 8) | (sb[2] << 16) | ((uint32_t)sb[3] << 24);
+    scale = half_bits_to_float((uint16_t)u);
+    bias = half_bits_to_float((uint16_t)(u >> 16));
   }
   const uint32_t mask = (1u << bits) - 1;
-  for (int j = lane; j < cols; j += 64) {
-    const uint32_t q = ((uint32_t)data[j / epb] >> ((j % epb) * bits)) & mask;
-    const float v = (float)((double)scale * (double)q + (double)bias);
-    const int64_t o = row * (int64_t)cols + j;
-    if (output_ty == ST_FP32) reinterpret_cast<float*>(output)[o] = v;
-    else if (output_ty == ST_FP16) reinterpret_cast<uint16_t*>(output)[o] = float_to_half_bits(v);
-    else reinterpret_cast<uint16_t*>(output)[o] = float_to_bf16_bits(v);
+  const int run_bytes = RUN / epb; // 8, 4 or 2
+  for (int j0 = sub * RUN; j0 < cols; j0 += lpr * RUN) {
+    const uint8_t* p = data + j0 / epb;
+    const int nb = data_bytes - j0 / epb < run_bytes ? data_bytes - j0 / epb : run_bytes;
+    uint64_t packed = 0;
+    const uintptr_t pa = reinterpret_cast<uintptr_t>(p);
+    if (nb == 8 && (pa & 3) == 0) packed = (uint64_t) reinterpret_cast<const uint32_t*>(p)[0] | ((uint64_t) reinterpret_cast<const uint32_t*>(p)[1] << 32);
+    else if (nb == 4 && (pa & 3) == 0) packed = *reinterpret_cast<const uint32_t*>(p);
+    else if (nb == 2 && (pa & 1) == 0) packed = *reinterpret_cast<const uint16_t*>(p);
+    else for (int b = 0; b < nb; ++b) packed |= (uint64_t)p[b] << (8 * b);
+    float v[RUN];
+    for (int k = 0; k < RUN; ++k) {
+      const uint32_t q = (uint32_t)(packed >> (k * bits)) & mask;
+      v[k] = (float)((double)scale * (double)q + (double)bias);
+    }
+    const int n = cols - j0 < RUN ? cols - j0 : RUN;
+    const int64_t o = row * (int64_t)cols + j0;
+    if (output_ty == ST_FP32) {
+      float* op = reinterpret_cast<float*>(output) + o;
+      if (n == RUN && (reinterpret_cast<uintptr_t>(op) & 15) == 0) {
+        reinterpret_cast<float4*>(op)[0] = make_float4(v[0], v[1], v[2], v[3]);
+        reinterpret_cast<float4*>(op)[1] = make_float4(v[4], v[5], v[6], v[7]);
+      } else {
+        for (int k = 0; k < RUN; ++k) if (k < n) op[k] = v[k];
+      }
+    } else {
+      uint16_t h[RUN];
+      for (int k = 0; k < RUN; ++k) h[k] = output_ty == ST_FP16 ? float_to_half_bits(v[k]) : float_to_bf16_bits(v[k]);
+      uint16_t* op = reinterpret_cast<uint16_t*>(output) + o;
+      if (n == RUN && (reinterpret_cast<uintptr_t>(op) & 15) == 0) {
+        *reinterpret_cast<uint4*>(op) = make_uint4(h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16),
+                                                   h[4] | ((uint32_t)h[5] << 16), h[6] | ((uint32_t)h[7] << 16));
+      } else {
+        for (int k = 0; k < RUN; ++k) if (k < n) op[k] = h[k];
+      }
+    }
   }
+  }
+}
+
+// enough workgroups to fill the device several times over, no more than there is work
+unsigned stream_blocks(int64_t needed) {
+  const int64_t cap = 256 * 64;
+  return (unsigned)(needed < cap ? (needed < 1 ? 1 : needed) : cap);
+}
+
+// lanes per row: the power of two (1..64) that gives a lane about one run
+int lanes_per_row(int32_t cols) {
+  int lpr = 1;
+  while (lpr < 64 && lpr * RUN < cols) lpr <<= 1;
+  return lpr;
 }
 
 } // namespace
@@ -239,14 +351,23 @@ hipError_t launch_quantize_rowwise(const void* input, bool half_in, int64_t rows
                                    int32_t sb_float, int32_t layout, int64_t out_stride, void* output,
                                    hipStream_t stream) {
   if (rows <= 0 || cols <= 0) return hipSuccess;
-  const int64_t blocks = (rows + 3) / 4;
-  if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
-  if (half_in)
-    hipLaunchKernelGGL(quantize_rowwise_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, stream, input, rows, cols,
-                       bits, sb_float, layout, out_stride, (uint8_t*)output);
-  else
-    hipLaunchKernelGGL(quantize_rowwise_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, stream, input, rows, cols,
-                       bits, sb_float, layout, out_stride, (uint8_t*)output);
+  const int lpr = lanes_per_row(cols);
+  const int64_t rows_per_block = 4 * (64 / lpr);
+  const int64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
+  const dim3 grid(stream_blocks(blocks)), block(256);
+#define FBGEMM_AMD_LAUNCH_Q(H, B) \
+  hipLaunchKernelGGL((quantize_rowwise_kernel<H, B>), grid, block, 0, stream, input, rows, cols, sb_float, layout, \
+                     out_stride, (uint8_t*)output, lpr)
+  if (half_in) {
+    if (bits == 2) FBGEMM_AMD_LAUNCH_Q(true, 2);
+    else if (bits == 4) FBGEMM_AMD_LAUNCH_Q(true, 4);
+    else FBGEMM_AMD_LAUNCH_Q(true, 8);
+  } else {
+    if (bits == 2) FBGEMM_AMD_LAUNCH_Q(false, 2);
+    else if (bits == 4) FBGEMM_AMD_LAUNCH_Q(false, 4);
+    else FBGEMM_AMD_LAUNCH_Q(false, 8);
+  }
+#undef FBGEMM_AMD_LAUNCH_Q
   return hipGetLastError();
 }
 
@@ -254,10 +375,17 @@ hipError_t launch_dequantize_rowwise(const void* input, int64_t rows, int64_t in
                                      int32_t sb_float, int32_t layout, int32_t output_ty, void* output,
                                      hipStream_t stream) {
   if (rows <= 0 || cols <= 0) return hipSuccess;
-  const int64_t blocks = (rows + 3) / 4;
-  if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
-  hipLaunchKernelGGL(dequantize_rowwise_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (const uint8_t*)input,
-                     rows, in_stride, cols, bits, sb_float, layout, output_ty, output);
+  const int lpr = lanes_per_row(cols);
+  const int64_t rows_per_block = 4 * (64 / lpr);
+  const int64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
+  const dim3 grid(stream_blocks(blocks)), block(256);
+#define FBGEMM_AMD_LAUNCH_D(B) \
+  hipLaunchKernelGGL((dequantize_rowwise_kernel<B>), grid, block, 0, stream, (const uint8_t*)input, rows, in_stride, \
+                     cols, sb_float, layout, output_ty, output, lpr)
+  if (bits == 2) FBGEMM_AMD_LAUNCH_D(2);
+  else if (bits == 4) FBGEMM_AMD_LAUNCH_D(4);
+  else FBGEMM_AMD_LAUNCH_D(8);
+#undef FBGEMM_AMD_LAUNCH_D
   return hipGetLastError();
 }
 
