@@ -253,7 +253,9 @@ __global__ __launch_bounds__(256) void quantize_rowwise_kernel(
 }
 
 // output_ty: ST_FP32, ST_FP16, ST_BF16. `lpr` lanes share a row; a lane turns
-// runs of 8 packed elements into 8 outputs.
+// runs of 4 packed elements into 4 outputs (one 16-byte store of fp32: every
+// store instruction of the wave then writes whole contiguous lines).
+constexpr int DRUN = 4;
 template <int BITS>
 __global__ __launch_bounds__(256) void dequantize_rowwise_kernel(
     const uint8_t* input, int64_t rows, int64_t in_stride, int32_t cols, int32_t sb_float,
@@ -292,40 +294,37 @@ __global__ __launch_bounds__(256) void dequantize_rowwise_kernel(
     bias = half_bits_to_float((uint16_t)(u >> 16));
   }
   const uint32_t mask = (1u << bits) - 1;
-  const int run_bytes = RUN / epb; // 8, 4 or 2
-  for (int j0 = sub * RUN; j0 < cols; j0 += lpr * RUN) {
+  const int run_bytes = DRUN / epb; // 4, 2 or 1
+  for (int j0 = sub * DRUN; j0 < cols; j0 += lpr * DRUN) {
     const uint8_t* p = data + j0 / epb;
     const int nb = data_bytes - j0 / epb < run_bytes ? data_bytes - j0 / epb : run_bytes;
-    uint64_t packed = 0;
+    uint32_t packed = 0;
     const uintptr_t pa = reinterpret_cast<uintptr_t>(p);
-    if (nb == 8 && (pa & 3) == 0) packed = (uint64_t) reinterpret_cast<const uint32_t*>(p)[0] | ((uint64_t) reinterpret_cast<const uint32_t*>(p)[1] << 32);
-    else if (nb == 4 && (pa & 3) == 0) packed = *reinterpret_cast<const uint32_t*>(p);
+    if (nb == 4 && (pa & 3) == 0) packed = *reinterpret_cast<const uint32_t*>(p);
     else if (nb == 2 && (pa & 1) == 0) packed = *reinterpret_cast<const uint16_t*>(p);
-    else for (int b = 0; b < nb; ++b) packed |= (uint64_t)p[b] << (8 * b);
-    float v[RUN];
-    for (int k = 0; k < RUN; ++k) {
-      const uint32_t q = (uint32_t)(packed >> (k * bits)) & mask;
+    else for (int b = 0; b < nb; ++b) packed |= (uint32_t)p[b] << (8 * b);
+    float v[DRUN];
+    for (int k = 0; k < DRUN; ++k) {
+      const uint32_t q = (packed >> (k * bits)) & mask;
       v[k] = (float)((double)scale * (double)q + (double)bias);
     }
-    const int n = cols - j0 < RUN ? cols - j0 : RUN;
+    const int n = cols - j0 < DRUN ? cols - j0 : DRUN;
     const int64_t o = row * (int64_t)cols + j0;
     if (output_ty == ST_FP32) {
       float* op = reinterpret_cast<float*>(output) + o;
-      if (n == RUN && (reinterpret_cast<uintptr_t>(op) & 15) == 0) {
-        reinterpret_cast<float4*>(op)[0] = make_float4(v[0], v[1], v[2], v[3]);
-        reinterpret_cast<float4*>(op)[1] = make_float4(v[4], v[5], v[6], v[7]);
+      if (n == DRUN && (reinterpret_cast<uintptr_t>(op) & 15) == 0) {
+        *reinterpret_cast<float4*>(op) = make_float4(v[0], v[1], v[2], v[3]);
       } else {
-        for (int k = 0; k < RUN; ++k) if (k < n) op[k] = v[k];
+        for (int k = 0; k < DRUN; ++k) if (k < n) op[k] = v[k];
       }
     } else {
-      uint16_t h[RUN];
-      for (int k = 0; k < RUN; ++k) h[k] = output_ty == ST_FP16 ? float_to_half_bits(v[k]) : float_to_bf16_bits(v[k]);
+      uint16_t h[DRUN];
+      for (int k = 0; k < DRUN; ++k) h[k] = output_ty == ST_FP16 ? float_to_half_bits(v[k]) : float_to_bf16_bits(v[k]);
       uint16_t* op = reinterpret_cast<uint16_t*>(output) + o;
-      if (n == RUN && (reinterpret_cast<uintptr_t>(op) & 15) == 0) {
-        *reinterpret_cast<uint4*>(op) = make_uint4(h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16),
-                                                   h[4] | ((uint32_t)h[5] << 16), h[6] | ((uint32_t)h[7] << 16));
+      if (n == DRUN && (reinterpret_cast<uintptr_t>(op) & 7) == 0) {
+        *reinterpret_cast<uint2*>(op) = make_uint2(h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16));
       } else {
-        for (int k = 0; k < RUN; ++k) if (k < n) op[k] = h[k];
+        for (int k = 0; k < DRUN; ++k) if (k < n) op[k] = h[k];
       }
     }
   }
@@ -339,9 +338,9 @@ unsigned stream_blocks(int64_t needed) {
 }
 
 // lanes per row: the power of two (1..64) that gives a lane about one run
-int lanes_per_row(int32_t cols) {
+int lanes_per_row(int32_t cols, int run) {
   int lpr = 1;
-  while (lpr < 64 && lpr * RUN < cols) lpr <<= 1;
+  while (lpr < 64 && lpr * run < cols) lpr <<= 1;
   return lpr;
 }
 
@@ -351,7 +350,7 @@ hipError_t launch_quantize_rowwise(const void* input, bool half_in, int64_t rows
                                    int32_t sb_float, int32_t layout, int64_t out_stride, void* output,
                                    hipStream_t stream) {
   if (rows <= 0 || cols <= 0) return hipSuccess;
-  const int lpr = lanes_per_row(cols);
+  const int lpr = lanes_per_row(cols, RUN);
   const int64_t rows_per_block = 4 * (64 / lpr);
   const int64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
   const dim3 grid(stream_blocks(blocks)), block(256);
@@ -375,7 +374,7 @@ hipError_t launch_dequantize_rowwise(const void* input, int64_t rows, int64_t in
                                      int32_t sb_float, int32_t layout, int32_t output_ty, void* output,
                                      hipStream_t stream) {
   if (rows <= 0 || cols <= 0) return hipSuccess;
-  const int lpr = lanes_per_row(cols);
+  const int lpr = lanes_per_row(cols, DRUN);
   const int64_t rows_per_block = 4 * (64 / lpr);
   const int64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
   const dim3 grid(stream_blocks(blocks)), block(256);
