@@ -19,6 +19,9 @@ hipError_t launch_lookup(const LookupArgs& a, bool idx64, hipStream_t stream);
 hipError_t launch_lengths_to_offsets(const void* lengths, bool is64, int64_t n, int64_t* offsets, hipStream_t stream);
 hipError_t launch_status_clear(Status* st, hipStream_t stream);
 hipError_t launch_bag_order(const void* offsets, bool off64, int32_t B, int32_t T, BagEntry* order, hipStream_t stream);
+hipError_t launch_sequence_lookup(const TableDesc* tables, const uint8_t* w0, const uint8_t* w1, const void* indices,
+                                  bool idx64, const void* offsets, int32_t B, int32_t T, int64_t total_L, int32_t D,
+                                  int32_t out_ty, void* out, Status* status, hipStream_t stream);
 hipError_t launch_calibration_copy(const void* src, void* dst, int64_t bytes, hipStream_t stream);
 hipError_t launch_bounds_check(const int64_t* rows_per_table, int32_t T, void* indices, void* offsets, bool is64,
                                int64_t num_indices, int64_t total_B, int64_t B, const int32_t* B_offsets, int mode,
@@ -732,6 +735,40 @@ int fbgemm_amd_tbe_forward_pruned(
     }
   }
 #endif
+  return 0;
+}
+
+int fbgemm_amd_tbe_forward_nobag(
+    fbgemm_amd_tbe_plan* plan, const void* d_dev_weights, const void* d_uvm_weights,
+    const void* d_indices, const void* d_offsets, int32_t index_bits,
+    int64_t indices_numel, int64_t offsets_numel, int32_t D, int32_t output_ty,
+    void* d_output, void* d_status, void* stream) {
+  if (!plan) return fail(FBGEMM_AMD_E_ARG, "plan is null");
+  if (index_bits != 32 && index_bits != 64) return fail(FBGEMM_AMD_E_ARG, "index_bits must be 32 or 64");
+  const bool copy_rows = output_ty == ST_INT8 || output_ty == ST_INT4;
+  if (!copy_rows && output_ty != ST_FP32 && output_ty != ST_FP16 && output_ty != ST_BF16)
+    return fail(FBGEMM_AMD_E_UNSUPPORTED, "output type %d is not supported", output_ty);
+  if (!d_status) return fail(FBGEMM_AMD_E_ARG, "d_status is null");
+  if (D <= 0) return fail(FBGEMM_AMD_E_ARG, "D must be positive");
+  if (offsets_numel < 1 || (offsets_numel - 1) % plan->T != 0)
+    return fail(FBGEMM_AMD_E_ARG, "offsets must hold T*B+1 entries");
+  const int64_t B64 = (offsets_numel - 1) / plan->T;
+  if (B64 > 0x7fffffffLL) return fail(FBGEMM_AMD_E_ARG, "B exceeds 2^31-1");
+  if (B64 == 0 || indices_numel == 0) return 0;
+  if (!d_offsets || !d_output || !d_indices) return fail(FBGEMM_AMD_E_ARG, "null data pointer");
+  for (int t = 0; t < plan->T; ++t) {
+    const TableDesc& d = plan->tables[t];
+    if (d.D != D) return fail(FBGEMM_AMD_E_ARG, "table %d has D = %d: without pooling all tables share D = %d", t, d.D, D);
+    // embedding_forward_quantized_cpu_template.cpp:357-359
+    if (copy_rows && d.ty != output_ty)
+      return fail(FBGEMM_AMD_E_ARG, "table %d: int8 / int4 output copies rows and needs weights of the same type", t);
+    const int eb = type_bits(d.ty) / 8;
+    if (eb > 1 && (d.weights_offset % eb || d.row_stride % eb))
+      return fail(FBGEMM_AMD_E_ARG, "table %d: rows are not aligned to their elements", t);
+  }
+  HIP_TRY(launch_sequence_lookup(plan->d_tables, (const uint8_t*)d_dev_weights, (const uint8_t*)d_uvm_weights, d_indices,
+                                 index_bits == 64, d_offsets, (int32_t)B64, plan->T, indices_numel, D, output_ty,
+                                 d_output, (Status*)d_status, (hipStream_t)stream));
   return 0;
 }
 

@@ -1,0 +1,171 @@
+// gfx950 kernel of the table-batched forward without pooling
+// (PoolingMode.NONE, "sequence" output): one output row per index.
+//
+// What the reference's CPU operator does for this mode
+// (fbgemm_gpu/codegen/inference/embedding_forward_quantized_cpu_template.cpp:283-296,390-420):
+// every index is a bag of length one, so row i of the [total_L, D] output is
+//     out[i][j] = convert(fma(1.0f * scale, q[j], 0.0f + 1.0f * bias))     (quantised rows)
+//     out[i][j] = convert(fma(1.0f, x[j], 0.0f))                           (fp16 / fp32 rows)
+// of row indices[i] of the table position i belongs to (the table whose slice
+// of `offsets` holds i); an index of -1 (pruned row) leaves zeros. With an
+// int8 or int4 output type the row's bytes (fp16 scale/bias first, then the
+// elements) are copied as they are (src/RefImplementations.cc:1235-1253,
+// 1466-1484): all tables then hold rows of that type.
+//
+// `lpr` lanes share an output row; a lane turns runs of 4 elements into one
+// store. The table of a position is found by bisection over the T + 1 table
+// boundaries, which the workgroup keeps in LDS.
+#include <hip/hip_runtime.h>
+
+#include "lookup_common.h"
+
+namespace fbgemm_amd {
+
+namespace {
+
+constexpr int SRUN = 4;
+constexpr int MAX_LDS_TABLES = 4096; // boundaries kept in LDS; beyond that they are read from memory
+
+__device__ __forceinline__ float s_bits_to_float(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t s_float_to_bits(float f) { return __builtin_bit_cast(uint32_t, f); }
+__device__ __forceinline__ float s_half_to_float(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
+__device__ __forceinline__ uint16_t s_to_half(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }
+__device__ __forceinline__ uint16_t s_to_bf16(float f) { return (uint16_t)((s_float_to_bits(f) + 0x8000u) >> 16); }
+
+__device__ __forceinline__ int64_t s_read(const void* p, bool is64, int64_t i) {
+  return is64 ? reinterpret_cast<const int64_t*>(p)[i] : (int64_t) reinterpret_cast<const int32_t*>(p)[i];
+}
+
+__device__ __forceinline__ int s_type_bits(int ty) {
+  return ty == ST_FP32 ? 32 : (ty == ST_FP16 || ty == ST_BF16) ? 16 : ty == ST_INT8 ? 8 : ty == ST_INT4 ? 4 : 2;
+}
+
+template <typename index_t>
+__global__ __launch_bounds__(256) void sequence_lookup_kernel(
+    const TableDesc* tables, const uint8_t* w0, const uint8_t* w1, const index_t* indices, const void* offsets,
+    int off64, int32_t B, int32_t T, int64_t total_L, int32_t D, int32_t out_ty, void* out, int32_t lpr,
+    Status* status) {
+  __shared__ int64_t bounds[MAX_LDS_TABLES + 1];
+  const bool in_lds = T <= MAX_LDS_TABLES;
+  if (in_lds) {
+    for (int t = threadIdx.x; t <= T; t += blockDim.x) bounds[t] = s_read(offsets, off64, (int64_t)t * B);
+  }
+  __syncthreads();
+  const int lane = threadIdx.x & 63;
+  const int sub = lane & (lpr - 1);
+  const int per_wave = 64 / lpr;
+  const int64_t nwaves = (int64_t)gridDim.x * (blockDim.x >> 6);
+  const int64_t ngroups = (total_L + per_wave - 1) / per_wave;
+  const bool copy_rows = out_ty == ST_INT8 || out_ty == ST_INT4;
+  // bytes of an output row
+  const int64_t out_row_bytes = out_ty == ST_FP32 ? (int64_t)D * 4 : (out_ty == ST_FP16 || out_ty == ST_BF16) ? (int64_t)D * 2
+      : out_ty == ST_INT8 ? (int64_t)D + 4 : (int64_t)(D + 8 + 1) / 2;
+  for (int64_t g = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6); g < ngroups; g += nwaves) {
+    const int64_t pos = g * per_wave + lane / lpr;
+    if (pos >= total_L) continue;
+    // largest t with bounds[t] <= pos (empty tables share a boundary: the last of them wins)
+    int lo = 0, hi = T; // invariant: bounds[lo] <= pos < bounds[hi] once the input is well formed
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      const int64_t b = in_lds ? bounds[mid] : s_read(offsets, off64, (int64_t)mid * B);
+      if (b <= pos) lo = mid;
+      else hi = mid;
+    }
+    const TableDesc d = tables[lo];
+    uint8_t* orow = reinterpret_cast<uint8_t*>(out) + pos * out_row_bytes;
+    const int64_t idx = (int64_t)indices[pos];
+    bool ok = true;
+    if (idx == -1) {
+      ok = false; // pruned row: zeros
+    } else if (idx < 0 || idx >= d.num_rows) {
+      if (sub == 0) {
+        atomicOr(&status->bits, ERR_INDEX_OUT_OF_RANGE);
+        atomicMin(&status->first_bad_pos, (unsigned long long)pos);
+      }
+      ok = false;
+    }
+    const uint8_t* row = (d.placement ? w1 : w0) + d.weights_offset + (ok ? idx : 0) * d.row_stride;
+    if (copy_rows) {
+      // the row as it is stored: header, then elements (what fits the output row)
+      const int64_t in_bytes = d.data_off + d.data_bytes;
+      const int64_t n = in_bytes < out_row_bytes ? in_bytes : out_row_bytes;
+      for (int64_t b0 = (int64_t)sub * 4; b0 < out_row_bytes; b0 += (int64_t)lpr * 4) {
+        uint32_t v = 0;
+        if (ok && b0 + 4 <= n && (reinterpret_cast<uintptr_t>(row + b0) & 3) == 0) v = *reinterpret_cast<const uint32_t*>(row + b0);
+        else if (ok) for (int k = 0; k < 4; ++k) if (b0 + k < n) v |= (uint32_t)row[b0 + k] << (8 * k);
+        if (b0 + 4 <= out_row_bytes && (reinterpret_cast<uintptr_t>(orow + b0) & 3) == 0) *reinterpret_cast<uint32_t*>(orow + b0) = v;
+        else for (int k = 0; k < 4; ++k) if (b0 + k < out_row_bytes) orow[b0 + k] = (uint8_t)(v >> (8 * k));
+      }
+      continue;
+    }
+    const int bits = s_type_bits(d.ty);
+    const bool quant = bits <= 8;
+    float scale = 1.0f, bias = 0.0f;
+    if (quant && ok) {
+      const uint8_t* ph = row + d.sb_off;
+      uint32_t h;
+      if ((reinterpret_cast<uintptr_t>(ph) & 3) == 0) h = *reinterpret_cast<const uint32_t*>(ph);
+      else h = ph[0] | (ph[1] << 8) | (ph[2] << 16) | ((uint32_t)ph[3] << 24);
+      scale = 1.0f * s_half_to_float((uint16_t)h);
+      bias = 1.0f * s_half_to_float((uint16_t)(h >> 16));
+    }
+    const uint8_t* data = row + d.data_off;
+    const int Dt = d.D < D ? d.D : D; // columns the table has (all tables share D in this mode)
+    for (int j0 = sub * SRUN; j0 < D; j0 += lpr * SRUN) {
+      float v[SRUN];
+      for (int k = 0; k < SRUN; ++k) {
+        const int j = j0 + k;
+        float x = 0.0f;
+        if (ok && j < Dt) {
+          if (bits == 32) {
+            x = __builtin_fmaf(1.0f, reinterpret_cast<const float*>(data)[j], 0.0f);
+          } else if (bits == 16) {
+            const uint16_t u = reinterpret_cast<const uint16_t*>(data)[j];
+            x = __builtin_fmaf(1.0f, d.ty == ST_BF16 ? s_bits_to_float((uint32_t)u << 16) : s_half_to_float(u), 0.0f);
+          } else {
+            const int epb = 8 / bits;
+            const uint32_t q = ((uint32_t)data[j / epb] >> ((j % epb) * bits)) & ((1u << bits) - 1);
+            x = __builtin_fmaf(scale, (float)q, 0.0f + bias);
+          }
+        }
+        v[k] = x;
+      }
+      const int n = D - j0 < SRUN ? D - j0 : SRUN;
+      if (out_ty == ST_FP32) {
+        float* op = reinterpret_cast<float*>(orow) + j0;
+        if (n == SRUN && (reinterpret_cast<uintptr_t>(op) & 15) == 0) *reinterpret_cast<float4*>(op) = make_float4(v[0], v[1], v[2], v[3]);
+        else for (int k = 0; k < n; ++k) op[k] = v[k];
+      } else {
+        uint16_t h[SRUN];
+        for (int k = 0; k < SRUN; ++k) h[k] = out_ty == ST_FP16 ? s_to_half(v[k]) : s_to_bf16(v[k]);
+        uint16_t* op = reinterpret_cast<uint16_t*>(orow) + j0;
+        if (n == SRUN && (reinterpret_cast<uintptr_t>(op) & 7) == 0) *reinterpret_cast<uint2*>(op) = make_uint2(h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16));
+        else for (int k = 0; k < n; ++k) op[k] = h[k];
+      }
+    }
+  }
+}
+
+} // namespace
+
+hipError_t launch_sequence_lookup(const TableDesc* tables, const uint8_t* w0, const uint8_t* w1, const void* indices,
+                                  bool idx64, const void* offsets, int32_t B, int32_t T, int64_t total_L, int32_t D,
+                                  int32_t out_ty, void* out, Status* status, hipStream_t stream) {
+  if (total_L <= 0 || D <= 0) return hipSuccess;
+  const int64_t row_units = out_ty == ST_INT8 ? (D + 4 + 3) / 4 : out_ty == ST_INT4 ? ((D + 9) / 2 + 3) / 4 : (D + SRUN - 1) / SRUN;
+  int lpr = 1;
+  while (lpr < 64 && lpr < row_units) lpr <<= 1;
+  const int64_t per_block = 4 * (64 / lpr);
+  int64_t blocks = (total_L + per_block - 1) / per_block;
+  if (blocks > 256 * 64) blocks = 256 * 64;
+  const dim3 grid((unsigned)blocks), block(256);
+  if (idx64)
+    hipLaunchKernelGGL(sequence_lookup_kernel<int64_t>, grid, block, 0, stream, tables, w0, w1, (const int64_t*)indices,
+                       offsets, 1, B, T, total_L, D, out_ty, out, lpr, status);
+  else
+    hipLaunchKernelGGL(sequence_lookup_kernel<int32_t>, grid, block, 0, stream, tables, w0, w1, (const int32_t*)indices,
+                       offsets, 0, B, T, total_L, D, out_ty, out, lpr, status);
+  return hipGetLastError();
+}
+
+} // namespace fbgemm_amd

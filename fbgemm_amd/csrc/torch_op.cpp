@@ -10,6 +10,7 @@
 #include <c10/hip/HIPStream.h>
 #include <torch/library.h>
 
+#include <algorithm>
 #include <map>
 #include <mutex>
 #include <tuple>
@@ -35,7 +36,11 @@ struct PlanKey {
   }
 };
 std::mutex g_mu;
-std::map<PlanKey, fbgemm_amd_tbe_plan*> g_plans;
+struct PlanEntry {
+  fbgemm_amd_tbe_plan* plan;
+  Tensor keep[4]; // the key's tensors: alive while cached, so their addresses are not handed to other tensors
+};
+std::map<PlanKey, PlanEntry> g_plans;
 std::map<int, Tensor> g_status; // one status block per device, never freed
 
 Tensor& status_block(const Tensor& like) {
@@ -55,7 +60,7 @@ fbgemm_amd_tbe_plan* plan_for(const Tensor& dev_weights, const Tensor& uvm_weigh
   PlanKey key{weights_offsets.data_ptr(), weights_tys.data_ptr(), D_offsets.data_ptr(), placements.data_ptr(),
               D_offsets.numel() - 1, dev_weights.numel(), uvm_weights.numel(), row_alignment};
   auto it = g_plans.find(key);
-  if (it != g_plans.end()) return it->second;
+  if (it != g_plans.end()) return it->second.plan;
   const Tensor wo = weights_offsets.to(at::kCPU, at::kLong).contiguous();
   const Tensor wt = weights_tys.to(at::kCPU, at::kByte).contiguous();
   const Tensor dofs = D_offsets.to(at::kCPU, at::kInt).contiguous();
@@ -65,7 +70,7 @@ fbgemm_amd_tbe_plan* plan_for(const Tensor& dev_weights, const Tensor& uvm_weigh
       &plan, (int32_t)(dofs.numel() - 1), wo.data_ptr<int64_t>(), wt.data_ptr<uint8_t>(), dofs.data_ptr<int32_t>(),
       wp.data_ptr<int32_t>(), dev_weights.numel(), uvm_weights.numel(), row_alignment);
   TORCH_CHECK(rc == 0, "fbgemm_amd: ", fbgemm_amd_last_error());
-  g_plans.emplace(key, plan);
+  g_plans.emplace(key, PlanEntry{plan, {weights_offsets, weights_tys, D_offsets, placements}});
   return plan;
 }
 
@@ -80,15 +85,15 @@ at::ScalarType out_scalar_type(int64_t output_dtype) {
 
 Tensor int_nbit_split_embedding_codegen_lookup_function_hip(
     Tensor dev_weights, Tensor uvm_weights, Tensor weights_placements, Tensor weights_offsets, Tensor weights_tys,
-    Tensor D_offsets, int64_t total_D, int64_t /*max_int2_D*/, int64_t /*max_int4_D*/, int64_t /*max_int8_D*/,
-    int64_t /*max_float16_D*/, int64_t /*max_float32_D*/, Tensor indices, Tensor offsets, int64_t pooling_mode,
+    Tensor D_offsets, int64_t total_D, int64_t max_int2_D, int64_t max_int4_D, int64_t max_int8_D,
+    int64_t max_float16_D, int64_t max_float32_D, Tensor indices, Tensor offsets, int64_t pooling_mode,
     std::optional<Tensor> indice_weights, int64_t output_dtype, std::optional<Tensor> /*lxu_cache_weights*/,
     std::optional<Tensor> lxu_cache_locations, std::optional<int64_t> row_alignment,
     std::optional<int64_t> max_float8_D, std::optional<int64_t> /*fp8_exponent_bits*/,
     std::optional<int64_t> /*fp8_exponent_bias*/) {
   TORCH_CHECK(dev_weights.is_cuda() && indices.is_cuda() && offsets.is_cuda(), "fbgemm_amd: tensors must be on the GPU");
-  TORCH_CHECK(pooling_mode == FBGEMM_AMD_POOL_SUM || pooling_mode == FBGEMM_AMD_POOL_MEAN,
-              "fbgemm_amd: PoolingMode.NONE (sequence output) is not on this path");
+  TORCH_CHECK(pooling_mode == FBGEMM_AMD_POOL_SUM || pooling_mode == FBGEMM_AMD_POOL_MEAN || pooling_mode == FBGEMM_AMD_POOL_NONE,
+              "fbgemm_amd: unknown pooling mode ", pooling_mode);
   TORCH_CHECK(!max_float8_D || *max_float8_D == 0, "fbgemm_amd: FP8 tables are not on this path");
   TORCH_CHECK(!lxu_cache_locations || lxu_cache_locations->numel() == 0,
               "fbgemm_amd: the LXU cache is not on this path (tables are resident in HBM)");
@@ -109,6 +114,24 @@ Tensor int_nbit_split_embedding_codegen_lookup_function_hip(
   TORCH_CHECK(T > 0 && total_D > 0);
   const int64_t B = (offsets.numel() - 1) / T;
   TORCH_CHECK(B >= 0);
+  if (pooling_mode == FBGEMM_AMD_POOL_NONE) {
+    // embedding_forward_quantized_host_cpu.cpp:113-139: one row per index, D = the largest max_*_D
+    const int64_t D = std::max({max_int2_D, max_int4_D, max_int8_D, max_float16_D, max_float32_D});
+    const int64_t total_L = indices.numel();
+    Tensor out;
+    if (output_dtype == FBGEMM_AMD_INT8 || output_dtype == FBGEMM_AMD_INT4)
+      out = at::zeros({total_L, output_dtype == FBGEMM_AMD_INT8 ? D + 4 : (D + 9) / 2}, dev_weights.options().dtype(at::kByte));
+    else
+      out = at::zeros({total_L, D}, dev_weights.options().dtype(out_scalar_type(output_dtype)));
+    if (total_L == 0 || B == 0) return out;
+    Tensor& st = status_block(dev_weights);
+    const int rc = fbgemm_amd_tbe_forward_nobag(
+        plan, dev_weights.data_ptr(), uvm_weights.numel() ? uvm_weights.data_ptr() : nullptr, indices.data_ptr(),
+        offsets.data_ptr(), indices.scalar_type() == at::kLong ? 64 : 32, indices.numel(), offsets.numel(), (int32_t)D,
+        (int32_t)output_dtype, out.data_ptr(), st.data_ptr(), current_stream(dev_weights));
+    TORCH_CHECK(rc == 0, "fbgemm_amd: ", fbgemm_amd_last_error());
+    return out;
+  }
   Tensor out = at::empty({B, total_D}, dev_weights.options().dtype(out_scalar_type(output_dtype)));
   if (B == 0) return out;
   Tensor& st = status_block(dev_weights);

@@ -218,14 +218,15 @@ def _plan_for(dev_weights, uvm_weights, weights_placements, weights_offsets, wei
            weights_placements.data_ptr(), weights_offsets._version, D_offsets._version,
            weights_tys._version, D_offsets.numel(), dev_weights.numel(), uvm_weights.numel(),
            row_alignment)
-    plan = _plans.get(key)
-    if plan is None:
+    entry = _plans.get(key)
+    if entry is None:
         plan = TbePlan(weights_offsets, weights_tys, D_offsets, weights_placements,
                        dev_weights.numel(), uvm_weights.numel(), row_alignment)
         if len(_plans) > 64:
             _plans.clear()
-        _plans[key] = plan
-    return plan
+        # the entry keeps the tensors alive: while it is cached their addresses cannot be handed to other tensors
+        entry = _plans[key] = (plan, (weights_offsets, weights_tys, D_offsets, weights_placements))
+    return entry[0]
 
 
 def int_nbit_split_embedding_codegen_lookup_function(
@@ -245,16 +246,42 @@ def int_nbit_split_embedding_codegen_lookup_function(
     ``pruned_array_lookup``) fuse the pruned-row remap into the forward:
     ``indices`` are then logical ids."""
     _require_cuda(dev_weights, indices, offsets, indice_weights)
-    if pooling_mode == POOL_NONE:
-        raise NotImplementedError("PoolingMode.NONE (sequence output) is not on this path")
     if max_float8_D:
         raise NotImplementedError("FP8 tables are not on this path")
     if lxu_cache_locations is not None and lxu_cache_locations.numel() > 0:
         raise NotImplementedError("the LXU cache is not on this path: tables are resident in HBM")
-    if output_dtype not in _OUT_TORCH:
-        raise NotImplementedError(f"output_dtype {output_dtype} is not on this path")
     if offsets.dtype != indices.dtype:
         offsets = offsets.to(indices.dtype)  # as embedding_forward_quantized_host_cpu.cpp:111-113
+    if pooling_mode == POOL_NONE:
+        # embedding_forward_quantized_host_cpu.cpp:113-139: one row per index, unweighted, D = the largest max_*_D
+        if row_alignment is None:
+            row_alignment = 16
+        if plan is None:
+            plan = _plan_for(dev_weights, uvm_weights, weights_placements, weights_offsets, weights_tys,
+                             D_offsets, row_alignment)
+        D = max(max_int2_D, max_int4_D, max_int8_D, max_float16_D, max_float32_D)
+        total_L = indices.numel()
+        if output_dtype in _OUT_TORCH:
+            out = torch.zeros((total_L, D), dtype=_OUT_TORCH[output_dtype], device=dev_weights.device)
+        elif output_dtype in (INT8, INT4):
+            out = torch.zeros((total_L, D + 4 if output_dtype == INT8 else (D + 9) // 2), dtype=torch.uint8,
+                              device=dev_weights.device)
+        else:
+            raise NotImplementedError(f"output_dtype {output_dtype} is not on this path")
+        if total_L == 0 or (offsets.numel() - 1) // plan.T == 0:
+            return out
+        own = status is None
+        st = Status(dev_weights.device) if own else status
+        check(_lib.lib().fbgemm_amd_tbe_forward_nobag(
+            plan.handle, _ptr(dev_weights), _ptr(uvm_weights), _ptr(indices.contiguous()), _ptr(offsets.contiguous()),
+            _bits(indices), indices.numel(), offsets.numel(), D, output_dtype, _ptr(out), _ptr(st.buf), _stream()))
+        if own:
+            bits, pos = st.read()
+            if bits:
+                _raise_embedding_error(bits, pos, indices, offsets, plan, (offsets.numel() - 1) // plan.T)
+        return out
+    if output_dtype not in _OUT_TORCH:
+        raise NotImplementedError(f"output_dtype {output_dtype} is not on this path")
     if indice_weights is not None and indice_weights.numel() == 0:
         indice_weights = None
     if indice_weights is not None and indice_weights.dtype != torch.float32:

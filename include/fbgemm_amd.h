@@ -32,8 +32,9 @@ enum {
   FBGEMM_AMD_BF16 = 5
 };
 
-/* Pooling modes (embedding_common.h:34). NONE is not on this path. */
-enum { FBGEMM_AMD_POOL_SUM = 0, FBGEMM_AMD_POOL_MEAN = 1 };
+/* Pooling modes (embedding_common.h:34). NONE (one output row per index) has its own entry point,
+ * fbgemm_amd_tbe_forward_nobag. */
+enum { FBGEMM_AMD_POOL_SUM = 0, FBGEMM_AMD_POOL_MEAN = 1, FBGEMM_AMD_POOL_NONE = 2 };
 
 /* Error codes returned by the entry points. */
 enum {
@@ -171,6 +172,22 @@ int fbgemm_amd_tbe_forward_pruned(
     const float* d_indice_weights, int32_t output_ty, void* d_output,
     const void* d_index_remappings, int32_t remap_bits,
     const int64_t* d_index_remappings_offsets, void* d_status, void* stream);
+
+/* The forward without pooling (PoolingMode.NONE, "sequence" output;
+ * embedding_forward_quantized_host_cpu.cpp:113-139 and
+ * embedding_forward_quantized_cpu_template.cpp:283-296,390-420): d_output is
+ * [indices_numel, D] of output_ty, row i the row d_indices[i] of the table
+ * whose slice of d_offsets holds position i, converted like a bag of one
+ * (unweighted); an index of -1 gives a row of zeros. All tables share D (the
+ * operator passes the largest of its max_*_D). output_ty FBGEMM_AMD_INT8 /
+ * FBGEMM_AMD_INT4 copies the stored row (fp16 scale, fp16 bias, elements:
+ * D + 4 bytes, resp. (D + 8) / 2 bytes per output row) and needs every table
+ * to be of that type (src/RefImplementations.cc:1235-1253,1466-1484). */
+int fbgemm_amd_tbe_forward_nobag(
+    fbgemm_amd_tbe_plan* plan, const void* d_dev_weights, const void* d_uvm_weights,
+    const void* d_indices, const void* d_offsets, int32_t index_bits,
+    int64_t indices_numel, int64_t offsets_numel, int32_t D, int32_t output_ty,
+    void* d_output, void* d_status, void* stream);
 
 /* Timing of the lookup kernel alone (without the bag scheduler that runs
  * before it), for benchmarks: after fbgemm_amd_tbe_plan_profile(plan, slots)

@@ -328,6 +328,53 @@ def tbe_forward(dev_weights, weights_offsets, weights_tys, D_offsets, total_D, i
     return rc, out
 
 
+def tbe_forward_nobag(dev_weights, weights_offsets, weights_tys, rows_per_table, D, indices, offsets,
+                      out_ty, row_alignment):
+    """PoolingMode.NONE on the CPU, the way the reference's operator runs it
+    (embedding_forward_quantized_cpu_template.cpp:390-420): per table, the pooled
+    kernel over virtual bags of length one. int8 / int4 output types copy the
+    stored rows (src/RefImplementations.cc:1235-1253,1466-1484). Returns
+    (ok, out[total_L, D]) resp. uint8 [total_L, row bytes]."""
+    dev_weights = np.ascontiguousarray(dev_weights, dtype=np.uint8)
+    indices = np.ascontiguousarray(indices)
+    T = len(weights_tys)
+    B = (len(offsets) - 1) // T
+    total_L = len(indices)
+    copy_rows = out_ty in (ST_INT8, ST_INT4)
+    width = (D + 4 if out_ty == ST_INT8 else (D + 9) // 2) if copy_rows else D
+    out = np.zeros((total_L, width), np.uint8 if copy_rows else out_dtype(out_ty))
+    ok_all = True
+    for t in range(T):
+        s, e = int(offsets[t * B]), int(offsets[(t + 1) * B])
+        ty = int(weights_tys[t])
+        rb = padded_row_bytes(D, ty, row_alignment)
+        tbl = dev_weights[int(weights_offsets[t]):int(weights_offsets[t]) + int(rows_per_table[t]) * rb]
+        idx = indices[s:e]
+        if copy_rows:
+            rows2d = tbl.reshape(-1, rb)
+            for i, r in enumerate(idx.tolist()):
+                if r == -1:
+                    continue  # our operator leaves zeros for a pruned row
+                if r < 0 or r >= rows_per_table[t]:
+                    ok_all = False
+                    continue
+                n = min(width, unpadded_row_bytes(D, ty))
+                out[s + i, :n] = rows2d[r, :n]
+            continue
+        elem = 4 if ty == ST_FP32 else 2 if ty in (ST_FP16, ST_BF16) else 1
+        ok, o = spmdm(ty, D, tbl, idx, np.arange(e - s + 1, dtype=indices.dtype), out_ty=out_ty,
+                      input_stride=rb // elem, scale_bias_last=False, data_size=int(rows_per_table[t]),
+                      output_size=e - s)
+        ok_all = ok_all and ok
+        out[s:e] = o.reshape(e - s, D)
+    return ok_all, out
+
+
+def unpadded_row_bytes(dim, ty, scale_bias_bytes=4):
+    bits = {ST_FP32: 32, ST_FP16: 16, ST_BF16: 16, ST_INT8: 8, ST_INT4: 4, ST_INT2: 2}[ty]
+    return (dim * bits + 7) // 8 + (scale_bias_bytes if bits <= 8 else 0)
+
+
 def _conv(name, arr, in_dt, out_dt, impl):
     arr = np.ascontiguousarray(arr, dtype=in_dt)
     out = np.empty(arr.shape, dtype=out_dt)

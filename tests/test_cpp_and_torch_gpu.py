@@ -158,3 +158,23 @@ def test_torch_rowwise_quantize_ops(torch_ops, oracle):
             assert (g == want.view(g.dtype)).all()
     with pytest.raises(RuntimeError):
         torch_ops.FloatToFusedNBitRowwiseQuantizedSBHalf(cu(x[:, :3]), 4)
+
+
+def test_torch_operator_without_pooling(torch_ops, oracle):
+    from test_tbe_gpu import build_weights
+    rng = np.random.default_rng(78)
+    D = 64
+    specs = [(120, D, INT4), (90, D, INT8), (70, D, FP16)]
+    T, B = len(specs), 11
+    weights, wo, _ = build_weights(rng, specs, 16)
+    tys = np.array([s[2] for s in specs], np.uint8)
+    D_offsets = (np.arange(T + 1) * D).astype(np.int32)
+    lens = rng.integers(0, 6, size=T * B)
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    idx = np.concatenate([rng.integers(0, specs[t][0], size=int(lens[t * B:(t + 1) * B].sum())) for t in range(T)]).astype(np.int64)
+    got = torch_ops.int_nbit_split_embedding_codegen_lookup_function(
+        cu(weights), torch.zeros(0, dtype=torch.uint8, device="cuda"), cu(np.zeros(T, np.int32)), cu(wo), cu(tys),
+        cu(D_offsets), T * D, 0, D, D, D, 0, cu(idx), cu(off), 2, None, FP16, None, None, 16)
+    ok, want = oracle.tbe_forward_nobag(weights, wo, tys, [s[0] for s in specs], D, idx, off, FP16, 16)
+    assert ok and tuple(got.shape) == (len(idx), D)
+    H.assert_same_bits(got.cpu().view(torch.int16).numpy().view(np.uint16), want, "torch op, no pooling")

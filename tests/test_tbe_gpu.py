@@ -276,3 +276,74 @@ def test_config4_batched_scaled(ops, oracle):
                                   p.total_D, dense, p.host_offsets, p.pooling_mode, None, p.output_dtype, p.row_alignment)
     assert rc == 0
     H.assert_same_bits(got.cpu().numpy(), want, "config4 batched @ 0.02")
+
+
+@pytest.mark.parametrize("dt", [np.int32, np.int64])
+@pytest.mark.parametrize("D", [4, 32, 56, 128, 260])
+def test_no_pooling_matches_oracle(ops, oracle, dt, D):
+    """PoolingMode.NONE (sequence output): every index is a bag of one
+    (embedding_forward_quantized_cpu_template.cpp:390-420); after
+    nbit_forward_test.py:1060-1160 (nobag equals bags of length one)."""
+    rng = np.random.default_rng(900 + D)
+    tys = [INT4, INT8, FP16, INT2, FP32, INT4]
+    specs = [(int(rng.integers(20, 300)), D, ty) for ty in tys]
+    T, B = len(specs), 13
+    for row_alignment in (16, 1):
+        weights, wo, _ = build_weights(rng, specs, row_alignment)
+        lens = rng.integers(0, 7, size=T * B)
+        off = np.concatenate([[0], np.cumsum(lens)]).astype(dt)
+        idx = np.concatenate([rng.integers(0, specs[t][0], size=int(lens[t * B:(t + 1) * B].sum())) for t in range(T)]).astype(dt)
+        idx[rng.random(len(idx)) < 0.1] = -1
+        wt = np.array(tys, np.uint8)
+        D_offsets = (np.arange(T + 1) * D).astype(np.int32)
+        maxd = lambda ty: D if ty in tys else 0
+        for out_ty, tdt in ((FP32, torch.float32), (FP16, torch.float16), (BF16, torch.bfloat16)):
+            got = ops.int_nbit_split_embedding_codegen_lookup_function(
+                cu(weights), torch.zeros(0, dtype=torch.uint8, device="cuda"), cu(np.zeros(T, np.int32)), cu(wo), cu(wt),
+                cu(D_offsets), T * D, maxd(INT2), maxd(INT4), maxd(INT8), maxd(FP16), maxd(FP32), cu(idx), cu(off),
+                ops.POOL_NONE, None, out_ty, row_alignment=row_alignment)
+            assert got.dtype == tdt and tuple(got.shape) == (len(idx), D)
+            ok, want = oracle.tbe_forward_nobag(weights, wo, wt, [s[0] for s in specs], D, idx, off, out_ty, row_alignment)
+            assert ok
+            g = got.cpu()
+            g = g.numpy() if out_ty == FP32 else g.view(torch.int16).numpy().view(np.uint16)
+            H.assert_same_bits(g, want, f"no pooling D={D} out={out_ty} align={row_alignment}")
+        # an index past the table is reported
+        if len(idx):
+            bad = idx.copy()
+            bad[len(bad) // 2] = 10 ** 6
+            with pytest.raises(RuntimeError, match="out of bounds"):
+                ops.int_nbit_split_embedding_codegen_lookup_function(
+                    cu(weights), torch.zeros(0, dtype=torch.uint8, device="cuda"), cu(np.zeros(T, np.int32)), cu(wo), cu(wt),
+                    cu(D_offsets), T * D, maxd(INT2), maxd(INT4), maxd(INT8), maxd(FP16), maxd(FP32), cu(bad), cu(off),
+                    ops.POOL_NONE, None, FP16, row_alignment=row_alignment)
+
+
+@pytest.mark.parametrize("ty", [INT8, INT4])
+def test_no_pooling_quantized_output_copies_rows(ops, oracle, ty):
+    rng = np.random.default_rng(950 + ty)
+    D, T, B = 64, 3, 9
+    specs = [(int(rng.integers(20, 100)), D, ty) for _ in range(T)]
+    weights, wo, rbs = build_weights(rng, specs, 16)
+    lens = rng.integers(0, 6, size=T * B)
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    idx = np.concatenate([rng.integers(0, specs[t][0], size=int(lens[t * B:(t + 1) * B].sum())) for t in range(T)]).astype(np.int64)
+    wt = np.full(T, ty, np.uint8)
+    D_offsets = (np.arange(T + 1) * D).astype(np.int32)
+    got = ops.int_nbit_split_embedding_codegen_lookup_function(
+        cu(weights), torch.zeros(0, dtype=torch.uint8, device="cuda"), cu(np.zeros(T, np.int32)), cu(wo), cu(wt),
+        cu(D_offsets), T * D, 0, D if ty == INT4 else 0, D if ty == INT8 else 0, 0, 0, cu(idx), cu(off),
+        ops.POOL_NONE, None, ty, row_alignment=16).cpu().numpy()
+    ok, want = oracle.tbe_forward_nobag(weights, wo, wt, [s[0] for s in specs], D, idx, off, ty, 16)
+    assert ok and got.shape == want.shape and (got == want).all()
+    # the copied rows are the stored rows: header first, then the packed elements
+    t0_rows = weights[wo[0]:wo[0] + specs[0][0] * rbs[0]].reshape(-1, rbs[0])
+    n0 = int(off[B])
+    assert (got[:n0] == t0_rows[idx[:n0], :got.shape[1]]).all()
+    # a table of another type is refused
+    wt2 = wt.copy()
+    wt2[1] = FP16
+    with pytest.raises(RuntimeError, match="same type"):
+        ops.int_nbit_split_embedding_codegen_lookup_function(
+            cu(weights), torch.zeros(0, dtype=torch.uint8, device="cuda"), cu(np.zeros(T, np.int32)), cu(wo), cu(wt2),
+            cu(D_offsets), T * D, 0, D, D, D, 0, cu(idx), cu(off), ops.POOL_NONE, None, ty, row_alignment=16)
