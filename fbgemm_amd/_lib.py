@@ -40,6 +40,7 @@ SYMBOLS = {
     "fbgemm_amd_tbe_plan_profile_read": (C.c_int, [_P, _P, _I32, _P]),
     "fbgemm_amd_bounds_check_indices": (C.c_int, [_P, _I32, _P, _P, _I32, _I64, _I64, _I32, _P, _P, _P, _P]),
     "fbgemm_amd_pruned_hashmap_lookup": (C.c_int, [_P, _P, _I32, _I64, _P, _I32, _P, _I32, _P, _P]),
+    "fbgemm_amd_pruned_hashmap_insert_host": (C.c_int, [_P, _P, _P, _I32, _I64, _P, _I32, _P, _I32]),
     "fbgemm_amd_quantize_rowwise": (C.c_int, [_P, _I32, _I64, _I32, _I32, _I32, _I32, _I64, _P, _P]),
     "fbgemm_amd_dequantize_rowwise": (C.c_int, [_P, _I64, _I64, _I32, _I32, _I32, _I32, _I32, _P, _P]),
     "fbgemm_amd_tbe_plan_num_rows": (_I64, [_P, _I32]),

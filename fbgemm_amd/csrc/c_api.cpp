@@ -868,6 +868,71 @@ int fbgemm_amd_bounds_check_indices(
   return 0;
 }
 
+namespace {
+inline uint64_t host_pruned_hash(uint64_t k, bool wide) {
+  if (wide) { // MurmurHash3's 64-bit finalizer
+    k ^= k >> 33;
+    k *= 0xff51afd7ed558ccdull;
+    k ^= k >> 33;
+    k *= 0xc4ceb9fe1a85ec53ull;
+    k ^= k >> 33;
+    return k;
+  }
+  uint32_t h = (uint32_t)k; // and its 32-bit one
+  h ^= h >> 16;
+  h *= 0x85ebca6bu;
+  h ^= h >> 13;
+  h *= 0xc2b2ae35u;
+  h ^= h >> 16;
+  return h;
+}
+inline int64_t host_read(const void* p, bool wide, int64_t i) {
+  return wide ? ((const int64_t*)p)[i] : (int64_t)((const int32_t*)p)[i];
+}
+inline void host_write(void* p, bool wide, int64_t i, int64_t v) {
+  if (wide) ((int64_t*)p)[i] = v;
+  else ((int32_t*)p)[i] = (int32_t)v;
+}
+} // namespace
+
+int fbgemm_amd_pruned_hashmap_insert_host(
+    const void* h_indices, const void* h_dense_indices, const void* h_offsets, int32_t index_bits,
+    int64_t offsets_numel, void* h_hash_table, int32_t hash_bits, const int64_t* h_hash_table_offsets, int32_t T) {
+  if (T <= 0 || offsets_numel < 1 || (offsets_numel - 1) % T != 0) return fail(FBGEMM_AMD_E_ARG, "offsets must hold T*B+1 entries");
+  if ((index_bits != 32 && index_bits != 64) || (hash_bits != 32 && hash_bits != 64))
+    return fail(FBGEMM_AMD_E_ARG, "index_bits/hash_bits must be 32 or 64");
+  const int64_t B = (offsets_numel - 1) / T;
+  if (B <= 0) return fail(FBGEMM_AMD_E_ARG, "pruned_hashmap_insert needs B > 0");
+  if (!h_indices || !h_dense_indices || !h_offsets || !h_hash_table || !h_hash_table_offsets)
+    return fail(FBGEMM_AMD_E_ARG, "null data pointer");
+  const bool iw = index_bits == 64, hw = hash_bits == 64;
+  for (int32_t t = 0; t < T; ++t) {
+    const int64_t table_start = h_hash_table_offsets[t];
+    const int64_t capacity = h_hash_table_offsets[t + 1] - table_start;
+    if (capacity <= 0) continue;
+    const int64_t lo = host_read(h_offsets, iw, (int64_t)t * B), hi = host_read(h_offsets, iw, (int64_t)(t + 1) * B);
+    for (int64_t i = lo; i < hi; ++i) {
+      const int64_t idx = host_read(h_indices, iw, i);
+      const int64_t dense = host_read(h_dense_indices, iw, i);
+      if (dense == -1) continue; // a pruned row is not in the map
+      // the hash is taken of the id at the index width, as the reference takes it
+      int64_t slot = (int64_t)(host_pruned_hash(iw ? (uint64_t)idx : (uint64_t)(uint32_t)idx, iw) % (uint64_t)capacity);
+      int64_t probes = 0;
+      for (;; ++probes) {
+        if (probes == capacity) return fail(FBGEMM_AMD_E_ARG, "hash table of table %d is full", t);
+        const int64_t key = host_read(h_hash_table, hw, 2 * (table_start + slot));
+        if (key == -1 || key == idx) {
+          host_write(h_hash_table, hw, 2 * (table_start + slot), idx);
+          host_write(h_hash_table, hw, 2 * (table_start + slot) + 1, dense);
+          break;
+        }
+        slot = slot + 1 == capacity ? 0 : slot + 1;
+      }
+    }
+  }
+  return 0;
+}
+
 int fbgemm_amd_pruned_hashmap_lookup(
     const void* d_indices, const void* d_offsets, int32_t index_bits, int64_t offsets_numel,
     const void* d_hash_table, int32_t hash_bits, const int64_t* d_hash_table_offsets, int32_t T,

@@ -447,3 +447,24 @@ def dequantize_rowwise(input, cols, bit_rate, sb_float=False, layout=QLAYOUT_TRA
         _ptr(input), rows, input.stride(0) if rows > 1 else input.size(1), cols, bit_rate, int(sb_float), layout,
         _TORCH_OUT[output_dtype], _ptr(out), _stream()))
     return out
+
+
+def pruned_hashmap_insert(indices, dense_indices, offsets, hash_table, hash_table_offsets):
+    """pruned_hashmap_insert (embedding_forward_quantized_host_cpu.cpp:331-334;
+    embedding_forward_quantized_cpu_template.cpp:124-201): HOST tensors, in place
+    on ``hash_table`` ([slots, 2], -1 = empty), as in the reference, whose GPU
+    module builds the map on the CPU too."""
+    for t in (indices, dense_indices, offsets, hash_table, hash_table_offsets):
+        if t.is_cuda:
+            raise ValueError("pruned_hashmap_insert works on host tensors")
+    if indices.dtype != offsets.dtype:
+        raise TypeError("indices and offsets must have the same dtype")
+    if not hash_table.is_contiguous() or hash_table.dim() != 2 or hash_table.size(1) != 2:
+        raise ValueError("hash_table must be a contiguous [slots, 2] tensor")
+    indices = indices.contiguous()
+    dense = dense_indices.to(indices.dtype).contiguous()
+    offsets = offsets.contiguous()
+    hto = hash_table_offsets.to(torch.int64).contiguous()
+    check(_lib.lib().fbgemm_amd_pruned_hashmap_insert_host(
+        _ptr(indices), _ptr(dense), _ptr(offsets), _bits(indices), offsets.numel(), _ptr(hash_table),
+        _bits(hash_table), _ptr(hto), hto.numel() - 1))

@@ -255,6 +255,18 @@ int fbgemm_amd_pruned_hashmap_lookup(
     const void* d_hash_table, int32_t hash_bits, const int64_t* d_hash_table_offsets, int32_t T,
     void* d_dense, void* stream);
 
+/* pruned_hashmap_insert (embedding_forward_quantized_cpu_template.cpp:124-201;
+ * the reference has this operator on the CPU only and its GPU module calls
+ * it there, split_table_batched_embeddings_ops_inference.py:2001-2010): HOST
+ * pointers, runs on the calling thread. Inserts (indices[i], dense_indices[i])
+ * of every table's slice into that table's slots of h_hash_table ([slots][2],
+ * -1 = empty), skipping pairs whose dense id is -1, by linear probing from the
+ * same hash as the lookup. Returns FBGEMM_AMD_E_ARG when a table has no empty
+ * slot left (the reference would not return). */
+int fbgemm_amd_pruned_hashmap_insert_host(
+    const void* h_indices, const void* h_dense_indices, const void* h_offsets, int32_t index_bits,
+    int64_t offsets_numel, void* h_hash_table, int32_t hash_bits, const int64_t* h_hash_table_offsets, int32_t T);
+
 /* ---- row-wise quantizers: producers and readers of the row formats ---------- *
  *
  * fp32 / fp16 rows [rows][cols] -> fused quantized rows, bit for bit what the

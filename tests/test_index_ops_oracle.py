@@ -185,3 +185,35 @@ def test_hashmap_probe_wraps_and_handles_collisions():
         assert (table[2] == [keys[0], 10]).all() and (table[0] == [keys[1], 20]).all() and (table[1] == [keys[2], 30]).all()
         got = oracle.pruned_hashmap_lookup(np.array(keys + [k + 1], dt), np.array([0, 4], dt), table, np.array([0, cap], np.int64))
         assert list(got) == [10, 20, 30, -1]  # the absent key ends after one trip round the full table
+
+
+@pytest.mark.parametrize("idt", [np.int32, np.int64])
+@pytest.mark.parametrize("hdt", [np.int32, np.int64])
+def test_library_host_insert_builds_the_oracles_table(idt, hdt):
+    """fbgemm_amd_pruned_hashmap_insert_host is host code (the reference builds the
+    map on the CPU as well): its table equals the oracle's, slot for slot."""
+    import ctypes as C
+
+    from fbgemm_amd import _lib
+    rng = np.random.default_rng(31)
+    T = 4
+    ns = [0, 57, 300, 1]
+    caps = [0 if n == 0 else int(n / 0.5) + 3 for n in ns]
+    hto = np.concatenate([[0], np.cumsum(caps)]).astype(np.int64)
+    keys = np.concatenate([rng.choice(10 ** 6, size=n, replace=False) for n in ns]).astype(idt)
+    dense = np.concatenate([np.arange(n) for n in ns]).astype(idt)
+    dense[rng.random(len(dense)) < 0.2] = -1  # pruned rows are not inserted
+    off = np.concatenate([[0], np.cumsum(ns)]).astype(idt)
+    want = np.full((int(hto[-1]), 2), -1, hdt)
+    oracle.pruned_hashmap_insert(keys, dense, off, want, hto)
+    got = np.full((int(hto[-1]), 2), -1, hdt)
+    p = lambda a: C.c_void_p(a.ctypes.data)
+    rc = _lib.lib().fbgemm_amd_pruned_hashmap_insert_host(
+        p(keys), p(dense), p(off), 8 * keys.itemsize, len(off), p(got), 8 * got.itemsize, p(hto), T)
+    assert rc == 0 and (got == want).all()
+    # a full table is refused instead of probing for ever
+    tiny = np.full((2, 2), -1, hdt)
+    rc = _lib.lib().fbgemm_amd_pruned_hashmap_insert_host(
+        p(np.arange(3, dtype=idt)), p(np.arange(3, dtype=idt)), p(np.asarray([0, 3], idt)), 8 * keys.itemsize, 2,
+        p(tiny), 8 * tiny.itemsize, p(np.asarray([0, 2], np.int64)), 1)
+    assert rc < 0
