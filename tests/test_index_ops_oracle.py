@@ -213,7 +213,7 @@ def test_library_host_insert_builds_the_oracles_table(idt, hdt):
     assert rc == 0 and (got == want).all()
     # a full table is refused instead of probing for ever
     tiny = np.full((2, 2), -1, hdt)
+    k3, o3, h3 = np.arange(3, dtype=idt), np.asarray([0, 3], idt), np.asarray([0, 2], np.int64)
     rc = _lib.lib().fbgemm_amd_pruned_hashmap_insert_host(
-        p(np.arange(3, dtype=idt)), p(np.arange(3, dtype=idt)), p(np.asarray([0, 3], idt)), 8 * keys.itemsize, 2,
-        p(tiny), 8 * tiny.itemsize, p(np.asarray([0, 2], np.int64)), 1)
+        p(k3), p(k3), p(o3), 8 * k3.itemsize, 2, p(tiny), 8 * tiny.itemsize, p(h3), 1)
     assert rc < 0
