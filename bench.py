@@ -224,6 +224,20 @@ def cpu_baseline_tbe(p, seconds, torch):
     }
 
 
+def calibration_copy(a, torch):
+    """One plain copy of a known size: the yardstick the hardware byte counters are scaled against."""
+    if not a.calibration_copy_mib:
+        return
+    from fbgemm_amd import _lib
+    n = a.calibration_copy_mib << 20
+    src = torch.zeros(n, dtype=torch.uint8, device="cuda")
+    dst = torch.empty_like(src)
+    _lib.check(_lib.lib().fbgemm_amd_calibration_copy(
+        C.c_void_p(src.data_ptr()), C.c_void_p(dst.data_ptr()), n,
+        C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    torch.cuda.synchronize()
+
+
 def side_op(a):
     """One operator beside the lookup, timed with events on the launch stream.
 
@@ -311,6 +325,7 @@ def side_op(a):
     ev1.record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / a.steps
+    calibration_copy(a, torch)
     ms = ev0.elapsed_time(ev1) / a.steps
     gbps = alg_bytes / (ms * 1e-3) / 1e9
     res = {"metric": f"achieved HBM GB/s, {a.op} on 1 MI355X", "value": round(gbps, 2), "unit": "GB/s", "n_gpus": 1,
@@ -396,15 +411,7 @@ def main():
     wall = time.perf_counter() - t0
     bits, pos = st.read()
     assert bits == 0, f"the lookup rejected its inputs: status {bits:#x} at {pos}"
-    if a.calibration_copy_mib:
-        from fbgemm_amd import _lib
-        n = a.calibration_copy_mib << 20
-        src = torch.zeros(n, dtype=torch.uint8, device="cuda")
-        dst = torch.empty_like(src)
-        _lib.check(_lib.lib().fbgemm_amd_calibration_copy(
-            C.c_void_p(src.data_ptr()), C.c_void_p(dst.data_ptr()), n,
-            C.c_void_p(torch.cuda.current_stream().cuda_stream)))
-        torch.cuda.synchronize()
+    calibration_copy(a, torch)
     ms_per_step = wall * 1e3 / a.steps
     forward_ms = ev0.elapsed_time(ev1) / a.steps  # events on the launch stream, back-to-back forwards
     kernel_ms, kernel_name = forward_ms, "lookup_kernel (+ bag_order_kernel), per forward"

@@ -1,6 +1,7 @@
 #!/bin/bash
 # Collect the rocprofv3 evidence for one benchmark configuration and condense it.
 #   bash fbgemm_amd/profile_run.sh <config id> <output summary file> [extra bench.py args]
+# (extra args "--op quantize" etc. profile an operator beside the lookup; the config id is then unused)
 # Runs from the repository root on a machine with the GPU. One rocprofv3 run per
 # counter group (the hardware cannot collect them together); raw CSVs go to /tmp.
 set -o pipefail

@@ -2,8 +2,7 @@
 
     python -m fbgemm_amd.profile_summary <rocprofv3 output dir> [more dirs...]
 
-Prints, for every kernel whose name contains ``lookup_kernel`` or
-``calibration_copy_kernel`` (and the totals row of --stats), the call count and
+Prints, for every kernel of this library (and the totals row of --stats), the call count and
 average duration, and the per-dispatch average of every hardware counter
 collected. Raw CSVs hold every torch kernel of the run and are large; this is
 the part worth keeping.
@@ -14,7 +13,9 @@ import os
 import sys
 from collections import defaultdict
 
-OURS = ("lookup_kernel", "calibration_copy_kernel", "bag_order_kernel", "lengths_to_offsets", "pruned_array_lookup")
+OURS = ("sequence_lookup_kernel", "lookup_kernel", "calibration_copy_kernel", "bag_order_kernel", "lengths_to_offsets",
+        "pruned_array_lookup", "pruned_hashmap_lookup", "bounds_partial_max", "bounds_carry", "bounds_fix_offsets",
+        "bounds_check_bags", "dequantize_rowwise", "quantize_rowwise")
 
 
 def short(name):
