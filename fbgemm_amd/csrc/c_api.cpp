@@ -91,7 +91,7 @@ int sort_bags_default() {
 // Choose how lanes split a row. Wide 16-byte lanes need every row's data and
 // scale/bias to sit on 4-byte boundaries; anything else falls back to 4-byte
 // lanes and finally to element-sized lanes, which accept any layout.
-void plan_lanes(TableDesc& d, uintptr_t base_addr, int64_t out_stride, bool has_sb) {
+void plan_lanes(TableDesc& d, uintptr_t base_addr, int64_t out_stride, bool has_sb, bool allow_packed) {
   const int bits = type_bits(d.ty);
   d.data_bytes = (int32_t)(((int64_t)d.D * bits + 7) / 8);
   const bool a4 = base_addr % 4 == 0 && d.weights_offset % 4 == 0 && d.row_stride % 4 == 0 &&
@@ -127,10 +127,13 @@ void plan_lanes(TableDesc& d, uintptr_t base_addr, int64_t out_stride, bool has_
     const int nchunks = (d.data_bytes + 4 + 15) / 16;
     const int Ci = (d.ty == ST_INT8 && max_chunks >= 2 && nchunks >= 4) ? 2 : 1;
     const int lanes = std::max(2, (nchunks + Ci - 1) / Ci);
-    // lanes that would idle because a bag may not straddle a quarter of the wave
+    // lanes that would idle because a bag may not straddle a quarter of the wave:
+    // too many (9 lanes per bag) and the bags are laid end to end instead
     const int used = lanes <= 16 ? (16 / lanes) * lanes : 16;
-    if (lanes <= 32 && (int64_t)nchunks * 16 <= d.row_stride && used >= 14) {
+    const bool pack = used < 14 && allow_packed && (64 / lanes) * lanes >= 56;
+    if (lanes <= 32 && (int64_t)nchunks * 16 <= d.row_stride && (used >= 14 || pack)) {
       d.inline_hdr = 1;
+      d.packed = pack ? 1 : 0;
       d.vb = 16;
       d.chunks = Ci;
       d.lanes = lanes;
@@ -192,6 +195,7 @@ double row_cost(const TableDesc& d) {
   }
   lines /= (double)(128 / g);
   if (q && !d.inline_hdr) lines += 0.5;
+  if (d.packed) lines += 0.4; // bags that straddle a quarter of the wave ask for some lines twice
   return lines + 0.35;
 }
 
@@ -356,7 +360,8 @@ int fbgemm_amd_spmdm_launch(
   const int64_t out_stride = cfg->output_stride == -1 ? D : cfg->output_stride;
   if ((ty == ST_FP16 || ty == ST_BF16) && (uintptr_t)d_input % 2) return fail(FBGEMM_AMD_E_ARG, "fp16 table must be 2-byte aligned");
   if (ty == ST_FP32 && (uintptr_t)d_input % 4) return fail(FBGEMM_AMD_E_ARG, "fp32 table must be 4-byte aligned");
-  plan_lanes(d, (uintptr_t)d_input, out_stride, has_sb);
+  plan_lanes(d, (uintptr_t)d_input, out_stride, has_sb, false);
+  d.lanes_recip = (65536 + d.lanes - 1) / d.lanes;
 
   a.tables = nullptr;
   a.weights[0] = (const uint8_t*)d_input;
@@ -381,7 +386,7 @@ int fbgemm_amd_spmdm_launch(
   a.check_total = 1;
   a.out_aligned = (uintptr_t)d_out % 16 == 0;
   a.status = (Status*)d_status;
-  const int G = bags_per_wave(d.lanes);
+  const int G = bags_per_wave(d.lanes, d.packed);
   a.num_waves = (output_size + G - 1) / G;
 
   // Ordering the bags pays once several waves' worth of bags exist.
@@ -442,6 +447,10 @@ struct fbgemm_amd_tbe_plan {
   int64_t row_alignment = 16;
   std::vector<TableDesc> tables; // host copy
   TableDesc* d_tables = nullptr;
+  // the same tables with bags laid end to end where that saves a request per row
+  // (see bags_per_wave); empty when no table has such a shape. Used for long bags.
+  std::vector<TableDesc> tables_packed;
+  TableDesc* d_tables_packed = nullptr;
   int device = 0;
   // per-B work lists
   struct Work {
@@ -450,7 +459,7 @@ struct fbgemm_amd_tbe_plan {
     int64_t* d_xcd_start = nullptr;
     int64_t num_waves = 0;
   };
-  std::map<int32_t, Work> work;
+  std::map<std::pair<int32_t, int>, Work> work; // per (B, lane-shape set)
   std::mutex mu;
   // optional timing of the lookup kernel alone: a ring of (start, stop) event pairs
   std::vector<hipEvent_t> prof_ev;
@@ -509,10 +518,25 @@ int fbgemm_amd_tbe_plan_create(
     d.sb_off = 0;
     d.data_off = q ? 4 : 0;
     // weights buffers come from hipMalloc / torch: at least 256-byte aligned
-    plan_lanes(d, 0, plan->total_D, q);
+    plan_lanes(d, 0, plan->total_D, q, false);
+    d.lanes_recip = (65536 + d.lanes - 1) / d.lanes;
   }
   HIP_TRY(hipMalloc((void**)&plan->d_tables, sizeof(TableDesc) * T));
   HIP_TRY(hipMemcpy(plan->d_tables, plan->tables.data(), sizeof(TableDesc) * T, hipMemcpyHostToDevice));
+  plan->tables_packed = plan->tables;
+  bool any_packed = false;
+  for (int t = 0; t < T; ++t) {
+    TableDesc& d = plan->tables_packed[t];
+    plan_lanes(d, 0, plan->total_D, quantised(d.ty), true);
+    d.lanes_recip = (65536 + d.lanes - 1) / d.lanes;
+    any_packed = any_packed || d.packed;
+  }
+  if (any_packed) {
+    HIP_TRY(hipMalloc((void**)&plan->d_tables_packed, sizeof(TableDesc) * T));
+    HIP_TRY(hipMemcpy(plan->d_tables_packed, plan->tables_packed.data(), sizeof(TableDesc) * T, hipMemcpyHostToDevice));
+  } else {
+    plan->tables_packed.clear();
+  }
   *out = plan;
   return 0;
 }
@@ -527,6 +551,7 @@ void fbgemm_amd_tbe_plan_destroy(fbgemm_amd_tbe_plan* plan) {
     if (kv.second.d_xcd_start) (void)hipFree(kv.second.d_xcd_start);
   }
   if (plan->d_tables) (void)hipFree(plan->d_tables);
+  if (plan->d_tables_packed) (void)hipFree(plan->d_tables_packed);
   for (hipEvent_t e : plan->prof_ev) (void)hipEventDestroy(e);
   delete plan;
 }
@@ -578,10 +603,18 @@ int fbgemm_amd_tbe_forward_pruned(
     return fail(FBGEMM_AMD_E_ARG, "weights buffers must be 16-byte aligned");
   hipStream_t stream = (hipStream_t)stream_;
 
+  // Bags laid end to end save a line request per row and cost about a fifth more
+  // arithmetic on the tables they apply to. With short bags the per-bag work
+  // makes the kernel arithmetic-bound and the saving does not pay (measured: 15
+  // rows per bag loses 9 %, 30 rows per bag gains 5 %).
+  static const int packed_mode = env_int("FBGEMM_AMD_PACKED", 1); // 0 never, 1 by bag length, 2 always
+  const bool use_packed = !plan->tables_packed.empty() &&
+      (packed_mode == 2 || (packed_mode == 1 && indices_numel >= 20 * (int64_t)plan->T * B));
+  const std::vector<TableDesc>& tables = use_packed ? plan->tables_packed : plan->tables;
   fbgemm_amd_tbe_plan::Work w;
   {
     std::lock_guard<std::mutex> lk(plan->mu);
-    auto it = plan->work.find(B);
+    auto it = plan->work.find({B, use_packed ? 1 : 0});
     if (it == plan->work.end()) {
       // The work list is 8 runs, one per XCD (see lookup_kernel). Tables are
       // cut into slices of waves, the slices are dealt to the XCDs so that
@@ -598,8 +631,8 @@ int fbgemm_amd_tbe_forward_pruned(
       std::vector<double> wave_cost(plan->T);
       std::vector<int> nwaves(plan->T);
       for (int t = 0; t < plan->T; ++t) {
-        const TableDesc& d = plan->tables[t];
-        const int G = bags_per_wave(d.lanes);
+        const TableDesc& d = tables[t];
+        const int G = bags_per_wave(d.lanes, d.packed);
         nwaves[t] = (B + G - 1) / G;
         wave_cost[t] = G * row_cost(d);
         total_cost += wave_cost[t] * nwaves[t];
@@ -636,7 +669,7 @@ int fbgemm_amd_tbe_forward_pruned(
         std::vector<std::pair<double, WaveWork>> keyed;
         std::map<std::pair<int, int>, std::vector<Slice>> shapes; // slices of a shape, largest first (per_x order)
         for (const Slice& sl : per_x[x]) {
-          const TableDesc& d = plan->tables[sl.t];
+          const TableDesc& d = tables[sl.t];
           shapes[(interleave && by_shape) ? std::make_pair((int)d.ty, (int)d.D) : std::make_pair(0, 0)].push_back(sl);
         }
         size_t depth = 0;
@@ -646,7 +679,7 @@ int fbgemm_amd_tbe_forward_pruned(
           for (auto& kv : shapes) {
             if (i >= kv.second.size()) continue;
             const Slice& sl = kv.second[i];
-            const int G = bags_per_wave(plan->tables[sl.t].lanes);
+            const int G = bags_per_wave(tables[sl.t].lanes, tables[sl.t].packed);
             // one shape only (or no interleaving asked for): slice after slice
             const double base = (interleave && by_shape) ? (double)gidx : (interleave ? 0.0 : (double)gidx++);
             for (int k = 0; k < sl.count; ++k)
@@ -670,14 +703,14 @@ int fbgemm_amd_tbe_forward_pruned(
         HIP_TRY(hipMemcpy(nw.d_xcd_start, xcd_start.data(), sizeof(int64_t) * 9, hipMemcpyHostToDevice));
       }
       HIP_TRY(hipMalloc((void**)&nw.d_order, sizeof(BagEntry) * (size_t)plan->T * (size_t)B));
-      it = plan->work.emplace(B, nw).first;
+      it = plan->work.emplace(std::make_pair(B, use_packed ? 1 : 0), nw).first;
     }
     w = it->second;
   }
 
   LookupArgs a;
   memset(&a, 0, sizeof(a));
-  a.tables = plan->d_tables;
+  a.tables = use_packed ? plan->d_tables_packed : plan->d_tables;
   a.weights[0] = (const uint8_t*)d_dev_weights;
   a.weights[1] = (const uint8_t*)d_uvm_weights;
   a.indices = d_indices;

@@ -57,17 +57,22 @@ struct TableDesc {
   int32_t inline_hdr;     // 1: lanes own 16-byte chunks of the WHOLE row (fp16 scale/bias
                           // header first, then data), so the header arrives with the data
                           // and costs no request of its own; `lanes` need not divide 64
+  int32_t packed;         // 1: bags lie end to end in the wave (see bags_per_wave)
+  int32_t lanes_recip;    // ceil(65536 / lanes): j / lanes == (j * lanes_recip) >> 16 for 0 <= j <= 64
 };
 
 // Bags a wave pools side by side when `lanes` lanes share a bag. The memory
 // pipeline merges the addresses of a 16-byte-per-lane load 16 lanes at a time,
-// so a bag's lanes must not straddle a multiple of 16: each quarter of the wave
-// holds 16 / lanes whole bags and leaves the rest of its lanes idle. (For the
-// powers of two this is 64 / lanes.)
+// so a bag's lanes should not straddle a multiple of 16: with `packed` = 0 each
+// quarter of the wave holds 16 / lanes whole bags and leaves the rest of its
+// lanes idle (for the powers of two this is 64 / lanes). Where that would idle
+// too many lanes (9 lanes per bag: 7 of every 16), `packed` = 1 lays the bags
+// end to end instead: 64 / lanes bags, some of which straddle a quarter and
+// cost an extra line request now and then.
 #if defined(__HIPCC__)
 __host__ __device__
 #endif
-inline int bags_per_wave(int lanes) { return lanes <= 16 ? 4 * (16 / lanes) : 64 / lanes; }
+inline int bags_per_wave(int lanes, int packed) { return (lanes <= 16 && !packed) ? 4 * (16 / lanes) : 64 / lanes; }
 
 // What the bag scheduler leaves per bag, in the order waves take the bags.
 struct __attribute__((aligned(16))) BagEntry {

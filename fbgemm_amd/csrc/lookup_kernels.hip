@@ -250,6 +250,11 @@ __device__ __forceinline__ uint32_t to_half_bits(float f) {
 // the reference's bf16 writer: add 0x8000 to the pattern, keep the top half
 // (include/fbgemm/FloatConversion.h:312-315)
 __device__ __forceinline__ uint32_t to_bf16_bits(float f) { return (float_to_bits(f) + 0x8000u) >> 16; }
+// two outputs in one word: bytes 2, 3 of each rounded-up pattern, picked by one byte permute
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  return __builtin_amdgcn_perm(float_to_bits(hi) + 0x8000u, float_to_bits(lo) + 0x8000u, 0x07060302u);
+}
+__device__ __forceinline__ uint32_t pack_half2(float lo, float hi) { return to_half_bits(lo) | (to_half_bits(hi) << 16); }
 
 template <int NBYTES>
 __device__ __forceinline__ void store_words(void* p, const uint32_t* w) {
@@ -287,11 +292,12 @@ __device__ __forceinline__ void write_out(const LookupArgs& a, const float (&acc
     const bool bf = a.out_ty == ST_BF16;
     if (vec_ok && E >= 2) {
       uint32_t w[(E + 1) / 2];
+      if (bf) {
 #pragma unroll
-      for (int e = 0; e + 1 < E; e += 2) {
-        const uint32_t lo = bf ? to_bf16_bits(acc[e]) : to_half_bits(acc[e]);
-        const uint32_t hi = bf ? to_bf16_bits(acc[e + 1]) : to_half_bits(acc[e + 1]);
-        w[e / 2] = lo | (hi << 16);
+        for (int e = 0; e + 1 < E; e += 2) w[e / 2] = pack_bf16x2(acc[e], acc[e + 1]);
+      } else {
+#pragma unroll
+        for (int e = 0; e + 1 < E; e += 2) w[e / 2] = pack_half2(acc[e], acc[e + 1]);
       }
       store_words<E * 2>(o, w);
     } else {
@@ -330,11 +336,12 @@ __device__ __forceinline__ void write_out_runs(const LookupArgs& a, const float 
       const bool bf = a.out_ty == ST_BF16;
       if (whole && vec_ok) {
         uint32_t w[GE / 2];
+        if (bf) {
 #pragma unroll
-        for (int e = 0; e < GE; e += 2) {
-          const uint32_t lo = bf ? to_bf16_bits(acc[j * GE + e]) : to_half_bits(acc[j * GE + e]);
-          const uint32_t hi = bf ? to_bf16_bits(acc[j * GE + e + 1]) : to_half_bits(acc[j * GE + e + 1]);
-          w[e / 2] = lo | (hi << 16);
+          for (int e = 0; e < GE; e += 2) w[e / 2] = pack_bf16x2(acc[j * GE + e], acc[j * GE + e + 1]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < GE; e += 2) w[e / 2] = pack_half2(acc[j * GE + e], acc[j * GE + e + 1]);
         }
         store_words<GE * 2>(o, w);
       } else {
@@ -411,19 +418,21 @@ __device__ __forceinline__ bool pool_bags(const LookupArgs& a, const TableDesc& 
 
   static_assert(!INHDR || (VB == 16 && QUANT), "whole-row chunks are 16 bytes of a quantised row");
   const int S = d.lanes;
-  const int G = bags_per_wave(S);
+  const int G = bags_per_wave(S, d.packed);
   // quarter q of the wave holds bags q * (16 / S) ...; its last 16 % S lanes idle
   int grp, sub;
   bool idle;
-  if (S <= 16) {
-    const int per_q = 16 / S;
+  // divisions by S through the table's reciprocal (exact for arguments up to 64)
+  const uint32_t recip = (uint32_t)d.lanes_recip;
+  if (S <= 16 && !d.packed) {
+    const int per_q = (int)((16u * recip) >> 16);
     const int j = lane & 15;
-    const int gq = j / S;
+    const int gq = (int)(((uint32_t)j * recip) >> 16);
     idle = gq >= per_q;
     grp = (lane >> 4) * per_q + (idle ? per_q - 1 : gq);
     sub = j - gq * S;
   } else {
-    grp = lane / S;
+    grp = (int)(((uint32_t)lane * recip) >> 16);
     sub = lane - grp * S;
     idle = grp >= G;
   }
@@ -815,7 +824,7 @@ __device__ __forceinline__ void run_item(const LookupArgs& a, int64_t wave, int 
     table = ww.table;
     first_slot = ww.first_bag;
   } else {
-    first_slot = (int)(wave * bags_per_wave(a.single.lanes));
+    first_slot = (int)(wave * bags_per_wave(a.single.lanes, a.single.packed));
   }
   const TableDesc d = a.tables ? a.tables[table] : a.single;
 #ifdef FBGEMM_AMD_ONLY_TY // register-budget experiments: compile a single row type

@@ -347,3 +347,23 @@ def test_no_pooling_quantized_output_copies_rows(ops, oracle, ty):
         ops.int_nbit_split_embedding_codegen_lookup_function(
             cu(weights), torch.zeros(0, dtype=torch.uint8, device="cuda"), cu(np.zeros(T, np.int32)), cu(wo), cu(wt2),
             cu(D_offsets), T * D, 0, D, D, D, 0, cu(idx), cu(off), ops.POOL_NONE, None, ty, row_alignment=16)
+
+
+@pytest.mark.parametrize("out_ty", [FP32, FP16, BF16])
+def test_long_bags_of_nine_chunk_rows(ops, oracle, out_ty):
+    """Rows of 9 or 17 sixteen-byte chunks (int4 / int8, D = 256) with long bags:
+    the plan lays 7 bags of 9 lanes end to end in a wave, so bags straddle the
+    quarters of the wave and one lane idles."""
+    rng = np.random.default_rng(1200 + out_ty)
+    specs = [(400, 256, INT4), (300, 256, INT8), (350, 128, INT4), (200, 256, INT4)]
+    T, B = len(specs), 45  # 45 bags: 6 full waves of 7 and a ragged one
+    weights, wo, _ = build_weights(rng, specs, 16)
+    lens = rng.integers(20, 60, size=T * B)
+    lens[3] = 0
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    idx = np.concatenate([rng.integers(0, specs[t][0], size=int(lens[t * B:(t + 1) * B].sum())) for t in range(T)]).astype(np.int64)
+    idx[rng.random(len(idx)) < 0.05] = -1
+    psw = rng.uniform(0, 1, len(idx)).astype(np.float32)
+    for pooling, w in ((0, psw), (1, None), (0, None)):
+        got, want = run_both(ops, oracle, weights, wo, specs, idx, off, pooling, w, out_ty, 16)
+        H.assert_same_bits(got, want, f"nine-chunk rows pooling={pooling} weighted={w is not None} out={out_ty}")
