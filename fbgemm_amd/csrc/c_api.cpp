@@ -82,6 +82,8 @@ int env_int(const char* name, int dflt) {
 // Tunables, read once per process (the reference reads its FBGEMM_* switches
 // the same way, src/Utils.cc:773-875).
 
+constexpr int64_t SORT_MIN_LOOKUPS = 1 << 21;
+
 // 1: order each table's bags by length on the device before the lookup.
 int sort_bags_default() {
   static int v = env_int("FBGEMM_AMD_SORT_BAGS", 1);
@@ -389,8 +391,9 @@ int fbgemm_amd_spmdm_launch(
   const int G = bags_per_wave(d.lanes, d.packed);
   a.num_waves = (output_size + G - 1) / G;
 
-  // Ordering the bags pays once several waves' worth of bags exist.
-  const bool sort = sort_bags_default() && output_size > 2 * G;
+  // Ordering the bags pays once several waves' worth of bags and enough lookups exist
+  // (the scheduler launch costs 6-8 us and buys ~5 % of the lookup: it pays from a few million lookups on)
+  const bool sort = sort_bags_default() && output_size > 2 * G && index_size >= (int64_t)SORT_MIN_LOOKUPS;
   if (cfg->use_offsets) {
     a.offsets = d_offsets_or_lengths;
     a.off64 = cfg->offset_bits == 64;
@@ -733,7 +736,7 @@ int fbgemm_amd_tbe_forward_pruned(
   a.check_total = 0;
   a.out_aligned = (uintptr_t)d_output % 16 == 0;
   a.status = (Status*)d_status;
-  if (sort_bags_default()) {
+  if (sort_bags_default() && indices_numel >= (int64_t)SORT_MIN_LOOKUPS) {
     HIP_TRY(launch_bag_order(d_offsets, index_bits == 64, B, plan->T, w.d_order, stream));
     a.order = w.d_order;
   }

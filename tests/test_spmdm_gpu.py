@@ -236,3 +236,17 @@ def test_closed_forms(ops, oracle):
         assert ok
         got = out.view(np.float16).reshape(nb, D).astype(np.float32)
         assert (got == lens.astype(np.float32)[:, None]).all()
+
+
+def test_large_call_takes_the_ordered_path(ops, oracle):
+    """More than two million lookups in one single-table call: the library
+    orders the bags by length first (it skips that for smaller calls)."""
+    rng = np.random.default_rng(77)
+    rows, D, nb = 5000, 32, 90_000
+    table, _ = H.make_table(rng, INT4, rows, D, True)
+    lens = rng.integers(0, 60, size=nb)
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    idx = rng.integers(0, rows, size=int(off[-1])).astype(np.int32)
+    assert len(idx) > (1 << 21)
+    check_case(ops, oracle, ty=INT4, D=D, table=table, idx=idx, off_or_len=off, normalize=True, out_ty=FP16,
+               data_size=rows, output_size=nb, what="2.6 M lookups, ordered bags")
