@@ -28,6 +28,7 @@ SYMBOLS = {
     "fbgemm_amd_last_error": (C.c_char_p, []),
     "fbgemm_amd_version": (C.c_char_p, []),
     "fbgemm_amd_status_clear": (C.c_int, [_P, _P]),
+    "fbgemm_amd_stream_synchronize": (C.c_int, [_P]),
     "fbgemm_amd_status_read": (C.c_int, [_P, _P, C.POINTER(_I32), C.POINTER(_I64)]),
     "fbgemm_amd_spmdm_launch": (C.c_int, [C.POINTER(SpmdmConfig), _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _P, _P]),
     "fbgemm_amd_spmdm_run": (C.c_int, [C.POINTER(SpmdmConfig), _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _P]),

@@ -277,6 +277,11 @@ int fbgemm_amd_status_read(const void* d_status, void* stream, int32_t* bits, in
   return 0;
 }
 
+int fbgemm_amd_stream_synchronize(void* stream) {
+  HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+  return 0;
+}
+
 int fbgemm_amd_calibration_copy(const void* d_src, void* d_dst, int64_t bytes, void* stream) {
   if (!d_src || !d_dst || bytes < 0 || bytes % 16) return fail(FBGEMM_AMD_E_ARG, "copy needs 16-byte multiples");
   HIP_TRY(launch_calibration_copy(d_src, d_dst, bytes, (hipStream_t)stream));

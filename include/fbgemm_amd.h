@@ -294,6 +294,10 @@ int fbgemm_amd_dequantize_rowwise(
     const void* d_input, int64_t rows, int64_t in_row_stride, int32_t cols, int32_t bit_rate, int32_t sb_float,
     int32_t layout, int32_t output_ty, void* d_output, void* stream);
 
+/* Wait for everything enqueued on `stream` (hipStreamSynchronize), for callers
+ * of the asynchronous entry points that hold no HIP headers. */
+int fbgemm_amd_stream_synchronize(void* stream);
+
 /* ---- measurement aid -------------------------------------------------------- *
  * No counterpart in the reference. A plain device-to-device copy of `bytes`
  * (a multiple of 16) by a kernel named calibration_copy_kernel: profiles scale

@@ -12,6 +12,7 @@
 // Header-only; link against libfbgemm_amd.so.
 #pragma once
 
+#include <cstddef>
 #include <cstdint>
 #include <functional>
 #include <stdexcept>
@@ -225,6 +226,69 @@ GenerateEmbeddingSpMDMNBitRowWiseSparse(int bit_rate, const std::int64_t block_s
     return detail::run(cfg, output_size, index_size, uncompressed_data_size, input, indices, offsets_or_lengths,
                        weights, out, compressed_indices_table, has_weight);
   };
+}
+
+// ---- row-wise quantizers (include/fbgemm/QuantUtils.h:276-334 of the reference) ----
+// Same names and argument lists; every pointer is a DEVICE pointer; the call
+// returns when the work is done. `rowwise_min_max` (precomputed extremes) is
+// not supported and must be null.
+
+namespace detail {
+template <typename T>
+constexpr int float_ty() {
+  if constexpr (std::is_same_v<T, float>) return FBGEMM_AMD_FP32;
+  else if constexpr (std::is_same_v<T, float16> || std::is_same_v<T, std::uint16_t>) return FBGEMM_AMD_FP16;
+  else if constexpr (std::is_same_v<T, bfloat16>) return FBGEMM_AMD_BF16;
+  else static_assert(sizeof(T) == 0, "type must be float, float16, uint16_t or bfloat16");
+}
+inline void done(int rc) {
+  if (rc < 0) throw std::runtime_error(std::string("fbgemm_amd: ") + fbgemm_amd_last_error());
+  fbgemm_amd_stream_synchronize(stream_ref());
+}
+} // namespace detail
+
+template <typename InputType>
+void FloatOrHalfToFusedNBitRowwiseQuantizedSBHalf(int bit_rate, const InputType* input, std::size_t input_rows,
+                                                  int input_columns, std::uint8_t* output,
+                                                  const InputType* rowwise_min_max = nullptr) {
+  static_assert(!std::is_same_v<InputType, bfloat16>, "input is float or float16");
+  if (rowwise_min_max) throw std::invalid_argument("fbgemm_amd: rowwise_min_max is not supported");
+  const int epb = 8 / bit_rate;
+  detail::done(fbgemm_amd_quantize_rowwise(input, detail::float_ty<InputType>(), (std::int64_t)input_rows, input_columns,
+                                           bit_rate, 0, FBGEMM_AMD_QLAYOUT_TRAILER, (input_columns + epb - 1) / epb + 4,
+                                           output, stream_ref()));
+}
+
+template <typename OutputType>
+void FusedNBitRowwiseQuantizedSBHalfToFloatOrHalf(int bit_rate, const std::uint8_t* input, std::size_t input_rows,
+                                                  int input_columns, OutputType* output, bool scale_bias_last = true) {
+  // input_columns counts the bytes of a fused row (QuantUtils.cc:758-760)
+  const int cols = (input_columns - 4) * (8 / bit_rate);
+  detail::done(fbgemm_amd_dequantize_rowwise(input, (std::int64_t)input_rows, input_columns, cols, bit_rate, 0,
+                                             scale_bias_last ? FBGEMM_AMD_QLAYOUT_TRAILER : FBGEMM_AMD_QLAYOUT_TBE,
+                                             detail::float_ty<OutputType>(), output, stream_ref()));
+}
+
+template <typename InputType>
+void FloatOrHalfToFused8BitRowwiseQuantizedSBFloat(const InputType* input, std::size_t input_rows, int input_columns,
+                                                   std::uint8_t* output, const InputType* rowwise_min_max = nullptr) {
+  static_assert(!std::is_same_v<InputType, bfloat16>, "input is float or float16");
+  if (rowwise_min_max) throw std::invalid_argument("fbgemm_amd: rowwise_min_max is not supported");
+  detail::done(fbgemm_amd_quantize_rowwise(input, detail::float_ty<InputType>(), (std::int64_t)input_rows, input_columns,
+                                           8, 1, FBGEMM_AMD_QLAYOUT_TRAILER, input_columns + 8, output, stream_ref()));
+}
+
+template <typename OutputType>
+void Fused8BitRowwiseQuantizedSBFloatToFloatOrHalf(const std::uint8_t* input, std::size_t input_rows, int input_columns,
+                                                   OutputType* output, const bool scale_bias_last = true,
+                                                   const bool quant_padding_float_type = true) {
+  if (scale_bias_last != quant_padding_float_type)
+    throw std::invalid_argument("fbgemm_amd: rows are (data, fp32 scale, fp32 bias) or (fp16 scale, fp16 bias, data)");
+  const int sb = quant_padding_float_type ? 8 : 4;
+  detail::done(fbgemm_amd_dequantize_rowwise(input, (std::int64_t)input_rows, input_columns, input_columns - sb, 8,
+                                             quant_padding_float_type ? 1 : 0,
+                                             scale_bias_last ? FBGEMM_AMD_QLAYOUT_TRAILER : FBGEMM_AMD_QLAYOUT_TBE,
+                                             detail::float_ty<OutputType>(), output, stream_ref()));
 }
 
 } // namespace fbgemm_amd

@@ -20,6 +20,11 @@ extern "C" int oracle_embedding_spmdm(
     int normalize_by_lengths, void* out, int out_ty, int is_weight_positional, int use_offsets,
     int64_t output_stride, int64_t input_stride, int scale_bias_last, const int32_t* remap);
 extern "C" uint16_t oracle_float2half_rn(float f);
+extern "C" void oracle_quantize_rowwise(const void* input, int half_in, int64_t rows, int32_t cols, int32_t bit_rate,
+                                        int32_t sb_float, int32_t layout, int64_t out_stride, uint8_t* output);
+extern "C" void oracle_dequantize_rowwise(const uint8_t* input, int64_t rows, int64_t in_stride, int32_t cols,
+                                          int32_t bit_rate, int32_t sb_float, int32_t layout, int32_t output_ty,
+                                          void* output);
 
 #define HIP_OK(x) do { hipError_t e_ = (x); if (e_ != hipSuccess) { printf("%s: %s\n", #x, hipGetErrorString(e_)); return 2; } } while (0)
 
@@ -134,6 +139,42 @@ void run_8bit(int64_t D, int batch, int rows, int avg_len, bool weighted, bool n
         (long)D, weighted, normalize);
 }
 
+// The quantizer templates (names and arguments of include/fbgemm/QuantUtils.h:276-334)
+// against the oracle, after test/QuantUtilsTest.cc's fused row-wise cases.
+void run_quantizers(int rows, int cols, unsigned seed) {
+  std::mt19937 rng(seed);
+  std::vector<float> x((size_t)rows * cols);
+  for (auto& v : x) v = (float)((int)(rng() % 20001) - 10000) / 1000.f;
+  Dev<float> d_x(x);
+  for (int bit_rate : {2, 4, 8}) {
+    const int epb = 8 / bit_rate;
+    if (cols % epb) continue;
+    const int stride = cols / epb + 4;
+    std::vector<uint8_t> want((size_t)rows * stride), zero((size_t)rows * stride, 0);
+    oracle_quantize_rowwise(x.data(), 0, rows, cols, bit_rate, 0, 0, stride, want.data());
+    Dev<uint8_t> d_q(zero);
+    fbgemm_amd::FloatOrHalfToFusedNBitRowwiseQuantizedSBHalf<float>(bit_rate, d_x.p, rows, cols, d_q.p);
+    CHECK(d_q.host() == want, "%d-bit rows differ (%d x %d)", bit_rate, rows, cols);
+    std::vector<float> back_want((size_t)rows * cols), back_init((size_t)rows * cols, -3.f);
+    oracle_dequantize_rowwise(want.data(), rows, stride, cols, bit_rate, 0, 0, FBGEMM_AMD_FP32, back_want.data());
+    Dev<float> d_back(back_init);
+    fbgemm_amd::FusedNBitRowwiseQuantizedSBHalfToFloatOrHalf<float>(bit_rate, d_q.p, rows, stride, d_back.p);
+    auto got = d_back.host();
+    CHECK(memcmp(got.data(), back_want.data(), got.size() * 4) == 0, "%d-bit rows dequantize differently", bit_rate);
+  }
+  const int stride8 = cols + 8;
+  std::vector<uint8_t> want8((size_t)rows * stride8), zero8((size_t)rows * stride8, 0);
+  oracle_quantize_rowwise(x.data(), 0, rows, cols, 8, 1, 0, stride8, want8.data());
+  Dev<uint8_t> d_q8(zero8);
+  fbgemm_amd::FloatOrHalfToFused8BitRowwiseQuantizedSBFloat<float>(d_x.p, rows, cols, d_q8.p);
+  CHECK(d_q8.host() == want8, "8-bit rows with fp32 scale/bias differ (%d x %d)", rows, cols);
+  std::vector<uint16_t> half_want((size_t)rows * cols), half_init((size_t)rows * cols, 0xBEEF);
+  oracle_dequantize_rowwise(want8.data(), rows, stride8, cols, 8, 1, 0, FBGEMM_AMD_FP16, half_want.data());
+  Dev<uint16_t> d_half(half_init);
+  fbgemm_amd::Fused8BitRowwiseQuantizedSBFloatToFloatOrHalf<std::uint16_t>(d_q8.p, rows, stride8, d_half.p);
+  CHECK(d_half.host() == half_want, "8-bit rows dequantize to fp16 differently");
+}
+
 int main() {
   int ndev = 0;
   HIP_OK(hipGetDeviceCount(&ndev));
@@ -158,6 +199,8 @@ int main() {
         run_8bit<int64_t, int32_t>(s[2], s[0], s[1], s[3], weighted, normalize, ++seed);
         run_8bit<int32_t, int32_t>(s[2], s[0], s[1], s[3], weighted, normalize, ++seed);
       }
+  for (int cols : {4, 8, 64, 100, 128, 260})
+    for (int rows : {1, 7, 130}) run_quantizers(rows, cols, ++seed);
   printf("%s: %d failure(s)\n", failures ? "FAILED" : "PASSED", failures);
   return failures ? 1 : 0;
 }
