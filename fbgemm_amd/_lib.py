@@ -36,6 +36,7 @@ SYMBOLS = {
     "fbgemm_amd_tbe_plan_destroy": (None, [_P]),
     "fbgemm_amd_tbe_forward": (C.c_int, [_P, _P, _P, _P, _P, _I32, _I64, _I64, _I32, _P, _I32, _P, _P, _P]),
     "fbgemm_amd_tbe_forward_pruned": (C.c_int, [_P, _P, _P, _P, _P, _I32, _I64, _I64, _I32, _P, _I32, _P, _P, _I32, _P, _P, _P]),
+    "fbgemm_amd_tbe_plan_set_fp8": (C.c_int, [_P, _I32, _I32]),
     "fbgemm_amd_tbe_forward_nobag": (C.c_int, [_P, _P, _P, _P, _P, _I32, _I64, _I64, _I32, _I32, _P, _P, _P]),
     "fbgemm_amd_tbe_plan_profile": (C.c_int, [_P, _I32]),
     "fbgemm_amd_tbe_plan_profile_read": (C.c_int, [_P, _P, _I32, _P]),

@@ -21,7 +21,8 @@ hipError_t launch_status_clear(Status* st, hipStream_t stream);
 hipError_t launch_bag_order(const void* offsets, bool off64, int32_t B, int32_t T, BagEntry* order, hipStream_t stream);
 hipError_t launch_sequence_lookup(const TableDesc* tables, const uint8_t* w0, const uint8_t* w1, const void* indices,
                                   bool idx64, const void* offsets, int32_t B, int32_t T, int64_t total_L, int32_t D,
-                                  int32_t out_ty, void* out, Status* status, hipStream_t stream);
+                                  int32_t out_ty, void* out, int32_t fp8_shift, float fp8_mult, Status* status,
+                                  hipStream_t stream);
 hipError_t launch_calibration_copy(const void* src, void* dst, int64_t bytes, hipStream_t stream);
 hipError_t launch_bounds_check(const int64_t* rows_per_table, int32_t T, void* indices, void* offsets, bool is64,
                                int64_t num_indices, int64_t total_B, int64_t B, const int32_t* B_offsets, int mode,
@@ -65,7 +66,7 @@ int type_bits(int ty) {
   switch (ty) {
     case ST_FP32: return 32;
     case ST_FP16: case ST_BF16: return 16;
-    case ST_INT8: return 8;
+    case ST_INT8: case ST_FP8: return 8;
     case ST_INT4: return 4;
     case ST_INT2: return 2;
     default: return 0;
@@ -245,7 +246,7 @@ int grow(T** buf, int64_t* cap, int64_t need, hipStream_t stream) {
 
 int check_cfg(const fbgemm_amd_spmdm_config* c) {
   if (!c) return fail(FBGEMM_AMD_E_ARG, "config is null");
-  if (type_bits(c->weight_ty) == 0) return fail(FBGEMM_AMD_E_ARG, "unsupported weight_ty %d", c->weight_ty);
+  if (type_bits(c->weight_ty) == 0 || c->weight_ty == ST_FP8) return fail(FBGEMM_AMD_E_ARG, "unsupported weight_ty %d", c->weight_ty);
   if (c->output_ty != ST_FP32 && c->output_ty != ST_FP16 && c->output_ty != ST_BF16)
     return fail(FBGEMM_AMD_E_ARG, "unsupported output_ty %d", c->output_ty);
   if ((c->index_bits != 32 && c->index_bits != 64) || (c->offset_bits != 32 && c->offset_bits != 64))
@@ -292,6 +293,7 @@ int32_t fbgemm_amd_unpadded_row_size_in_bytes(int32_t dim, int32_t ty, int32_t s
   switch (ty) {
     case ST_FP32: return dim * 4;
     case ST_FP16: case ST_BF16: return dim * 2;
+    case ST_FP8: return dim;
     case ST_INT8: return dim + sb;
     case ST_INT4: return dim / 2 + sb;
     case ST_INT2: return dim / 4 + sb;
@@ -470,6 +472,9 @@ struct fbgemm_amd_tbe_plan {
   std::map<std::pair<int32_t, int>, Work> work; // per (B, lane-shape set)
   std::mutex mu;
   // optional timing of the lookup kernel alone: a ring of (start, stop) event pairs
+  int32_t fp8_shift = 0; // FP8 rows: set by fbgemm_amd_tbe_plan_set_fp8
+  float fp8_mult = 0.0f;
+  bool has_fp8 = false;
   std::vector<hipEvent_t> prof_ev;
   int64_t prof_count = 0;
 };
@@ -521,6 +526,7 @@ int fbgemm_amd_tbe_plan_create(
     const int64_t next = it != p.end() ? *it : (d.placement ? uvm_bytes : dev_bytes);
     d.num_rows = std::max<int64_t>(0, (next - d.weights_offset) / d.row_stride);
     d.skip_minus_one = 1;
+    plan->has_fp8 = plan->has_fp8 || d.ty == ST_FP8;
     const bool q = quantised(d.ty);
     d.sb_fp32 = 0;
     d.sb_off = 0;
@@ -562,6 +568,18 @@ void fbgemm_amd_tbe_plan_destroy(fbgemm_amd_tbe_plan* plan) {
   if (plan->d_tables_packed) (void)hipFree(plan->d_tables_packed);
   for (hipEvent_t e : plan->prof_ev) (void)hipEventDestroy(e);
   delete plan;
+}
+
+int fbgemm_amd_tbe_plan_set_fp8(fbgemm_amd_tbe_plan* plan, int32_t exponent_bits, int32_t exponent_bias) {
+  if (!plan) return fail(FBGEMM_AMD_E_ARG, "plan is null");
+  // embedding_forward_quantized_cpu_template.cpp (check_fp8_params): both must be given
+  if (exponent_bits < 1 || exponent_bits > 6 || exponent_bias < 0 || exponent_bias > 253)
+    return fail(FBGEMM_AMD_E_ARG, "fp8 needs 1..6 exponent bits and a bias in 0..253");
+  std::lock_guard<std::mutex> lk(plan->mu);
+  plan->fp8_shift = 16 + exponent_bits;
+  const uint32_t mult_bits = (uint32_t)(127 + (127 - exponent_bias)) << 23; // 2^(127 - bias)
+  memcpy(&plan->fp8_mult, &mult_bits, 4);
+  return 0;
 }
 
 int64_t fbgemm_amd_tbe_plan_num_rows(const fbgemm_amd_tbe_plan* plan, int32_t t) {
@@ -610,6 +628,8 @@ int fbgemm_amd_tbe_forward_pruned(
   if ((uintptr_t)d_dev_weights % 16 || (uintptr_t)d_uvm_weights % 16)
     return fail(FBGEMM_AMD_E_ARG, "weights buffers must be 16-byte aligned");
   hipStream_t stream = (hipStream_t)stream_;
+  if (plan->has_fp8 && plan->fp8_shift == 0)
+    return fail(FBGEMM_AMD_E_ARG, "the plan holds FP8 tables: set their exponent bits and bias first (fbgemm_amd_tbe_plan_set_fp8)");
 
   // Bags laid end to end save a line request per row and cost about a fifth more
   // arithmetic on the tables they apply to. With short bags the per-bag work
@@ -741,6 +761,8 @@ int fbgemm_amd_tbe_forward_pruned(
   a.check_total = 0;
   a.out_aligned = (uintptr_t)d_output % 16 == 0;
   a.status = (Status*)d_status;
+  a.fp8_shift = plan->fp8_shift;
+  a.fp8_mult = plan->fp8_mult;
   if (sort_bags_default() && indices_numel >= (int64_t)SORT_MIN_LOOKUPS) {
     HIP_TRY(launch_bag_order(d_offsets, index_bits == 64, B, plan->T, w.d_order, stream));
     a.order = w.d_order;
@@ -797,6 +819,8 @@ int fbgemm_amd_tbe_forward_nobag(
   if (B64 > 0x7fffffffLL) return fail(FBGEMM_AMD_E_ARG, "B exceeds 2^31-1");
   if (B64 == 0 || indices_numel == 0) return 0;
   if (!d_offsets || !d_output || !d_indices) return fail(FBGEMM_AMD_E_ARG, "null data pointer");
+  if (plan->has_fp8 && plan->fp8_shift == 0)
+    return fail(FBGEMM_AMD_E_ARG, "the plan holds FP8 tables: set their exponent bits and bias first (fbgemm_amd_tbe_plan_set_fp8)");
   for (int t = 0; t < plan->T; ++t) {
     const TableDesc& d = plan->tables[t];
     if (d.D != D) return fail(FBGEMM_AMD_E_ARG, "table %d has D = %d: without pooling all tables share D = %d", t, d.D, D);
@@ -809,7 +833,7 @@ int fbgemm_amd_tbe_forward_nobag(
   }
   HIP_TRY(launch_sequence_lookup(plan->d_tables, (const uint8_t*)d_dev_weights, (const uint8_t*)d_uvm_weights, d_indices,
                                  index_bits == 64, d_offsets, (int32_t)B64, plan->T, indices_numel, D, output_ty,
-                                 d_output, (Status*)d_status, (hipStream_t)stream));
+                                 d_output, plan->fp8_shift, plan->fp8_mult, (Status*)d_status, (hipStream_t)stream));
   return 0;
 }
 

@@ -13,6 +13,7 @@ enum : int32_t {
   ST_INT4 = 3,
   ST_INT2 = 4,
   ST_BF16 = 5,
+  ST_FP8 = 6, // 8-bit floats (1 sign, e exponent, 7 - e mantissa bits; exponent bias given per call)
 };
 
 // Bits of the status word a lookup ORs in when it meets an input the reference
@@ -120,6 +121,8 @@ struct LookupArgs {
   int32_t check_total;       // single-table call: positions are relative to offsets[0] and
                              // offsets[last] - offsets[0] must equal index_size
   int32_t out_aligned;       // `out` is 16-byte aligned (vector stores allowed)
+  int32_t fp8_shift;         // FP8 rows: 16 + exponent bits (moves the 7 low bits to fp32's exponent/mantissa)
+  float fp8_mult;            // FP8 rows: 2^(127 - exponent bias)
   Status* status;
 #ifdef FBGEMM_AMD_WAVE_TRACE
   // diagnostic build only: 4 words per workgroup (start, end of the wave on the

@@ -46,7 +46,7 @@ __device__ __forceinline__ float half_hi(uint32_t u) {
 }
 
 __device__ __forceinline__ constexpr int type_bits(int ty) {
-  return ty == ST_FP32 ? 32 : (ty == ST_FP16 || ty == ST_BF16) ? 16 : ty == ST_INT8 ? 8 : ty == ST_INT4 ? 4 : 2;
+  return ty == ST_FP32 ? 32 : (ty == ST_FP16 || ty == ST_BF16) ? 16 : (ty == ST_INT8 || ty == ST_FP8) ? 8 : ty == ST_INT4 ? 4 : 2;
 }
 
 __device__ __forceinline__ void report(Status* st, int32_t bit) {
@@ -182,6 +182,27 @@ struct Accum<ST_BF16, VB> {
     }
   }
   __device__ __forceinline__ static void slow(float (&acc)[E], const uint32_t* raw, float a, float b) { fast(acc, raw, a, b); }
+};
+
+// 8-bit floats: the 7 low bits are moved to fp32's exponent and mantissa
+// fields, the value is scaled by 2^(127 - bias) and the sign bit is put back
+// (Float8ToFloat_ref, src/RefImplementations.cc:184-214); then acc = fma(w, x, acc).
+// `shift` and `mult` come with the call (they are the same for all lanes).
+template <int VB>
+struct Accum<ST_FP8, VB> {
+  static constexpr int E = VB;
+  static constexpr bool kPrescaled = false;
+  __device__ __forceinline__ static void fp8(float (&acc)[E], const uint32_t* raw, float w, int shift, float mult) {
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const uint32_t b = (raw[e / 4] >> (8 * (e % 4))) & 0xffu;
+      const float mag = bits_to_float((b & 0x7fu) << shift) * mult;
+      const float x = bits_to_float(float_to_bits(mag) | ((b & 0x80u) << 24));
+      acc[e] = __builtin_fmaf(w, x, acc[e]);
+    }
+  }
+  __device__ __forceinline__ static void fast(float (&)[E], const uint32_t*, float, float) {}
+  __device__ __forceinline__ static void slow(float (&)[E], const uint32_t*, float, float) {}
 };
 
 template <int VB>
@@ -722,7 +743,8 @@ __device__ __forceinline__ bool pool_bags(const LookupArgs& a, const TableDesc& 
           }
 #pragma unroll
           for (int c = 0; c < C; ++c) {
-            if constexpr (PRESCALE) Acc::fast(acc[c], raw[e][c], m.scale, m.bias);
+            if constexpr (TY == ST_FP8) Acc::fp8(acc[c], raw[e][c], m.scale, a.fp8_shift, a.fp8_mult);
+            else if constexpr (PRESCALE) Acc::fast(acc[c], raw[e][c], m.scale, m.bias);
             else Acc::slow(acc[c], raw[e][c], m.scale, m.bias);
           }
         }
@@ -837,6 +859,7 @@ __device__ __forceinline__ void run_item(const LookupArgs& a, int64_t wave, int 
     case ST_INT2: pool_dispatch_vb<index_t, GENERAL, ST_INT2>(a, d, table, first_slot, lane, stage_row, stage_mul); break;
     case ST_FP32: pool_dispatch_vb<index_t, GENERAL, ST_FP32>(a, d, table, first_slot, lane, stage_row, stage_mul); break;
     case ST_BF16: pool_dispatch_vb<index_t, GENERAL, ST_BF16>(a, d, table, first_slot, lane, stage_row, stage_mul); break;
+    case ST_FP8: pool_dispatch_vb<index_t, GENERAL, ST_FP8>(a, d, table, first_slot, lane, stage_row, stage_mul); break;
     default: break;
   }
 #endif

@@ -37,14 +37,14 @@ __device__ __forceinline__ int64_t s_read(const void* p, bool is64, int64_t i) {
 }
 
 __device__ __forceinline__ int s_type_bits(int ty) {
-  return ty == ST_FP32 ? 32 : (ty == ST_FP16 || ty == ST_BF16) ? 16 : ty == ST_INT8 ? 8 : ty == ST_INT4 ? 4 : 2;
+  return ty == ST_FP32 ? 32 : (ty == ST_FP16 || ty == ST_BF16) ? 16 : (ty == ST_INT8 || ty == ST_FP8) ? 8 : ty == ST_INT4 ? 4 : 2;
 }
 
 template <typename index_t>
 __global__ __launch_bounds__(256) void sequence_lookup_kernel(
     const TableDesc* tables, const uint8_t* w0, const uint8_t* w1, const index_t* indices, const void* offsets,
     int off64, int32_t B, int32_t T, int64_t total_L, int32_t D, int32_t out_ty, void* out, int32_t lpr,
-    Status* status) {
+    int32_t fp8_shift, float fp8_mult, Status* status) {
   __shared__ int64_t bounds[MAX_LDS_TABLES + 1];
   const bool in_lds = T <= MAX_LDS_TABLES;
   if (in_lds) {
@@ -99,7 +99,7 @@ __global__ __launch_bounds__(256) void sequence_lookup_kernel(
       continue;
     }
     const int bits = s_type_bits(d.ty);
-    const bool quant = bits <= 8;
+    const bool quant = bits <= 8 && d.ty != ST_FP8;
     float scale = 1.0f, bias = 0.0f;
     if (quant && ok) {
       const uint8_t* ph = row + d.sb_off;
@@ -122,6 +122,11 @@ __global__ __launch_bounds__(256) void sequence_lookup_kernel(
           } else if (bits == 16) {
             const uint16_t u = reinterpret_cast<const uint16_t*>(data)[j];
             x = __builtin_fmaf(1.0f, d.ty == ST_BF16 ? s_bits_to_float((uint32_t)u << 16) : s_half_to_float(u), 0.0f);
+          } else if (d.ty == ST_FP8) {
+            // Float8ToFloat_ref (src/RefImplementations.cc:184-214), then the bag of one: fma(1, x, 0)
+            const uint32_t b = data[j];
+            const float mag = s_bits_to_float((b & 0x7fu) << fp8_shift) * fp8_mult;
+            x = __builtin_fmaf(1.0f, s_bits_to_float(s_float_to_bits(mag) | ((b & 0x80u) << 24)), 0.0f);
           } else {
             const int epb = 8 / bits;
             const uint32_t q = ((uint32_t)data[j / epb] >> ((j % epb) * bits)) & ((1u << bits) - 1);
@@ -150,7 +155,8 @@ __global__ __launch_bounds__(256) void sequence_lookup_kernel(
 
 hipError_t launch_sequence_lookup(const TableDesc* tables, const uint8_t* w0, const uint8_t* w1, const void* indices,
                                   bool idx64, const void* offsets, int32_t B, int32_t T, int64_t total_L, int32_t D,
-                                  int32_t out_ty, void* out, Status* status, hipStream_t stream) {
+                                  int32_t out_ty, void* out, int32_t fp8_shift, float fp8_mult, Status* status,
+                                  hipStream_t stream) {
   if (total_L <= 0 || D <= 0) return hipSuccess;
   const int64_t row_units = out_ty == ST_INT8 ? (D + 4 + 3) / 4 : out_ty == ST_INT4 ? ((D + 9) / 2 + 3) / 4 : (D + SRUN - 1) / SRUN;
   int lpr = 1;
@@ -161,10 +167,10 @@ hipError_t launch_sequence_lookup(const TableDesc* tables, const uint8_t* w0, co
   const dim3 grid((unsigned)blocks), block(256);
   if (idx64)
     hipLaunchKernelGGL(sequence_lookup_kernel<int64_t>, grid, block, 0, stream, tables, w0, w1, (const int64_t*)indices,
-                       offsets, 1, B, T, total_L, D, out_ty, out, lpr, status);
+                       offsets, 1, B, T, total_L, D, out_ty, out, lpr, fp8_shift, fp8_mult, status);
   else
     hipLaunchKernelGGL(sequence_lookup_kernel<int32_t>, grid, block, 0, stream, tables, w0, w1, (const int32_t*)indices,
-                       offsets, 0, B, T, total_L, D, out_ty, out, lpr, status);
+                       offsets, 0, B, T, total_L, D, out_ty, out, lpr, fp8_shift, fp8_mult, status);
   return hipGetLastError();
 }
 

@@ -89,12 +89,11 @@ Tensor int_nbit_split_embedding_codegen_lookup_function_hip(
     int64_t max_float16_D, int64_t max_float32_D, Tensor indices, Tensor offsets, int64_t pooling_mode,
     std::optional<Tensor> indice_weights, int64_t output_dtype, std::optional<Tensor> /*lxu_cache_weights*/,
     std::optional<Tensor> lxu_cache_locations, std::optional<int64_t> row_alignment,
-    std::optional<int64_t> max_float8_D, std::optional<int64_t> /*fp8_exponent_bits*/,
-    std::optional<int64_t> /*fp8_exponent_bias*/) {
+    std::optional<int64_t> max_float8_D, std::optional<int64_t> fp8_exponent_bits,
+    std::optional<int64_t> fp8_exponent_bias) {
   TORCH_CHECK(dev_weights.is_cuda() && indices.is_cuda() && offsets.is_cuda(), "fbgemm_amd: tensors must be on the GPU");
   TORCH_CHECK(pooling_mode == FBGEMM_AMD_POOL_SUM || pooling_mode == FBGEMM_AMD_POOL_MEAN || pooling_mode == FBGEMM_AMD_POOL_NONE,
               "fbgemm_amd: unknown pooling mode ", pooling_mode);
-  TORCH_CHECK(!max_float8_D || *max_float8_D == 0, "fbgemm_amd: FP8 tables are not on this path");
   TORCH_CHECK(!lxu_cache_locations || lxu_cache_locations->numel() == 0,
               "fbgemm_amd: the LXU cache is not on this path (tables are resident in HBM)");
   TORCH_CHECK(indices.scalar_type() == at::kInt || indices.scalar_type() == at::kLong, "indices must be int32 or int64");
@@ -110,13 +109,19 @@ Tensor int_nbit_split_embedding_codegen_lookup_function_hip(
   std::lock_guard<std::mutex> lk(g_mu);
   fbgemm_amd_tbe_plan* plan = plan_for(dev_weights, uvm_weights, weights_placements, weights_offsets, weights_tys,
                                        D_offsets, align);
+  if (max_float8_D && *max_float8_D > 0) {
+    TORCH_CHECK(fp8_exponent_bits && fp8_exponent_bias && *fp8_exponent_bits > 0 && *fp8_exponent_bias >= 0,
+                "FP8 tables need fp8_exponent_bits and fp8_exponent_bias");
+    TORCH_CHECK(fbgemm_amd_tbe_plan_set_fp8(plan, (int32_t)*fp8_exponent_bits, (int32_t)*fp8_exponent_bias) == 0,
+                "fbgemm_amd: ", fbgemm_amd_last_error());
+  }
   const int64_t T = D_offsets.numel() - 1;
   TORCH_CHECK(T > 0 && total_D > 0);
   const int64_t B = (offsets.numel() - 1) / T;
   TORCH_CHECK(B >= 0);
   if (pooling_mode == FBGEMM_AMD_POOL_NONE) {
     // embedding_forward_quantized_host_cpu.cpp:113-139: one row per index, D = the largest max_*_D
-    const int64_t D = std::max({max_int2_D, max_int4_D, max_int8_D, max_float16_D, max_float32_D});
+    const int64_t D = std::max({max_int2_D, max_int4_D, max_int8_D, max_float16_D, max_float32_D, max_float8_D.value_or(0)});
     const int64_t total_L = indices.numel();
     Tensor out;
     if (output_dtype == FBGEMM_AMD_INT8 || output_dtype == FBGEMM_AMD_INT4)
@@ -142,6 +147,30 @@ Tensor int_nbit_split_embedding_codegen_lookup_function_hip(
       st.data_ptr(), current_stream(dev_weights));
   TORCH_CHECK(rc == 0, "fbgemm_amd: ", fbgemm_amd_last_error());
   return out;
+}
+
+// The operator the reference's module calls when it owns a UVM cache
+// (embedding_forward_quantized_host_cpu.cpp:323-329): the same forward. Here
+// every table is resident in HBM, so the cache arguments must be absent.
+Tensor int_nbit_split_embedding_uvm_caching_codegen_lookup_function_hip(
+    Tensor dev_weights, Tensor uvm_weights, Tensor weights_placements, Tensor weights_offsets, Tensor weights_tys,
+    Tensor D_offsets, int64_t total_D, int64_t max_int2_D, int64_t max_int4_D, int64_t max_int8_D,
+    int64_t max_float16_D, int64_t max_float32_D, Tensor indices, Tensor offsets, int64_t pooling_mode,
+    std::optional<Tensor> indice_weights, int64_t output_dtype, std::optional<Tensor> lxu_cache_weights,
+    std::optional<Tensor> lxu_cache_locations, std::optional<int64_t> row_alignment,
+    std::optional<int64_t> max_float8_D, std::optional<int64_t> fp8_exponent_bits,
+    std::optional<int64_t> fp8_exponent_bias, std::optional<Tensor> cache_hash_size_cumsum,
+    std::optional<int64_t> total_cache_hash_size, std::optional<Tensor> /*cache_index_table_map*/,
+    std::optional<Tensor> /*lxu_cache_state*/, std::optional<Tensor> /*lxu_state*/) {
+  TORCH_CHECK((!cache_hash_size_cumsum || cache_hash_size_cumsum->numel() == 0) &&
+                  (!total_cache_hash_size || *total_cache_hash_size <= 0),
+              "fbgemm_amd: the UVM cache is not on this path (tables are resident in HBM)");
+  return int_nbit_split_embedding_codegen_lookup_function_hip(
+      std::move(dev_weights), std::move(uvm_weights), std::move(weights_placements), std::move(weights_offsets),
+      std::move(weights_tys), std::move(D_offsets), total_D, max_int2_D, max_int4_D, max_int8_D, max_float16_D,
+      max_float32_D, std::move(indices), std::move(offsets), pooling_mode, std::move(indice_weights), output_dtype,
+      std::move(lxu_cache_weights), std::move(lxu_cache_locations), row_alignment.value_or(-1) > 0 ? row_alignment : std::nullopt,
+      max_float8_D, fp8_exponent_bits, fp8_exponent_bias);
 }
 
 // Out-of-range indices are recorded on the device and do not stop the stream
@@ -319,6 +348,12 @@ TORCH_LIBRARY_FRAGMENT(fbgemm, m) {
   m.def(
       "pruned_array_lookup(Tensor indices, Tensor offsets, Tensor index_remappings, Tensor index_remappings_offsets) -> Tensor");
 #endif
+#ifndef FBGEMM_AMD_IMPL_ONLY
+  m.def(
+      "int_nbit_split_embedding_uvm_caching_codegen_lookup_function(Tensor dev_weights, Tensor uvm_weights, Tensor weights_placements, Tensor weights_offsets, Tensor weights_tys, Tensor D_offsets, SymInt total_D, int max_int2_D, int max_int4_D, int max_int8_D, int max_float16_D, int max_float32_D, Tensor indices, Tensor offsets, int pooling_mode, Tensor? indice_weights=None, int output_dtype=1, Tensor? lxu_cache_weights=None, Tensor? lxu_cache_locations=None, int? row_alignment=-1, int? max_float8_D=0, int? fp8_exponent_bits=-1, int? fp8_exponent_bias=-1, Tensor? cache_hash_size_cumsum=None, int? total_cache_hash_size=-1, Tensor? cache_index_table_map=None, Tensor? lxu_cache_state=None, Tensor? lxu_state=None) -> Tensor");
+#endif
+  m.impl("int_nbit_split_embedding_uvm_caching_codegen_lookup_function",
+         torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(int_nbit_split_embedding_uvm_caching_codegen_lookup_function_hip)));
   m.impl("int_nbit_split_embedding_codegen_lookup_function",
          torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(int_nbit_split_embedding_codegen_lookup_function_hip)));
   m.impl("pruned_array_lookup", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(pruned_array_lookup_hip)));

@@ -25,15 +25,16 @@ class SparseType(enum.Enum):
     INT4 = "int4"
     INT2 = "int2"
     BF16 = "bf16"
+    FP8 = "fp8"
 
     def as_int(self):
-        return {"fp32": 0, "fp16": 1, "int8": 2, "int4": 3, "int2": 4, "bf16": 5}[self.value]
+        return {"fp32": 0, "fp16": 1, "int8": 2, "int4": 3, "int2": 4, "bf16": 5, "fp8": 6}[self.value]
 
     def bit_rate(self):
-        return {"fp32": 32, "fp16": 16, "int8": 8, "int4": 4, "int2": 2, "bf16": 16}[self.value]
+        return {"fp32": 32, "fp16": 16, "int8": 8, "int4": 4, "int2": 2, "bf16": 16, "fp8": 8}[self.value]
 
     def is_float(self):
-        return self.value in ("fp32", "fp16", "bf16")
+        return self.value in ("fp32", "fp16", "bf16", "fp8")
 
 
 class PoolingMode(enum.IntEnum):
@@ -74,7 +75,8 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(torch.nn.Module):
     def __init__(self, embedding_specs, feature_table_map=None, index_remapping=None,
                  pooling_mode=PoolingMode.SUM, device=None, bounds_check_mode=BoundsCheckMode.WARNING,
                  weight_lists=None, pruning_hash_load_factor=0.5, use_array_for_index_remapping=True,
-                 output_dtype=SparseType.FP16, row_alignment=None, scale_bias_size_in_bytes=4,
+                 output_dtype=SparseType.FP16, row_alignment=None, fp8_exponent_bits=None, fp8_exponent_bias=None,
+                 scale_bias_size_in_bytes=4,
                  cacheline_alignment=True, reverse_qparam=False, indices_dtype=torch.int32):
         super().__init__()
         self.current_device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
@@ -115,6 +117,12 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(torch.nn.Module):
 
         self.max_int2_D, self.max_int4_D, self.max_int8_D = max_ty_D(SparseType.INT2), max_ty_D(SparseType.INT4), max_ty_D(SparseType.INT8)
         self.max_float16_D, self.max_float32_D = max(max_ty_D(SparseType.FP16), max_ty_D(SparseType.BF16)), max_ty_D(SparseType.FP32)
+        self.max_float8_D = max_ty_D(SparseType.FP8)
+        if self.max_float8_D > 0:
+            # split_table_batched_embeddings_ops_inference.py: FP8 tables need both parameters
+            assert fp8_exponent_bits is not None and fp8_exponent_bias is not None, "FP8 tables need fp8_exponent_bits and fp8_exponent_bias"
+        self.fp8_exponent_bits = -1 if fp8_exponent_bits is None else fp8_exponent_bits
+        self.fp8_exponent_bias = -1 if fp8_exponent_bias is None else fp8_exponent_bias
         dev = self.current_device
         self.register_buffer("D_offsets", torch.tensor(D_offsets, device=dev, dtype=torch.int32))
         self.register_buffer("rows_per_table", torch.tensor([rows[t] for t in self.feature_table_map], device=dev, dtype=torch.int64))
@@ -208,6 +216,8 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(torch.nn.Module):
             src = src.to(self.current_device)
             assert tuple(src.shape) == (n, dim)
             if ty.is_float():
+                if ty == SparseType.FP8:
+                    raise NotImplementedError("FP8 rows are assigned as bytes (assign_embedding_weights)")
                 want = {SparseType.FP32: torch.float32, SparseType.FP16: torch.float16, SparseType.BF16: torch.bfloat16}[ty]
                 whole[:, :dim * ty.bit_rate() // 8].copy_(src.to(want).contiguous().view(torch.uint8).view(n, -1))
             else:
@@ -281,6 +291,7 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(torch.nn.Module):
             self.weights_dev, self.weights_uvm, self.weights_placements, self.weights_offsets, self.weights_tys,
             self.D_offsets, self.total_D, self.max_int2_D, self.max_int4_D, self.max_int8_D, self.max_float16_D,
             self.max_float32_D, indices, offsets, int(self.pooling_mode), per_sample_weights, self.output_dtype,
-            row_alignment=self.row_alignment,
+            row_alignment=self.row_alignment, max_float8_D=self.max_float8_D,
+            fp8_exponent_bits=self.fp8_exponent_bits, fp8_exponent_bias=self.fp8_exponent_bias,
             index_remappings=self.index_remappings_array if fuse_remap else None,
             index_remappings_offsets=self.index_remappings_array_offsets if fuse_remap else None)

@@ -18,7 +18,7 @@ import torch
 from . import _lib
 from ._lib import SpmdmConfig, check
 
-FP32, FP16, INT8, INT4, INT2, BF16 = 0, 1, 2, 3, 4, 5
+FP32, FP16, INT8, INT4, INT2, BF16, FP8 = 0, 1, 2, 3, 4, 5, 6
 POOL_SUM, POOL_MEAN, POOL_NONE = 0, 1, 2
 
 _OUT_TORCH = {FP32: torch.float32, FP16: torch.float16, BF16: torch.bfloat16}
@@ -246,8 +246,6 @@ def int_nbit_split_embedding_codegen_lookup_function(
     ``pruned_array_lookup``) fuse the pruned-row remap into the forward:
     ``indices`` are then logical ids."""
     _require_cuda(dev_weights, indices, offsets, indice_weights)
-    if max_float8_D:
-        raise NotImplementedError("FP8 tables are not on this path")
     if lxu_cache_locations is not None and lxu_cache_locations.numel() > 0:
         raise NotImplementedError("the LXU cache is not on this path: tables are resident in HBM")
     if offsets.dtype != indices.dtype:
@@ -259,7 +257,8 @@ def int_nbit_split_embedding_codegen_lookup_function(
         if plan is None:
             plan = _plan_for(dev_weights, uvm_weights, weights_placements, weights_offsets, weights_tys,
                              D_offsets, row_alignment)
-        D = max(max_int2_D, max_int4_D, max_int8_D, max_float16_D, max_float32_D)
+        D = max(max_int2_D, max_int4_D, max_int8_D, max_float16_D, max_float32_D, max_float8_D or 0)
+        _set_fp8(plan, max_float8_D, fp8_exponent_bits, fp8_exponent_bias)
         total_L = indices.numel()
         if output_dtype in _OUT_TORCH:
             out = torch.zeros((total_L, D), dtype=_OUT_TORCH[output_dtype], device=dev_weights.device)
@@ -291,6 +290,7 @@ def int_nbit_split_embedding_codegen_lookup_function(
     if plan is None:
         plan = _plan_for(dev_weights, uvm_weights, weights_placements, weights_offsets, weights_tys,
                          D_offsets, row_alignment)
+    _set_fp8(plan, max_float8_D, fp8_exponent_bits, fp8_exponent_bias)
     T = plan.T
     if total_D != plan.total_D:
         raise ValueError(f"total_D {total_D} does not match D_offsets[-1] {plan.total_D}")
@@ -314,6 +314,14 @@ def int_nbit_split_embedding_codegen_lookup_function(
         if bits:
             _raise_embedding_error(bits, pos, indices, offsets, plan, B)
     return out
+
+
+def _set_fp8(plan, max_float8_D, exponent_bits, exponent_bias):
+    """FP8 tables need the operator's exponent bits and bias (check_fp8_params of the reference)."""
+    if max_float8_D:
+        if exponent_bits is None or exponent_bias is None or exponent_bits <= 0 or exponent_bias < 0:
+            raise RuntimeError("FP8 tables need fp8_exponent_bits and fp8_exponent_bias")
+        check(_lib.lib().fbgemm_amd_tbe_plan_set_fp8(plan.handle, exponent_bits, exponent_bias))
 
 
 def _raise_embedding_error(bits, pos, indices, offsets, plan, B):

@@ -29,7 +29,8 @@ enum {
   FBGEMM_AMD_INT8 = 2,
   FBGEMM_AMD_INT4 = 3,
   FBGEMM_AMD_INT2 = 4,
-  FBGEMM_AMD_BF16 = 5
+  FBGEMM_AMD_BF16 = 5,
+  FBGEMM_AMD_FP8 = 6
 };
 
 /* Pooling modes (embedding_common.h:34). NONE (one output row per index) has its own entry point,
@@ -172,6 +173,14 @@ int fbgemm_amd_tbe_forward_pruned(
     const float* d_indice_weights, int32_t output_ty, void* d_output,
     const void* d_index_remappings, int32_t remap_bits,
     const int64_t* d_index_remappings_offsets, void* d_status, void* stream);
+
+/* Tables of FBGEMM_AMD_FP8 rows (D bytes per row, no scale/bias) are decoded
+ * with the operator's fp8_exponent_bits / fp8_exponent_bias
+ * (Float8ToFloat_ref, src/RefImplementations.cc:184-214; the pooled arithmetic
+ * is EmbeddingSpMDMFP8_ref's, :1544-1616: acc = fma(w, value, acc)). Set them
+ * before the first forward of a plan that holds such tables; an index of -1 is
+ * skipped as for every other row type. */
+int fbgemm_amd_tbe_plan_set_fp8(fbgemm_amd_tbe_plan* plan, int32_t exponent_bits, int32_t exponent_bias);
 
 /* The forward without pooling (PoolingMode.NONE, "sequence" output;
  * embedding_forward_quantized_host_cpu.cpp:113-139 and

@@ -169,6 +169,50 @@ def spmdm(in_ty, block_size, table, indices, offsets_or_lengths, *, weights=None
     return bool(ok), out
 
 
+def float8_to_float(b, exponent_bits, exponent_bias, impl="oracle"):
+    lib = _lib(impl)
+    fn = lib.oracle_float8_to_float if impl == "oracle" else lib.ref_float8_to_float
+    fn.restype = _c.c_float
+    fn.argtypes = [_c.c_uint8, _c.c_int, _c.c_int]
+    return fn(int(b), exponent_bits, exponent_bias)
+
+
+def spmdm_fp8(block_size, table, indices, offsets_or_lengths, *, weights=None, normalize=False, out_ty=ST_FP32,
+              positional=False, use_offsets=True, output_stride=-1, input_stride=-1, exponent_bits=4,
+              exponent_bias=7, skip_minus_one=False, data_size, output_size=None, impl="oracle"):
+    """Pooled lookup over 8-bit float rows (EmbeddingSpMDMFP8_ref). ``impl="ref"`` takes int64 indices / offsets."""
+    table = np.ascontiguousarray(table, dtype=np.uint8)
+    indices = np.ascontiguousarray(indices)
+    offsets_or_lengths = np.ascontiguousarray(offsets_or_lengths)
+    if output_size is None:
+        output_size = len(offsets_or_lengths) - (1 if use_offsets else 0)
+    stride = block_size if output_stride == -1 else output_stride
+    out = np.zeros(max(output_size, 0) * stride, dtype=out_dtype(out_ty))
+    if weights is not None:
+        weights = np.ascontiguousarray(weights, dtype=np.float32)
+    lib = _lib(impl)
+    if impl == "oracle":
+        fn = lib.oracle_embedding_spmdm_fp8
+        fn.restype = _c.c_int
+        fn.argtypes = [_c.c_int64] * 4 + [_c.c_void_p, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_int, _c.c_void_p,
+                                          _c.c_int, _c.c_void_p, _c.c_int, _c.c_int, _c.c_int, _c.c_int64, _c.c_int64,
+                                          _c.c_int, _c.c_int, _c.c_int]
+        ok = fn(block_size, output_size, len(indices), data_size, _ptr(table), _ptr(indices), _is64(indices),
+                _ptr(offsets_or_lengths), _is64(offsets_or_lengths), _ptr(weights), int(normalize), _ptr(out), out_ty,
+                int(positional), int(use_offsets), output_stride, input_stride, exponent_bits, exponent_bias,
+                int(skip_minus_one))
+    else:
+        assert indices.dtype == np.int64 and offsets_or_lengths.dtype == np.int64 and not skip_minus_one
+        fn = lib.ref_embedding_spmdm_fp8
+        fn.restype = _c.c_int
+        fn.argtypes = [_c.c_int64] * 4 + [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int, _c.c_void_p,
+                                          _c.c_int, _c.c_int, _c.c_int, _c.c_int64, _c.c_int64, _c.c_int, _c.c_int]
+        ok = fn(block_size, output_size, len(indices), data_size, _ptr(table), _ptr(indices), _ptr(offsets_or_lengths),
+                _ptr(weights), int(normalize), _ptr(out), out_ty, int(positional), int(use_offsets), output_stride,
+                input_stride, exponent_bits, exponent_bias)
+    return bool(ok), out
+
+
 def compressed_indices_remap(indices, mapping, offsets, weights=None, impl="oracle"):
     """Compacting remap. Returns (out_indices[:n], out_offsets, out_weights[:n])."""
     indices = np.ascontiguousarray(indices)

@@ -371,3 +371,69 @@ void oracle_float2half_rn_array(const float* in, uint16_t* out, int64_t n) {
 void oracle_float2bf16_array(const float* in, uint16_t* out, int64_t n) {
   for (int64_t i = 0; i < n; ++i) out[i] = oracle_float2bf16(in[i]);
 }
+
+/* ---- 8-bit float rows (hfp8) ------------------------------------------------
+ * Float8ToFloat_ref (src/RefImplementations.cc:184-214): the 7 low bits go to
+ * fp32's exponent / mantissa fields, the value is multiplied by
+ * 2^(127 - exponent_bias), the sign bit is ORed back in. */
+float oracle_float8_to_float(uint8_t input, int exponent_bits, int exponent_bias) {
+  union { uint32_t i; float f; } val, mult;
+  const uint32_t sign = ((uint32_t)input & 0x80u) << 24;
+  val.i = ((uint32_t)input & 0x7fu) << (24 - (8 - exponent_bits));
+  mult.i = (uint32_t)(127 + (127 - exponent_bias)) << 23;
+  val.f *= mult.f;
+  val.i |= sign;
+  return val.f;
+}
+
+/* EmbeddingSpMDMFP8_ref (src/RefImplementations.cc:1544-1616): buf[j] =
+ * fma(w, value(row[j]), buf[j]); no scale/bias; mean and output conversion as
+ * the other kernels. skip_minus_one = 0 is the reference (an index of -1 is
+ * out of range); 1 models the table-batched operator, which skips pruned rows
+ * for every row type. Returns 1, or 0 where the reference returns false. */
+int oracle_embedding_spmdm_fp8(
+    int64_t block_size, int64_t output_size, int64_t index_size, int64_t data_size, const uint8_t* input,
+    const void* indices, int idx64, const void* offsets_or_lengths, int off64, const float* weights,
+    int normalize_by_lengths, void* out, int out_ty, int is_weight_positional, int use_offsets,
+    int64_t output_stride, int64_t input_stride, int exponent_bits, int exponent_bias, int skip_minus_one) {
+  if (output_stride == -1) output_stride = block_size;
+  if (input_stride == -1) input_stride = block_size;
+  float* buf = (float*)malloc(sizeof(float) * (size_t)(block_size > 0 ? block_size : 1));
+  int64_t current = 0;
+  int ok = 1;
+  for (int64_t m = 0; m < output_size && ok; ++m) {
+    memset(buf, 0, sizeof(float) * (size_t)block_size);
+    const int64_t o0 = off64 ? ((const int64_t*)offsets_or_lengths)[m] : ((const int32_t*)offsets_or_lengths)[m];
+    int len;
+    if (use_offsets) {
+      const int64_t o1 = off64 ? ((const int64_t*)offsets_or_lengths)[m + 1] : ((const int32_t*)offsets_or_lengths)[m + 1];
+      len = (int)(o1 - o0);
+    } else {
+      len = (int)o0;
+    }
+    if (current + len > index_size) { ok = 0; break; }
+    for (int i = 0; i < len; ++i) {
+      const int64_t idx = idx64 ? ((const int64_t*)indices)[current] : ((const int32_t*)indices)[current];
+      if (skip_minus_one && idx == -1) { ++current; continue; }
+      if (idx < 0 || idx >= data_size) { ok = 0; break; }
+      float w = 1.0f;
+      if (weights) w = weights[is_weight_positional ? i : current];
+      for (int64_t j = 0; j < block_size; ++j)
+        buf[j] = fmaf(w, oracle_float8_to_float(input[input_stride * idx + j], exponent_bits, exponent_bias), buf[j]);
+      ++current;
+    }
+    if (!ok) break;
+    if (normalize_by_lengths && len) {
+      const float scale = 1.0f / (float)len;
+      for (int64_t j = 0; j < block_size; ++j) buf[j] *= scale;
+    }
+    for (int64_t j = 0; j < block_size; ++j) {
+      const int64_t o = m * output_stride + j;
+      if (out_ty == ST_FP32) ((float*)out)[o] = buf[j];
+      else if (out_ty == ST_BF16) ((uint16_t*)out)[o] = oracle_float2bf16(buf[j]);
+      else ((uint16_t*)out)[o] = oracle_float2half_rn(buf[j]);
+    }
+  }
+  free(buf);
+  return ok && current == index_size;
+}

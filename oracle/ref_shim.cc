@@ -12,6 +12,11 @@
 #include "fbgemm/FloatConversion.h"
 #include "src/RefImplementations.h"
 
+namespace fbgemm {
+// defined in src/RefImplementations.cc with external linkage
+void Float8ToFloat_ref(const uint8_t input, float* output, int exponent_bits, int exponent_bias);
+} // namespace fbgemm
+
 namespace {
 
 enum { ST_FP32 = 0, ST_FP16 = 1, ST_INT8 = 2, ST_INT4 = 3, ST_INT2 = 4, ST_BF16 = 5 };
@@ -146,6 +151,29 @@ void ref_compressed_indices_remap(
         static_cast<int32_t*>(out_indices), static_cast<int32_t*>(out_offsets),
         out_weights);
   }
+}
+
+float ref_float8_to_float(uint8_t input, int exponent_bits, int exponent_bias) {
+  float f = 0.0f;
+  fbgemm::Float8ToFloat_ref(input, &f, exponent_bits, exponent_bias);
+  return f;
+}
+
+// EmbeddingSpMDMFP8_ref (src/RefImplementations.h:275-292); int64 indices and offsets, fp32 or 16-bit output
+int ref_embedding_spmdm_fp8(
+    int64_t block_size, int64_t output_size, int64_t index_size, int64_t data_size, const uint8_t* input,
+    const int64_t* indices, const int64_t* offsets_or_lengths, const float* weights, int normalize_by_lengths,
+    void* out, int out_ty, int is_weight_positional, int use_offsets, int64_t output_stride, int64_t input_stride,
+    int exponent_bits, int exponent_bias) {
+  if (out_ty == ST_FP32)
+    return fbgemm::EmbeddingSpMDMFP8_ref<int64_t, int64_t, float>(
+        block_size, output_size, index_size, data_size, input, indices, offsets_or_lengths, weights,
+        normalize_by_lengths != 0, static_cast<float*>(out), is_weight_positional != 0, use_offsets != 0,
+        output_stride, input_stride, exponent_bits, exponent_bias, false);
+  return fbgemm::EmbeddingSpMDMFP8_ref<int64_t, int64_t, uint16_t>(
+      block_size, output_size, index_size, data_size, input, indices, offsets_or_lengths, weights,
+      normalize_by_lengths != 0, static_cast<uint16_t*>(out), is_weight_positional != 0, use_offsets != 0,
+      output_stride, input_stride, exponent_bits, exponent_bias, out_ty == ST_BF16);
 }
 
 float ref_half2float(uint16_t h) { return fbgemm::cpu_half2float(fbgemm::float16{h}); }
