@@ -13,8 +13,8 @@ import os
 import sys
 from collections import defaultdict
 
-OURS = ("sequence_lookup_kernel", "lookup_kernel", "calibration_copy_kernel", "bag_order_kernel", "lengths_to_offsets",
-        "pruned_array_lookup", "pruned_hashmap_lookup", "bounds_partial_max", "bounds_carry", "bounds_fix_offsets",
+OURS = ("sequence_lookup_kernel", "pruned_array_lookup", "pruned_hashmap_lookup", "lookup_kernel", "calibration_copy_kernel",
+        "bag_order_kernel", "lengths_to_offsets", "bounds_partial_max", "bounds_carry", "bounds_fix_offsets",
         "bounds_check_bags", "dequantize_rowwise", "quantize_rowwise")
 
 

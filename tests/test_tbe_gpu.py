@@ -355,7 +355,8 @@ def test_long_bags_of_nine_chunk_rows(ops, oracle, out_ty):
     the plan lays 7 bags of 9 lanes end to end in a wave, so bags straddle the
     quarters of the wave and one lane idles."""
     rng = np.random.default_rng(1200 + out_ty)
-    specs = [(400, 256, INT4), (300, 256, INT8), (350, 128, INT4), (200, 256, INT4)]
+    # 9, 9 (17 chunks, two per lane), 5, 9, 10 and 12 lanes per bag
+    specs = [(400, 256, INT4), (300, 256, INT8), (350, 128, INT4), (200, 256, INT4), (100, 288, INT4), (100, 352, INT4)]
     T, B = len(specs), 45  # 45 bags: 6 full waves of 7 and a ragged one
     weights, wo, _ = build_weights(rng, specs, 16)
     lens = rng.integers(20, 60, size=T * B)
