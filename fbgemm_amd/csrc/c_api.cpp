@@ -731,6 +731,17 @@ int fbgemm_amd_tbe_forward_pruned(
         HIP_TRY(hipMemcpy(nw.d_xcd_start, xcd_start.data(), sizeof(int64_t) * 9, hipMemcpyHostToDevice));
       }
       HIP_TRY(hipMalloc((void**)&nw.d_order, sizeof(BagEntry) * (size_t)plan->T * (size_t)B));
+      // A caller whose batch size keeps changing would grow this cache without bound: past 16
+      // batch sizes, wait for the launches that may still read the old lists and drop them all.
+      if (plan->work.size() >= 16) {
+        HIP_TRY(hipDeviceSynchronize());
+        for (auto& kv : plan->work) {
+          if (kv.second.d_work) (void)hipFree(kv.second.d_work);
+          if (kv.second.d_order) (void)hipFree(kv.second.d_order);
+          if (kv.second.d_xcd_start) (void)hipFree(kv.second.d_xcd_start);
+        }
+        plan->work.clear();
+      }
       it = plan->work.emplace(std::make_pair(B, use_packed ? 1 : 0), nw).first;
     }
     w = it->second;

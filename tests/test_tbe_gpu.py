@@ -368,3 +368,26 @@ def test_long_bags_of_nine_chunk_rows(ops, oracle, out_ty):
     for pooling, w in ((0, psw), (1, None), (0, None)):
         got, want = run_both(ops, oracle, weights, wo, specs, idx, off, pooling, w, out_ty, 16)
         H.assert_same_bits(got, want, f"nine-chunk rows pooling={pooling} weighted={w is not None} out={out_ty}")
+
+
+def test_many_batch_sizes_reuse_and_recycle_work_lists(ops, oracle):
+    """One plan, 40 different batch sizes (the plan keeps a work list per batch
+    size and recycles them past 16), then the first size again."""
+    rng = np.random.default_rng(1300)
+    specs = [(120, 64, INT4), (80, 32, FP16), (60, 128, INT8)]
+    T = len(specs)
+    weights, wo, _ = build_weights(rng, specs, 16)
+    tys = np.array([s[2] for s in specs], np.uint8)
+    D_offsets = np.concatenate([[0], np.cumsum([s[1] for s in specs])]).astype(np.int32)
+    total_D = int(D_offsets[-1])
+    d = [cu(weights), torch.zeros(0, dtype=torch.uint8, device="cuda"), cu(np.zeros(T, np.int32)), cu(wo), cu(tys), cu(D_offsets)]
+    for B in list(range(1, 41)) + [1, 7]:
+        lens = rng.integers(0, 9, size=T * B)
+        off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+        idx = np.concatenate([rng.integers(0, specs[t][0], size=int(lens[t * B:(t + 1) * B].sum())) for t in range(T)]
+                             + [np.zeros(0, np.int64)]).astype(np.int64)
+        got = ops.int_nbit_split_embedding_codegen_lookup_function(
+            *d, total_D, 0, 64, 128, 32, 0, cu(idx), cu(off), 0, None, FP32, row_alignment=16).cpu().numpy()
+        rc, want = oracle.tbe_forward(weights, wo, tys, D_offsets, total_D, idx, off, 0, None, FP32, 16)
+        assert rc == 0
+        H.assert_same_bits(got, want, f"B={B}")
