@@ -21,6 +21,7 @@ class SpmdmConfig(C.Structure):
         ("block_size", _I64), ("output_stride", _I64), ("input_stride", _I64),
         ("normalize_by_lengths", _I32), ("is_weight_positional", _I32),
         ("use_offsets", _I32), ("scale_bias_last", _I32),
+        ("no_bag", _I32), ("fp8_exponent_bits", _I32), ("fp8_exponent_bias", _I32), ("reserved", _I32),
     ]
 
 

@@ -23,6 +23,9 @@ hipError_t launch_sequence_lookup(const TableDesc* tables, const uint8_t* w0, co
                                   bool idx64, const void* offsets, int32_t B, int32_t T, int64_t total_L, int32_t D,
                                   int32_t out_ty, void* out, int32_t fp8_shift, float fp8_mult, Status* status,
                                   hipStream_t stream);
+hipError_t launch_row_lookup(const TableDesc& d, const uint8_t* table, const void* indices, bool idx64,
+                             const float* weights, int64_t n, int32_t out_ty, void* out, int64_t out_stride_bytes,
+                             int64_t copy_bytes, int32_t fp8_shift, float fp8_mult, Status* status, hipStream_t stream);
 hipError_t launch_calibration_copy(const void* src, void* dst, int64_t bytes, hipStream_t stream);
 hipError_t launch_bounds_check(const int64_t* rows_per_table, int32_t T, void* indices, void* offsets, bool is64,
                                int64_t num_indices, int64_t total_B, int64_t B, const int32_t* B_offsets, int mode,
@@ -246,9 +249,20 @@ int grow(T** buf, int64_t* cap, int64_t need, hipStream_t stream) {
 
 int check_cfg(const fbgemm_amd_spmdm_config* c) {
   if (!c) return fail(FBGEMM_AMD_E_ARG, "config is null");
-  if (type_bits(c->weight_ty) == 0 || c->weight_ty == ST_FP8) return fail(FBGEMM_AMD_E_ARG, "unsupported weight_ty %d", c->weight_ty);
-  if (c->output_ty != ST_FP32 && c->output_ty != ST_FP16 && c->output_ty != ST_BF16)
+  if (type_bits(c->weight_ty) == 0) return fail(FBGEMM_AMD_E_ARG, "unsupported weight_ty %d", c->weight_ty);
+  if (c->weight_ty == ST_FP8 &&
+      (c->fp8_exponent_bits < 1 || c->fp8_exponent_bits > 6 || c->fp8_exponent_bias < 0 || c->fp8_exponent_bias > 253))
+    return fail(FBGEMM_AMD_E_ARG, "fp8 rows need 1..6 exponent bits and a bias in 0..253");
+  const bool float_out = c->output_ty == ST_FP32 || c->output_ty == ST_FP16 || c->output_ty == ST_BF16;
+  if (c->no_bag) {
+    // the combinations the reference has (src/RefImplementations.cc:1235-1288,1352-1376,1466-1484)
+    if (c->weight_ty == ST_INT4 ? c->output_ty != ST_INT4
+                                : (c->weight_ty == ST_INT2 || c->weight_ty == ST_FP8 ||
+                                   !(float_out || (c->weight_ty == ST_INT8 && c->output_ty == ST_INT8))))
+      return fail(FBGEMM_AMD_E_ARG, "no_bag: weight_ty %d has no output_ty %d", c->weight_ty, c->output_ty);
+  } else if (!float_out) {
     return fail(FBGEMM_AMD_E_ARG, "unsupported output_ty %d", c->output_ty);
+  }
   if ((c->index_bits != 32 && c->index_bits != 64) || (c->offset_bits != 32 && c->offset_bits != 64))
     return fail(FBGEMM_AMD_E_ARG, "index_bits/offset_bits must be 32 or 64");
   if (c->block_size <= 0 || c->block_size > (1 << 24)) return fail(FBGEMM_AMD_E_ARG, "bad block_size");
@@ -319,15 +333,16 @@ int fbgemm_amd_spmdm_launch(
   hipStream_t stream = (hipStream_t)stream_;
   if (output_size == 0) {
     // the reference returns (0 == index_size) without touching anything
-    if (index_size != 0) {
+    if (index_size != 0 && !cfg->no_bag) {
       Status h{ERR_LENGTH_MISMATCH, 0, ~0ull};
       HIP_TRY(hipMemcpyAsync(d_status, &h, sizeof(h), hipMemcpyHostToDevice, stream));
       HIP_TRY(hipStreamSynchronize(stream));
     }
     return 0;
   }
-  if (!d_input || !d_out || !d_offsets_or_lengths || (index_size > 0 && !d_indices))
+  if (!d_input || !d_out || (!cfg->no_bag && !d_offsets_or_lengths) || ((index_size > 0 || cfg->no_bag) && !d_indices))
     return fail(FBGEMM_AMD_E_ARG, "null data pointer");
+  if (cfg->no_bag && d_remap) return fail(FBGEMM_AMD_E_ARG, "no_bag has no row-wise-sparse variant");
   if (d_remap && !cfg->scale_bias_last && quantised(cfg->weight_ty))
     return fail(FBGEMM_AMD_E_ARG, "row-wise-sparse lookups use the scale_bias_last layout");
   if (d_remap && cfg->output_ty != ST_FP32)
@@ -369,6 +384,34 @@ int fbgemm_amd_spmdm_launch(
   const int64_t out_stride = cfg->output_stride == -1 ? D : cfg->output_stride;
   if ((ty == ST_FP16 || ty == ST_BF16) && (uintptr_t)d_input % 2) return fail(FBGEMM_AMD_E_ARG, "fp16 table must be 2-byte aligned");
   if (ty == ST_FP32 && (uintptr_t)d_input % 4) return fail(FBGEMM_AMD_E_ARG, "fp32 table must be 4-byte aligned");
+  if (ty == ST_FP8) {
+    a.fp8_shift = 16 + cfg->fp8_exponent_bits;
+    const uint32_t mult_bits = (uint32_t)(127 + (127 - cfg->fp8_exponent_bias)) << 23; // 2^(127 - bias)
+    memcpy(&a.fp8_mult, &mult_bits, 4);
+    d.skip_minus_one = 0; // EmbeddingSpMDMFP8_ref has no pruned-row skip (src/RefImplementations.cc:1584-1587)
+  }
+  if (cfg->no_bag) {
+    // one output row per index; the reference reads exactly output_size indices
+    d.data_bytes = (int32_t)((D * bits + 7) / 8);
+    int64_t out_stride_bytes, copy_bytes = 0;
+    if (ty == ST_INT4) {
+      copy_bytes = d.row_stride;
+      out_stride_bytes = d.row_stride;
+    } else if (cfg->output_ty == ST_INT8) {
+      copy_bytes = std::min(out_stride, d.row_stride);
+      out_stride_bytes = out_stride;
+    } else {
+      out_stride_bytes = out_stride * (cfg->output_ty == ST_FP32 ? 4 : 2);
+      if ((uintptr_t)d_out % (cfg->output_ty == ST_FP32 ? 4 : 2)) return fail(FBGEMM_AMD_E_ARG, "output is not aligned to its elements");
+    }
+    if (ty == ST_FP16 || ty == ST_BF16 || ty == ST_FP32) {
+      if (d.row_stride % (bits / 8)) return fail(FBGEMM_AMD_E_ARG, "rows are not aligned to their elements");
+    }
+    HIP_TRY(launch_row_lookup(d, (const uint8_t*)d_input, d_indices, cfg->index_bits == 64, d_weights, output_size,
+                              cfg->output_ty, d_out, out_stride_bytes, copy_bytes, a.fp8_shift, a.fp8_mult,
+                              (Status*)d_status, stream));
+    return 0;
+  }
   plan_lanes(d, (uintptr_t)d_input, out_stride, has_sb, false);
   d.lanes_recip = (65536 + d.lanes - 1) / d.lanes;
 

@@ -1,5 +1,6 @@
-// gfx950 kernel of the table-batched forward without pooling
-// (PoolingMode.NONE, "sequence" output): one output row per index.
+// gfx950 kernels that write one output row per index: the table-batched
+// forward without pooling (PoolingMode.NONE, "sequence" output) and, at the end
+// of the file, the no_bag mode of the single-table kernels.
 //
 // What the reference's CPU operator does for this mode
 // (fbgemm_gpu/codegen/inference/embedding_forward_quantized_cpu_template.cpp:283-296,390-420):
@@ -38,6 +39,88 @@ __device__ __forceinline__ int64_t s_read(const void* p, bool is64, int64_t i) {
 
 __device__ __forceinline__ int s_type_bits(int ty) {
   return ty == ST_FP32 ? 32 : (ty == ST_FP16 || ty == ST_BF16) ? 16 : (ty == ST_INT8 || ty == ST_FP8) ? 8 : ty == ST_INT4 ? 4 : 2;
+}
+
+// Copy `n_out` bytes of an output row: the first `n_in` from the table row, zeros after.
+__device__ __forceinline__ void copy_row_bytes(const uint8_t* row, bool ok, int64_t n_in, int64_t n_out, uint8_t* orow,
+                                               int sub, int lpr) {
+  for (int64_t b0 = (int64_t)sub * 4; b0 < n_out; b0 += (int64_t)lpr * 4) {
+    uint32_t v = 0;
+    if (ok && b0 + 4 <= n_in && (reinterpret_cast<uintptr_t>(row + b0) & 3) == 0) v = *reinterpret_cast<const uint32_t*>(row + b0);
+    else if (ok) for (int k = 0; k < 4; ++k) if (b0 + k < n_in) v |= (uint32_t)row[b0 + k] << (8 * k);
+    if (b0 + 4 <= n_out && (reinterpret_cast<uintptr_t>(orow + b0) & 3) == 0) *reinterpret_cast<uint32_t*>(orow + b0) = v;
+    else for (int k = 0; k < 4; ++k) if (b0 + k < n_out) orow[b0 + k] = (uint8_t)(v >> (8 * k));
+  }
+}
+
+// One output row of D columns from one table row, as a bag of one with weight w:
+//   quantised rows  out[j] = convert(fma(w * scale, q[j], 0 + w * bias))
+//   plain rows      out[j] = convert(fma(w, x[j], 0))
+// `lpr` lanes share the row, lane `sub` takes runs of SRUN columns. A row that
+// is not there (!ok) gives zeros; columns past the table's own width give zeros.
+__device__ __forceinline__ void emit_row(const TableDesc& d, const uint8_t* row, bool ok, float w, int D, int out_ty,
+                                         uint8_t* orow, int sub, int lpr, int fp8_shift, float fp8_mult) {
+  const int bits = s_type_bits(d.ty);
+  const bool quant = bits <= 8 && d.ty != ST_FP8;
+  float scale = w, bias = 0.0f;
+  if (quant && ok) {
+    const uint8_t* ph = row + d.sb_off;
+    if (d.sb_fp32) {
+      uint32_t h[2];
+      for (int k = 0; k < 2; ++k) {
+        const uint8_t* q = ph + 4 * k;
+        if ((reinterpret_cast<uintptr_t>(q) & 3) == 0) h[k] = *reinterpret_cast<const uint32_t*>(q);
+        else h[k] = q[0] | (q[1] << 8) | (q[2] << 16) | ((uint32_t)q[3] << 24);
+      }
+      scale = w * s_bits_to_float(h[0]);
+      bias = w * s_bits_to_float(h[1]);
+    } else {
+      uint32_t h;
+      if ((reinterpret_cast<uintptr_t>(ph) & 3) == 0) h = *reinterpret_cast<const uint32_t*>(ph);
+      else h = ph[0] | (ph[1] << 8) | (ph[2] << 16) | ((uint32_t)ph[3] << 24);
+      scale = w * s_half_to_float((uint16_t)h);
+      bias = w * s_half_to_float((uint16_t)(h >> 16));
+    }
+  }
+  const uint8_t* data = row + d.data_off;
+  const int Dt = d.D < D ? d.D : D;
+  for (int j0 = sub * SRUN; j0 < D; j0 += lpr * SRUN) {
+    float v[SRUN];
+    for (int k = 0; k < SRUN; ++k) {
+      const int j = j0 + k;
+      float x = 0.0f;
+      if (ok && j < Dt) {
+        if (bits == 32) {
+          x = __builtin_fmaf(w, reinterpret_cast<const float*>(data)[j], 0.0f);
+        } else if (bits == 16) {
+          const uint16_t u = reinterpret_cast<const uint16_t*>(data)[j];
+          x = __builtin_fmaf(w, d.ty == ST_BF16 ? s_bits_to_float((uint32_t)u << 16) : s_half_to_float(u), 0.0f);
+        } else if (d.ty == ST_FP8) {
+          // Float8ToFloat_ref (src/RefImplementations.cc:184-214), then the bag of one: fma(w, x, 0)
+          const uint32_t b = data[j];
+          const float mag = s_bits_to_float((b & 0x7fu) << fp8_shift) * fp8_mult;
+          x = __builtin_fmaf(w, s_bits_to_float(s_float_to_bits(mag) | ((b & 0x80u) << 24)), 0.0f);
+        } else {
+          const int epb = 8 / bits;
+          const uint32_t q = ((uint32_t)data[j / epb] >> ((j % epb) * bits)) & ((1u << bits) - 1);
+          x = __builtin_fmaf(scale, (float)q, 0.0f + bias);
+        }
+      }
+      v[k] = x;
+    }
+    const int n = D - j0 < SRUN ? D - j0 : SRUN;
+    if (out_ty == ST_FP32) {
+      float* op = reinterpret_cast<float*>(orow) + j0;
+      if (n == SRUN && (reinterpret_cast<uintptr_t>(op) & 15) == 0) *reinterpret_cast<float4*>(op) = make_float4(v[0], v[1], v[2], v[3]);
+      else for (int k = 0; k < n; ++k) op[k] = v[k];
+    } else {
+      uint16_t h[SRUN];
+      for (int k = 0; k < SRUN; ++k) h[k] = out_ty == ST_FP16 ? s_to_half(v[k]) : s_to_bf16(v[k]);
+      uint16_t* op = reinterpret_cast<uint16_t*>(orow) + j0;
+      if (n == SRUN && (reinterpret_cast<uintptr_t>(op) & 7) == 0) *reinterpret_cast<uint2*>(op) = make_uint2(h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16));
+      else for (int k = 0; k < n; ++k) op[k] = h[k];
+    }
+  }
 }
 
 template <typename index_t>
@@ -88,66 +171,45 @@ __global__ __launch_bounds__(256) void sequence_lookup_kernel(
     if (copy_rows) {
       // the row as it is stored: header, then elements (what fits the output row)
       const int64_t in_bytes = d.data_off + d.data_bytes;
-      const int64_t n = in_bytes < out_row_bytes ? in_bytes : out_row_bytes;
-      for (int64_t b0 = (int64_t)sub * 4; b0 < out_row_bytes; b0 += (int64_t)lpr * 4) {
-        uint32_t v = 0;
-        if (ok && b0 + 4 <= n && (reinterpret_cast<uintptr_t>(row + b0) & 3) == 0) v = *reinterpret_cast<const uint32_t*>(row + b0);
-        else if (ok) for (int k = 0; k < 4; ++k) if (b0 + k < n) v |= (uint32_t)row[b0 + k] << (8 * k);
-        if (b0 + 4 <= out_row_bytes && (reinterpret_cast<uintptr_t>(orow + b0) & 3) == 0) *reinterpret_cast<uint32_t*>(orow + b0) = v;
-        else for (int k = 0; k < 4; ++k) if (b0 + k < out_row_bytes) orow[b0 + k] = (uint8_t)(v >> (8 * k));
-      }
+      copy_row_bytes(row, ok, in_bytes < out_row_bytes ? in_bytes : out_row_bytes, out_row_bytes, orow, sub, lpr);
       continue;
     }
-    const int bits = s_type_bits(d.ty);
-    const bool quant = bits <= 8 && d.ty != ST_FP8;
-    float scale = 1.0f, bias = 0.0f;
-    if (quant && ok) {
-      const uint8_t* ph = row + d.sb_off;
-      uint32_t h;
-      if ((reinterpret_cast<uintptr_t>(ph) & 3) == 0) h = *reinterpret_cast<const uint32_t*>(ph);
-      else h = ph[0] | (ph[1] << 8) | (ph[2] << 16) | ((uint32_t)ph[3] << 24);
-      scale = 1.0f * s_half_to_float((uint16_t)h);
-      bias = 1.0f * s_half_to_float((uint16_t)(h >> 16));
+    emit_row(d, row, ok, 1.0f, D, out_ty, orow, sub, lpr, fp8_shift, fp8_mult);
+  }
+}
+
+// The single-table kernels' no_bag mode (src/RefImplementations.cc:1235-1288,
+// 1352-1376, 1466-1484): output row m comes from table row indices[m], scaled
+// by weights[m] when weights are given; any index outside [0, num_rows) is an
+// error (-1 included). copy_bytes > 0 selects the byte-copy outputs: that many
+// bytes of the stored row go to the output row and the rest of it stays as it was.
+template <typename index_t>
+__global__ __launch_bounds__(256) void row_lookup_kernel(
+    TableDesc d, const uint8_t* table, const index_t* indices, const float* weights, int64_t n, int32_t out_ty,
+    void* out, int64_t out_stride_bytes, int64_t copy_bytes, int32_t lpr, int32_t fp8_shift, float fp8_mult,
+    Status* status) {
+  const int lane = threadIdx.x & 63;
+  const int sub = lane & (lpr - 1);
+  const int per_wave = 64 / lpr;
+  const int64_t nwaves = (int64_t)gridDim.x * (blockDim.x >> 6);
+  const int64_t ngroups = (n + per_wave - 1) / per_wave;
+  for (int64_t g = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6); g < ngroups; g += nwaves) {
+    const int64_t pos = g * per_wave + lane / lpr;
+    if (pos >= n) continue;
+    const int64_t idx = (int64_t)indices[pos];
+    const bool ok = idx >= 0 && idx < d.num_rows;
+    if (!ok && sub == 0) {
+      atomicOr(&status->bits, ERR_INDEX_OUT_OF_RANGE);
+      atomicMin(&status->first_bad_pos, (unsigned long long)pos);
     }
-    const uint8_t* data = row + d.data_off;
-    const int Dt = d.D < D ? d.D : D; // columns the table has (all tables share D in this mode)
-    for (int j0 = sub * SRUN; j0 < D; j0 += lpr * SRUN) {
-      float v[SRUN];
-      for (int k = 0; k < SRUN; ++k) {
-        const int j = j0 + k;
-        float x = 0.0f;
-        if (ok && j < Dt) {
-          if (bits == 32) {
-            x = __builtin_fmaf(1.0f, reinterpret_cast<const float*>(data)[j], 0.0f);
-          } else if (bits == 16) {
-            const uint16_t u = reinterpret_cast<const uint16_t*>(data)[j];
-            x = __builtin_fmaf(1.0f, d.ty == ST_BF16 ? s_bits_to_float((uint32_t)u << 16) : s_half_to_float(u), 0.0f);
-          } else if (d.ty == ST_FP8) {
-            // Float8ToFloat_ref (src/RefImplementations.cc:184-214), then the bag of one: fma(1, x, 0)
-            const uint32_t b = data[j];
-            const float mag = s_bits_to_float((b & 0x7fu) << fp8_shift) * fp8_mult;
-            x = __builtin_fmaf(1.0f, s_bits_to_float(s_float_to_bits(mag) | ((b & 0x80u) << 24)), 0.0f);
-          } else {
-            const int epb = 8 / bits;
-            const uint32_t q = ((uint32_t)data[j / epb] >> ((j % epb) * bits)) & ((1u << bits) - 1);
-            x = __builtin_fmaf(scale, (float)q, 0.0f + bias);
-          }
-        }
-        v[k] = x;
-      }
-      const int n = D - j0 < SRUN ? D - j0 : SRUN;
-      if (out_ty == ST_FP32) {
-        float* op = reinterpret_cast<float*>(orow) + j0;
-        if (n == SRUN && (reinterpret_cast<uintptr_t>(op) & 15) == 0) *reinterpret_cast<float4*>(op) = make_float4(v[0], v[1], v[2], v[3]);
-        else for (int k = 0; k < n; ++k) op[k] = v[k];
-      } else {
-        uint16_t h[SRUN];
-        for (int k = 0; k < SRUN; ++k) h[k] = out_ty == ST_FP16 ? s_to_half(v[k]) : s_to_bf16(v[k]);
-        uint16_t* op = reinterpret_cast<uint16_t*>(orow) + j0;
-        if (n == SRUN && (reinterpret_cast<uintptr_t>(op) & 7) == 0) *reinterpret_cast<uint2*>(op) = make_uint2(h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16));
-        else for (int k = 0; k < n; ++k) op[k] = h[k];
-      }
+    const uint8_t* row = table + (ok ? idx : 0) * d.row_stride;
+    uint8_t* orow = reinterpret_cast<uint8_t*>(out) + pos * out_stride_bytes;
+    if (copy_bytes > 0) {
+      if (ok) copy_row_bytes(row, true, copy_bytes, copy_bytes, orow, sub, lpr);
+      continue;
     }
+    const float w = weights ? weights[pos] : 1.0f;
+    emit_row(d, row, ok, w, d.D, out_ty, orow, sub, lpr, fp8_shift, fp8_mult);
   }
 }
 
@@ -171,6 +233,26 @@ hipError_t launch_sequence_lookup(const TableDesc* tables, const uint8_t* w0, co
   else
     hipLaunchKernelGGL(sequence_lookup_kernel<int32_t>, grid, block, 0, stream, tables, w0, w1, (const int32_t*)indices,
                        offsets, 0, B, T, total_L, D, out_ty, out, lpr, fp8_shift, fp8_mult, status);
+  return hipGetLastError();
+}
+
+hipError_t launch_row_lookup(const TableDesc& d, const uint8_t* table, const void* indices, bool idx64,
+                             const float* weights, int64_t n, int32_t out_ty, void* out, int64_t out_stride_bytes,
+                             int64_t copy_bytes, int32_t fp8_shift, float fp8_mult, Status* status, hipStream_t stream) {
+  if (n <= 0) return hipSuccess;
+  const int64_t row_units = copy_bytes > 0 ? (copy_bytes + 3) / 4 : (d.D + SRUN - 1) / SRUN;
+  int lpr = 1;
+  while (lpr < 64 && lpr < row_units) lpr <<= 1;
+  const int64_t per_block = 4 * (64 / lpr);
+  int64_t blocks = (n + per_block - 1) / per_block;
+  if (blocks > 256 * 64) blocks = 256 * 64;
+  const dim3 grid((unsigned)blocks), block(256);
+  if (idx64)
+    hipLaunchKernelGGL(row_lookup_kernel<int64_t>, grid, block, 0, stream, d, table, (const int64_t*)indices, weights, n,
+                       out_ty, out, out_stride_bytes, copy_bytes, lpr, fp8_shift, fp8_mult, status);
+  else
+    hipLaunchKernelGGL(row_lookup_kernel<int32_t>, grid, block, 0, stream, d, table, (const int32_t*)indices, weights, n,
+                       out_ty, out, out_stride_bytes, copy_bytes, lpr, fp8_shift, fp8_mult, status);
   return hipGetLastError();
 }
 

@@ -67,13 +67,14 @@ class Status:
 
 
 def _make_kernel(weight_ty, block_size, normalize_by_lengths, is_weight_positional, use_offsets,
-                 output_stride, input_stride, scale_bias_last, output_ty, has_weight, sparse):
+                 output_stride, input_stride, scale_bias_last, output_ty, has_weight, sparse, no_bag=False,
+                 fp8=(0, 0)):
     def kernel(output_size, index_size, data_size, input, indices, offsets_or_lengths, weights, out,
                compressed_indices_table=None, status=None):
         _require_cuda(input, indices, offsets_or_lengths, weights, out, compressed_indices_table)
         if sparse and compressed_indices_table is None:
             raise ValueError("row-wise-sparse kernels need compressed_indices_table")
-        if has_weight != (weights is not None):
+        if has_weight is not None and has_weight != (weights is not None):
             # the reference's generated code is specialised on has_weight; a mismatch is a caller bug
             raise ValueError("weights must be given exactly when has_weight was set")
         if weights is not None and weights.dtype != torch.float32:
@@ -82,11 +83,12 @@ def _make_kernel(weight_ty, block_size, normalize_by_lengths, is_weight_position
             raise TypeError("compressed_indices_table must be int32")
         cfg = SpmdmConfig(
             weight_ty=weight_ty, output_ty=output_ty, index_bits=_bits(indices),
-            offset_bits=_bits(offsets_or_lengths), block_size=block_size,
+            offset_bits=32 if offsets_or_lengths is None else _bits(offsets_or_lengths), block_size=block_size,
             output_stride=output_stride, input_stride=input_stride,
             normalize_by_lengths=int(normalize_by_lengths),
             is_weight_positional=int(is_weight_positional), use_offsets=int(use_offsets),
-            scale_bias_last=int(scale_bias_last))
+            scale_bias_last=int(scale_bias_last), no_bag=int(no_bag), fp8_exponent_bits=fp8[0],
+            fp8_exponent_bias=fp8[1])
         lib = _lib.lib()
         if status is not None:
             check(lib.fbgemm_amd_spmdm_launch(
@@ -110,15 +112,15 @@ def generate_embedding_spmdm_with_strides(
     """GenerateEmbeddingSpMDMWithStrides (FbgemmEmbedding.h:94-117). ``in_ty`` is
     INT8 (fused 8-bit rows), FP16 or FP32; ``out_ty`` FP32 or FP16 (BF16 via
     ``is_bf16_out``). ``prefetch`` is accepted and ignored: the GPU hides
-    latency with loads in flight, not software prefetch."""
-    if no_bag:
-        raise NotImplementedError("no_bag (sequence output) is not on this path")
+    latency with loads in flight, not software prefetch. With ``no_bag`` the
+    kernel writes one row per index (``offsets_or_lengths`` may be None) and
+    ``out_ty`` INT8 copies the rows as stored (the reference's uint8_t output)."""
     if in_ty == FP16 and is_bf16_in:
         in_ty = BF16
     if is_bf16_out:
         out_ty = BF16
     return _make_kernel(in_ty, block_size, normalize_by_lengths, is_weight_positional, use_offsets,
-                        output_stride, input_stride, scale_bias_last, out_ty, has_weight, False)
+                        output_stride, input_stride, scale_bias_last, out_ty, has_weight, False, no_bag)
 
 
 def generate_embedding_spmdm(in_ty, block_size, has_weight, normalize_by_lengths, prefetch=16,
@@ -137,13 +139,28 @@ def generate_embedding_spmdm_nbit_with_strides(
     """GenerateEmbeddingSpMDMNBitWithStrides (FbgemmEmbedding.h:151-174)."""
     if input_bit_rate not in (2, 4):
         raise ValueError("input_bit_rate must be 2 or 4")
-    if no_bag:
-        raise NotImplementedError("no_bag (sequence output) is not on this path")
     if is_bf16_out:
         out_ty = BF16
+    if no_bag:
+        # 4-bit rows copied to a 4-bit output is the one form the reference has
+        # (src/RefImplementations.cc:1466-1474); it returns false for the others
+        if input_bit_rate != 4 or output_bit_rate != 4:
+            return lambda *args, **kwargs: False
+        out_ty = INT4
     return _make_kernel(INT4 if input_bit_rate == 4 else INT2, block_size, normalize_by_lengths,
                         is_weight_positional, use_offsets, output_stride, input_stride,
-                        scale_bias_last, out_ty, has_weight, False)
+                        scale_bias_last, out_ty, has_weight, False, no_bag)
+
+
+def generate_embedding_spmdm_fp8_with_strides(
+        block_size, normalize_by_lengths, is_weight_positional=False, use_offsets=True, output_stride=-1,
+        input_stride=-1, exponent_bits=4, exponent_bias=7, is_bf16_out=False, out_ty=FP32):
+    """GenerateEmbeddingSpMDMFP8WithStrides (FbgemmEmbedding.h:185-203): rows of 8-bit
+    floats without scale/bias. The kernel takes ``weights`` as it comes (None = unweighted)."""
+    if is_bf16_out:
+        out_ty = BF16
+    return _make_kernel(FP8, block_size, normalize_by_lengths, is_weight_positional, use_offsets, output_stride,
+                        input_stride, True, out_ty, None, False, False, (exponent_bits, exponent_bias))
 
 
 def generate_embedding_spmdm_nbit(bit_rate, block_size, has_weight, normalize_by_lengths, prefetch=16,

@@ -74,15 +74,15 @@ int fbgemm_amd_status_read(const void* d_status, void* stream, int32_t* bits, in
 /* ---- single-table pooled lookup ----------------------------------------- *
  *
  * Replaces the kernels returned by fbgemm::GenerateEmbeddingSpMDMWithStrides,
- * GenerateEmbeddingSpMDMNBitWithStrides, GenerateEmbeddingSpMDMRowWiseSparse
- * and GenerateEmbeddingSpMDMNBitRowWiseSparse
- * (include/fbgemm/FbgemmEmbedding.h:94-117,151-174,229-262): the config holds
+ * GenerateEmbeddingSpMDMNBitWithStrides, GenerateEmbeddingSpMDMFP8WithStrides,
+ * GenerateEmbeddingSpMDMRowWiseSparse and GenerateEmbeddingSpMDMNBitRowWiseSparse
+ * (include/fbgemm/FbgemmEmbedding.h:94-117,151-174,185-203,229-262): the config holds
  * what those factories fix at generation time, the launch takes what
  * EmbeddingSpMDMKernelSignature::Type takes (FbgemmEmbedding.h:41-49,211-221).
  */
 typedef struct fbgemm_amd_spmdm_config {
-  int32_t weight_ty;            /* FBGEMM_AMD_INT8/INT4/INT2/FP16/BF16/FP32 */
-  int32_t output_ty;            /* FBGEMM_AMD_FP32/FP16/BF16 */
+  int32_t weight_ty;            /* FBGEMM_AMD_INT8/INT4/INT2/FP16/BF16/FP32/FP8 */
+  int32_t output_ty;            /* FBGEMM_AMD_FP32/FP16/BF16 (no_bag: also INT8/INT4) */
   int32_t index_bits;           /* 32 or 64 */
   int32_t offset_bits;          /* 32 or 64 */
   int64_t block_size;           /* elements per row (D) */
@@ -96,6 +96,19 @@ typedef struct fbgemm_amd_spmdm_config {
   int32_t scale_bias_last;      /* 1: scale/bias after the row data (fp32 pair for
                                    INT8, fp16 pair for INT4/INT2); 0: fp16 pair in
                                    front of the data, and index -1 is skipped */
+  int32_t no_bag;               /* 1: no pooling, one output row per index (the
+                                   factories' no_bag flag, FbgemmEmbedding.h:113,170;
+                                   src/RefImplementations.cc:1235-1288,1352-1376,
+                                   1466-1484): output_size indices, offsets unused,
+                                   d_weights[m] scales row m, -1 is out of range.
+                                   output_ty INT8 (8-bit rows) copies the first
+                                   min(output_stride, input_stride) bytes of each row
+                                   to rows output_stride bytes apart; output_ty INT4
+                                   (4-bit rows, the only output they have) copies
+                                   input_stride bytes to rows input_stride apart */
+  int32_t fp8_exponent_bits;    /* weight_ty FP8 (GenerateEmbeddingSpMDMFP8WithStrides, */
+  int32_t fp8_exponent_bias;    /* FbgemmEmbedding.h:185-203): the format of the rows */
+  int32_t reserved;             /* 0 */
 } fbgemm_amd_spmdm_config;
 
 /* Enqueue one pooled lookup. d_weights may be NULL (unweighted).

@@ -76,7 +76,9 @@ constexpr int output_ty(bool is_bf16_out) {
   else if constexpr (std::is_same_v<OutType, float16> || std::is_same_v<OutType, std::uint16_t>)
     return is_bf16_out ? FBGEMM_AMD_BF16 : FBGEMM_AMD_FP16;
   else if constexpr (std::is_same_v<OutType, bfloat16>) return FBGEMM_AMD_BF16;
-  else static_assert(sizeof(OutType) == 0, "OutType must be float, float16, uint16_t or bfloat16");
+  // rows copied as stored (no_bag only): the C ABI rejects this type for the pooled kernels
+  else if constexpr (std::is_same_v<OutType, std::uint8_t>) return FBGEMM_AMD_INT8;
+  else static_assert(sizeof(OutType) == 0, "OutType must be float, float16, uint16_t, bfloat16 or (no_bag) uint8_t");
 }
 
 inline bool run(const fbgemm_amd_spmdm_config& cfg, std::int64_t output_size, std::int64_t index_size,
@@ -101,8 +103,8 @@ GenerateEmbeddingSpMDMWithStrides(const std::int64_t block_size, bool has_weight
                                   std::int64_t output_stride = -1, std::int64_t input_stride = -1,
                                   bool scale_bias_last = true, bool no_bag = false, bool is_bf16_out = false,
                                   bool is_bf16_in = false) {
-  if (no_bag) throw std::invalid_argument("fbgemm_amd: no_bag (sequence output) is not on this path");
   fbgemm_amd_spmdm_config cfg{};
+  cfg.no_bag = no_bag;
   cfg.weight_ty = detail::weight_ty<InType>(is_bf16_in);
   cfg.output_ty = detail::output_ty<OutType>(is_bf16_out);
   cfg.index_bits = detail::bits_of<IndexType>();
@@ -142,12 +144,19 @@ GenerateEmbeddingSpMDMNBitWithStrides(const int input_bit_rate, const std::int64
                                       bool is_weight_positional = false, bool use_offsets = true,
                                       std::int64_t output_stride = -1, std::int64_t input_stride = -1,
                                       bool scale_bias_last = true, const bool is_bf16_out = false,
-                                      const bool no_bag = false, int /*output_bit_rate*/ = -1) {
+                                      const bool no_bag = false, int output_bit_rate = -1) {
   if (input_bit_rate != 2 && input_bit_rate != 4) throw std::invalid_argument("fbgemm_amd: input_bit_rate must be 2 or 4");
-  if (no_bag) throw std::invalid_argument("fbgemm_amd: no_bag (sequence output) is not on this path");
+  if (output_bit_rate == -1) output_bit_rate = 8 * (int)sizeof(OutType);
   fbgemm_amd_spmdm_config cfg{};
+  cfg.no_bag = no_bag;
   cfg.weight_ty = input_bit_rate == 4 ? FBGEMM_AMD_INT4 : FBGEMM_AMD_INT2;
-  cfg.output_ty = detail::output_ty<OutType>(is_bf16_out);
+  // 4-bit rows to a 4-bit output (bytes copied) is the one no_bag form the reference has
+  // (src/RefImplementations.cc:1466-1474); the call returns false for the others, as the reference does
+  cfg.output_ty = (std::is_same_v<OutType, std::uint8_t> && output_bit_rate == 4) ? FBGEMM_AMD_INT4
+                                                                                     : detail::output_ty<OutType>(is_bf16_out);
+  if (no_bag && !(input_bit_rate == 4 && output_bit_rate == 4 && std::is_same_v<OutType, std::uint8_t>))
+    return [](std::int64_t, std::int64_t, std::int64_t, const std::uint8_t*, const IndexType*, const OffsetType*,
+              const float*, OutType*) { return false; };
   cfg.index_bits = detail::bits_of<IndexType>();
   cfg.offset_bits = detail::bits_of<OffsetType>();
   cfg.block_size = block_size;
@@ -172,6 +181,35 @@ GenerateEmbeddingSpMDMNBit(int bit_rate, const std::int64_t block_size, bool has
                            int prefetch = 16, bool is_weight_positional = false, bool use_offsets = true) {
   return GenerateEmbeddingSpMDMNBitWithStrides<IndexType, OffsetType, OutType>(
       bit_rate, block_size, has_weight, normalize_by_lengths, prefetch, is_weight_positional, use_offsets);
+}
+
+// GenerateEmbeddingSpMDMFP8WithStrides (FbgemmEmbedding.h:185-203): rows of 8-bit floats, no scale/bias
+template <typename IndexType, typename OffsetType = std::int32_t, typename OutType = float>
+typename EmbeddingSpMDMKernelSignature<std::uint8_t, IndexType, OffsetType, OutType>::Type
+GenerateEmbeddingSpMDMFP8WithStrides(const std::int64_t block_size, bool normalize_by_lengths,
+                                     bool is_weight_positional = false, bool use_offsets = true,
+                                     std::int64_t output_stride = -1, std::int64_t input_stride = -1,
+                                     int exponent_bits = 4, int exponent_bias = 7, bool is_bf16_out = false) {
+  fbgemm_amd_spmdm_config cfg{};
+  cfg.weight_ty = FBGEMM_AMD_FP8;
+  cfg.output_ty = detail::output_ty<OutType>(is_bf16_out);
+  cfg.index_bits = detail::bits_of<IndexType>();
+  cfg.offset_bits = detail::bits_of<OffsetType>();
+  cfg.block_size = block_size;
+  cfg.output_stride = output_stride;
+  cfg.input_stride = input_stride;
+  cfg.normalize_by_lengths = normalize_by_lengths;
+  cfg.is_weight_positional = is_weight_positional;
+  cfg.use_offsets = use_offsets;
+  cfg.scale_bias_last = 1;
+  cfg.fp8_exponent_bits = exponent_bits;
+  cfg.fp8_exponent_bias = exponent_bias;
+  // the reference's kernel takes the weights pointer as it comes (no has_weight flag)
+  return [cfg](std::int64_t output_size, std::int64_t index_size, std::int64_t data_size, const std::uint8_t* input,
+               const IndexType* indices, const OffsetType* offsets_or_lengths, const float* weights, OutType* out) {
+    return detail::run(cfg, output_size, index_size, data_size, input, indices, offsets_or_lengths, weights, out,
+                       nullptr, weights != nullptr);
+  };
 }
 
 // GenerateEmbeddingSpMDMRowWiseSparse (FbgemmEmbedding.h:229-243)

@@ -213,6 +213,41 @@ def spmdm_fp8(block_size, table, indices, offsets_or_lengths, *, weights=None, n
     return bool(ok), out
 
 
+def spmdm_nobag(in_ty, block_size, table, indices, *, weights=None, out_ty=ST_FP32, output_stride=-1, input_stride=-1,
+                scale_bias_last=True, data_size, impl="oracle", out=None):
+    """One output row per index (the no_bag mode of EmbeddingSpMDM_ref / EmbeddingSpMDMNBit_ref).
+    out_ty ST_INT8 (8-bit rows) / ST_INT4 (4-bit rows) copy row bytes; the result is then uint8.
+    Returns (ok, out) with out flat, output rows output_stride (INT4: input_stride) elements apart."""
+    table = np.ascontiguousarray(table)
+    indices = np.ascontiguousarray(indices)
+    n = len(indices)
+    if in_ty in (ST_INT4, ST_INT2):
+        stride = (block_size + 1) // 2 + 4 if input_stride == -1 else input_stride
+    else:
+        stride = block_size if output_stride == -1 else output_stride
+    if out is None:
+        out = np.zeros(n * stride, dtype=np.uint8 if out_ty in (ST_INT8, ST_INT4) else out_dtype(out_ty))
+    if weights is not None:
+        weights = np.ascontiguousarray(weights, dtype=np.float32)
+    lib = _lib(impl)
+    if impl == "oracle":
+        fn = lib.oracle_embedding_spmdm_nobag
+        fn.restype = _c.c_int
+        fn.argtypes = [_c.c_int, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_void_p, _c.c_void_p, _c.c_int, _c.c_void_p,
+                       _c.c_void_p, _c.c_int, _c.c_int64, _c.c_int64, _c.c_int]
+        ok = fn(in_ty, block_size, n, data_size, _ptr(table), _ptr(indices), _is64(indices), _ptr(weights), _ptr(out),
+                out_ty, output_stride, input_stride, int(scale_bias_last))
+    else:
+        assert indices.dtype == np.int64
+        fn = lib.ref_embedding_spmdm_nobag
+        fn.restype = _c.c_int
+        fn.argtypes = [_c.c_int, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p,
+                       _c.c_int, _c.c_int64, _c.c_int64, _c.c_int]
+        ok = fn(in_ty, block_size, n, data_size, _ptr(table), _ptr(indices), _ptr(weights), _ptr(out), out_ty,
+                output_stride, input_stride, int(scale_bias_last))
+    return bool(ok), out
+
+
 def compressed_indices_remap(indices, mapping, offsets, weights=None, impl="oracle"):
     """Compacting remap. Returns (out_indices[:n], out_offsets, out_weights[:n])."""
     indices = np.ascontiguousarray(indices)

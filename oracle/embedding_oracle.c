@@ -16,6 +16,8 @@
  * Reference files followed (paths relative to the reference tree):
  *   src/RefImplementations.cc:1196-1425  EmbeddingSpMDM_ref (8-bit, fp16, fp32 rows)
  *   src/RefImplementations.cc:1427-1541  EmbeddingSpMDMNBit_ref (int4 / int2 rows)
+ *   src/RefImplementations.cc:1235-1288,1352-1376,1466-1484  the no_bag branches of both
+ *   src/RefImplementations.cc:184-214,1544-1616  Float8ToFloat_ref, EmbeddingSpMDMFP8_ref
  *   src/RefImplementations.cc:1617-1822  row-wise-sparse variants
  *   src/RefImplementations.cc:2308-2333  compressed_indices_remap_ref
  *   src/RefImplementations.h:428-453     float <-> storage conversions
@@ -436,4 +438,88 @@ int oracle_embedding_spmdm_fp8(
   }
   free(buf);
   return ok && current == index_size;
+}
+
+/* ---- no_bag (one output row per index) of the single-table kernels -------
+ * EmbeddingSpMDM_ref with no_bag (src/RefImplementations.cc:1235-1288 8-bit
+ * rows, :1352-1376 fp16 / bf16 / fp32 rows) and EmbeddingSpMDMNBit_ref with
+ * no_bag (:1466-1484). output_size indices, no offsets:
+ *   8-bit rows, 8-bit output (out_ty == ST_INT8): the first
+ *     min(output_stride, input_stride) bytes of the row are copied, output
+ *     rows are output_stride bytes apart;
+ *   8-bit rows, float output: out[j] = convert(fma(w*scale, q[j], 0 + w*bias));
+ *   plain rows: out[j] = convert(fma(w, x[j], 0));
+ *   4-bit rows (out_ty == ST_INT4, the only combination the reference has):
+ *     input_stride bytes are copied and output rows are input_stride apart.
+ *     The reference lets idx == data_size through there (`idx > data_size`,
+ *     :1478); this restatement keeps that, tests stay away from it.
+ * An index of -1 is out of range in this mode whatever the layout.
+ * Returns 1, or 0 where the reference returns false. */
+int oracle_embedding_spmdm_nobag(
+    int in_ty, int64_t block_size, int64_t output_size, int64_t data_size, const void* input, const void* indices,
+    int idx64, const float* weights, void* out, int out_ty, int64_t output_stride, int64_t input_stride,
+    int scale_bias_last) {
+  const uint8_t* in8 = (const uint8_t*)input;
+  if (output_stride == -1) output_stride = block_size;
+  if (in_ty == ST_INT4 || in_ty == ST_INT2) {
+    if (in_ty != ST_INT4 || out_ty != ST_INT4) return 0;
+    if (input_stride == -1) input_stride = (block_size + 1) / 2 + 4;
+    uint8_t* o = (uint8_t*)out;
+    for (int64_t i = 0; i < output_size; ++i) {
+      const int64_t idx = read_index(indices, idx64, i);
+      if (idx < 0 || idx > data_size) return 0;
+      memcpy(o, in8 + input_stride * idx, (size_t)input_stride);
+      o += input_stride;
+    }
+    return 1;
+  }
+  if (in_ty == ST_INT8) {
+    const int64_t sb = scale_bias_last ? 8 : 4;
+    if (input_stride == -1) input_stride = block_size + sb;
+    for (int64_t m = 0; m < output_size; ++m) {
+      const int64_t idx = read_index(indices, idx64, m);
+      if (idx < 0 || idx >= data_size) return 0;
+      const uint8_t* row = in8 + input_stride * idx;
+      if (out_ty == ST_INT8) {
+        const int64_t w = output_stride < input_stride ? output_stride : input_stride;
+        memcpy((uint8_t*)out + m * output_stride, row, (size_t)w);
+        continue;
+      }
+      float weight = 1.0f;
+      if (weights) weight = weights[m];
+      float scale, bias;
+      if (scale_bias_last) {
+        float f[2];
+        memcpy(f, row + block_size, 8);
+        scale = weight * f[0];
+        bias = weight * f[1];
+      } else {
+        uint16_t h[2];
+        memcpy(h, row, 4);
+        scale = weight * oracle_half2float(h[0]);
+        bias = weight * oracle_half2float(h[1]);
+      }
+      const uint8_t* q = row + (scale_bias_last ? 0 : 4);
+      for (int64_t j = 0; j < block_size; ++j)
+        store_out(out, out_ty, m * output_stride + j, fmaf(scale, (float)q[j], 0.0f + bias));
+    }
+    return 1;
+  }
+  if (input_stride == -1) input_stride = block_size;
+  for (int64_t m = 0; m < output_size; ++m) {
+    const int64_t idx = read_index(indices, idx64, m);
+    if (idx < 0 || idx >= data_size) return 0;
+    float w = 1.0f;
+    if (weights) w = weights[m];
+    for (int64_t j = 0; j < block_size; ++j) {
+      float x;
+      if (in_ty == ST_FP32) x = ((const float*)input)[input_stride * idx + j];
+      else {
+        const uint16_t u = ((const uint16_t*)input)[input_stride * idx + j];
+        x = in_ty == ST_BF16 ? oracle_bf162float(u) : oracle_half2float(u);
+      }
+      store_out(out, out_ty, m * output_stride + j, fmaf(w, x, 0.0f));
+    }
+  }
+  return 1;
 }

@@ -176,6 +176,43 @@ int ref_embedding_spmdm_fp8(
       output_stride, input_stride, exponent_bits, exponent_bias, out_ty == ST_BF16);
 }
 
+// The no_bag branches of EmbeddingSpMDM_ref / EmbeddingSpMDMNBit_ref (src/RefImplementations.cc:1235-1288,
+// 1352-1376, 1466-1484); int64 indices. out_ty ST_INT8 / ST_INT4 select the byte-copy outputs.
+int ref_embedding_spmdm_nobag(
+    int in_ty, int64_t block_size, int64_t output_size, int64_t data_size, const void* input, const int64_t* indices,
+    const float* weights, void* out, int out_ty, int64_t output_stride, int64_t input_stride, int scale_bias_last) {
+  const bool sbl = scale_bias_last != 0;
+  const bool bf16_out = out_ty == ST_BF16;
+  const int32_t* no_offsets = nullptr;
+#define NOBAG(IN, OUT, BF16IN)                                                                              \
+  fbgemm::EmbeddingSpMDM_ref<IN, int64_t, int32_t, OUT>(                                                     \
+      block_size, output_size, output_size, data_size, static_cast<const IN*>(input), indices, no_offsets, \
+      weights, false, static_cast<OUT*>(out), false, true, output_stride, input_stride, sbl, /*no_bag=*/true, \
+      bf16_out, BF16IN)
+  switch (in_ty) {
+    case ST_INT4:
+    case ST_INT2:
+      return fbgemm::EmbeddingSpMDMNBit_ref<int64_t, int32_t, uint8_t>(
+          in_ty == ST_INT4 ? 4 : 2, block_size, output_size, output_size, data_size,
+          static_cast<const uint8_t*>(input), indices, no_offsets, weights, false, static_cast<uint8_t*>(out), false,
+          true, output_stride, input_stride, sbl, false, /*no_bag=*/true, out_ty == ST_INT4 ? 4 : -1);
+    case ST_INT8:
+      if (out_ty == ST_INT8) return NOBAG(uint8_t, uint8_t, false);
+      if (out_ty == ST_FP32) return NOBAG(uint8_t, float, false);
+      return NOBAG(uint8_t, uint16_t, false);
+    case ST_FP32:
+      if (out_ty == ST_FP32) return NOBAG(float, float, false);
+      return NOBAG(float, uint16_t, false);
+    case ST_FP16:
+    case ST_BF16:
+      if (out_ty == ST_FP32) return NOBAG(uint16_t, float, in_ty == ST_BF16);
+      return NOBAG(uint16_t, uint16_t, in_ty == ST_BF16);
+    default:
+      return 0;
+  }
+#undef NOBAG
+}
+
 float ref_half2float(uint16_t h) { return fbgemm::cpu_half2float(fbgemm::float16{h}); }
 uint16_t ref_float2half_rn(float f) { return fbgemm::cpu_float2half_rn(f).val; }
 uint16_t ref_float2bf16(float f) { return fbgemm::cpu_float2bfloat16(f).val; }

@@ -20,6 +20,15 @@ extern "C" int oracle_embedding_spmdm(
     int normalize_by_lengths, void* out, int out_ty, int is_weight_positional, int use_offsets,
     int64_t output_stride, int64_t input_stride, int scale_bias_last, const int32_t* remap);
 extern "C" uint16_t oracle_float2half_rn(float f);
+extern "C" int oracle_embedding_spmdm_nobag(
+    int in_ty, int64_t block_size, int64_t output_size, int64_t data_size, const void* input, const void* indices,
+    int idx64, const float* weights, void* out, int out_ty, int64_t output_stride, int64_t input_stride,
+    int scale_bias_last);
+extern "C" int oracle_embedding_spmdm_fp8(
+    int64_t block_size, int64_t output_size, int64_t index_size, int64_t data_size, const uint8_t* input,
+    const void* indices, int idx64, const void* offsets_or_lengths, int off64, const float* weights,
+    int normalize_by_lengths, void* out, int out_ty, int is_weight_positional, int use_offsets,
+    int64_t output_stride, int64_t input_stride, int exponent_bits, int exponent_bias, int skip_minus_one);
 extern "C" void oracle_quantize_rowwise(const void* input, int half_in, int64_t rows, int32_t cols, int32_t bit_rate,
                                         int32_t sb_float, int32_t layout, int64_t out_stride, uint8_t* output);
 extern "C" void oracle_dequantize_rowwise(const uint8_t* input, int64_t rows, int64_t in_stride, int32_t cols,
@@ -139,6 +148,85 @@ void run_8bit(int64_t D, int batch, int rows, int avg_len, bool weighted, bool n
         (long)D, weighted, normalize);
 }
 
+// no_bag of the 8-bit factory (float rows out, and rows copied as stored) and of the 4-bit one,
+// and the 8-bit-float factory, against the oracle.
+template <typename IndexType>
+void run_no_bag_and_fp8(int64_t D, int n, int rows, unsigned seed) {
+  std::mt19937 rng(seed);
+  const int64_t stride = D + 8;
+  std::vector<uint8_t> table(rows * stride);
+  for (auto& b : table) b = rng() & 0xff;
+  for (int r = 0; r < rows; ++r) {
+    float sb[2] = {0.001f + 0.009f * (rng() % 1000) / 1000.f, -1.f + 2.f * (rng() % 1000) / 1000.f};
+    memcpy(&table[r * stride + D], sb, 8);
+  }
+  std::vector<IndexType> indices(n);
+  for (auto& i : indices) i = rng() % rows;
+  std::vector<float> w(n);
+  for (auto& x : w) x = (float)(rng() % 2000) / 1000.f - 1.f;
+  Dev<uint8_t> d_table(table);
+  Dev<IndexType> d_idx(indices);
+  Dev<float> d_w(w);
+  const int idx64 = sizeof(IndexType) == 8;
+  {
+    std::vector<float> want(n * D, -7.f), init(n * D, -7.f);
+    const int ok_ref = oracle_embedding_spmdm_nobag(FBGEMM_AMD_INT8, D, n, rows, table.data(), indices.data(), idx64, w.data(),
+                                                    want.data(), FBGEMM_AMD_FP32, -1, -1, 1);
+    Dev<float> d_out(init);
+    auto kernel = fbgemm_amd::GenerateEmbeddingSpMDMWithStrides<uint8_t, IndexType, int32_t, float>(
+        D, true, false, 16, false, true, -1, -1, true, /*no_bag=*/true);
+    const bool ok = kernel(n, n, rows, d_table.p, d_idx.p, nullptr, d_w.p, d_out.p);
+    auto got = d_out.host();
+    CHECK(ok && ok_ref && memcmp(got.data(), want.data(), got.size() * 4) == 0, "no_bag 8-bit -> float differs (D %ld)", (long)D);
+  }
+  {
+    std::vector<uint8_t> want(n * stride, 0xA5), init(n * stride, 0xA5);
+    const int ok_ref = oracle_embedding_spmdm_nobag(FBGEMM_AMD_INT8, D, n, rows, table.data(), indices.data(), idx64, nullptr,
+                                                    want.data(), FBGEMM_AMD_INT8, stride, -1, 1);
+    Dev<uint8_t> d_out(init);
+    auto kernel = fbgemm_amd::GenerateEmbeddingSpMDMWithStrides<uint8_t, IndexType, int32_t, uint8_t>(
+        D, false, false, 16, false, true, stride, -1, true, /*no_bag=*/true);
+    const bool ok = kernel(n, n, rows, d_table.p, d_idx.p, nullptr, nullptr, d_out.p);
+    auto got = d_out.host();
+    CHECK(ok && ok_ref && got == want, "no_bag 8-bit row copy differs (D %ld)", (long)D);
+  }
+  if (D % 2 == 0) {
+    const int64_t s4 = D / 2 + 4;
+    std::vector<uint8_t> t4(rows * s4);
+    for (auto& b : t4) b = rng() & 0xff;
+    std::vector<uint8_t> want(n * s4, 0xA5), init(n * s4, 0xA5);
+    const int ok_ref = oracle_embedding_spmdm_nobag(FBGEMM_AMD_INT4, D, n, rows, t4.data(), indices.data(), idx64, nullptr,
+                                                    want.data(), FBGEMM_AMD_INT4, -1, -1, 0);
+    Dev<uint8_t> d_t4(t4), d_out(init);
+    auto kernel = fbgemm_amd::GenerateEmbeddingSpMDMNBitWithStrides<IndexType, int32_t, uint8_t>(
+        4, D, false, false, 16, false, true, -1, -1, false, false, /*no_bag=*/true, /*output_bit_rate=*/4);
+    const bool ok = kernel(n, n, rows, d_t4.p, d_idx.p, nullptr, nullptr, d_out.p);
+    auto got = d_out.host();
+    CHECK(ok && ok_ref && got == want, "no_bag 4-bit row copy differs (D %ld)", (long)D);
+    auto none = fbgemm_amd::GenerateEmbeddingSpMDMNBitWithStrides<IndexType, int32_t, float>(
+        4, D, false, false, 16, false, true, -1, -1, false, false, /*no_bag=*/true);
+    CHECK(!none(n, n, rows, d_t4.p, d_idx.p, nullptr, nullptr, nullptr), "no_bag 4-bit -> float must return false");
+  }
+  {
+    // pooled 8-bit floats: bags of up to 7, weighted, mean
+    std::vector<int32_t> offsets(1, 0);
+    while (offsets.back() < n) offsets.push_back(std::min<int32_t>(n, offsets.back() + rng() % 8));
+    const int batch = (int)offsets.size() - 1;
+    std::vector<uint8_t> t8(rows * D);
+    for (auto& b : t8) b = rng() & 0xff;
+    std::vector<uint16_t> want(batch * D, 0), init(batch * D, 0xBEEF);
+    const int ok_ref = oracle_embedding_spmdm_fp8(D, batch, n, rows, t8.data(), indices.data(), idx64, offsets.data(), 0,
+                                                  w.data(), 1, want.data(), FBGEMM_AMD_FP16, 0, 1, -1, -1, 4, 7, 0);
+    Dev<uint8_t> d_t8(t8);
+    Dev<int32_t> d_off(offsets);
+    Dev<uint16_t> d_out(init);
+    auto kernel = fbgemm_amd::GenerateEmbeddingSpMDMFP8WithStrides<IndexType, int32_t, uint16_t>(D, true);
+    const bool ok = kernel(batch, n, rows, d_t8.p, d_idx.p, d_off.p, d_w.p, d_out.p);
+    auto got = d_out.host();
+    CHECK(ok && ok_ref && got == want, "8-bit-float pooled lookup differs (D %ld)", (long)D);
+  }
+}
+
 // The quantizer templates (names and arguments of include/fbgemm/QuantUtils.h:276-334)
 // against the oracle, after test/QuantUtilsTest.cc's fused row-wise cases.
 void run_quantizers(int rows, int cols, unsigned seed) {
@@ -199,6 +287,10 @@ int main() {
         run_8bit<int64_t, int32_t>(s[2], s[0], s[1], s[3], weighted, normalize, ++seed);
         run_8bit<int32_t, int32_t>(s[2], s[0], s[1], s[3], weighted, normalize, ++seed);
       }
+  for (int D : {2, 8, 40, 86, 128, 256}) {
+    run_no_bag_and_fp8<int64_t>(D, 77, 300, ++seed);
+    run_no_bag_and_fp8<int32_t>(D, 500, 1000, ++seed);
+  }
   for (int cols : {4, 8, 64, 100, 128, 260})
     for (int rows : {1, 7, 130}) run_quantizers(rows, cols, ++seed);
   printf("%s: %d failure(s)\n", failures ? "FAILED" : "PASSED", failures);

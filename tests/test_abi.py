@@ -75,8 +75,11 @@ def test_ops_refuse_cpu_tensors():
         kern(1, 4, 10, t, idx, off, None, torch.zeros(32))
     with pytest.raises(ValueError, match="input_bit_rate"):
         ops.generate_embedding_spmdm_nbit_with_strides(3, 32, False, False)
-    with pytest.raises(NotImplementedError):
-        ops.generate_embedding_spmdm_nbit_with_strides(4, 32, False, False, no_bag=True)
+    # no_bag of 4-bit rows exists for a 4-bit output only; the others return false, as the reference does
+    assert ops.generate_embedding_spmdm_nbit_with_strides(4, 32, False, False, no_bag=True)(0, 0, 0, t, idx, None, None, t) is False
+    with pytest.raises(ValueError, match="no CPU path"):
+        ops.generate_embedding_spmdm_nbit_with_strides(4, 32, False, False, no_bag=True, output_bit_rate=4)(
+            4, 4, 10, t, idx, None, None, torch.zeros(80, dtype=torch.uint8))
 
 
 def test_workload_generators_are_seeded():
