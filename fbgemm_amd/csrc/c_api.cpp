@@ -26,6 +26,9 @@ hipError_t launch_sequence_lookup(const TableDesc* tables, const uint8_t* w0, co
 hipError_t launch_row_lookup(const TableDesc& d, const uint8_t* table, const void* indices, bool idx64,
                              const float* weights, int64_t n, int32_t out_ty, void* out, int64_t out_stride_bytes,
                              int64_t copy_bytes, int32_t fp8_shift, float fp8_mult, Status* status, hipStream_t stream);
+hipError_t launch_float_to_hfp8(const float* input, int64_t n, int32_t ebits, int32_t bias, float max_pos, uint8_t* output,
+                                hipStream_t stream);
+hipError_t launch_hfp8_to_float(const uint8_t* input, int64_t n, int32_t ebits, int32_t bias, float* output, hipStream_t stream);
 hipError_t launch_calibration_copy(const void* src, void* dst, int64_t bytes, hipStream_t stream);
 hipError_t launch_bounds_check(const int64_t* rows_per_table, int32_t T, void* indices, void* offsets, bool is64,
                                int64_t num_indices, int64_t total_B, int64_t B, const int32_t* B_offsets, int mode,
@@ -956,6 +959,27 @@ int fbgemm_amd_dequantize_rowwise(
   if (!d_input || !d_output) return fail(FBGEMM_AMD_E_ARG, "null data pointer");
   HIP_TRY(launch_dequantize_rowwise(d_input, rows, in_row_stride, cols, bit_rate, sb_float, layout, output_ty, d_output,
                                     (hipStream_t)stream));
+  return 0;
+}
+
+int fbgemm_amd_float_to_hfp8(const float* d_input, int64_t n, int32_t ebits, int32_t exponent_bias, float max_pos,
+                             uint8_t* d_output, void* stream) {
+  if (n < 0) return fail(FBGEMM_AMD_E_ARG, "n must not be negative");
+  if (ebits < 1 || ebits > 6 || exponent_bias < 0 || exponent_bias > 126) return fail(FBGEMM_AMD_E_ARG, "hfp8 needs 1..6 exponent bits and a bias in 0..126");
+  if (!(max_pos > 0.0f)) return fail(FBGEMM_AMD_E_ARG, "max_pos must be positive");
+  if (n == 0) return 0;
+  if (!d_input || !d_output) return fail(FBGEMM_AMD_E_ARG, "null data pointer");
+  HIP_TRY(launch_float_to_hfp8(d_input, n, ebits, exponent_bias, max_pos, d_output, (hipStream_t)stream));
+  return 0;
+}
+
+int fbgemm_amd_hfp8_to_float(const uint8_t* d_input, int64_t n, int32_t ebits, int32_t exponent_bias, float* d_output,
+                             void* stream) {
+  if (n < 0) return fail(FBGEMM_AMD_E_ARG, "n must not be negative");
+  if (ebits < 1 || ebits > 6 || exponent_bias < 0 || exponent_bias > 253) return fail(FBGEMM_AMD_E_ARG, "hfp8 needs 1..6 exponent bits and a bias in 0..253");
+  if (n == 0) return 0;
+  if (!d_input || !d_output) return fail(FBGEMM_AMD_E_ARG, "null data pointer");
+  HIP_TRY(launch_hfp8_to_float(d_input, n, ebits, exponent_bias, d_output, (hipStream_t)stream));
   return 0;
 }
 

@@ -24,6 +24,8 @@
 // when one run per lane covers the row.
 #include <hip/hip_runtime.h>
 
+#include <cstring>
+
 #include "lookup_common.h"
 
 namespace fbgemm_amd {
@@ -331,6 +333,68 @@ __global__ __launch_bounds__(256) void dequantize_rowwise_kernel(
   }
 }
 
+// fp32 -> 8-bit float (hfp8), the reference's float_to_hfp8
+// (fbgemm_gpu/include/fbgemm_gpu/quantize_ops_utils.h:29-81; the same steps as
+// FloatToFloat8_ref, src/RefImplementations.cc:126-182): |x| clamped to max_pos;
+// in the normal range a power of two 23 - mbits binades above x is added and
+// subtracted, so that fp32's round-to-nearest-even rounds x to mbits mantissa
+// bits; below the smallest normal 2^(24 - bias - mbits) is added and the low
+// bits of the sum are the code. The sign goes to bit 7.
+__device__ __forceinline__ uint32_t float_to_hfp8(float x, int ebits, int bias, float max_pos) {
+  const int mbits = 7 - ebits;
+  uint32_t u = __builtin_bit_cast(uint32_t, x);
+  const uint32_t sign = u & 0x80000000u;
+  u &= 0x7fffffffu;
+  const float v = __builtin_fminf(__builtin_bit_cast(float, u), max_pos);
+  u = __builtin_bit_cast(uint32_t, v);
+  const float smallest_normal = __builtin_bit_cast(float, (uint32_t)(127 - bias + 1) << 23);
+  if (v >= smallest_normal) {
+    const float bouncer = __builtin_bit_cast(float, (u & 0xff800000u) + ((uint32_t)(23 - mbits) << 23));
+    const float r = (bouncer + v) - bouncer;
+    uint32_t o = (__builtin_bit_cast(uint32_t, r) - ((uint32_t)(127 - bias) << 23)) << (8 - ebits);
+    return ((o | sign) >> 24) & 0xffu;
+  }
+  const float bouncer = __builtin_bit_cast(float, (uint32_t)(127 + (23 + (1 - bias - mbits))) << 23);
+  const float r = bouncer + v;
+  return (__builtin_bit_cast(uint32_t, r) | (sign >> 24)) & 0xffu;
+}
+
+// hfp8 -> fp32 (hfp8_to_float, quantize_ops_utils.h:83-110; Float8ToFloat_ref)
+__device__ __forceinline__ float hfp8_to_float(uint32_t b, int shift, float mult) {
+  const float mag = __builtin_bit_cast(float, (b & 0x7fu) << shift) * mult;
+  return __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, mag) | ((b & 0x80u) << 24));
+}
+
+// Four elements per lane and step: one 16-byte load or store on the fp32 side,
+// one 4-byte access on the code side; the tail (and unaligned buffers) element by element.
+__global__ __launch_bounds__(256) void float_to_hfp8_kernel(const float* in, uint8_t* out, int64_t n, int ebits,
+                                                            int bias, float max_pos) {
+  const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t nthreads = (int64_t)gridDim.x * blockDim.x;
+  const bool vec = (reinterpret_cast<uintptr_t>(in) & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 3) == 0;
+  const int64_t n4 = vec ? n / 4 : 0;
+  for (int64_t i = tid; i < n4; i += nthreads) {
+    const float4 x = reinterpret_cast<const float4*>(in)[i];
+    const uint32_t c = float_to_hfp8(x.x, ebits, bias, max_pos) | (float_to_hfp8(x.y, ebits, bias, max_pos) << 8) |
+        (float_to_hfp8(x.z, ebits, bias, max_pos) << 16) | (float_to_hfp8(x.w, ebits, bias, max_pos) << 24);
+    reinterpret_cast<uint32_t*>(out)[i] = c;
+  }
+  for (int64_t i = n4 * 4 + tid; i < n; i += nthreads) out[i] = (uint8_t)float_to_hfp8(in[i], ebits, bias, max_pos);
+}
+
+__global__ __launch_bounds__(256) void hfp8_to_float_kernel(const uint8_t* in, float* out, int64_t n, int shift, float mult) {
+  const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t nthreads = (int64_t)gridDim.x * blockDim.x;
+  const bool vec = (reinterpret_cast<uintptr_t>(in) & 3) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+  const int64_t n4 = vec ? n / 4 : 0;
+  for (int64_t i = tid; i < n4; i += nthreads) {
+    const uint32_t c = reinterpret_cast<const uint32_t*>(in)[i];
+    reinterpret_cast<float4*>(out)[i] = make_float4(hfp8_to_float(c & 0xffu, shift, mult), hfp8_to_float((c >> 8) & 0xffu, shift, mult),
+                                                    hfp8_to_float((c >> 16) & 0xffu, shift, mult), hfp8_to_float(c >> 24, shift, mult));
+  }
+  for (int64_t i = n4 * 4 + tid; i < n; i += nthreads) out[i] = hfp8_to_float(in[i], shift, mult);
+}
+
 // enough workgroups to fill the device several times over, no more than there is work
 unsigned stream_blocks(int64_t needed) {
   const int64_t cap = 256 * 64;
@@ -385,6 +449,24 @@ hipError_t launch_dequantize_rowwise(const void* input, int64_t rows, int64_t in
   else if (bits == 4) FBGEMM_AMD_LAUNCH_D(4);
   else FBGEMM_AMD_LAUNCH_D(8);
 #undef FBGEMM_AMD_LAUNCH_D
+  return hipGetLastError();
+}
+
+hipError_t launch_float_to_hfp8(const float* input, int64_t n, int32_t ebits, int32_t bias, float max_pos, uint8_t* output,
+                                hipStream_t stream) {
+  if (n <= 0) return hipSuccess;
+  const dim3 grid(stream_blocks((n / 4 + 255) / 256)), block(256);
+  hipLaunchKernelGGL(float_to_hfp8_kernel, grid, block, 0, stream, input, output, n, ebits, bias, max_pos);
+  return hipGetLastError();
+}
+
+hipError_t launch_hfp8_to_float(const uint8_t* input, int64_t n, int32_t ebits, int32_t bias, float* output, hipStream_t stream) {
+  if (n <= 0) return hipSuccess;
+  const uint32_t mult_bits = (uint32_t)(127 + (127 - bias)) << 23; // 2^(127 - bias)
+  float mult;
+  memcpy(&mult, &mult_bits, 4);
+  const dim3 grid(stream_blocks((n / 4 + 255) / 256)), block(256);
+  hipLaunchKernelGGL(hfp8_to_float_kernel, grid, block, 0, stream, input, output, n, 16 + ebits, mult);
   return hipGetLastError();
 }
 

@@ -336,6 +336,30 @@ Tensor fusednbit_sbfront_to_float_or_half(const Tensor& t, int64_t bit_rate, int
   return dequantize_rows(t, bit_rate, false, false, output_dtype);
 }
 
+// FloatToHFP8Quantized / HFP8QuantizedToFloat (fbgemm_gpu/src/quantize_ops/quantize_ops_cpu.cpp:571-620)
+Tensor float_to_hfp8(const Tensor& input, int64_t ebits, int64_t exponent_bias, double max_pos) {
+  TORCH_CHECK(input.is_cuda(), "fbgemm_amd: tensors must be on the GPU");
+  TORCH_CHECK(input.dim() == 2, "Tensor 'input' must have 2 dimension(s). Found ", input.dim());
+  TORCH_CHECK(input.scalar_type() == at::kFloat, "input must be float32");
+  const Tensor in = input.contiguous();
+  Tensor out = at::empty(in.sizes(), in.options().dtype(at::kByte));
+  const int rc = fbgemm_amd_float_to_hfp8(in.data_ptr<float>(), in.numel(), (int32_t)ebits, (int32_t)exponent_bias,
+                                          (float)max_pos, out.data_ptr<uint8_t>(), current_stream(in));
+  TORCH_CHECK(rc == 0, "fbgemm_amd: ", fbgemm_amd_last_error());
+  return out;
+}
+Tensor hfp8_to_float(const Tensor& input, int64_t ebits, int64_t exponent_bias) {
+  TORCH_CHECK(input.is_cuda(), "fbgemm_amd: tensors must be on the GPU");
+  TORCH_CHECK(input.dim() == 2, "Tensor 'input' must have 2 dimension(s). Found ", input.dim());
+  TORCH_CHECK(input.scalar_type() == at::kByte, "input must be uint8");
+  const Tensor in = input.contiguous();
+  Tensor out = at::empty(in.sizes(), in.options().dtype(at::kFloat));
+  const int rc = fbgemm_amd_hfp8_to_float(in.data_ptr<uint8_t>(), in.numel(), (int32_t)ebits, (int32_t)exponent_bias,
+                                          out.data_ptr<float>(), current_stream(in));
+  TORCH_CHECK(rc == 0, "fbgemm_amd: ", fbgemm_amd_last_error());
+  return out;
+}
+
 } // namespace
 
 // The schema strings are the reference's, character for character. When a real
@@ -401,7 +425,12 @@ TORCH_LIBRARY_FRAGMENT(fbgemm, m) {
       "FusedNBitRowwiseQuantizedSBHalfToHalf(Tensor input, int bit_rate) -> Tensor");
   m.def(
       "FusedNBitRowwiseQuantizedSBHalfToFloatOrHalf(Tensor input, int bit_rate, int output_dtype=0, bool scale_bias_last=True) -> Tensor");
+  // quantize_ops_cpu.cpp:670-673
+  m.def("FloatToHFP8Quantized(Tensor input, int ebits, int exponent_bias, float max_pos) -> Tensor");
+  m.def("HFP8QuantizedToFloat(Tensor input, int ebits, int exponent_bias) -> Tensor");
 #endif
+  m.impl("FloatToHFP8Quantized", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(float_to_hfp8)));
+  m.impl("HFP8QuantizedToFloat", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(hfp8_to_float)));
   m.impl("pruned_hashmap_lookup", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(pruned_hashmap_lookup_hip)));
   m.impl("bounds_check_indices", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(bounds_check_indices_hip)));
   m.impl("FloatToFused8BitRowwiseQuantized", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(float_to_fused8bit)));

@@ -474,6 +474,29 @@ def dequantize_rowwise(input, cols, bit_rate, sb_float=False, layout=QLAYOUT_TRA
     return out
 
 
+def float_to_hfp8_quantized(input, ebits, exponent_bias, max_pos):
+    """FloatToHFP8Quantized (fbgemm_gpu/src/quantize_ops/quantize_ops_cpu.cpp:571-594):
+    fp32 ``[rows, cols]`` -> hfp8 codes, uint8, same shape."""
+    _require_cuda(input)
+    if input.dtype != torch.float32 or input.dim() != 2:
+        raise ValueError("input must be a 2-d float32 tensor")
+    input = input.contiguous()
+    out = torch.empty(input.shape, dtype=torch.uint8, device=input.device)
+    check(_lib.lib().fbgemm_amd_float_to_hfp8(_ptr(input), input.numel(), ebits, exponent_bias, float(max_pos), _ptr(out), _stream()))
+    return out
+
+
+def hfp8_quantized_to_float(input, ebits, exponent_bias):
+    """HFP8QuantizedToFloat (quantize_ops_cpu.cpp:596-620): hfp8 codes ``[rows, cols]`` -> fp32."""
+    _require_cuda(input)
+    if input.dtype != torch.uint8 or input.dim() != 2:
+        raise ValueError("input must be a 2-d uint8 tensor")
+    input = input.contiguous()
+    out = torch.empty(input.shape, dtype=torch.float32, device=input.device)
+    check(_lib.lib().fbgemm_amd_hfp8_to_float(_ptr(input), input.numel(), ebits, exponent_bias, _ptr(out), _stream()))
+    return out
+
+
 def pruned_hashmap_insert(indices, dense_indices, offsets, hash_table, hash_table_offsets):
     """pruned_hashmap_insert (embedding_forward_quantized_host_cpu.cpp:331-334;
     embedding_forward_quantized_cpu_template.cpp:124-201): HOST tensors, in place

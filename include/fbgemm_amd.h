@@ -316,6 +316,20 @@ int fbgemm_amd_dequantize_rowwise(
     const void* d_input, int64_t rows, int64_t in_row_stride, int32_t cols, int32_t bit_rate, int32_t sb_float,
     int32_t layout, int32_t output_ty, void* d_output, void* stream);
 
+/* fp32 <-> 8-bit float (hfp8) element-wise, `n` elements: the operators
+ * FloatToHFP8Quantized / HFP8QuantizedToFloat
+ * (fbgemm_gpu/src/quantize_ops/quantize_ops_cpu.cpp:531-620,
+ * fbgemm_gpu/include/fbgemm_gpu/quantize_ops_utils.h:29-110; the same arithmetic as
+ * FloatToFloat8_ref / Float8ToFloat_ref, src/RefImplementations.cc:126-214), which
+ * produce and read back the rows of FP8 tables (quantize_embs,
+ * fbgemm_gpu/fbgemm_gpu/tbe/utils/quantize.py:36-45). |x| is clamped to max_pos,
+ * rounding is to nearest even, values below the smallest normal keep gradual
+ * underflow. */
+int fbgemm_amd_float_to_hfp8(const float* d_input, int64_t n, int32_t ebits, int32_t exponent_bias, float max_pos,
+                             uint8_t* d_output, void* stream);
+int fbgemm_amd_hfp8_to_float(const uint8_t* d_input, int64_t n, int32_t ebits, int32_t exponent_bias, float* d_output,
+                             void* stream);
+
 /* Wait for everything enqueued on `stream` (hipStreamSynchronize), for callers
  * of the asynchronous entry points that hold no HIP headers. */
 int fbgemm_amd_stream_synchronize(void* stream);

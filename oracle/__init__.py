@@ -177,6 +177,35 @@ def float8_to_float(b, exponent_bits, exponent_bias, impl="oracle"):
     return fn(int(b), exponent_bits, exponent_bias)
 
 
+def hfp8_max_pos(exponent_bits, exponent_bias):
+    fn = _lib("oracle").oracle_hfp8_max_pos
+    fn.restype = _c.c_float
+    fn.argtypes = [_c.c_int, _c.c_int]
+    return fn(exponent_bits, exponent_bias)
+
+
+def float_to_hfp8(x, exponent_bits, exponent_bias, max_pos=None, impl="oracle"):
+    """fp32 array -> hfp8 codes (uint8). ``impl="ref"`` is the reference's FloatToFloat8_ref,
+    which computes max_pos itself."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty(x.shape, dtype=np.uint8)
+    lib = _lib(impl)
+    if impl == "oracle":
+        if max_pos is None:
+            max_pos = hfp8_max_pos(exponent_bits, exponent_bias)
+        fn = lib.oracle_float_to_hfp8_array
+        fn.restype = None
+        fn.argtypes = [_c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_int, _c.c_int, _c.c_float]
+        fn(_ptr(x), _ptr(out), x.size, exponent_bits, exponent_bias, max_pos)
+    else:
+        assert max_pos is None
+        fn = lib.ref_float_to_float8_array
+        fn.restype = None
+        fn.argtypes = [_c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_int, _c.c_int]
+        fn(_ptr(x), _ptr(out), x.size, exponent_bits, exponent_bias)
+    return out
+
+
 def spmdm_fp8(block_size, table, indices, offsets_or_lengths, *, weights=None, normalize=False, out_ty=ST_FP32,
               positional=False, use_offsets=True, output_stride=-1, input_stride=-1, exponent_bits=4,
               exponent_bias=7, skip_minus_one=False, data_size, output_size=None, impl="oracle"):

@@ -139,3 +139,45 @@ void oracle_dequantize_rowwise(const uint8_t* input, int64_t rows, int64_t in_st
     }
   }
 }
+
+/* ---- fp32 -> 8-bit float (hfp8) ----------------------------------------------
+ * float_to_hfp8 (fbgemm_gpu/include/fbgemm_gpu/quantize_ops_utils.h:29-81), which is
+ * FloatToFloat8_ref (src/RefImplementations.cc:126-182) with max_pos as an argument:
+ * clamp |x| to max_pos; normal range: round to 7 - ebits mantissa bits by adding and
+ * subtracting a power of two 23 - mbits binades above x (fp32's own round-to-nearest-
+ * even does the rounding), re-bias the exponent, shift the 7 code bits into place;
+ * below the smallest normal 2^(1 - bias): add 2^(24 - bias - mbits), whose low bits
+ * then are the code. The sign goes to bit 7. Pinned by tests/test_hfp8_oracle.py:
+ * against the reference's FloatToFloat8_ref compiled from its sources, and against
+ * "nearest of the 128 representable magnitudes, ties to the even code, saturating".
+ * The decoder is oracle_float8_to_float (embedding_oracle.c). */
+uint8_t oracle_float_to_hfp8(float x, int ebits, int exponent_bias, float max_pos) {
+  const int mbits = 7 - ebits;
+  union { uint32_t i; float f; } v, bouncer, smallest_normal;
+  v.f = x;
+  const uint32_t sign = v.i & 0x80000000u;
+  v.i &= 0x7fffffffu;
+  v.f = fminf(v.f, max_pos);
+  smallest_normal.i = (uint32_t)(127 - exponent_bias + 1) << 23;
+  if (v.f >= smallest_normal.f) {
+    bouncer.i = (v.i & 0xff800000u) + ((uint32_t)(23 - mbits) << 23);
+    volatile float t = bouncer.f + v.f; /* each step rounded to fp32 */
+    v.f = t - bouncer.f;
+    v.i = (v.i - ((uint32_t)(127 - exponent_bias) << 23)) << (8 - ebits);
+    v.i = (v.i | sign) >> 24;
+  } else {
+    bouncer.i = (uint32_t)(127 + (23 + (1 - exponent_bias - mbits))) << 23;
+    v.f = bouncer.f + v.f;
+    v.i = v.i | (sign >> 24);
+  }
+  return (uint8_t)v.i;
+}
+
+/* FloatToFloat8_ref's own max_pos (src/RefImplementations.cc:131-132) */
+float oracle_hfp8_max_pos(int ebits, int exponent_bias) {
+  return (float)((double)(1 << ((1 << ebits) - 2 - exponent_bias)) * (2.0 - pow(2.0, ebits - 7)));
+}
+
+void oracle_float_to_hfp8_array(const float* in, uint8_t* out, int64_t n, int ebits, int exponent_bias, float max_pos) {
+  for (int64_t i = 0; i < n; ++i) out[i] = oracle_float_to_hfp8(in[i], ebits, exponent_bias, max_pos);
+}

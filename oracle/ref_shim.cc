@@ -15,6 +15,7 @@
 namespace fbgemm {
 // defined in src/RefImplementations.cc with external linkage
 void Float8ToFloat_ref(const uint8_t input, float* output, int exponent_bits, int exponent_bias);
+void FloatToFloat8_ref(const float input, uint8_t* output, int exponent_bits, int exponent_bias);
 } // namespace fbgemm
 
 namespace {
@@ -211,6 +212,10 @@ int ref_embedding_spmdm_nobag(
       return 0;
   }
 #undef NOBAG
+}
+
+void ref_float_to_float8_array(const float* in, uint8_t* out, int64_t n, int exponent_bits, int exponent_bias) {
+  for (int64_t i = 0; i < n; ++i) fbgemm::FloatToFloat8_ref(in[i], out + i, exponent_bits, exponent_bias);
 }
 
 float ref_half2float(uint16_t h) { return fbgemm::cpu_half2float(fbgemm::float16{h}); }
