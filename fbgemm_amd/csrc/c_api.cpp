@@ -29,6 +29,11 @@ hipError_t launch_row_lookup(const TableDesc& d, const uint8_t* table, const voi
 hipError_t launch_float_to_hfp8(const float* input, int64_t n, int32_t ebits, int32_t bias, float max_pos, uint8_t* output,
                                 hipStream_t stream);
 hipError_t launch_hfp8_to_float(const uint8_t* input, int64_t n, int32_t ebits, int32_t bias, float* output, hipStream_t stream);
+int64_t prune_partials(int64_t rows);
+hipError_t launch_prune_map(const float* indicator, int64_t rows, double threshold, int use_abs, int64_t min_rows,
+                            bool idx64, void* remap, int64_t* num_kept, int64_t* partial, hipStream_t stream);
+hipError_t launch_prune_gather(const void* in, int64_t rows, int64_t row_bytes, const void* remap, bool idx64, void* out,
+                               int64_t out_rows, hipStream_t stream);
 hipError_t launch_calibration_copy(const void* src, void* dst, int64_t bytes, hipStream_t stream);
 hipError_t launch_bounds_check(const int64_t* rows_per_table, int32_t T, void* indices, void* offsets, bool is64,
                                int64_t num_indices, int64_t total_B, int64_t B, const int32_t* B_offsets, int mode,
@@ -980,6 +985,41 @@ int fbgemm_amd_hfp8_to_float(const uint8_t* d_input, int64_t n, int32_t ebits, i
   if (n == 0) return 0;
   if (!d_input || !d_output) return fail(FBGEMM_AMD_E_ARG, "null data pointer");
   HIP_TRY(launch_hfp8_to_float(d_input, n, ebits, exponent_bias, d_output, (hipStream_t)stream));
+  return 0;
+}
+
+int fbgemm_amd_rowwise_prune_map(const float* d_indicator, int64_t rows, double threshold, int32_t use_abs,
+                                 int64_t min_non_pruned_rows, int32_t index_bits, void* d_remap, int64_t* num_kept,
+                                 void* stream_) {
+  if (rows < 0) return fail(FBGEMM_AMD_E_ARG, "rows must not be negative");
+  if (!(threshold >= 0.0)) return fail(FBGEMM_AMD_E_ARG, "Threshold should be greater than or equal to zero.");
+  if (index_bits != 32 && index_bits != 64) return fail(FBGEMM_AMD_E_ARG, "index_bits must be 32 or 64");
+  if (index_bits == 32 && rows > 0x7fffffffLL) return fail(FBGEMM_AMD_E_ARG, "rows do not fit 32-bit ids");
+  if (!num_kept) return fail(FBGEMM_AMD_E_ARG, "num_kept is null");
+  *num_kept = 0;
+  if (rows == 0) return 0;
+  if (!d_indicator || !d_remap) return fail(FBGEMM_AMD_E_ARG, "null data pointer");
+  hipStream_t stream = (hipStream_t)stream_;
+  std::lock_guard<std::mutex> lk(g_mu);
+  DeviceScratch* s;
+  if (int rc = get_scratch(&s)) return rc;
+  // the block sums, and one more slot for the count that comes back
+  const int64_t np = prune_partials(rows);
+  if (int rc = grow(&s->partial, &s->partial_cap, np + 1, stream)) return rc;
+  HIP_TRY(launch_prune_map(d_indicator, rows, threshold, use_abs, min_non_pruned_rows, index_bits == 64, d_remap,
+                           s->partial + np, s->partial, stream));
+  HIP_TRY(hipMemcpyAsync(num_kept, s->partial + np, sizeof(int64_t), hipMemcpyDeviceToHost, stream));
+  HIP_TRY(hipStreamSynchronize(stream));
+  return 0;
+}
+
+int fbgemm_amd_rowwise_prune_gather(const void* d_weights, int64_t rows, int64_t row_bytes, const void* d_remap,
+                                    int32_t index_bits, void* d_output, int64_t output_rows, void* stream) {
+  if (rows < 0 || row_bytes < 0 || output_rows < 0) return fail(FBGEMM_AMD_E_ARG, "negative size");
+  if (index_bits != 32 && index_bits != 64) return fail(FBGEMM_AMD_E_ARG, "index_bits must be 32 or 64");
+  if (rows == 0 || row_bytes == 0 || output_rows == 0) return 0;
+  if (!d_weights || !d_remap || !d_output) return fail(FBGEMM_AMD_E_ARG, "null data pointer");
+  HIP_TRY(launch_prune_gather(d_weights, rows, row_bytes, d_remap, index_bits == 64, d_output, output_rows, (hipStream_t)stream));
   return 0;
 }
 

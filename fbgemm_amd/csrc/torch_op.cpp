@@ -360,6 +360,39 @@ Tensor hfp8_to_float(const Tensor& input, int64_t ebits, int64_t exponent_bias) 
   return out;
 }
 
+// embedding_bag_rowwise_prune (fbgemm_gpu/src/sparse_ops/sparse_ops_cpu.cpp:2773-2893)
+std::tuple<Tensor, Tensor> rowwise_prune(const Tensor& weights, const Tensor& indicator, double threshold,
+                                         at::ScalarType compressed_indices_dtype, bool abs, c10::SymInt min_non_pruned_rows_,
+                                         std::optional<double> min_save_ratio) {
+  TORCH_CHECK(weights.is_cuda() && indicator.is_cuda(), "fbgemm_amd: tensors must be on the GPU");
+  TORCH_CHECK(weights.dim() == 2, "Tensor 'weights' must have 2 dimension(s). Found ", weights.dim());
+  TORCH_CHECK(indicator.numel() == weights.size(0),
+              "Number of elements in 'indicator' should be equivalent to number of rows in 'weights'.");
+  TORCH_CHECK(threshold >= 0.0, "Threshold should be greater than or equal to zero.");
+  TORCH_CHECK(compressed_indices_dtype == at::kInt || compressed_indices_dtype == at::kLong,
+              "'compressed_indices_dtype' should be Int/Long.");
+  const int64_t min_rows = min_non_pruned_rows_.expect_int();
+  const int64_t rows = weights.size(0), cols = weights.size(1);
+  if (min_save_ratio.has_value() &&
+      !((double)(rows * 4 + min_rows * cols * 4) < *min_save_ratio * (double)(4 * weights.numel()))) {
+    Tensor one = at::zeros({1}, weights.options().dtype(compressed_indices_dtype));
+    return {weights, one};
+  }
+  const Tensor w = weights.contiguous();
+  const Tensor ind = indicator.to(at::kFloat).contiguous();
+  Tensor remap = at::empty({rows}, w.options().dtype(compressed_indices_dtype));
+  const int32_t bits = compressed_indices_dtype == at::kLong ? 64 : 32;
+  int64_t kept = 0;
+  int rc = fbgemm_amd_rowwise_prune_map(ind.data_ptr<float>(), rows, threshold, abs ? 1 : 0, min_rows, bits,
+                                        remap.data_ptr(), &kept, current_stream(w));
+  TORCH_CHECK(rc == 0, "fbgemm_amd: ", fbgemm_amd_last_error());
+  Tensor out = at::empty({kept, cols}, w.options());
+  rc = fbgemm_amd_rowwise_prune_gather(w.data_ptr(), rows, cols * (int64_t)w.element_size(), remap.data_ptr(), bits,
+                                       out.data_ptr(), kept, current_stream(w));
+  TORCH_CHECK(rc == 0, "fbgemm_amd: ", fbgemm_amd_last_error());
+  return {out, remap};
+}
+
 } // namespace
 
 // The schema strings are the reference's, character for character. When a real
@@ -425,10 +458,14 @@ TORCH_LIBRARY_FRAGMENT(fbgemm, m) {
       "FusedNBitRowwiseQuantizedSBHalfToHalf(Tensor input, int bit_rate) -> Tensor");
   m.def(
       "FusedNBitRowwiseQuantizedSBHalfToFloatOrHalf(Tensor input, int bit_rate, int output_dtype=0, bool scale_bias_last=True) -> Tensor");
+  // fbgemm_gpu/src/sparse_ops/sparse_ops_cpu.cpp:3891-3892
+  m.def(
+      "embedding_bag_rowwise_prune(Tensor weight, Tensor indicator, float threshold, ScalarType compressed_indices_dtype, bool abs=True, SymInt min_num_rows=0, float? min_save_ratio=1.0) -> (Tensor, Tensor)");
   // quantize_ops_cpu.cpp:670-673
   m.def("FloatToHFP8Quantized(Tensor input, int ebits, int exponent_bias, float max_pos) -> Tensor");
   m.def("HFP8QuantizedToFloat(Tensor input, int ebits, int exponent_bias) -> Tensor");
 #endif
+  m.impl("embedding_bag_rowwise_prune", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(rowwise_prune)));
   m.impl("FloatToHFP8Quantized", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(float_to_hfp8)));
   m.impl("HFP8QuantizedToFloat", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(hfp8_to_float)));
   m.impl("pruned_hashmap_lookup", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(pruned_hashmap_lookup_hip)));

@@ -206,9 +206,11 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(torch.nn.Module):
             else:
                 assert dest[1] is None
 
-    def quantize_and_assign(self, fp_weight_list):
+    def quantize_and_assign(self, fp_weight_list, fp8_max_position=None):
         """fp32 / fp16 tables -> this module's rows, on the GPU (the producer the
-        reference runs on the CPU: tbe/utils/quantize.py:20-72)."""
+        reference runs on the CPU: tbe/utils/quantize.py:20-72). FP8 tables take the
+        clamp of FP8QuantizationConfig (``fp8_max_position``; default: the largest
+        value the format holds below its top exponent)."""
         self.initialize_weights()
         assert len(fp_weight_list) == len(self.embedding_specs)
         rows = self.split_embedding_weights_with_scale_bias(0)
@@ -217,7 +219,12 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(torch.nn.Module):
             assert tuple(src.shape) == (n, dim)
             if ty.is_float():
                 if ty == SparseType.FP8:
-                    raise NotImplementedError("FP8 rows are assigned as bytes (assign_embedding_weights)")
+                    eb, bias = self.fp8_exponent_bits, self.fp8_exponent_bias
+                    max_pos = fp8_max_position
+                    if max_pos is None:  # split_embedding_configs.py:317-318
+                        max_pos = (1 << ((1 << eb) - 2 - bias)) * (2 - 2 ** (eb - 7))
+                    whole[:, :dim].copy_(ops.float_to_hfp8_quantized(src.float(), eb, bias, max_pos))
+                    continue
                 want = {SparseType.FP32: torch.float32, SparseType.FP16: torch.float16, SparseType.BF16: torch.bfloat16}[ty]
                 whole[:, :dim * ty.bit_rate() // 8].copy_(src.to(want).contiguous().view(torch.uint8).view(n, -1))
             else:

@@ -497,6 +497,39 @@ def hfp8_quantized_to_float(input, ebits, exponent_bias):
     return out
 
 
+def embedding_bag_rowwise_prune(weight, indicator, threshold, compressed_indices_dtype, abs=True, min_num_rows=0,
+                                min_save_ratio=1.0):
+    """embedding_bag_rowwise_prune (fbgemm_gpu/src/sparse_ops/sparse_ops_cpu.cpp:2836-2893), on the GPU:
+    keeps the rows of ``weight`` whose ``indicator`` exceeds ``threshold`` (and the last rows needed to
+    reach ``min_num_rows``); returns (kept rows, remap) with remap[i] the new row id or -1. When
+    pruning would not save memory (``min_save_ratio``) the weights come back whole with the map [0]."""
+    _require_cuda(weight, indicator)
+    if weight.dim() != 2:
+        raise ValueError("Tensor 'weights' must have 2 dimension(s)")
+    if indicator.numel() != weight.size(0):
+        raise ValueError("Number of elements in 'indicator' should be equivalent to number of rows in 'weights'.")
+    if not threshold >= 0.0:
+        raise ValueError("Threshold should be greater than or equal to zero.")
+    if compressed_indices_dtype not in (torch.int32, torch.int64):
+        raise ValueError("'compressed_indices_dtype' should be Int/Long.")
+    rows, cols = weight.shape
+    if min_save_ratio is not None:
+        # should_prune (sparse_ops_cpu.cpp:2773-2794): sized as fp32 rows plus a 4-byte map entry per
+        # original row, with min_num_rows standing for the rows that stay
+        if not rows * 4 + min_num_rows * cols * 4 < min_save_ratio * 4 * rows * cols:
+            return weight, torch.zeros(1, dtype=compressed_indices_dtype, device=weight.device)
+    weight = weight.contiguous()
+    indicator = indicator.to(torch.float32).contiguous()
+    remap = torch.empty(rows, dtype=compressed_indices_dtype, device=weight.device)
+    kept = C.c_int64(0)
+    check(_lib.lib().fbgemm_amd_rowwise_prune_map(_ptr(indicator), rows, float(threshold), int(bool(abs)), int(min_num_rows),
+                                                  _bits(remap), _ptr(remap), C.byref(kept), _stream()))
+    out = torch.empty((kept.value, cols), dtype=weight.dtype, device=weight.device)
+    check(_lib.lib().fbgemm_amd_rowwise_prune_gather(_ptr(weight), rows, cols * weight.element_size(), _ptr(remap),
+                                                     _bits(remap), _ptr(out), kept.value, _stream()))
+    return out, remap
+
+
 def pruned_hashmap_insert(indices, dense_indices, offsets, hash_table, hash_table_offsets):
     """pruned_hashmap_insert (embedding_forward_quantized_host_cpu.cpp:331-334;
     embedding_forward_quantized_cpu_template.cpp:124-201): HOST tensors, in place

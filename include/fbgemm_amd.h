@@ -330,6 +330,22 @@ int fbgemm_amd_float_to_hfp8(const float* d_input, int64_t n, int32_t ebits, int
 int fbgemm_amd_hfp8_to_float(const uint8_t* d_input, int64_t n, int32_t ebits, int32_t exponent_bias, float* d_output,
                              void* stream);
 
+/* embedding_bag_rowwise_prune (fbgemm_gpu/src/sparse_ops/sparse_ops_cpu.cpp:2836-2893,
+ * which ends in at::native::_rowwise_prune; the converter's pruning step,
+ * fbgemm_gpu/fbgemm_gpu/split_embedding_inference_converter.py:75-93), in two calls
+ * because the size of the result depends on the data.
+ * _map: row i stays when indicator[i] (|indicator[i]| with use_abs) > threshold, or
+ * when the rows kept so far plus all rows still to come do not exceed
+ * min_non_pruned_rows; d_remap[rows] (int32 or int64) receives the new row id or -1,
+ * *num_kept (host) the number of rows that stay. Synchronizes `stream`.
+ * _gather: d_output[remap[i]] = d_weights[i] for the rows that stay; rows of
+ * row_bytes bytes, output_rows = the num_kept the map gave. */
+int fbgemm_amd_rowwise_prune_map(const float* d_indicator, int64_t rows, double threshold, int32_t use_abs,
+                                 int64_t min_non_pruned_rows, int32_t index_bits, void* d_remap, int64_t* num_kept,
+                                 void* stream);
+int fbgemm_amd_rowwise_prune_gather(const void* d_weights, int64_t rows, int64_t row_bytes, const void* d_remap,
+                                    int32_t index_bits, void* d_output, int64_t output_rows, void* stream);
+
 /* Wait for everything enqueued on `stream` (hipStreamSynchronize), for callers
  * of the asynchronous entry points that hold no HIP headers. */
 int fbgemm_amd_stream_synchronize(void* stream);

@@ -326,6 +326,22 @@ def bounds_check_indices(rows_per_table, indices, offsets, mode, warning, B_offs
         indices.size, offsets.size, int(mode), _ptr(warning), _ptr(bo))
 
 
+def rowwise_prune(weights, indicator, threshold, index_dtype=np.int32, use_abs=True, min_non_pruned_rows=0):
+    """embedding_bag_rowwise_prune without its min_save_ratio early exit: returns (kept rows, remap)."""
+    weights = np.ascontiguousarray(weights, dtype=np.float32)
+    indicator = np.ascontiguousarray(indicator, dtype=np.float32)
+    rows, cols = weights.shape
+    remap = np.empty(rows, dtype=index_dtype)
+    out = np.empty((rows, cols), dtype=np.float32)
+    fn = _lib("oracle").oracle_rowwise_prune
+    fn.restype = _c.c_int64
+    fn.argtypes = [_c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_int64, _c.c_double, _c.c_int, _c.c_int64, _c.c_int,
+                   _c.c_void_p, _c.c_void_p]
+    kept = fn(_ptr(weights), _ptr(indicator), rows, cols, float(threshold), int(use_abs), int(min_non_pruned_rows),
+              _is64(remap), _ptr(remap), _ptr(out))
+    return out[:kept].copy(), remap
+
+
 def pruned_hash(x, bits):
     lib = _lib("oracle")
     return lib.oracle_pruned_hash64(x) if bits == 64 else lib.oracle_pruned_hash32(x)

@@ -19,7 +19,10 @@
  *   - the hash functions against the published MurmurHash3 finalizers' known
  *     answers (fmix32 / fmix64) and the map against a Python dict (every
  *     inserted key is found with its value, every other key gives -1),
- *     including colliding keys and a wrapped probe sequence.
+ *     including colliding keys and a wrapped probe sequence;
+ * tests/test_prune_oracle.py checks oracle_rowwise_prune against
+ * torch._rowwise_prune (the ATen routine the reference's operator ends in) and
+ * its keep rule by brute force over short inputs.
  *
  * Reference files followed:
  *   fbgemm_gpu/codegen/utils/embedding_bounds_check_host_cpu.cpp:48-219
@@ -27,8 +30,12 @@
  *                                        (hash functions, pruned_hashmap_insert)
  *   fbgemm_gpu/codegen/inference/embedding_forward_quantized_cpu_template.cpp:524-603
  *                                        (pruned_hashmap_lookup)
+ *   fbgemm_gpu/src/sparse_ops/sparse_ops_cpu.cpp:2836-2893  embedding_bag_rowwise_prune
  */
+#include <math.h>
+#include <stddef.h>
 #include <stdint.h>
+#include <string.h>
 
 static int64_t rd(const void* p, int is64, int64_t i) {
   return is64 ? ((const int64_t*)p)[i] : (int64_t)((const int32_t*)p)[i];
@@ -201,4 +208,31 @@ void oracle_pruned_hashmap_lookup(
       wr(dense_indices, idx64, i, out);
     }
   }
+}
+
+/* ---- embedding_bag_rowwise_prune ---------------------------------------------
+ * fbgemm_gpu/src/sparse_ops/sparse_ops_cpu.cpp:2836-2893: the sequential loop that
+ * decides which rows stay (indicator above the threshold, compared in double; once
+ * the rows kept so far plus all rows still to come do not exceed
+ * min_non_pruned_rows, every remaining row stays), followed by what
+ * at::native::_rowwise_prune does with that mask: kept rows are copied in order,
+ * remap[i] is the new row id or -1. Returns the number of rows kept; out_weights
+ * may be NULL (mask and remap only). Pinned by tests/test_prune_oracle.py against
+ * torch._rowwise_prune (the ATen routine the reference calls) and by brute force
+ * over all masks of short inputs. */
+int64_t oracle_rowwise_prune(const float* weights, const float* indicator, int64_t rows, int64_t cols, double threshold,
+                             int use_abs, int64_t min_non_pruned_rows, int idx64, void* remap, float* out_weights) {
+  int64_t num_kept = 0;
+  for (int64_t i = 0; i < rows; ++i) {
+    const float val = use_abs ? fabsf(indicator[i]) : indicator[i];
+    int keep = (double)val > threshold;
+    if (num_kept < min_non_pruned_rows && num_kept + (rows - i) <= min_non_pruned_rows) keep = 1;
+    const int64_t id = keep ? num_kept : -1;
+    if (idx64) ((int64_t*)remap)[i] = id;
+    else ((int32_t*)remap)[i] = (int32_t)id;
+    if (!keep) continue;
+    if (out_weights) memcpy(out_weights + num_kept * cols, weights + i * cols, sizeof(float) * (size_t)cols);
+    ++num_kept;
+  }
+  return num_kept;
 }
