@@ -48,6 +48,7 @@ SYMBOLS = {
     "fbgemm_amd_dequantize_rowwise": (C.c_int, [_P, _I64, _I64, _I32, _I32, _I32, _I32, _I32, _P, _P]),
     "fbgemm_amd_float_to_hfp8": (C.c_int, [_P, _I64, _I32, _I32, C.c_float, _P, _P]),
     "fbgemm_amd_hfp8_to_float": (C.c_int, [_P, _I64, _I32, _I32, _P, _P]),
+    "fbgemm_amd_compressed_indices_remap": (C.c_int, [_I32, _P, _I32, _P, _I64, _P, _P, _P, _P, _P, _P, _P]),
     "fbgemm_amd_rowwise_prune_map": (C.c_int, [_P, _I64, C.c_double, _I32, _I64, _I32, _P, C.POINTER(_I64), _P]),
     "fbgemm_amd_rowwise_prune_gather": (C.c_int, [_P, _I64, _I64, _P, _I32, _P, _I64, _P]),
     "fbgemm_amd_tbe_plan_num_rows": (_I64, [_P, _I32]),

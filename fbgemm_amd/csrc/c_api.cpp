@@ -34,6 +34,10 @@ hipError_t launch_prune_map(const float* indicator, int64_t rows, double thresho
                             bool idx64, void* remap, int64_t* num_kept, int64_t* partial, hipStream_t stream);
 hipError_t launch_prune_gather(const void* in, int64_t rows, int64_t row_bytes, const void* remap, bool idx64, void* out,
                                int64_t out_rows, hipStream_t stream);
+hipError_t launch_compressed_indices_remap(const void* indices, bool idx64, const int32_t* mapping, int64_t mapping_numel,
+                                           const void* offsets, int64_t offsets_numel, const float* weights, int64_t first,
+                                           int64_t n, void* out_indices, void* out_offsets, float* out_weights,
+                                           int64_t* before, int64_t* partial, Status* status, hipStream_t stream);
 hipError_t launch_calibration_copy(const void* src, void* dst, int64_t bytes, hipStream_t stream);
 hipError_t launch_bounds_check(const int64_t* rows_per_table, int32_t T, void* indices, void* offsets, bool is64,
                                int64_t num_indices, int64_t total_B, int64_t B, const int32_t* B_offsets, int mode,
@@ -1020,6 +1024,41 @@ int fbgemm_amd_rowwise_prune_gather(const void* d_weights, int64_t rows, int64_t
   if (rows == 0 || row_bytes == 0 || output_rows == 0) return 0;
   if (!d_weights || !d_remap || !d_output) return fail(FBGEMM_AMD_E_ARG, "null data pointer");
   HIP_TRY(launch_prune_gather(d_weights, rows, row_bytes, d_remap, index_bits == 64, d_output, output_rows, (hipStream_t)stream));
+  return 0;
+}
+
+int fbgemm_amd_compressed_indices_remap(
+    int32_t offsets_numel, const void* d_indices, int32_t index_bits, const int32_t* d_mapping, int64_t mapping_numel,
+    const void* d_offsets, const float* d_weights, void* d_out_indices, void* d_out_offsets, float* d_out_weights,
+    void* d_status, void* stream_) {
+  if (index_bits != 32 && index_bits != 64) return fail(FBGEMM_AMD_E_ARG, "index_bits must be 32 or 64");
+  if (offsets_numel < 1) return fail(FBGEMM_AMD_E_ARG, "offsets must hold at least one entry");
+  if (!d_offsets || !d_out_offsets || !d_mapping) return fail(FBGEMM_AMD_E_ARG, "null data pointer");
+  if (mapping_numel < 0) return fail(FBGEMM_AMD_E_ARG, "mapping_numel must not be negative");
+  hipStream_t stream = (hipStream_t)stream_;
+  // the positions the reference walks: offsets[0] .. offsets[last] - 1
+  const size_t eb = index_bits / 8;
+  int64_t ends[2] = {0, 0};
+  HIP_TRY(hipMemcpyAsync(&ends[0], d_offsets, eb, hipMemcpyDeviceToHost, stream));
+  HIP_TRY(hipMemcpyAsync(&ends[1], (const char*)d_offsets + (size_t)(offsets_numel - 1) * eb, eb, hipMemcpyDeviceToHost, stream));
+  HIP_TRY(hipStreamSynchronize(stream));
+  if (index_bits == 32) {
+    ends[0] = (int32_t)ends[0];
+    ends[1] = (int32_t)ends[1];
+  }
+  const int64_t first = ends[0];
+  const int64_t n = ends[1] > first ? ends[1] - first : 0;
+  if (first < 0) return fail(FBGEMM_AMD_E_ARG, "offsets[0] is negative");
+  if (n > 0 && (!d_indices || !d_out_indices)) return fail(FBGEMM_AMD_E_ARG, "null data pointer");
+  if (n > 0 && d_weights && !d_out_weights) return fail(FBGEMM_AMD_E_ARG, "weights need out_weights");
+  std::lock_guard<std::mutex> lk(g_mu);
+  DeviceScratch* s;
+  if (int rc = get_scratch(&s)) return rc;
+  if (int rc = grow(&s->fixed, &s->fixed_cap, n + 1, stream)) return rc;
+  if (int rc = grow(&s->partial, &s->partial_cap, prune_partials(n + 1), stream)) return rc;
+  HIP_TRY(launch_compressed_indices_remap(d_indices, index_bits == 64, d_mapping, mapping_numel, d_offsets, offsets_numel,
+                                          d_weights, first, n, d_out_indices, d_out_offsets, d_out_weights, s->fixed,
+                                          s->partial, d_status ? (Status*)d_status : s->status, stream));
   return 0;
 }
 

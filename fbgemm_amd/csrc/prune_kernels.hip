@@ -35,6 +35,20 @@ __device__ __forceinline__ bool passes(const float* indicator, int64_t i, double
   return (double)(use_abs ? __builtin_fabsf(v) : v) > threshold;
 }
 
+// compressed_indices_remap: position k of the index array stays when its row is not pruned.
+// An index outside the mapping cannot be looked up: it is dropped and reported.
+template <typename index_t>
+__device__ __forceinline__ int32_t mapped_row(const index_t* indices, const int32_t* mapping, int64_t mapping_numel, int64_t k,
+                                              Status* status) {
+  const int64_t idx = (int64_t)indices[k];
+  if (idx < 0 || idx >= mapping_numel) {
+    atomicOr(&status->bits, ERR_INDEX_OUT_OF_RANGE);
+    atomicMin(&status->first_bad_pos, (unsigned long long)k);
+    return -1;
+  }
+  return mapping[idx];
+}
+
 // inclusive sum over the workgroup's threads; returns this thread's inclusive value
 __device__ __forceinline__ int64_t block_inclusive_sum(int64_t mine, int64_t* lds) {
   lds[threadIdx.x] = mine;
@@ -133,6 +147,73 @@ __global__ __launch_bounds__(256) void prune_gather_kernel(const uint8_t* in, in
   }
 }
 
+// ---- compressed_indices_remap ----------------------------------------------
+// src/RefImplementations.cc:2308-2333 (AVX-512 twin: src/EmbeddingSpMDMAvx512.cc):
+// the entries of the bags whose row is pruned (mapping[index] == -1) are dropped,
+// the others are replaced by their physical row and moved up, per-sample weights
+// move with them, and out_offsets[i] counts the entries that stay before bag i
+// (out_offsets[0] = offsets[0], as the reference writes it). With offsets that
+// do not decrease the reference visits positions offsets[0] .. offsets[last]-1
+// in order, so the new position of an entry is the number of entries that stay
+// before it: one exclusive prefix sum.
+
+// pass 1: entries of every block of PSCAN_BLOCK positions that stay
+template <typename index_t>
+__global__ __launch_bounds__(PSCAN_THREADS) void remap_count_kernel(const index_t* indices, const int32_t* mapping,
+                                                                    int64_t mapping_numel, int64_t first, int64_t n,
+                                                                    int64_t* partial, Status* status) {
+  __shared__ int64_t lds[PSCAN_THREADS];
+  const int64_t base = (int64_t)blockIdx.x * PSCAN_BLOCK + (int64_t)threadIdx.x * PSCAN_ITEMS;
+  int64_t local = 0;
+  for (int i = 0; i < PSCAN_ITEMS; ++i)
+    if (base + i < n && mapped_row(indices, mapping, mapping_numel, first + base + i, status) != -1) ++local;
+  const int64_t incl = block_inclusive_sum(local, lds);
+  if (threadIdx.x == PSCAN_THREADS - 1) partial[blockIdx.x] = incl;
+}
+
+// pass 3: move the entries; before[k] = entries that stay in front of position first + k (k = 0 .. n)
+template <typename index_t>
+__global__ __launch_bounds__(PSCAN_THREADS) void remap_move_kernel(const index_t* indices, const int32_t* mapping,
+                                                                   int64_t mapping_numel, const float* weights, int64_t first,
+                                                                   int64_t n, const int64_t* carry_in, index_t* out_indices,
+                                                                   float* out_weights, int64_t* before_out, Status* status) {
+  __shared__ int64_t lds[PSCAN_THREADS];
+  const int64_t base = (int64_t)blockIdx.x * PSCAN_BLOCK + (int64_t)threadIdx.x * PSCAN_ITEMS;
+  int32_t row[PSCAN_ITEMS];
+  int64_t local = 0;
+  for (int i = 0; i < PSCAN_ITEMS; ++i) {
+    row[i] = base + i < n ? mapped_row(indices, mapping, mapping_numel, first + base + i, status) : -1;
+    local += row[i] != -1 ? 1 : 0;
+  }
+  const int64_t incl = block_inclusive_sum(local, lds);
+  int64_t before = carry_in[blockIdx.x] + incl - local;
+  for (int i = 0; i < PSCAN_ITEMS; ++i) {
+    const int64_t k = base + i;
+    if (k > n) break;
+    before_out[k] = before; // k == n: the total
+    if (k == n) break;
+    if (row[i] != -1) {
+      out_indices[before] = (index_t)row[i];
+      if (weights) out_weights[before] = weights[first + k];
+      ++before;
+    }
+  }
+}
+
+template <typename index_t>
+__global__ __launch_bounds__(256) void remap_offsets_kernel(const index_t* offsets, int64_t offsets_numel, int64_t first,
+                                                            int64_t n, const int64_t* before, index_t* out_offsets) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= offsets_numel) return;
+  if (i == 0) {
+    out_offsets[0] = offsets[0];
+    return;
+  }
+  int64_t k = (int64_t)offsets[i] - first;
+  k = k < 0 ? 0 : (k > n ? n : k);
+  out_offsets[i] = (index_t)before[k];
+}
+
 } // namespace
 
 int64_t prune_partials(int64_t rows) { return (rows + PSCAN_BLOCK - 1) / PSCAN_BLOCK; }
@@ -169,6 +250,34 @@ hipError_t launch_prune_gather(const void* in, int64_t rows, int64_t row_bytes, 
   else
     hipLaunchKernelGGL(prune_gather_kernel<int32_t>, dim3((unsigned)blocks), dim3(256), 0, stream, (const uint8_t*)in, rows,
                        row_bytes, (const int32_t*)remap, (uint8_t*)out, out_rows, lpr, vec);
+  return hipGetLastError();
+}
+
+// n = offsets[last] - offsets[0] positions starting at `first` = offsets[0]; `before` holds n + 1 entries,
+// `partial` prune_partials(n + 1).
+hipError_t launch_compressed_indices_remap(const void* indices, bool idx64, const int32_t* mapping, int64_t mapping_numel,
+                                           const void* offsets, int64_t offsets_numel, const float* weights, int64_t first,
+                                           int64_t n, void* out_indices, void* out_offsets, float* out_weights,
+                                           int64_t* before, int64_t* partial, Status* status, hipStream_t stream) {
+  const int64_t nblocks = prune_partials(n + 1);
+  const unsigned oblocks = (unsigned)((offsets_numel + 255) / 256);
+  if (idx64) {
+    hipLaunchKernelGGL(remap_count_kernel<int64_t>, dim3((unsigned)nblocks), dim3(PSCAN_THREADS), 0, stream, (const int64_t*)indices,
+                       mapping, mapping_numel, first, n, partial, status);
+    hipLaunchKernelGGL(prune_carry_kernel, dim3(1), dim3(PSCAN_THREADS), 0, stream, partial, nblocks);
+    hipLaunchKernelGGL(remap_move_kernel<int64_t>, dim3((unsigned)nblocks), dim3(PSCAN_THREADS), 0, stream, (const int64_t*)indices,
+                       mapping, mapping_numel, weights, first, n, partial, (int64_t*)out_indices, out_weights, before, status);
+    hipLaunchKernelGGL(remap_offsets_kernel<int64_t>, dim3(oblocks), dim3(256), 0, stream, (const int64_t*)offsets, offsets_numel,
+                       first, n, before, (int64_t*)out_offsets);
+  } else {
+    hipLaunchKernelGGL(remap_count_kernel<int32_t>, dim3((unsigned)nblocks), dim3(PSCAN_THREADS), 0, stream, (const int32_t*)indices,
+                       mapping, mapping_numel, first, n, partial, status);
+    hipLaunchKernelGGL(prune_carry_kernel, dim3(1), dim3(PSCAN_THREADS), 0, stream, partial, nblocks);
+    hipLaunchKernelGGL(remap_move_kernel<int32_t>, dim3((unsigned)nblocks), dim3(PSCAN_THREADS), 0, stream, (const int32_t*)indices,
+                       mapping, mapping_numel, weights, first, n, partial, (int32_t*)out_indices, out_weights, before, status);
+    hipLaunchKernelGGL(remap_offsets_kernel<int32_t>, dim3(oblocks), dim3(256), 0, stream, (const int32_t*)offsets, offsets_numel,
+                       first, n, before, (int32_t*)out_offsets);
+  }
   return hipGetLastError();
 }
 

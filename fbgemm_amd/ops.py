@@ -497,6 +497,33 @@ def hfp8_quantized_to_float(input, ebits, exponent_bias):
     return out
 
 
+def compressed_indices_remap(indices, compressed_indices_mapping, offsets, weights=None):
+    """fbgemm::compressed_indices_remap (FbgemmEmbedding.h:392-401; src/RefImplementations.cc:2308-2333):
+    drops the entries of pruned rows, maps the others to physical rows, rewrites offsets (and weights).
+    Returns (out_indices, out_offsets, out_weights or None); the outputs have the inputs' sizes, their
+    first out_offsets[-1] entries are meaningful. Raises on an index outside the mapping."""
+    _require_cuda(indices, compressed_indices_mapping, offsets, weights)
+    if indices.dtype != offsets.dtype:
+        raise TypeError("indices and offsets must have the same dtype")
+    if compressed_indices_mapping.dtype != torch.int32:
+        raise TypeError("compressed_indices_mapping must be int32")
+    if weights is not None and weights.dtype != torch.float32:
+        raise TypeError("weights must be float32")
+    indices, offsets, mapping = indices.contiguous(), offsets.contiguous(), compressed_indices_mapping.contiguous()
+    out_indices = torch.empty_like(indices)
+    out_offsets = torch.empty_like(offsets)
+    out_weights = None if weights is None else torch.empty_like(weights)
+    st = Status(indices.device)
+    check(_lib.lib().fbgemm_amd_compressed_indices_remap(
+        offsets.numel(), _ptr(indices), _bits(indices), _ptr(mapping), mapping.numel(), _ptr(offsets),
+        _ptr(None if weights is None else weights.contiguous()), _ptr(out_indices), _ptr(out_offsets), _ptr(out_weights),
+        _ptr(st.buf), _stream()))
+    bits, pos = st.read()
+    if bits:
+        raise IndexError(f"compressed_indices_remap: index at position {pos} is outside the mapping")
+    return out_indices, out_offsets, out_weights
+
+
 def embedding_bag_rowwise_prune(weight, indicator, threshold, compressed_indices_dtype, abs=True, min_num_rows=0,
                                 min_save_ratio=1.0):
     """embedding_bag_rowwise_prune (fbgemm_gpu/src/sparse_ops/sparse_ops_cpu.cpp:2836-2893), on the GPU:

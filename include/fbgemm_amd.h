@@ -330,6 +330,23 @@ int fbgemm_amd_float_to_hfp8(const float* d_input, int64_t n, int32_t ebits, int
 int fbgemm_amd_hfp8_to_float(const uint8_t* d_input, int64_t n, int32_t ebits, int32_t exponent_bias, float* d_output,
                              void* stream);
 
+/* fbgemm::compressed_indices_remap (include/fbgemm/FbgemmEmbedding.h:392-401,
+ * src/RefImplementations.cc:2308-2333): the core library's pruned-row remap, which
+ * compacts. Entries whose row is pruned (d_mapping[index] == -1) are dropped, the
+ * others become their physical row and move up, per-sample weights (optional) move
+ * with them; d_out_offsets[i] = entries that stay before bag i, d_out_offsets[0] =
+ * offsets[0]. Indices and offsets share index_bits; offsets must not decrease (the
+ * reference then walks positions offsets[0] .. offsets[last]-1 in order). Beyond the
+ * reference: mapping_numel bounds the indices (an index outside the mapping is dropped
+ * and recorded in d_status instead of being read; d_status may be NULL: then it is
+ * only dropped). Outputs must not alias inputs.
+ * Reads offsets[0] and offsets[last] back first (synchronizes `stream`), then runs
+ * asynchronously; uses library-owned scratch (calls must be ordered on one stream). */
+int fbgemm_amd_compressed_indices_remap(
+    int32_t offsets_numel, const void* d_indices, int32_t index_bits, const int32_t* d_mapping, int64_t mapping_numel,
+    const void* d_offsets, const float* d_weights, void* d_out_indices, void* d_out_offsets, float* d_out_weights,
+    void* d_status, void* stream);
+
 /* embedding_bag_rowwise_prune (fbgemm_gpu/src/sparse_ops/sparse_ops_cpu.cpp:2836-2893,
  * which ends in at::native::_rowwise_prune; the converter's pruning step,
  * fbgemm_gpu/fbgemm_gpu/split_embedding_inference_converter.py:75-93), in two calls

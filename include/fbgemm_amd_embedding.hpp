@@ -285,6 +285,18 @@ inline void done(int rc) {
 }
 } // namespace detail
 
+// compressed_indices_remap (FbgemmEmbedding.h:392-401): device pointers; returns when the work is done.
+// As in the reference, nothing bounds the indices: every index must lie inside the mapping.
+template <typename IndexType>
+void compressed_indices_remap(std::int32_t offsets_numel, const IndexType* indices,
+                              const std::int32_t* compressed_indices_mapping, const IndexType* offsets,
+                              const float* weights, // optional, can be null
+                              IndexType* out_indices, IndexType* out_offsets, float* out_weights) {
+  detail::done(fbgemm_amd_compressed_indices_remap(offsets_numel, indices, detail::bits_of<IndexType>(),
+                                                   compressed_indices_mapping, INT64_MAX, offsets, weights, out_indices,
+                                                   out_offsets, out_weights, nullptr, stream_ref()));
+}
+
 template <typename InputType>
 void FloatOrHalfToFusedNBitRowwiseQuantizedSBHalf(int bit_rate, const InputType* input, std::size_t input_rows,
                                                   int input_columns, std::uint8_t* output,

@@ -7,6 +7,7 @@
 // returning false. Exit code 0 = all cases passed.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstdio>
 #include <cstring>
 #include <random>
@@ -227,6 +228,41 @@ void run_no_bag_and_fp8(int64_t D, int n, int rows, unsigned seed) {
   }
 }
 
+extern "C" void oracle_compressed_indices_remap(
+    int32_t offsets_len, const void* indices, int idx64, const int32_t* mapping, const void* offsets, const float* weights,
+    void* out_indices, void* out_offsets, float* out_weights);
+
+// compressed_indices_remap against the oracle (after test/EmbeddingSpMDMTest.cc:1040-1192: half of the rows pruned)
+template <typename IndexType>
+void run_remap(int batch, int rows, int avg_len, bool weighted, unsigned seed) {
+  std::mt19937 rng(seed);
+  std::vector<int32_t> mapping(rows);
+  int32_t next = 0;
+  for (auto& m : mapping) m = (rng() & 1) ? next++ : -1;
+  std::vector<IndexType> offsets(batch + 1, 0);
+  for (int b = 0; b < batch; ++b) offsets[b + 1] = offsets[b] + rng() % (2 * avg_len + 1);
+  std::vector<IndexType> indices(offsets[batch]);
+  for (auto& i : indices) i = rng() % rows;
+  std::vector<float> w(indices.size());
+  for (auto& x : w) x = (float)(rng() % 2000) / 1000.f - 1.f;
+  std::vector<IndexType> want_i(indices.size(), 0), want_o(offsets.size(), 0);
+  std::vector<float> want_w(w.size(), 0.f);
+  oracle_compressed_indices_remap((int32_t)offsets.size(), indices.data(), sizeof(IndexType) == 8, mapping.data(),
+                                  offsets.data(), weighted ? w.data() : nullptr, want_i.data(), want_o.data(), want_w.data());
+  Dev<IndexType> d_idx(indices), d_off(offsets), d_oi(want_i), d_oo(want_o);
+  Dev<int32_t> d_map(mapping);
+  Dev<float> d_w(w), d_ow(want_w);
+  fbgemm_amd::compressed_indices_remap<IndexType>((int32_t)offsets.size(), d_idx.p, d_map.p, d_off.p, weighted ? d_w.p : nullptr,
+                                                  d_oi.p, d_oo.p, weighted ? d_ow.p : nullptr);
+  const auto got_i = d_oi.host();
+  const auto got_o = d_oo.host();
+  const auto got_w = d_ow.host();
+  const size_t n = (size_t)want_o.back();
+  CHECK(got_o == want_o, "remap offsets differ (batch %d)", batch);
+  CHECK(std::equal(got_i.begin(), got_i.begin() + n, want_i.begin()), "remap indices differ (batch %d)", batch);
+  if (weighted) CHECK(memcmp(got_w.data(), want_w.data(), n * 4) == 0, "remap weights differ (batch %d)", batch);
+}
+
 // The quantizer templates (names and arguments of include/fbgemm/QuantUtils.h:276-334)
 // against the oracle, after test/QuantUtilsTest.cc's fused row-wise cases.
 void run_quantizers(int rows, int cols, unsigned seed) {
@@ -290,6 +326,10 @@ int main() {
   for (int D : {2, 8, 40, 86, 128, 256}) {
     run_no_bag_and_fp8<int64_t>(D, 77, 300, ++seed);
     run_no_bag_and_fp8<int32_t>(D, 500, 1000, ++seed);
+  }
+  for (int weighted = 0; weighted < 2; ++weighted) {
+    run_remap<int32_t>(10, 400, 5, weighted, ++seed);
+    run_remap<int64_t>(1000, 4000, 20, weighted, ++seed);
   }
   for (int cols : {4, 8, 64, 100, 128, 260})
     for (int rows : {1, 7, 130}) run_quantizers(rows, cols, ++seed);
