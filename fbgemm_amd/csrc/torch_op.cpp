@@ -360,6 +360,35 @@ Tensor hfp8_to_float(const Tensor& input, int64_t ebits, int64_t exponent_bias) 
   return out;
 }
 
+// Shape functions for tracing (DispatchKey::Meta), after the reference's
+// fbgemm_gpu/fbgemm_gpu/sparse_ops.py:503-581: the output of a pooled lookup is
+// [B, total_D], of a lookup without pooling [number of indices, D]; the copied-row
+// outputs of the latter have the shapes this library writes.
+Tensor lookup_meta(
+    Tensor dev_weights, Tensor /*uvm_weights*/, Tensor /*weights_placements*/, Tensor /*weights_offsets*/,
+    Tensor /*weights_tys*/, Tensor D_offsets, c10::SymInt total_D_, int64_t max_int2_D, int64_t max_int4_D,
+    int64_t max_int8_D, int64_t max_float16_D, int64_t max_float32_D, Tensor indices, Tensor offsets, int64_t pooling_mode,
+    std::optional<Tensor> /*indice_weights*/, int64_t output_dtype, std::optional<Tensor> /*lxu_cache_weights*/,
+    std::optional<Tensor> /*lxu_cache_locations*/, std::optional<int64_t> /*row_alignment*/,
+    std::optional<int64_t> max_float8_D, std::optional<int64_t> /*fp8_exponent_bits*/,
+    std::optional<int64_t> /*fp8_exponent_bias*/) {
+  if (pooling_mode == FBGEMM_AMD_POOL_NONE) {
+    const int64_t D = std::max({max_int2_D, max_int4_D, max_int8_D, max_float16_D, max_float32_D, max_float8_D.value_or(0)});
+    TORCH_CHECK(D > 0);
+    if (output_dtype == FBGEMM_AMD_INT8 || output_dtype == FBGEMM_AMD_INT4)
+      return at::empty({indices.numel(), output_dtype == FBGEMM_AMD_INT8 ? D + 4 : (D + 9) / 2},
+                       dev_weights.options().dtype(at::kByte));
+    return at::empty({indices.numel(), D}, dev_weights.options().dtype(out_scalar_type(output_dtype)));
+  }
+  const int64_t T = D_offsets.numel() - 1;
+  const int64_t total_D = total_D_.expect_int();
+  TORCH_CHECK(T > 0 && total_D > 0);
+  return at::empty({(offsets.size(0) - 1) / T, total_D}, dev_weights.options().dtype(out_scalar_type(output_dtype)));
+}
+Tensor same_shape_as_indices_meta(Tensor indices, Tensor /*offsets*/, Tensor /*table*/, Tensor /*table_offsets*/) {
+  return at::empty_like(indices);
+}
+
 // embedding_bag_rowwise_prune (fbgemm_gpu/src/sparse_ops/sparse_ops_cpu.cpp:2773-2893)
 std::tuple<Tensor, Tensor> rowwise_prune(const Tensor& weights, const Tensor& indicator, double threshold,
                                          at::ScalarType compressed_indices_dtype, bool abs, c10::SymInt min_non_pruned_rows_,
@@ -414,6 +443,8 @@ TORCH_LIBRARY_FRAGMENT(fbgemm, m) {
   m.impl("int_nbit_split_embedding_codegen_lookup_function",
          torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(int_nbit_split_embedding_codegen_lookup_function_hip)));
   m.impl("pruned_array_lookup", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(pruned_array_lookup_hip)));
+  m.impl("int_nbit_split_embedding_codegen_lookup_function", torch::dispatch(c10::DispatchKey::Meta, TORCH_FN(lookup_meta)));
+  m.impl("pruned_array_lookup", torch::dispatch(c10::DispatchKey::Meta, TORCH_FN(same_shape_as_indices_meta)));
 #ifndef FBGEMM_AMD_IMPL_ONLY
   // embedding_forward_quantized_host_cpu.cpp:338-341
   m.def(
@@ -469,6 +500,7 @@ TORCH_LIBRARY_FRAGMENT(fbgemm, m) {
   m.impl("FloatToHFP8Quantized", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(float_to_hfp8)));
   m.impl("HFP8QuantizedToFloat", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(hfp8_to_float)));
   m.impl("pruned_hashmap_lookup", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(pruned_hashmap_lookup_hip)));
+  m.impl("pruned_hashmap_lookup", torch::dispatch(c10::DispatchKey::Meta, TORCH_FN(same_shape_as_indices_meta)));
   m.impl("bounds_check_indices", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(bounds_check_indices_hip)));
   m.impl("FloatToFused8BitRowwiseQuantized", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(float_to_fused8bit)));
   m.impl("HalfToFused8BitRowwiseQuantized", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(float_to_fused8bit)));
