@@ -45,7 +45,8 @@ def parse():
     ap.add_argument("--check", action="store_true", help="verify a sample of the output against the oracle first")
     ap.add_argument("--op", default="lookup",
                     choices=["lookup", "quantize", "dequantize", "bounds_check", "pruned_array_lookup",
-                             "pruned_hashmap_lookup"],
+                             "pruned_hashmap_lookup", "float_to_hfp8", "hfp8_to_float", "rowwise_prune",
+                             "compressed_indices_remap", "sequence", "no_bag"],
                     help="lookup = the table-batched forward (the metric); the others time one operator beside "
                          "the path at the shape config 4 / config 3 gives it and print the same kind of line")
     return ap.parse_args()
@@ -243,7 +244,10 @@ def side_op(a):
 
     Shapes: the index operators see config 4's batch (32 tables x 4096 bags,
     3.6 M int64 indices, 2 M-row mappings); the quantizers see 1 M rows x 128
-    columns (a table of config 2's shape), 4-bit rows in the table-batched layout."""
+    columns (a table of config 2's shape), 4-bit rows in the table-batched layout;
+    so do the hfp8 converters and the single-table no_bag kernel (8-bit rows);
+    rowwise_prune sees 2 M x 64 fp32 with half of the rows kept; sequence
+    (PoolingMode.NONE) sees 32 int4 tables x 1 M rows x 128 with config 4's bags."""
     import numpy as np
     import torch
 
@@ -281,6 +285,57 @@ def side_op(a):
             dt = time.perf_counter() - t0
             return {"value": round(n * row_bytes / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
                     "sample": f"first {n} rows, one pass"}
+    elif a.op in ("float_to_hfp8", "hfp8_to_float"):
+        rows, cols = int((1 << 20) * a.scale), 128
+        x = torch.randn(rows, cols, device="cuda", dtype=torch.float32)
+        codes = ops.float_to_hfp8_quantized(x, 4, 7, 240.0)
+        if a.op == "float_to_hfp8":
+            launch = lambda: ops.float_to_hfp8_quantized(x, 4, 7, 240.0)
+            kernel, workload = "float_to_hfp8_kernel", f"fp32 [{rows}, {cols}] -> hfp8 (4 exponent bits, bias 7)"
+        else:
+            launch = lambda: ops.hfp8_quantized_to_float(codes, 4, 7)
+            kernel, workload = "hfp8_to_float_kernel", f"hfp8 (4 exponent bits, bias 7) [{rows}, {cols}] -> fp32"
+        alg_bytes, units = rows * cols * 5, rows
+    elif a.op == "rowwise_prune":
+        rows, cols = int(2_000_000 * a.scale), 64
+        w = torch.randn(rows, cols, device="cuda", dtype=torch.float32)
+        ind = torch.rand(rows, device="cuda", dtype=torch.float32)
+        kept = int((ind > 0.5).sum())
+        launch = lambda: ops.embedding_bag_rowwise_prune(w, ind, 0.5, torch.int32, True, 0, None)
+        # indicator in, remap out, the kept rows in and out
+        alg_bytes, units = 4 * rows + 4 * rows + 2 * kept * cols * 4, rows
+        kernel, workload = "prune_gather_kernel", f"fp32 [{rows}, {cols}], {kept} rows kept, int32 remap (map + gather, output allocated per call)"
+    elif a.op == "no_bag":
+        rows, cols = int((1 << 20) * a.scale), 128
+        table = torch.randint(0, 256, (rows, cols + 8), dtype=torch.uint8, device="cuda")
+        table[:, cols:] = torch.tensor([0.01, -0.5], dtype=torch.float32).view(torch.uint8).cuda()
+        n = rows
+        idx = torch.randint(0, rows, (n,), dtype=torch.int64, device="cuda")
+        out = torch.empty(n, cols, dtype=torch.float32, device="cuda")
+        kern = ops.generate_embedding_spmdm_with_strides(ops.INT8, cols, False, False, no_bag=True)
+        st = ops.Status()
+        launch = lambda: kern(n, n, rows, table, idx, None, None, out, status=st)
+        alg_bytes, units = n * (cols + 8 + cols * 4 + 8), n
+        kernel, workload = "row_lookup_kernel", f"8-bit rows [{rows}, {cols}] (fp32 scale/bias last), {n} int64 indices -> fp32 rows"
+    elif a.op == "sequence":
+        T, B, D = 32, max(1, int(4096 * a.scale)), 128
+        E = max(1000, int(1_000_000 * a.scale))
+        rb = ops.padded_row_size_in_bytes(D, ops.INT4, 16)
+        lens = rng.integers(5, 51, size=T * B)
+        off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+        n = int(off[-1])
+        idx = rng.integers(0, E, size=n).astype(np.int64)
+        weights = torch.randint(0, 256, (T * E * rb,), dtype=torch.uint8, device="cuda")
+        weights.view(T * E, rb)[:, :4] = torch.tensor([0.01, -0.5], dtype=torch.float16).view(torch.uint8).cuda()
+        wo = torch.arange(T, dtype=torch.int64) * (E * rb)
+        args = (weights, torch.zeros(0, dtype=torch.uint8, device="cuda"), torch.zeros(T, dtype=torch.int32, device="cuda"),
+                wo.cuda(), torch.full((T,), ops.INT4, dtype=torch.uint8, device="cuda"),
+                torch.arange(T + 1, dtype=torch.int32, device="cuda") * D, T * D, 0, D, 0, 0, 0, cu(idx), cu(off), ops.POOL_NONE,
+                None, ops.FP16)
+        st = ops.Status()
+        launch = lambda: ops.int_nbit_split_embedding_codegen_lookup_function(*args, row_alignment=16, status=st)
+        alg_bytes, units = n * (D // 2 + 4 + D * 2 + 8), n
+        kernel, workload = "sequence_lookup_kernel", f"PoolingMode.NONE, {T} int4 tables x {E} rows x {D}, {n} int64 indices -> fp16 rows (output allocated per call)"
     else:
         T, B = 32, max(1, int(4096 * a.scale))
         E = max(1000, int(2_000_000 * a.scale))
@@ -296,6 +351,16 @@ def side_op(a):
             launch = lambda: ops.bounds_check_indices(rows_per_table, d_idx, d_off, ops.BOUNDS_WARNING, warning)
             alg_bytes = 8 * n + 8 * (T * B + 1)
             kernel, workload = "bounds_check_bags_kernel", f"WARNING mode, {T} tables x {B} bags, {n} int64 indices in range"
+        elif a.op == "compressed_indices_remap":
+            # one table's mapping, all bags: the core library's remap takes one table at a time
+            mapping = np.where(rng.random(E) < 0.5, -1, 1).astype(np.int32)
+            mapping[mapping > 0] = np.arange(int((mapping > 0).sum()), dtype=np.int32)
+            d_map = cu(mapping)
+            w = torch.rand(n, device="cuda", dtype=torch.float32)
+            launch = lambda: ops.compressed_indices_remap(d_idx, d_map, d_off, w)
+            kept = int((mapping[idx] != -1).sum())
+            alg_bytes = 8 * n + 4 * n + 4 * n + 12 * kept + 16 * (T * B + 1)
+            kernel, workload = "remap_move_kernel", f"one mapping of {E} int32 entries (half pruned), {T * B} bags, {n} int64 indices + weights (outputs allocated per call)"
         elif a.op == "pruned_array_lookup":
             remap = cu(np.where(rng.random(T * E) < 0.5, -1, 1).astype(np.int32))
             ro = cu(np.arange(T + 1, dtype=np.int64) * E)
@@ -330,7 +395,7 @@ def side_op(a):
     gbps = alg_bytes / (ms * 1e-3) / 1e9
     res = {"metric": f"achieved HBM GB/s, {a.op} on 1 MI355X", "value": round(gbps, 2), "unit": "GB/s", "n_gpus": 1,
            "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(wall_ms, 5), "higher_is_better": True,
-           "scaling": "weak", "vs_baseline": None, "dtype": "f32" if "quant" in a.op else "int64", "data": "synthetic",
+           "scaling": "weak", "vs_baseline": None, "dtype": "f32" if a.op in ("quantize", "dequantize", "float_to_hfp8", "hfp8_to_float", "sequence", "no_bag") else "int64", "data": "synthetic",
            "config": {"workload": workload, "units_per_step": units},
            "roofline": {"bound": "hbm", "achieved": round(gbps, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                         "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None, "kernel": kernel,

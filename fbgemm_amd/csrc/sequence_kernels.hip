@@ -24,8 +24,8 @@ namespace fbgemm_amd {
 
 namespace {
 
-constexpr int SRUN = 4;
-constexpr int MAX_LDS_TABLES = 4096; // boundaries kept in LDS; beyond that they are read from memory
+constexpr int SRUN = 8; // columns per lane and step: a whole number of bytes for every row type
+constexpr int MAX_LDS_TABLES = 1024; // boundaries kept in LDS; beyond that they are read from memory
 
 __device__ __forceinline__ float s_bits_to_float(uint32_t u) { return __builtin_bit_cast(float, u); }
 __device__ __forceinline__ uint32_t s_float_to_bits(float f) { return __builtin_bit_cast(uint32_t, f); }
@@ -53,15 +53,41 @@ __device__ __forceinline__ void copy_row_bytes(const uint8_t* row, bool ok, int6
   }
 }
 
+// dword-aligned groups of words: rows sit on 4-byte boundaries at best, which is all a wide load needs
+struct __attribute__((aligned(4))) Words4 { uint32_t v[4]; };
+struct __attribute__((aligned(4))) Words2 { uint32_t v[2]; };
+
+// The bytes [b0, b0 + nbytes) of a row (nbytes <= 32) into w[], little end first:
+// whole dwords where the address allows it, single bytes otherwise and at the tail.
+__device__ __forceinline__ void load_run_bytes(const uint8_t* p, int nbytes, uint32_t (&w)[8]) {
+  const bool a4 = (reinterpret_cast<uintptr_t>(p) & 3) == 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    uint32_t v = 0;
+    if (i * 4 + 4 <= nbytes && a4) {
+      v = *reinterpret_cast<const uint32_t*>(p + i * 4);
+    } else {
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        if (i * 4 + k < nbytes) v |= (uint32_t)p[i * 4 + k] << (8 * k);
+    }
+    w[i] = v;
+  }
+}
+
 // One output row of D columns from one table row, as a bag of one with weight w:
 //   quantised rows  out[j] = convert(fma(w * scale, q[j], 0 + w * bias))
 //   plain rows      out[j] = convert(fma(w, x[j], 0))
-// `lpr` lanes share the row, lane `sub` takes runs of SRUN columns. A row that
-// is not there (!ok) gives zeros; columns past the table's own width give zeros.
-__device__ __forceinline__ void emit_row(const TableDesc& d, const uint8_t* row, bool ok, float w, int D, int out_ty,
-                                         uint8_t* orow, int sub, int lpr, int fp8_shift, float fp8_mult) {
-  const int bits = s_type_bits(d.ty);
-  const bool quant = bits <= 8 && d.ty != ST_FP8;
+// `lpr` lanes share the row, lane `sub` takes runs of SRUN columns (one to eight
+// dword loads, one or two 16-byte stores). A row that is not there (!ok) gives
+// zeros; columns past the table's own width give zeros. TY is the row type, so
+// that widths and bit positions are constants.
+template <int TY>
+__device__ __forceinline__ void emit_row_t(const TableDesc& d, const uint8_t* row, bool ok, float w, int D, int out_ty,
+                                           uint8_t* orow, int sub, int lpr, int fp8_shift, float fp8_mult) {
+  constexpr int bits = TY == ST_FP32 ? 32 : (TY == ST_FP16 || TY == ST_BF16) ? 16 : (TY == ST_INT8 || TY == ST_FP8) ? 8 : TY == ST_INT4 ? 4 : 2;
+  constexpr bool quant = TY == ST_INT8 || TY == ST_INT4 || TY == ST_INT2;
+  constexpr int run_bytes = (SRUN * bits) >> 3; // 2 .. 32
   float scale = w, bias = 0.0f;
   if (quant && ok) {
     const uint8_t* ph = row + d.sb_off;
@@ -84,25 +110,51 @@ __device__ __forceinline__ void emit_row(const TableDesc& d, const uint8_t* row,
   }
   const uint8_t* data = row + d.data_off;
   const int Dt = d.D < D ? d.D : D;
+  const int data_bytes = (Dt * bits + 7) >> 3; // the bytes of the row that hold columns < Dt
   for (int j0 = sub * SRUN; j0 < D; j0 += lpr * SRUN) {
+    // SRUN is a multiple of 8 / bits for every type, so a run starts on a byte
+    const int b0 = (j0 * bits) >> 3;
+    uint32_t raw[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) raw[i] = 0;
+    const uint8_t* p = data + b0;
+    if (ok && b0 + run_bytes <= data_bytes && (reinterpret_cast<uintptr_t>(p) & 3) == 0 && run_bytes >= 4) {
+      // a whole run on a dword boundary: the common case
+      if constexpr (run_bytes == 32) {
+        const Words4 a = *reinterpret_cast<const Words4*>(p), b = *reinterpret_cast<const Words4*>(p + 16);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { raw[i] = a.v[i]; raw[4 + i] = b.v[i]; }
+      } else if constexpr (run_bytes == 16) {
+        const Words4 a = *reinterpret_cast<const Words4*>(p);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) raw[i] = a.v[i];
+      } else if constexpr (run_bytes == 8) {
+        const Words2 a = *reinterpret_cast<const Words2*>(p);
+        raw[0] = a.v[0]; raw[1] = a.v[1];
+      } else {
+        raw[0] = *reinterpret_cast<const uint32_t*>(p);
+      }
+    } else if (ok && b0 < data_bytes) {
+      int nb = data_bytes - b0;
+      load_run_bytes(p, nb < run_bytes ? nb : run_bytes, raw);
+    }
     float v[SRUN];
+#pragma unroll
     for (int k = 0; k < SRUN; ++k) {
-      const int j = j0 + k;
       float x = 0.0f;
-      if (ok && j < Dt) {
-        if (bits == 32) {
-          x = __builtin_fmaf(w, reinterpret_cast<const float*>(data)[j], 0.0f);
-        } else if (bits == 16) {
-          const uint16_t u = reinterpret_cast<const uint16_t*>(data)[j];
-          x = __builtin_fmaf(w, d.ty == ST_BF16 ? s_bits_to_float((uint32_t)u << 16) : s_half_to_float(u), 0.0f);
-        } else if (d.ty == ST_FP8) {
+      if (ok && j0 + k < Dt) {
+        if constexpr (bits == 32) {
+          x = __builtin_fmaf(w, s_bits_to_float(raw[k]), 0.0f);
+        } else if constexpr (bits == 16) {
+          const uint16_t u = (uint16_t)(raw[k >> 1] >> (16 * (k & 1)));
+          x = __builtin_fmaf(w, TY == ST_BF16 ? s_bits_to_float((uint32_t)u << 16) : s_half_to_float(u), 0.0f);
+        } else if constexpr (TY == ST_FP8) {
           // Float8ToFloat_ref (src/RefImplementations.cc:184-214), then the bag of one: fma(w, x, 0)
-          const uint32_t b = data[j];
+          const uint32_t b = (raw[k >> 2] >> (8 * (k & 3))) & 0xffu;
           const float mag = s_bits_to_float((b & 0x7fu) << fp8_shift) * fp8_mult;
           x = __builtin_fmaf(w, s_bits_to_float(s_float_to_bits(mag) | ((b & 0x80u) << 24)), 0.0f);
         } else {
-          const int epb = 8 / bits;
-          const uint32_t q = ((uint32_t)data[j / epb] >> ((j % epb) * bits)) & ((1u << bits) - 1);
+          const uint32_t q = (raw[(k * bits) >> 5] >> ((k * bits) & 31)) & ((1u << bits) - 1);
           x = __builtin_fmaf(scale, (float)q, 0.0f + bias);
         }
       }
@@ -111,15 +163,41 @@ __device__ __forceinline__ void emit_row(const TableDesc& d, const uint8_t* row,
     const int n = D - j0 < SRUN ? D - j0 : SRUN;
     if (out_ty == ST_FP32) {
       float* op = reinterpret_cast<float*>(orow) + j0;
-      if (n == SRUN && (reinterpret_cast<uintptr_t>(op) & 15) == 0) *reinterpret_cast<float4*>(op) = make_float4(v[0], v[1], v[2], v[3]);
-      else for (int k = 0; k < n; ++k) op[k] = v[k];
+      if (n == SRUN && (reinterpret_cast<uintptr_t>(op) & 15) == 0) {
+#pragma unroll
+        for (int k = 0; k < SRUN; k += 4) *reinterpret_cast<float4*>(op + k) = make_float4(v[k], v[k + 1], v[k + 2], v[k + 3]);
+      } else {
+        for (int k = 0; k < n; ++k) op[k] = v[k];
+      }
     } else {
-      uint16_t h[SRUN];
-      for (int k = 0; k < SRUN; ++k) h[k] = out_ty == ST_FP16 ? s_to_half(v[k]) : s_to_bf16(v[k]);
+      uint32_t h[SRUN / 2];
+#pragma unroll
+      for (int k = 0; k < SRUN; k += 2) {
+        const uint32_t lo = out_ty == ST_FP16 ? s_to_half(v[k]) : s_to_bf16(v[k]);
+        const uint32_t hi = out_ty == ST_FP16 ? s_to_half(v[k + 1]) : s_to_bf16(v[k + 1]);
+        h[k >> 1] = lo | (hi << 16);
+      }
       uint16_t* op = reinterpret_cast<uint16_t*>(orow) + j0;
-      if (n == SRUN && (reinterpret_cast<uintptr_t>(op) & 7) == 0) *reinterpret_cast<uint2*>(op) = make_uint2(h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16));
-      else for (int k = 0; k < n; ++k) op[k] = h[k];
+      if (n == SRUN && (reinterpret_cast<uintptr_t>(op) & 15) == 0) {
+        *reinterpret_cast<uint4*>(op) = make_uint4(h[0], h[1], h[2], h[3]);
+      } else {
+        for (int k = 0; k < n; ++k) op[k] = (uint16_t)(h[k >> 1] >> (16 * (k & 1)));
+      }
     }
+  }
+}
+
+__device__ __forceinline__ void emit_row(const TableDesc& d, const uint8_t* row, bool ok, float w, int D, int out_ty,
+                                         uint8_t* orow, int sub, int lpr, int fp8_shift, float fp8_mult) {
+  switch (d.ty) {
+    case ST_INT4: emit_row_t<ST_INT4>(d, row, ok, w, D, out_ty, orow, sub, lpr, fp8_shift, fp8_mult); break;
+    case ST_INT8: emit_row_t<ST_INT8>(d, row, ok, w, D, out_ty, orow, sub, lpr, fp8_shift, fp8_mult); break;
+    case ST_FP16: emit_row_t<ST_FP16>(d, row, ok, w, D, out_ty, orow, sub, lpr, fp8_shift, fp8_mult); break;
+    case ST_INT2: emit_row_t<ST_INT2>(d, row, ok, w, D, out_ty, orow, sub, lpr, fp8_shift, fp8_mult); break;
+    case ST_FP32: emit_row_t<ST_FP32>(d, row, ok, w, D, out_ty, orow, sub, lpr, fp8_shift, fp8_mult); break;
+    case ST_BF16: emit_row_t<ST_BF16>(d, row, ok, w, D, out_ty, orow, sub, lpr, fp8_shift, fp8_mult); break;
+    case ST_FP8: emit_row_t<ST_FP8>(d, row, ok, w, D, out_ty, orow, sub, lpr, fp8_shift, fp8_mult); break;
+    default: break;
   }
 }
 
@@ -143,10 +221,9 @@ __global__ __launch_bounds__(256) void sequence_lookup_kernel(
   // bytes of an output row
   const int64_t out_row_bytes = out_ty == ST_FP32 ? (int64_t)D * 4 : (out_ty == ST_FP16 || out_ty == ST_BF16) ? (int64_t)D * 2
       : out_ty == ST_INT8 ? (int64_t)D + 4 : (int64_t)(D + 8 + 1) / 2;
-  for (int64_t g = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6); g < ngroups; g += nwaves) {
-    const int64_t pos = g * per_wave + lane / lpr;
-    if (pos >= total_L) continue;
-    // largest t with bounds[t] <= pos (empty tables share a boundary: the last of them wins)
+  // the table of position `pos`: the largest t with bounds[t] <= pos (empty tables
+  // share a boundary: the last of them wins)
+  auto table_of = [&](int64_t pos) -> int {
     int lo = 0, hi = T; // invariant: bounds[lo] <= pos < bounds[hi] once the input is well formed
     while (hi - lo > 1) {
       const int mid = (lo + hi) >> 1;
@@ -154,27 +231,48 @@ __global__ __launch_bounds__(256) void sequence_lookup_kernel(
       if (b <= pos) lo = mid;
       else hi = mid;
     }
-    const TableDesc d = tables[lo];
-    uint8_t* orow = reinterpret_cast<uint8_t*>(out) + pos * out_row_bytes;
-    const int64_t idx = (int64_t)indices[pos];
-    bool ok = true;
-    if (idx == -1) {
-      ok = false; // pruned row: zeros
-    } else if (idx < 0 || idx >= d.num_rows) {
-      if (sub == 0) {
-        atomicOr(&status->bits, ERR_INDEX_OUT_OF_RANGE);
-        atomicMin(&status->first_bad_pos, (unsigned long long)pos);
+    return lo;
+  };
+  // The index and the table descriptor of the NEXT group of positions are
+  // fetched while the rows of the current one are in flight, so that a wave
+  // waits for one memory round trip per group instead of two.
+  int64_t g = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  int64_t pos = g * per_wave + lane / lpr;
+  bool live = g < ngroups && pos < total_L;
+  int64_t idx = live ? (int64_t)indices[pos] : 0;
+  TableDesc d = tables[live ? table_of(pos) : 0];
+  while (g < ngroups) {
+    const int64_t g2 = g + nwaves;
+    const int64_t pos2 = g2 * per_wave + lane / lpr;
+    const bool live2 = g2 < ngroups && pos2 < total_L;
+    const int64_t idx2 = live2 ? (int64_t)indices[pos2] : 0;
+    const TableDesc d2 = tables[live2 ? table_of(pos2) : 0];
+    if (live) {
+      uint8_t* orow = reinterpret_cast<uint8_t*>(out) + pos * out_row_bytes;
+      bool ok = true;
+      if (idx == -1) {
+        ok = false; // pruned row: zeros
+      } else if (idx < 0 || idx >= d.num_rows) {
+        if (sub == 0) {
+          atomicOr(&status->bits, ERR_INDEX_OUT_OF_RANGE);
+          atomicMin(&status->first_bad_pos, (unsigned long long)pos);
+        }
+        ok = false;
       }
-      ok = false;
+      const uint8_t* row = (d.placement ? w1 : w0) + d.weights_offset + (ok ? idx : 0) * d.row_stride;
+      if (copy_rows) {
+        // the row as it is stored: header, then elements (what fits the output row)
+        const int64_t in_bytes = d.data_off + d.data_bytes;
+        copy_row_bytes(row, ok, in_bytes < out_row_bytes ? in_bytes : out_row_bytes, out_row_bytes, orow, sub, lpr);
+      } else {
+        emit_row(d, row, ok, 1.0f, D, out_ty, orow, sub, lpr, fp8_shift, fp8_mult);
+      }
     }
-    const uint8_t* row = (d.placement ? w1 : w0) + d.weights_offset + (ok ? idx : 0) * d.row_stride;
-    if (copy_rows) {
-      // the row as it is stored: header, then elements (what fits the output row)
-      const int64_t in_bytes = d.data_off + d.data_bytes;
-      copy_row_bytes(row, ok, in_bytes < out_row_bytes ? in_bytes : out_row_bytes, out_row_bytes, orow, sub, lpr);
-      continue;
-    }
-    emit_row(d, row, ok, 1.0f, D, out_ty, orow, sub, lpr, fp8_shift, fp8_mult);
+    g = g2;
+    pos = pos2;
+    live = live2;
+    idx = idx2;
+    d = d2;
   }
 }
 
@@ -193,23 +291,37 @@ __global__ __launch_bounds__(256) void row_lookup_kernel(
   const int per_wave = 64 / lpr;
   const int64_t nwaves = (int64_t)gridDim.x * (blockDim.x >> 6);
   const int64_t ngroups = (n + per_wave - 1) / per_wave;
-  for (int64_t g = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6); g < ngroups; g += nwaves) {
-    const int64_t pos = g * per_wave + lane / lpr;
-    if (pos >= n) continue;
-    const int64_t idx = (int64_t)indices[pos];
-    const bool ok = idx >= 0 && idx < d.num_rows;
-    if (!ok && sub == 0) {
-      atomicOr(&status->bits, ERR_INDEX_OUT_OF_RANGE);
-      atomicMin(&status->first_bad_pos, (unsigned long long)pos);
+  // the index and weight of the next group are fetched while this group's rows are in flight
+  int64_t g = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  int64_t pos = g * per_wave + lane / lpr;
+  bool live = g < ngroups && pos < n;
+  int64_t idx = live ? (int64_t)indices[pos] : 0;
+  float w = (live && weights) ? weights[pos] : 1.0f;
+  while (g < ngroups) {
+    const int64_t g2 = g + nwaves;
+    const int64_t pos2 = g2 * per_wave + lane / lpr;
+    const bool live2 = g2 < ngroups && pos2 < n;
+    const int64_t idx2 = live2 ? (int64_t)indices[pos2] : 0;
+    const float w2 = (live2 && weights) ? weights[pos2] : 1.0f;
+    if (live) {
+      const bool ok = idx >= 0 && idx < d.num_rows;
+      if (!ok && sub == 0) {
+        atomicOr(&status->bits, ERR_INDEX_OUT_OF_RANGE);
+        atomicMin(&status->first_bad_pos, (unsigned long long)pos);
+      }
+      const uint8_t* row = table + (ok ? idx : 0) * d.row_stride;
+      uint8_t* orow = reinterpret_cast<uint8_t*>(out) + pos * out_stride_bytes;
+      if (copy_bytes > 0) {
+        if (ok) copy_row_bytes(row, true, copy_bytes, copy_bytes, orow, sub, lpr);
+      } else {
+        emit_row(d, row, ok, w, d.D, out_ty, orow, sub, lpr, fp8_shift, fp8_mult);
+      }
     }
-    const uint8_t* row = table + (ok ? idx : 0) * d.row_stride;
-    uint8_t* orow = reinterpret_cast<uint8_t*>(out) + pos * out_stride_bytes;
-    if (copy_bytes > 0) {
-      if (ok) copy_row_bytes(row, true, copy_bytes, copy_bytes, orow, sub, lpr);
-      continue;
-    }
-    const float w = weights ? weights[pos] : 1.0f;
-    emit_row(d, row, ok, w, d.D, out_ty, orow, sub, lpr, fp8_shift, fp8_mult);
+    g = g2;
+    pos = pos2;
+    live = live2;
+    idx = idx2;
+    w = w2;
   }
 }
 

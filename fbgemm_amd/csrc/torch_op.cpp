@@ -125,10 +125,10 @@ Tensor int_nbit_split_embedding_codegen_lookup_function_hip(
     const int64_t total_L = indices.numel();
     Tensor out;
     if (output_dtype == FBGEMM_AMD_INT8 || output_dtype == FBGEMM_AMD_INT4)
-      out = at::zeros({total_L, output_dtype == FBGEMM_AMD_INT8 ? D + 4 : (D + 9) / 2}, dev_weights.options().dtype(at::kByte));
+      out = at::empty({total_L, output_dtype == FBGEMM_AMD_INT8 ? D + 4 : (D + 9) / 2}, dev_weights.options().dtype(at::kByte));
     else
-      out = at::zeros({total_L, D}, dev_weights.options().dtype(out_scalar_type(output_dtype)));
-    if (total_L == 0 || B == 0) return out;
+      out = at::empty({total_L, D}, dev_weights.options().dtype(out_scalar_type(output_dtype)));
+    if (total_L == 0 || B == 0) return out.zero_();
     Tensor& st = status_block(dev_weights);
     const int rc = fbgemm_amd_tbe_forward_nobag(
         plan, dev_weights.data_ptr(), uvm_weights.numel() ? uvm_weights.data_ptr() : nullptr, indices.data_ptr(),

@@ -278,14 +278,14 @@ def int_nbit_split_embedding_codegen_lookup_function(
         _set_fp8(plan, max_float8_D, fp8_exponent_bits, fp8_exponent_bias)
         total_L = indices.numel()
         if output_dtype in _OUT_TORCH:
-            out = torch.zeros((total_L, D), dtype=_OUT_TORCH[output_dtype], device=dev_weights.device)
+            out = torch.empty((total_L, D), dtype=_OUT_TORCH[output_dtype], device=dev_weights.device)
         elif output_dtype in (INT8, INT4):
-            out = torch.zeros((total_L, D + 4 if output_dtype == INT8 else (D + 9) // 2), dtype=torch.uint8,
+            out = torch.empty((total_L, D + 4 if output_dtype == INT8 else (D + 9) // 2), dtype=torch.uint8,
                               device=dev_weights.device)
         else:
             raise NotImplementedError(f"output_dtype {output_dtype} is not on this path")
         if total_L == 0 or (offsets.numel() - 1) // plan.T == 0:
-            return out
+            return out.zero_()
         own = status is None
         st = Status(dev_weights.device) if own else status
         check(_lib.lib().fbgemm_amd_tbe_forward_nobag(

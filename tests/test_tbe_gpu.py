@@ -319,6 +319,28 @@ def test_no_pooling_matches_oracle(ops, oracle, dt, D):
                     ops.POOL_NONE, None, FP16, row_alignment=row_alignment)
 
 
+def test_no_pooling_with_more_tables_than_the_kernel_keeps_in_lds(ops, oracle):
+    """1100 small tables (some without any index): the table boundaries no longer fit the
+    workgroup's LDS and the bisection reads them from memory."""
+    rng = np.random.default_rng(990)
+    D, T, B = 32, 1100, 2
+    tys = [INT4, INT8, FP16]
+    specs = [(int(rng.integers(3, 12)), D, tys[t % 3]) for t in range(T)]
+    weights, wo, _ = build_weights(rng, specs, 16)
+    lens = rng.integers(0, 4, size=T * B)
+    lens[5 * B:9 * B] = 0
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    idx = np.concatenate([rng.integers(0, specs[t][0], size=int(lens[t * B:(t + 1) * B].sum())) for t in range(T)]).astype(np.int64)
+    wt = np.array([s[2] for s in specs], np.uint8)
+    D_offsets = (np.arange(T + 1) * D).astype(np.int32)
+    got = ops.int_nbit_split_embedding_codegen_lookup_function(
+        cu(weights), torch.zeros(0, dtype=torch.uint8, device="cuda"), cu(np.zeros(T, np.int32)), cu(wo), cu(wt),
+        cu(D_offsets), T * D, 0, D, D, D, 0, cu(idx), cu(off), ops.POOL_NONE, None, FP32, row_alignment=16)
+    ok, want = oracle.tbe_forward_nobag(weights, wo, wt, [s[0] for s in specs], D, idx, off, FP32, 16)
+    assert ok
+    H.assert_same_bits(got.cpu().numpy(), want, "no pooling, 1100 tables")
+
+
 @pytest.mark.parametrize("ty", [INT8, INT4])
 def test_no_pooling_quantized_output_copies_rows(ops, oracle, ty):
     rng = np.random.default_rng(950 + ty)
