@@ -1125,8 +1125,10 @@ int fbgemm_amd_pruned_hashmap_insert_host(
     return fail(FBGEMM_AMD_E_ARG, "index_bits/hash_bits must be 32 or 64");
   const int64_t B = (offsets_numel - 1) / T;
   if (B <= 0) return fail(FBGEMM_AMD_E_ARG, "pruned_hashmap_insert needs B > 0");
-  if (!h_indices || !h_dense_indices || !h_offsets || !h_hash_table || !h_hash_table_offsets)
-    return fail(FBGEMM_AMD_E_ARG, "null data pointer");
+  if (!h_offsets || !h_hash_table_offsets) return fail(FBGEMM_AMD_E_ARG, "null data pointer");
+  // a map without slots (no table is pruned) has nothing to insert into: the reference's loop skips such tables
+  if (h_hash_table_offsets[T] - h_hash_table_offsets[0] <= 0) return 0;
+  if (!h_indices || !h_dense_indices || !h_hash_table) return fail(FBGEMM_AMD_E_ARG, "null data pointer");
   const bool iw = index_bits == 64, hw = hash_bits == 64;
   for (int32_t t = 0; t < T; ++t) {
     const int64_t table_start = h_hash_table_offsets[t];

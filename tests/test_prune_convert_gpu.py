@@ -157,3 +157,68 @@ def test_converter_matches_oracle_pipeline(ops, oracle, ty_name, ratio, use_arra
                                   m.D_offsets.cpu().numpy(), m.total_D, dense, off, 0, None, FP16, m.row_alignment)
     assert rc == 0
     H.assert_same_bits(got, want, f"converted {ty_name} ratio={ratio}")
+
+
+class FloatTables(torch.nn.Module):
+    """Test stand-in for the float module the reference's converter reads its tables from
+    (split_embedding_weights(), pooling_mode; forward = plain pooled sums in fp32)."""
+
+    def __init__(self, tables):
+        super().__init__()
+        self.tables = [t.cuda() for t in tables]
+        self.pooling_mode = 0
+
+    def split_embedding_weights(self):
+        return self.tables
+
+    def forward(self, indices, offsets):
+        T = len(self.tables)
+        B = (offsets.numel() - 1) // T
+        off = offsets.cpu().tolist()
+        out = torch.zeros(B, sum(t.size(1) for t in self.tables), device="cuda")
+        col = 0
+        for t, tbl in enumerate(self.tables):
+            for b in range(B):
+                s, e = off[t * B + b], off[t * B + b + 1]
+                if e > s:
+                    out[b, col:col + tbl.size(1)] = tbl[indices[s:e].long()].sum(0)
+            col += tbl.size(1)
+        return out
+
+
+class Arch(torch.nn.Module):
+    def __init__(self, tables):
+        super().__init__()
+        self.emb_module = FloatTables(tables)
+
+    def forward(self, indices, offsets):
+        return self.emb_module(indices, offsets)
+
+
+@pytest.mark.parametrize("use_array", [True, False])
+@pytest.mark.parametrize("ty_name", ["FP32", "FP16", "INT8", "INT4", "INT2"])
+def test_l2_norm_pruning_workflow_fixture(ty_name, use_array):
+    """The reference's fully specified pruning fixture
+    (fbgemm_gpu/test/tbe/inference/inference_converter_test.py:263-343): two tables of five constant rows,
+    pruning ratios 0.9 / 0.5 / 0.1; lookups through the converted module by original row id must equal the
+    float lookups over the indices the reference lists as surviving, to the reference's tolerance, and the
+    surviving rows must be the ones of largest norm."""
+    from fbgemm_amd import converter, module as M
+    D, E = 128, 5
+    indices = torch.tensor([3, 0, 2, 2, 3, 4, 2], dtype=torch.int32)
+    offsets = torch.tensor([0, 1, 4, 6, 7], dtype=torch.int32)
+    scales = [[0.4, 0.1, -0.2, 0.2, 0.3], [-0.8, 0.2, 0.5, -0.1, 0.9]]
+    weights = [torch.tensor(s).view(E, 1) * torch.ones(E, D) for s in scales]
+    cases = [(0.9, [0, 4], [0, 0, 1, 2, 2], [[0], [4]]),
+             (0.5, [3, 0, 2, 2, 4, 2], [0, 1, 4, 5, 6], [[0, 2, 3, 4], [0, 2, 4]]),
+             (0.1, indices.tolist(), offsets.tolist(), [[0, 1, 2, 3, 4], [0, 1, 2, 3, 4]])]
+    # ratio 0.5 keeps ceil(2.5) = 3 rows, and every row that ties with the third: |-0.2| == |0.2| keeps four in table 0
+    for ratio, rem_idx, rem_off, kept_rows in cases:
+        arch = Arch(weights)
+        want = arch(torch.tensor(rem_idx, dtype=torch.int32).cuda(), torch.tensor(rem_off, dtype=torch.int32).cuda())
+        conv = converter.SplitEmbInferenceConverter(getattr(M.SparseType, ty_name), ratio, use_array_for_index_remapping=use_array)
+        conv.convert_model(arch)
+        assert type(arch.emb_module) is M.IntNBitTableBatchedEmbeddingBagsCodegen
+        assert [e[1] for e in arch.emb_module.embedding_specs] == [len(k) for k in kept_rows]
+        got = arch(indices.cuda(), offsets.cuda())
+        torch.testing.assert_close(want.float().cpu(), got.float().cpu(), atol=1.0e-1, rtol=1.0e-1)
