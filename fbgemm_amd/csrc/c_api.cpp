@@ -38,6 +38,8 @@ hipError_t launch_compressed_indices_remap(const void* indices, bool idx64, cons
                                            const void* offsets, int64_t offsets_numel, const float* weights, int64_t first,
                                            int64_t n, void* out_indices, void* out_offsets, float* out_weights,
                                            int64_t* before, int64_t* partial, Status* status, hipStream_t stream);
+hipError_t launch_quantize_segments(const float* input, int64_t lines, int32_t T, const int32_t* d_seg_offsets,
+                                    int32_t total_D, int32_t max_D, uint8_t* output, hipStream_t stream);
 hipError_t launch_calibration_copy(const void* src, void* dst, int64_t bytes, hipStream_t stream);
 hipError_t launch_bounds_check(const int64_t* rows_per_table, int32_t T, void* indices, void* offsets, bool is64,
                                int64_t num_indices, int64_t total_B, int64_t B, const int32_t* B_offsets, int mode,
@@ -512,6 +514,10 @@ struct fbgemm_amd_tbe_plan {
   int64_t row_alignment = 16;
   std::vector<TableDesc> tables; // host copy
   TableDesc* d_tables = nullptr;
+  int32_t* d_D_offsets = nullptr; // the T + 1 output column offsets, for the 8-bit pooled output
+  int32_t max_D = 0;
+  float* pooled_tmp = nullptr;    // fp32 [B, total_D] the 8-bit pooled output is quantized from
+  int64_t pooled_tmp_cap = 0;
   // the same tables with bags laid end to end where that saves a request per row
   // (see bags_per_wave); empty when no table has such a shape. Used for long bags.
   std::vector<TableDesc> tables_packed;
@@ -590,6 +596,9 @@ int fbgemm_amd_tbe_plan_create(
     plan_lanes(d, 0, plan->total_D, q, false);
     d.lanes_recip = (65536 + d.lanes - 1) / d.lanes;
   }
+  HIP_TRY(hipMalloc((void**)&plan->d_D_offsets, sizeof(int32_t) * (T + 1)));
+  HIP_TRY(hipMemcpy(plan->d_D_offsets, D_offsets, sizeof(int32_t) * (T + 1), hipMemcpyHostToDevice));
+  for (int t = 0; t < T; ++t) plan->max_D = std::max(plan->max_D, D_offsets[t + 1] - D_offsets[t]);
   HIP_TRY(hipMalloc((void**)&plan->d_tables, sizeof(TableDesc) * T));
   HIP_TRY(hipMemcpy(plan->d_tables, plan->tables.data(), sizeof(TableDesc) * T, hipMemcpyHostToDevice));
   plan->tables_packed = plan->tables;
@@ -621,6 +630,8 @@ void fbgemm_amd_tbe_plan_destroy(fbgemm_amd_tbe_plan* plan) {
   }
   if (plan->d_tables) (void)hipFree(plan->d_tables);
   if (plan->d_tables_packed) (void)hipFree(plan->d_tables_packed);
+  if (plan->d_D_offsets) (void)hipFree(plan->d_D_offsets);
+  if (plan->pooled_tmp) (void)hipFree(plan->pooled_tmp);
   for (hipEvent_t e : plan->prof_ev) (void)hipEventDestroy(e);
   delete plan;
 }
@@ -666,6 +677,29 @@ int fbgemm_amd_tbe_forward_pruned(
   if (d_index_remappings && (!d_index_remappings_offsets || (remap_bits != 32 && remap_bits != 64)))
     return fail(FBGEMM_AMD_E_ARG, "a remap array needs its T+1 offsets and 32- or 64-bit entries");
   if (index_bits != 32 && index_bits != 64) return fail(FBGEMM_AMD_E_ARG, "index_bits must be 32 or 64");
+  if (output_ty == ST_INT8) {
+    // The reference's GPU operator quantizes every table's pooled vector row-wise to 8 bits in its
+    // output stage ([B, total_D + 8 T]: D_t bytes, fp32 scale, fp32 bias per table;
+    // embedding_forward_quantized_split_nbit_kernel_template.cu:535-566). Here: the fp32 forward into
+    // plan-owned scratch, then one launch that quantizes all (bag, table) segments.
+    if (offsets_numel < 1 || (offsets_numel - 1) % plan->T != 0) return fail(FBGEMM_AMD_E_ARG, "offsets must hold T*B+1 entries");
+    const int64_t B = (offsets_numel - 1) / plan->T;
+    if (B == 0) return 0;
+    if (!d_output) return fail(FBGEMM_AMD_E_ARG, "null data pointer");
+    float* tmp;
+    {
+      std::lock_guard<std::mutex> lk(plan->mu);
+      if (int rc = grow(&plan->pooled_tmp, &plan->pooled_tmp_cap, B * plan->total_D, (hipStream_t)stream_)) return rc;
+      tmp = plan->pooled_tmp;
+    }
+    if (int rc = fbgemm_amd_tbe_forward_pruned(plan, d_dev_weights, d_uvm_weights, d_indices, d_offsets, index_bits,
+                                               indices_numel, offsets_numel, pooling_mode, d_indice_weights, ST_FP32, tmp,
+                                               d_index_remappings, remap_bits, d_index_remappings_offsets, d_status, stream_))
+      return rc;
+    HIP_TRY(launch_quantize_segments(tmp, B, plan->T, plan->d_D_offsets, (int32_t)plan->total_D, plan->max_D,
+                                     (uint8_t*)d_output, (hipStream_t)stream_));
+    return 0;
+  }
   if (output_ty != ST_FP32 && output_ty != ST_FP16 && output_ty != ST_BF16)
     return fail(FBGEMM_AMD_E_UNSUPPORTED, "output type %d is not supported", output_ty);
   if (pooling_mode != FBGEMM_AMD_POOL_SUM && pooling_mode != FBGEMM_AMD_POOL_MEAN)

@@ -115,8 +115,8 @@ __device__ __forceinline__ void store_run(uint8_t* p, uint64_t v, int nbytes) {
 // layout: 0 = data then (scale, bias) trailer; 1 = fp16 (scale, bias) header then data
 template <bool HALF_IN, int BITS>
 __global__ __launch_bounds__(256) void quantize_rowwise_kernel(
-    const void* input, int64_t rows, int32_t cols, int32_t sb_float, int32_t layout,
-    int64_t out_stride, uint8_t* output, int32_t lpr) {
+    const void* input, int64_t rows, int32_t cols_arg, int32_t sb_float, int32_t layout,
+    int64_t out_stride, uint8_t* output, int32_t lpr, const int32_t* seg_offsets, int32_t seg_T, int64_t seg_in_stride) {
   constexpr int bits = BITS;
   const int lane = threadIdx.x & 63;
   const int sub = lane & (lpr - 1);
@@ -128,8 +128,24 @@ __global__ __launch_bounds__(256) void quantize_rowwise_kernel(
   const int64_t row_raw = wave * rows_per_wave + lane / lpr;
   const bool live = row_raw < rows;
   const int64_t row = live ? row_raw : rows - 1; // lanes past the end shadow the last row and store nothing
-  const void* in_row = reinterpret_cast<const uint8_t*>(input) + row * (int64_t)cols * (HALF_IN ? 2 : 4);
-  uint8_t* out_row = output + row * out_stride;
+  // Segment mode (seg_offsets != null): "row" r is the segment of table t = r % seg_T in
+  // line b = r / seg_T of a [lines, seg_in_stride] matrix: columns seg_offsets[t] .. seg_offsets[t+1],
+  // quantized to seg_offsets[t] + t * 8 bytes into line b of the output (every segment carries its
+  // own 8 bytes of scale and bias behind its data).
+  int32_t cols = cols_arg;
+  const void* in_row;
+  uint8_t* out_row;
+  if (seg_offsets) {
+    const int64_t b = row / seg_T;
+    const int32_t t = (int32_t)(row - b * seg_T);
+    const int32_t c0 = seg_offsets[t];
+    cols = seg_offsets[t + 1] - c0;
+    in_row = reinterpret_cast<const uint8_t*>(input) + (b * seg_in_stride + c0) * (HALF_IN ? 2 : 4);
+    out_row = output + b * out_stride + c0 + (int64_t)t * 8;
+  } else {
+    in_row = reinterpret_cast<const uint8_t*>(input) + row * (int64_t)cols * (HALF_IN ? 2 : 4);
+    out_row = output + row * out_stride;
+  }
   const bool single = cols <= lpr * RUN; // one run per lane covers the row
 
   // Fast pass: plain minimum / maximum. Which of several equal extremes is
@@ -420,7 +436,7 @@ hipError_t launch_quantize_rowwise(const void* input, bool half_in, int64_t rows
   const dim3 grid(stream_blocks(blocks)), block(256);
 #define FBGEMM_AMD_LAUNCH_Q(H, B) \
   hipLaunchKernelGGL((quantize_rowwise_kernel<H, B>), grid, block, 0, stream, input, rows, cols, sb_float, layout, \
-                     out_stride, (uint8_t*)output, lpr)
+                     out_stride, (uint8_t*)output, lpr, (const int32_t*)nullptr, 0, (int64_t)0)
   if (half_in) {
     if (bits == 2) FBGEMM_AMD_LAUNCH_Q(true, 2);
     else if (bits == 4) FBGEMM_AMD_LAUNCH_Q(true, 4);
@@ -431,6 +447,21 @@ hipError_t launch_quantize_rowwise(const void* input, bool half_in, int64_t rows
     else FBGEMM_AMD_LAUNCH_Q(false, 8);
   }
 #undef FBGEMM_AMD_LAUNCH_Q
+  return hipGetLastError();
+}
+
+// Every (line, table) segment of a [lines, total_D] fp32 matrix to 8-bit rows with an fp32
+// (scale, bias) trailer each: line b of the output holds, for t = 0 .. T-1, D_t bytes and 8 bytes.
+hipError_t launch_quantize_segments(const float* input, int64_t lines, int32_t T, const int32_t* d_seg_offsets,
+                                    int32_t total_D, int32_t max_D, uint8_t* output, hipStream_t stream) {
+  if (lines <= 0 || T <= 0 || max_D <= 0) return hipSuccess;
+  const int lpr = lanes_per_row(max_D, RUN);
+  const int64_t rows = lines * T;
+  const int64_t rows_per_block = 4 * (64 / lpr);
+  const int64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
+  const dim3 grid(stream_blocks(blocks)), block(256);
+  hipLaunchKernelGGL((quantize_rowwise_kernel<false, 8>), grid, block, 0, stream, (const void*)input, rows, max_D, 1, 0,
+                     (int64_t)total_D + 8 * (int64_t)T, output, lpr, d_seg_offsets, T, (int64_t)total_D);
   return hipGetLastError();
 }
 

@@ -137,7 +137,11 @@ Tensor int_nbit_split_embedding_codegen_lookup_function_hip(
     TORCH_CHECK(rc == 0, "fbgemm_amd: ", fbgemm_amd_last_error());
     return out;
   }
-  Tensor out = at::empty({B, total_D}, dev_weights.options().dtype(out_scalar_type(output_dtype)));
+  // 8-bit output: every table's pooled vector quantized row-wise, D_t bytes + fp32 scale + fp32 bias
+  // (fbgemm_gpu/fbgemm_gpu/sparse_ops.py:571-577)
+  Tensor out = output_dtype == FBGEMM_AMD_INT8
+      ? at::empty({B, total_D + 8 * T}, dev_weights.options().dtype(at::kByte))
+      : at::empty({B, total_D}, dev_weights.options().dtype(out_scalar_type(output_dtype)));
   if (B == 0) return out;
   Tensor& st = status_block(dev_weights);
   const int rc = fbgemm_amd_tbe_forward(
@@ -383,6 +387,8 @@ Tensor lookup_meta(
   const int64_t T = D_offsets.numel() - 1;
   const int64_t total_D = total_D_.expect_int();
   TORCH_CHECK(T > 0 && total_D > 0);
+  if (output_dtype == FBGEMM_AMD_INT8)
+    return at::empty({(offsets.size(0) - 1) / T, total_D + 8 * T}, dev_weights.options().dtype(at::kByte));
   return at::empty({(offsets.size(0) - 1) / T, total_D}, dev_weights.options().dtype(out_scalar_type(output_dtype)));
 }
 Tensor same_shape_as_indices_meta(Tensor indices, Tensor /*offsets*/, Tensor /*table*/, Tensor /*table_offsets*/) {

@@ -296,7 +296,7 @@ def int_nbit_split_embedding_codegen_lookup_function(
             if bits:
                 _raise_embedding_error(bits, pos, indices, offsets, plan, (offsets.numel() - 1) // plan.T)
         return out
-    if output_dtype not in _OUT_TORCH:
+    if output_dtype not in _OUT_TORCH and output_dtype != INT8:
         raise NotImplementedError(f"output_dtype {output_dtype} is not on this path")
     if indice_weights is not None and indice_weights.numel() == 0:
         indice_weights = None
@@ -312,7 +312,11 @@ def int_nbit_split_embedding_codegen_lookup_function(
     if total_D != plan.total_D:
         raise ValueError(f"total_D {total_D} does not match D_offsets[-1] {plan.total_D}")
     B = (offsets.numel() - 1) // T
-    out = torch.empty((B, total_D), dtype=_OUT_TORCH[output_dtype], device=dev_weights.device)
+    if output_dtype == INT8:
+        # every table's pooled vector quantized row-wise: D_t bytes, fp32 scale, fp32 bias (sparse_ops.py:571-577)
+        out = torch.empty((B, total_D + 8 * T), dtype=torch.uint8, device=dev_weights.device)
+    else:
+        out = torch.empty((B, total_D), dtype=_OUT_TORCH[output_dtype], device=dev_weights.device)
     if B == 0:
         return out
     own = status is None

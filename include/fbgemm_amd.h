@@ -161,7 +161,14 @@ void fbgemm_amd_tbe_plan_destroy(fbgemm_amd_tbe_plan* plan);
  * indices (index_bits). d_indice_weights NULL = unweighted. d_output is
  * [B, total_D] of output_ty, row-major; columns of table t start at
  * D_offsets[t]. The first forward with a new B uploads a per-wave work list
- * (allocates); later ones reuse it. */
+ * (allocates); later ones reuse it.
+ * output_ty FBGEMM_AMD_INT8 is the reference GPU operator's quantized pooled
+ * output (embedding_forward_quantized_split_nbit_kernel_template.cu:535-566;
+ * shape: fbgemm_gpu/fbgemm_gpu/sparse_ops.py:571-577): d_output is uint8
+ * [B, total_D + 8 T]; per bag and table, the pooled fp32 vector quantized
+ * row-wise to 8 bits as FloatToFused8BitRowwiseQuantized does (D_t bytes, fp32
+ * scale, fp32 bias), table t starting at byte D_offsets[t] + 8 t. Two launches
+ * more than the float outputs and a plan-owned fp32 [B, total_D] scratch. */
 int fbgemm_amd_tbe_forward(
     fbgemm_amd_tbe_plan* plan, const void* d_dev_weights, const void* d_uvm_weights,
     const void* d_indices, const void* d_offsets, int32_t index_bits,

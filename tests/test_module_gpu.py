@@ -178,3 +178,29 @@ def test_module_sequence_output(M, oracle):
                                         m.weights_tys.cpu().numpy(), [80, 60], 32, idx, off, FP16, 16)
     assert ok and tuple(got.shape) == (len(idx), 32)
     H.assert_same_bits(bits_of(got, FP16), want, "module, no pooling")
+
+
+def test_module_fused_pooled_embedding_quantization(M, oracle):
+    """The reference's check of the 8-bit pooled output
+    (fbgemm_gpu/test/tbe/inference/nbit_forward_test.py:293-340): per table, the dequantized 8-bit block
+    equals the fp32 module's block quantized and dequantized by the row-wise 8-bit operators, to 1e-2."""
+    from fbgemm_amd import ops
+    rng = np.random.default_rng(77)
+    S, L = M.SparseType, M.EmbeddingLocation.DEVICE
+    specs = [("a", 150, 64, S.INT4, L), ("b", 90, 32, S.INT8, L), ("c", 70, 16, S.FP16, L)]
+    tables = [torch.from_numpy(rng.normal(size=(n, d)).astype(np.float32)) for _, n, d, _, _ in specs]
+    mods = {}
+    for out in (S.INT8, S.FP32):
+        m = M.IntNBitTableBatchedEmbeddingBagsCodegen(specs, bounds_check_mode=M.BoundsCheckMode.NONE, output_dtype=out)
+        m.quantize_and_assign(tables)
+        mods[out] = m
+    idx, off = make_inputs(rng, [s[1] for s in specs], 9, 10, np.int32)
+    low = mods[S.INT8](cu(idx), cu(off))
+    ref = mods[S.FP32](cu(idx), cu(off))
+    Ds = [s[2] for s in specs]
+    assert low.dtype == torch.uint8 and tuple(low.shape) == (9, sum(Ds) + 8 * len(Ds))
+    for blk, want in zip(torch.split(low, [d + 8 for d in Ds], dim=1), torch.split(ref, Ds, dim=1)):
+        deq = ops.dequantize_rowwise(blk.contiguous(), want.size(1), 8, True)
+        requant = ops.dequantize_rowwise(ops.quantize_rowwise(want.contiguous(), 8, True), want.size(1), 8, True)
+        torch.testing.assert_close(deq, requant, rtol=1e-2, atol=1e-2)
+        assert torch.equal(deq, requant)  # here the two are the same arithmetic

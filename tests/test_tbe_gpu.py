@@ -413,3 +413,46 @@ def test_many_batch_sizes_reuse_and_recycle_work_lists(ops, oracle):
         rc, want = oracle.tbe_forward(weights, wo, tys, D_offsets, total_D, idx, off, 0, None, FP32, 16)
         assert rc == 0
         H.assert_same_bits(got, want, f"B={B}")
+
+
+@pytest.mark.parametrize("pooling", [0, 1])
+@pytest.mark.parametrize("dt", [np.int32, np.int64])
+def test_pooled_int8_output_is_the_rowwise_quantized_fp32_output(ops, oracle, pooling, dt):
+    """output_dtype INT8 of the pooled modes (the reference GPU operator's fused pooled-embedding
+    quantization; expected value after fbgemm_gpu/test/tbe/inference/nbit_forward_test.py:293-340):
+    every table's block is FloatToFused8BitRowwiseQuantized of that table's pooled fp32 vector,
+    D_t bytes + fp32 scale + fp32 bias. Byte for byte against the pooled oracle followed by the
+    quantizer oracle."""
+    rng = np.random.default_rng(1300 + pooling)
+    specs = [(200, 64, INT4), (150, 128, INT8), (90, 32, FP16), (300, 40, INT2), (60, 8, FP32), (120, 256, INT4), (50, 4, INT8)]
+    T, B = len(specs), 37
+    weights, wo, _ = build_weights(rng, specs, 16)
+    lens = rng.integers(0, 12, size=T * B)
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(dt)
+    idx = np.concatenate([rng.integers(0, specs[t][0], size=int(lens[t * B:(t + 1) * B].sum())) for t in range(T)]).astype(dt)
+    idx[rng.random(len(idx)) < 0.05] = -1
+    psw = rng.uniform(0, 1, len(idx)).astype(np.float32)
+    tys = np.array([s[2] for s in specs], np.uint8)
+    D_offsets = np.concatenate([[0], np.cumsum([s[1] for s in specs])]).astype(np.int32)
+    total_D = int(D_offsets[-1])
+    maxd = lambda ty: max([s[1] for s in specs if s[2] == ty], default=0)
+    for w in (None, psw):
+        got = ops.int_nbit_split_embedding_codegen_lookup_function(
+            cu(weights), torch.zeros(0, dtype=torch.uint8, device="cuda"), cu(np.zeros(T, np.int32)), cu(wo), cu(tys),
+            cu(D_offsets), total_D, maxd(INT2), maxd(INT4), maxd(INT8), maxd(FP16), maxd(FP32), cu(idx), cu(off),
+            pooling, None if w is None else cu(w), INT8, row_alignment=16)
+        assert got.dtype == torch.uint8 and tuple(got.shape) == (B, total_D + 8 * T)
+        got = got.cpu().numpy()
+        rc, pooled = oracle.tbe_forward(weights, wo, tys, D_offsets, total_D, idx, off, pooling, w, FP32, 16)
+        assert rc == 0
+        for t in range(T):
+            D = specs[t][1]
+            want = oracle.quantize_rowwise(np.ascontiguousarray(pooled[:, D_offsets[t]:D_offsets[t + 1]]), 8, True)
+            block = got[:, D_offsets[t] + 8 * t:D_offsets[t] + 8 * t + D + 8]
+            assert (block == want).all(), (t, np.argwhere(block != want)[:4])
+        # and the float forward on the same plan is not disturbed by the scratch the 8-bit one uses
+        f = ops.int_nbit_split_embedding_codegen_lookup_function(
+            cu(weights), torch.zeros(0, dtype=torch.uint8, device="cuda"), cu(np.zeros(T, np.int32)), cu(wo), cu(tys),
+            cu(D_offsets), total_D, maxd(INT2), maxd(INT4), maxd(INT8), maxd(FP16), maxd(FP32), cu(idx), cu(off),
+            pooling, None if w is None else cu(w), FP32, row_alignment=16)
+        H.assert_same_bits(f.cpu().numpy(), pooled, "fp32 forward after the 8-bit one")

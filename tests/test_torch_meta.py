@@ -40,8 +40,11 @@ def test_lookup_shapes(fb):
         assert tuple(seq.shape) == (40, 64) and seq.dtype == dt
     # rows copied as stored: 8-bit rows carry their 4 bytes of scale / bias
     assert tuple(lookup(fb, 2, 2).shape) == (40, 68) and lookup(fb, 2, 2).dtype == torch.uint8
+    # pooled 8-bit output: every table's block carries 8 bytes of scale and bias
+    q = lookup(fb, 0, 2)
+    assert tuple(q.shape) == (5, 96 + 8 * 3) and q.dtype == torch.uint8
     with pytest.raises(RuntimeError):
-        lookup(fb, 0, 2)
+        lookup(fb, 0, 3)
 
 
 def test_remap_shapes_and_schemas(fb):
