@@ -931,31 +931,53 @@ __global__ __launch_bounds__(1024) void bag_order_kernel(const void* offsets, in
   const int64_t ob = (int64_t)t * B;
   for (int i = tid; i < SORT_BINS; i += 1024) bins[i] = 0;
   __syncthreads();
-  auto bin_of = [&](int b) {
-    int64_t len = read_offset(offsets, off64, ob + b + 1) - read_offset(offsets, off64, ob + b);
-    if (len < 0) len = 0;
-    if (len > SORT_BINS - 1) len = SORT_BINS - 1;
-    return SORT_BINS - 1 - (int)len; // longest first
-  };
-  for (int b = tid; b < B; b += 1024) atomicAdd(&bins[bin_of(b)], 1);
-  __syncthreads();
-  // exclusive scan of the SORT_BINS (== blockDim) counters
-  const int mine = bins[tid];
-  partial[tid] = mine;
-  __syncthreads();
-  for (int step = 1; step < 1024; step <<= 1) {
-    const int v = tid >= step ? partial[tid - step] : 0;
-    __syncthreads();
-    partial[tid] += v;
-    __syncthreads();
+  // bin of a bag: SORT_BINS - 1 - min(length, SORT_BINS - 1), so that the longest come first
+  // the first two bags of every thread stay in registers between the two passes
+  int64_t a0 = 0, a1 = 0, b0 = 0, b1 = 0;
+  for (int b = tid, it = 0; b < B; b += 1024, ++it) {
+    const int64_t o0 = read_offset(offsets, off64, ob + b), o1 = read_offset(offsets, off64, ob + b + 1);
+    if (it == 0) {
+      a0 = o0;
+      a1 = o1;
+    } else if (it == 1) {
+      b0 = o0;
+      b1 = o1;
+    }
+    int64_t len = o1 - o0;
+    len = len < 0 ? 0 : (len > SORT_BINS - 1 ? SORT_BINS - 1 : len);
+    atomicAdd(&bins[SORT_BINS - 1 - (int)len], 1);
   }
-  bins[tid] = partial[tid] - mine;
   __syncthreads();
-  for (int b = tid; b < B; b += 1024) {
-    const int p = atomicAdd(&bins[bin_of(b)], 1);
+  // exclusive scan of the SORT_BINS (== blockDim) counters: inside each wave
+  // through lane shuffles, then over the 16 wave totals
+  const int mine = bins[tid];
+  int incl = mine;
+  const int lane = tid & 63;
+  for (int step = 1; step < 64; step <<= 1) {
+    const int v = __shfl_up(incl, step, 64);
+    if (lane >= step) incl += v;
+  }
+  if (lane == 63) partial[tid >> 6] = incl;
+  __syncthreads();
+  int before = 0;
+  for (int w = 0; w < (tid >> 6); ++w) before += partial[w];
+  bins[tid] = before + incl - mine;
+  __syncthreads();
+  for (int b = tid, it = 0; b < B; b += 1024, ++it) {
     BagEntry be;
-    be.o0 = read_offset(offsets, off64, ob + b);
-    be.o1 = read_offset(offsets, off64, ob + b + 1);
+    if (it == 0) {
+      be.o0 = a0;
+      be.o1 = a1;
+    } else if (it == 1) {
+      be.o0 = b0;
+      be.o1 = b1;
+    } else {
+      be.o0 = read_offset(offsets, off64, ob + b);
+      be.o1 = read_offset(offsets, off64, ob + b + 1);
+    }
+    int64_t len = be.o1 - be.o0;
+    len = len < 0 ? 0 : (len > SORT_BINS - 1 ? SORT_BINS - 1 : len);
+    const int p = atomicAdd(&bins[SORT_BINS - 1 - (int)len], 1);
     be.bag = b;
     be.pad0 = 0;
     be.pad1 = 0;
