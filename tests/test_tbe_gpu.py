@@ -456,3 +456,52 @@ def test_pooled_int8_output_is_the_rowwise_quantized_fp32_output(ops, oracle, po
             cu(D_offsets), total_D, maxd(INT2), maxd(INT4), maxd(INT8), maxd(FP16), maxd(FP32), cu(idx), cu(off),
             pooling, None if w is None else cu(w), FP32, row_alignment=16)
         H.assert_same_bits(f.cpu().numpy(), pooled, "fp32 forward after the 8-bit one")
+
+
+@pytest.mark.parametrize("pooling", [0, 2])
+def test_tables_in_both_weights_buffers(ops, oracle, pooling):
+    """weights_placements: tables 1 and 3 live in the second buffer (uvm_weights), whose offsets
+    count from its own start; the row bound of a table comes from the next table of the SAME buffer."""
+    rng = np.random.default_rng(1400 + pooling)
+    D = 64
+    specs = [(120, D, INT4), (80, D, INT8), (60, D, FP16), (200, D, INT4), (30, D, INT2)]
+    T, B = len(specs), 21
+    weights, wo, rbs = build_weights(rng, specs, 16)
+    # the same table bytes dealt to two buffers
+    bufs, offs = [[], []], [0, 0]
+    place = np.array([0, 1, 0, 1, 0], np.int32)
+    wo2 = np.zeros(T, np.int64)
+    for t, (rows, _, _) in enumerate(specs):
+        blob = weights[wo[t]:wo[t] + rows * rbs[t]]
+        pad = (-len(blob)) % 128
+        wo2[t] = offs[place[t]]
+        bufs[place[t]] += [blob, np.zeros(pad, np.uint8)]
+        offs[place[t]] += len(blob) + pad
+    dev, uvm = np.concatenate(bufs[0]), np.concatenate(bufs[1])
+    lens = rng.integers(0, 9, size=T * B)
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    idx = np.concatenate([rng.integers(0, specs[t][0], size=int(lens[t * B:(t + 1) * B].sum())) for t in range(T)]).astype(np.int64)
+    idx[0] = specs[0][0] - 1
+    tys = np.array([s[2] for s in specs], np.uint8)
+    D_offsets = (np.arange(T + 1) * D).astype(np.int32)
+    maxd = lambda ty: D if ty in tys else 0
+    got = ops.int_nbit_split_embedding_codegen_lookup_function(
+        cu(dev), cu(uvm), cu(place), cu(wo2), cu(tys), cu(D_offsets), T * D, maxd(INT2), maxd(INT4), maxd(INT8),
+        maxd(FP16), 0, cu(idx), cu(off), pooling, None, FP32, row_alignment=16).cpu().numpy()
+    if pooling == 2:
+        ok, want = oracle.tbe_forward_nobag(weights, wo, tys, [s[0] for s in specs], D, idx, off, FP32, 16)
+        assert ok
+    else:
+        rc, want = oracle.tbe_forward(weights, wo, tys, D_offsets, T * D, idx, off, pooling, None, FP32, 16)
+        assert rc == 0
+    H.assert_same_bits(got, want, f"two buffers, pooling {pooling}")
+    # the last row of the last table of each buffer is in range, the one after it is not
+    for t in (3, 4):
+        s = int(off[t * B])
+        if int(off[(t + 1) * B]) > s:
+            bad = idx.copy()
+            bad[s] = specs[t][0] + (128 // rbs[t]) + 1  # past the rows and past the buffer's padding
+            with pytest.raises(RuntimeError, match="out of bounds"):
+                ops.int_nbit_split_embedding_codegen_lookup_function(
+                    cu(dev), cu(uvm), cu(place), cu(wo2), cu(tys), cu(D_offsets), T * D, maxd(INT2), maxd(INT4), maxd(INT8),
+                    maxd(FP16), 0, cu(bad), cu(off), pooling, None, FP32, row_alignment=16)
