@@ -42,6 +42,9 @@ def parse():
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="also run one plain copy of this many MiB (yardstick for hardware byte counters)")
+    ap.add_argument("--graph", action="store_true",
+                    help="capture one forward in a HIP graph after the warm-up and time replays of it "
+                         "(what a serving loop would do; the default times eager launches)")
     ap.add_argument("--check", action="store_true", help="verify a sample of the output against the oracle first")
     ap.add_argument("--op", default="lookup",
                     choices=["lookup", "quantize", "dequantize", "bounds_check", "pruned_array_lookup",
@@ -100,7 +103,8 @@ def tbe_runner(p, torch):
             C.c_void_p(st.buf.data_ptr()), stream)
 
     def launch():
-        rc = lib.fbgemm_amd_tbe_forward_pruned(*args)
+        # the stream of the moment: under graph capture it is the capturing stream
+        rc = lib.fbgemm_amd_tbe_forward_pruned(*args[:-1], C.c_void_p(torch.cuda.current_stream().cuda_stream))
         if rc:
             raise RuntimeError(lib.fbgemm_amd_last_error().decode())
 
@@ -130,8 +134,9 @@ def spmdm_runner(probs, torch):
         outs.append(out)
 
     def launch():
+        now = C.c_void_p(torch.cuda.current_stream().cuda_stream)
         for cfg, a in calls:
-            rc = lib.fbgemm_amd_spmdm_launch(C.byref(cfg), *a)
+            rc = lib.fbgemm_amd_spmdm_launch(C.byref(cfg), *a[:-1], now)
             if rc:
                 raise RuntimeError(lib.fbgemm_amd_last_error().decode())
 
@@ -463,14 +468,25 @@ def main():
     for _ in range(a.warmup):
         launch()
     torch.cuda.synchronize()
-    if p is not None:  # HIP events around every lookup_kernel launch of the timed region, on its stream
+    step = launch
+    if a.graph:
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                launch()
+        torch.cuda.synchronize()
+        step = graph.replay
+        step()
+        torch.cuda.synchronize()
+    elif p is not None:  # HIP events around every lookup_kernel launch of the timed region, on its stream
         from fbgemm_amd import _lib
         _lib.check(_lib.lib().fbgemm_amd_tbe_plan_profile(plan.handle, a.steps))
     ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     ev0.record()
     for _ in range(a.steps):
-        launch()
+        step()
     ev1.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
@@ -480,7 +496,9 @@ def main():
     ms_per_step = wall * 1e3 / a.steps
     forward_ms = ev0.elapsed_time(ev1) / a.steps  # events on the launch stream, back-to-back forwards
     kernel_ms, kernel_name = forward_ms, "lookup_kernel (+ bag_order_kernel), per forward"
-    if p is not None:
+    if a.graph:
+        kernel_name = "lookup_kernel (+ bag_order_kernel), per graph replay"
+    elif p is not None:
         ms = (C.c_float * a.steps)()
         n = C.c_int32(0)
         _lib.check(_lib.lib().fbgemm_amd_tbe_plan_profile_read(plan.handle, ms, a.steps, C.byref(n)))
@@ -496,7 +514,7 @@ def main():
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": name, "config_id": a.config, "scale": a.scale, "lookups_per_step": lookups,
                    "useful_row_bytes_per_step": useful, "other_bytes_per_step": other,
-                   "output_dtype": dtype_out, "launches_per_step": launches_per_step},
+                   "output_dtype": dtype_out, "launches_per_step": launches_per_step, "hip_graph": bool(a.graph)},
         "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
         "pooled_rows_per_s": round(lookups / (ms_per_step * 1e-3), 1),
         "roofline": {"bound": "hbm", "achieved": round(kern_gbps, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
