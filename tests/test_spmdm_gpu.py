@@ -95,6 +95,14 @@ def check_case(ops, oracle, *, ty, D, table, idx, off_or_len, w=None, normalize=
     return ok_g
 
 
+@pytest.fixture(autouse=True, params=["wide", "narrow"])
+def lane_shape(request, monkeypatch):
+    """Small launches take 4-byte lanes by default; every test here runs with that policy and with the
+    16-byte lanes large launches get (the library reads the switch on every call)."""
+    monkeypatch.setenv("FBGEMM_AMD_NARROW_BELOW_WAVES", "0" if request.param == "wide" else "1024")
+    return request.param
+
+
 @pytest.fixture(scope="module")
 def ops():
     assert torch.cuda.is_available(), "these tests need the GPU"
