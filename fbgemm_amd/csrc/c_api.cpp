@@ -533,6 +533,9 @@ struct fbgemm_amd_tbe_plan {
   // (see bags_per_wave); empty when no table has such a shape. Used for long bags.
   std::vector<TableDesc> tables_packed;
   TableDesc* d_tables_packed = nullptr;
+  // the same tables with 4-byte lanes (see plan_lanes): for forwards too small to fill the device
+  std::vector<TableDesc> tables_narrow;
+  TableDesc* d_tables_narrow = nullptr;
   int device = 0;
   // per-B work lists
   struct Work {
@@ -626,6 +629,14 @@ int fbgemm_amd_tbe_plan_create(
   } else {
     plan->tables_packed.clear();
   }
+  plan->tables_narrow = plan->tables;
+  for (int t = 0; t < T; ++t) {
+    TableDesc& d = plan->tables_narrow[t];
+    plan_lanes(d, 0, plan->total_D, quantised(d.ty), false, true);
+    d.lanes_recip = (65536 + d.lanes - 1) / d.lanes;
+  }
+  HIP_TRY(hipMalloc((void**)&plan->d_tables_narrow, sizeof(TableDesc) * T));
+  HIP_TRY(hipMemcpy(plan->d_tables_narrow, plan->tables_narrow.data(), sizeof(TableDesc) * T, hipMemcpyHostToDevice));
   *out = plan;
   return 0;
 }
@@ -641,6 +652,7 @@ void fbgemm_amd_tbe_plan_destroy(fbgemm_amd_tbe_plan* plan) {
   }
   if (plan->d_tables) (void)hipFree(plan->d_tables);
   if (plan->d_tables_packed) (void)hipFree(plan->d_tables_packed);
+  if (plan->d_tables_narrow) (void)hipFree(plan->d_tables_narrow);
   if (plan->d_D_offsets) (void)hipFree(plan->d_D_offsets);
   if (plan->pooled_tmp) (void)hipFree(plan->pooled_tmp);
   for (hipEvent_t e : plan->prof_ev) (void)hipEventDestroy(e);
@@ -736,13 +748,23 @@ int fbgemm_amd_tbe_forward_pruned(
   // makes the kernel arithmetic-bound and the saving does not pay (measured: 15
   // rows per bag loses 9 %, 30 rows per bag gains 5 %).
   static const int packed_mode = env_int("FBGEMM_AMD_PACKED", 1); // 0 never, 1 by bag length, 2 always
-  const bool use_packed = !plan->tables_packed.empty() &&
+  // A forward of fewer than four waves per compute unit is bound by the chain of memory round
+  // trips inside a wave: 4-byte lanes spread its bags over four times the waves.
+  const int narrow_below = env_int("FBGEMM_AMD_NARROW_BELOW_WAVES", 1024); // read per call: tests switch it
+  int64_t wide_waves = 0;
+  for (const TableDesc& d : plan->tables) {
+    const int G = bags_per_wave(d.lanes, d.packed);
+    wide_waves += (B + G - 1) / G;
+  }
+  const bool use_narrow = wide_waves < narrow_below;
+  const bool use_packed = !use_narrow && !plan->tables_packed.empty() &&
       (packed_mode == 2 || (packed_mode == 1 && indices_numel >= 20 * (int64_t)plan->T * B));
-  const std::vector<TableDesc>& tables = use_packed ? plan->tables_packed : plan->tables;
+  const std::vector<TableDesc>& tables = use_narrow ? plan->tables_narrow : (use_packed ? plan->tables_packed : plan->tables);
+  const int variant = use_narrow ? 2 : (use_packed ? 1 : 0);
   fbgemm_amd_tbe_plan::Work w;
   {
     std::lock_guard<std::mutex> lk(plan->mu);
-    auto it = plan->work.find({B, use_packed ? 1 : 0});
+    auto it = plan->work.find({B, variant});
     if (it == plan->work.end()) {
       // The work list is 8 runs, one per XCD (see lookup_kernel). Tables are
       // cut into slices of waves, the slices are dealt to the XCDs so that
@@ -842,14 +864,14 @@ int fbgemm_amd_tbe_forward_pruned(
         }
         plan->work.clear();
       }
-      it = plan->work.emplace(std::make_pair(B, use_packed ? 1 : 0), nw).first;
+      it = plan->work.emplace(std::make_pair(B, variant), nw).first;
     }
     w = it->second;
   }
 
   LookupArgs a;
   memset(&a, 0, sizeof(a));
-  a.tables = use_packed ? plan->d_tables_packed : plan->d_tables;
+  a.tables = use_narrow ? plan->d_tables_narrow : (use_packed ? plan->d_tables_packed : plan->d_tables);
   a.weights[0] = (const uint8_t*)d_dev_weights;
   a.weights[1] = (const uint8_t*)d_uvm_weights;
   a.indices = d_indices;

@@ -17,7 +17,7 @@ import helpers as H
 from helpers import BF16, FP16, FP32, INT2, INT4, INT8
 
 torch = pytest.importorskip("torch")
-pytestmark = pytest.mark.gpu
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("lane_shape")]
 
 SENTINELS = 10
 
@@ -93,14 +93,6 @@ def check_case(ops, oracle, *, ty, D, table, idx, off_or_len, w=None, normalize=
     if ok_o:
         H.assert_same_bits(out_g, out_o, what)
     return ok_g
-
-
-@pytest.fixture(autouse=True, params=["wide", "narrow"])
-def lane_shape(request, monkeypatch):
-    """Small launches take 4-byte lanes by default; every test here runs with that policy and with the
-    16-byte lanes large launches get (the library reads the switch on every call)."""
-    monkeypatch.setenv("FBGEMM_AMD_NARROW_BELOW_WAVES", "0" if request.param == "wide" else "1024")
-    return request.param
 
 
 @pytest.fixture(scope="module")

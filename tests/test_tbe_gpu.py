@@ -12,7 +12,7 @@ import helpers as H
 from helpers import BF16, FP16, FP32, INT2, INT4, INT8
 
 torch = pytest.importorskip("torch")
-pytestmark = pytest.mark.gpu
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("lane_shape")]
 
 
 @pytest.fixture(scope="module")
