@@ -250,3 +250,65 @@ def test_large_call_takes_the_ordered_path(ops, oracle):
     assert len(idx) > (1 << 21)
     check_case(ops, oracle, ty=INT4, D=D, table=table, idx=idx, off_or_len=off, normalize=True, out_ty=FP16,
                data_size=rows, output_size=nb, what="2.6 M lookups, ordered bags")
+
+
+def same_bits_or_both_nan(got, want, what):
+    """Bit equality, except that any NaN matches any NaN (the sign and payload of a NaN an
+    invalid operation makes differ between the CPU and the GPU)."""
+    if got.dtype == np.float32:
+        gn, wn = np.isnan(got), np.isnan(want)
+        gb, wb = got.view(np.uint32), want.view(np.uint32)
+    else:  # fp16 / bf16 patterns
+        f = lambda a: (a & 0x7C00) == 0x7C00 if what.endswith("fp16") else (a & 0x7F80) == 0x7F80
+        gn = f(got) & ((got & (0x03FF if what.endswith("fp16") else 0x007F)) != 0)
+        wn = f(want) & ((want & (0x03FF if what.endswith("fp16") else 0x007F)) != 0)
+        gb, wb = got, want
+    assert (gn == wn).all(), f"{what}: NaNs in different places"
+    assert (gb[~wn] == wb[~wn]).all(), f"{what}: {np.argwhere(gb[~wn] != wb[~wn])[:4]}"
+
+
+@pytest.mark.parametrize("ty,sbl", [(INT8, True), (INT8, False), (INT4, True), (INT4, False), (INT2, False), (FP16, True), (FP32, True)])
+def test_special_values(ops, oracle, ty, sbl):
+    """Scales at and beyond 2^100 (where the 4- and 8-bit kernels leave their pre-scaled arithmetic and a
+    wave redoes its work the plain way), infinities, NaNs, denormals and signed zeros in scales, biases,
+    per-sample weights and float rows: every finite result bit for bit, NaN where the reference has NaN."""
+    rng = np.random.default_rng(31 + ty)
+    rows, D, nb = 40, 64, 30
+    table, stride = H.make_table(rng, ty, rows, D, sbl)
+    t2 = table.reshape(rows, stride)
+    specials32 = np.array([1e35, -3e33, np.inf, -np.inf, np.nan, 1e-40, -1e-42, 0.0, -0.0, 2.0 ** 100, np.nextafter(np.float32(2.0 ** 100), np.float32(0))], np.float32)
+    np.seterr(over="ignore")  # the casts of 1e35 to half give inf on purpose
+    if ty in (INT8, INT4, INT2):
+        pb = H.packed_bytes(ty, D)
+        for r in range(len(specials32)):
+            if ty == INT8 and sbl:  # fp32 pair behind the data
+                t2[r, pb:pb + 4] = specials32[r:r + 1].view(np.uint8)
+                t2[r + 12, pb + 4:pb + 8] = specials32[r:r + 1].view(np.uint8)
+            else:  # fp16 pair: behind (sbl) or in front of the data
+                o = pb if sbl else 0
+                t2[r, o:o + 2] = specials32[r:r + 1].astype(np.float16).view(np.uint8)
+                t2[r + 12, o + 2:o + 4] = specials32[r:r + 1].astype(np.float16).view(np.uint8)
+    elif ty == FP16:
+        t2.view(np.uint16)[:len(specials32), 3] = specials32.astype(np.float16).view(np.uint16)
+        t2.view(np.uint16)[5, 7] = 0x0001  # the smallest half denormal
+    else:
+        t2.view(np.float32)[:len(specials32), 3] = specials32
+    idx, off, lens = H.make_bags(rng, rows, nb, 6)
+    wts = rng.normal(size=len(idx)).astype(np.float32)
+    wts[::7] = 1e30   # times an fp16 scale of ~0.05: beyond 2^100
+    wts[3::11] = np.float32(1e-40)
+    wts[5::13] = np.inf
+    wts[6::17] = np.nan
+    wts[8::19] = -0.0
+    table = np.ascontiguousarray(t2).reshape(-1)
+    for w in (None, wts):
+        for out_ty, name in ((FP32, "fp32"), (FP16, "fp16"), (BF16, "bf16")):
+            for normalize in (False, True):
+                ok_g, out_g, sentinel = run_gpu(
+                    ops, ty=ty, D=D, table=table, idx=idx, off_or_len=off, w=w, normalize=normalize, out_ty=out_ty,
+                    positional=False, use_offsets=True, output_stride=-1, input_stride=-1, sbl=sbl, remap=None,
+                    data_size=rows, output_size=nb)
+                ok_o, out_o = oracle.spmdm(ty, D, table, idx, off, weights=w, normalize=normalize, out_ty=out_ty,
+                                           scale_bias_last=sbl, data_size=rows, output_size=nb)
+                assert ok_g and ok_o
+                same_bits_or_both_nan(out_g, out_o, f"special values ty={ty} sbl={sbl} weighted={w is not None} {name}")

@@ -505,3 +505,49 @@ def test_tables_in_both_weights_buffers(ops, oracle, pooling):
                 ops.int_nbit_split_embedding_codegen_lookup_function(
                     cu(dev), cu(uvm), cu(place), cu(wo2), cu(tys), cu(D_offsets), T * D, maxd(INT2), maxd(INT4), maxd(INT8),
                     maxd(FP16), 0, cu(bad), cu(off), pooling, None, FP32, row_alignment=16)
+
+
+@pytest.mark.parametrize("long_bags", [False, True])
+def test_special_values_in_the_table_batched_forward(ops, oracle, long_bags):
+    """Per-sample weights that push weight * scale beyond 2^100 (the 4- and 8-bit lanes then redo their
+    work without the pre-scaled arithmetic), infinite / NaN / denormal / signed-zero weights and fp16
+    scale-bias pairs: finite results bit for bit, NaN where the oracle has NaN. Long bags take the
+    end-to-end lane layout of the 9-chunk rows."""
+    from test_spmdm_gpu import same_bits_or_both_nan
+    np.seterr(over="ignore")
+    rng = np.random.default_rng(1500 + int(long_bags))
+    specs = [(60, 256, INT4), (50, 128, INT8), (40, 64, INT4), (30, 32, FP16), (45, 256, INT8), (25, 16, INT2)]
+    T, B = len(specs), 19
+    weights, wo, rbs = build_weights(rng, specs, 16)
+    specials = np.array([np.inf, -np.inf, np.nan, 6e-8, -6e-8, 0.0, -0.0, 65504.0], np.float32).astype(np.float16)
+    for t, (rows, D, ty) in enumerate(specs):
+        if ty == FP16:
+            continue
+        tbl = weights[wo[t]:wo[t] + rows * rbs[t]].reshape(rows, rbs[t])
+        for r in range(len(specials)):
+            tbl[r, 0:2] = specials[r:r + 1].view(np.uint8)
+            tbl[r + 10, 2:4] = specials[r:r + 1].view(np.uint8)
+    lens = rng.integers(20, 40, size=T * B) if long_bags else rng.integers(0, 9, size=T * B)
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    idx = np.concatenate([rng.integers(0, specs[t][0], size=int(lens[t * B:(t + 1) * B].sum())) for t in range(T)]).astype(np.int64)
+    psw = rng.normal(size=len(idx)).astype(np.float32)
+    psw[::9] = 1e30
+    psw[4::11] = np.float32(1e-40)
+    psw[5::23] = np.inf
+    psw[6::29] = np.nan
+    psw[7::31] = -0.0
+    tys = np.array([s[2] for s in specs], np.uint8)
+    D_offsets = np.concatenate([[0], np.cumsum([s[1] for s in specs])]).astype(np.int32)
+    total_D = int(D_offsets[-1])
+    maxd = lambda ty: max([s[1] for s in specs if s[2] == ty], default=0)
+    for w in (None, psw):
+        for pooling in (0, 1):
+            for out_ty, name in ((FP32, "fp32"), (FP16, "fp16"), (BF16, "bf16")):
+                got = ops.int_nbit_split_embedding_codegen_lookup_function(
+                    cu(weights), torch.zeros(0, dtype=torch.uint8, device="cuda"), cu(np.zeros(T, np.int32)), cu(wo), cu(tys),
+                    cu(D_offsets), total_D, maxd(INT2), maxd(INT4), maxd(INT8), maxd(FP16), 0, cu(idx), cu(off), pooling,
+                    None if w is None else cu(w), out_ty, row_alignment=16).cpu()
+                got = got.numpy() if out_ty == FP32 else got.view(torch.int16).numpy().view(np.uint16)
+                rc, want = oracle.tbe_forward(weights, wo, tys, D_offsets, total_D, idx, off, pooling, w, out_ty, 16)
+                assert rc == 0
+                same_bits_or_both_nan(got, want, f"special values weighted={w is not None} pooling={pooling} {name}")
