@@ -96,8 +96,9 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(torch.nn.Module):
         dims = [e[2] for e in self.embedding_specs]
         tys = [e[3] for e in self.embedding_specs]
         for e in self.embedding_specs:
-            if e[4] != EmbeddingLocation.DEVICE:
-                raise NotImplementedError("tables are resident in HBM (EmbeddingLocation.DEVICE); UVM and the cache are not on this path")
+            if e[4] not in (EmbeddingLocation.DEVICE, EmbeddingLocation.MANAGED):
+                raise NotImplementedError("tables are resident in HBM (DEVICE, or MANAGED = the operator's second weights "
+                                          "buffer, kept in HBM too); the UVM cache and host tables are not on this path")
         if self.pooling_mode == PoolingMode.NONE:
             assert all(d == dims[0] for d in dims), "Mixed dimension tables are only supported for pooling tables."
         T_ = len(self.embedding_specs)
@@ -130,17 +131,21 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(torch.nn.Module):
         self.register_buffer("weights_tys", torch.tensor([tys[t].as_int() for t in self.feature_table_map], device=dev, dtype=torch.uint8))
 
         # split_table_batched_embeddings_ops_inference.py:103-147 (nbit_construct_split_state)
-        offsets, size = [], 0
-        for _, n, dim, ty, _ in self.embedding_specs:
+        # one running offset per buffer: DEVICE tables in weights_dev, MANAGED ones in weights_uvm
+        offsets, sizes, places = [], [0, 0], []
+        for _, n, dim, ty, loc in self.embedding_specs:
             state = n * rounded_row_size_in_bytes(dim, ty, self.row_alignment)
             if cacheline_alignment:
                 state = round_up(state, 128)
-            offsets.append(size)
-            size += state
-        self.dev_size = size
+            buf = 1 if loc == EmbeddingLocation.MANAGED else 0
+            places.append(buf)
+            offsets.append(sizes[buf])
+            sizes[buf] += state
+        self.dev_size, self.uvm_size = sizes
         self.weights_physical_offsets = offsets
+        self.weights_physical_placements = places
         self.register_buffer("weights_offsets", torch.tensor([offsets[t] for t in self.feature_table_map], device=dev, dtype=torch.int64))
-        self.register_buffer("weights_placements", torch.zeros(T, device=dev, dtype=torch.int32))
+        self.register_buffer("weights_placements", torch.tensor([places[t] for t in self.feature_table_map], device=dev, dtype=torch.int32))
         self.weights_dev = torch.zeros(0, device=dev, dtype=torch.uint8)
         self.weights_uvm = torch.zeros(0, device=dev, dtype=torch.uint8)
         self.weight_initialized = False
@@ -160,6 +165,7 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(torch.nn.Module):
     def initialize_weights(self):
         if not self.weight_initialized:
             self.weights_dev = torch.zeros(self.dev_size, device=self.current_device, dtype=torch.uint8)
+            self.weights_uvm = torch.zeros(self.uvm_size, device=self.current_device, dtype=torch.uint8)
             self.weight_initialized = True
 
     def split_embedding_weights_with_scale_bias(self, split_scale_bias_mode=1):
@@ -170,7 +176,8 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(torch.nn.Module):
         for t, (_, n, dim, ty, _) in enumerate(self.embedding_specs):
             rb = rounded_row_size_in_bytes(dim, ty, self.row_alignment)
             off = self.weights_physical_offsets[t]
-            w = self.weights_dev.detach()[off:off + n * rb].view(n, rb)
+            buf = self.weights_uvm if self.weights_physical_placements[t] else self.weights_dev
+            w = buf.detach()[off:off + n * rb].view(n, rb)
             if split_scale_bias_mode == 0:
                 splits.append((w, None, None))
                 continue

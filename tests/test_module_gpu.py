@@ -204,3 +204,25 @@ def test_module_fused_pooled_embedding_quantization(M, oracle):
         requant = ops.dequantize_rowwise(ops.quantize_rowwise(want.contiguous(), 8, True), want.size(1), 8, True)
         torch.testing.assert_close(deq, requant, rtol=1e-2, atol=1e-2)
         assert torch.equal(deq, requant)  # here the two are the same arithmetic
+
+
+def test_module_with_managed_tables(M, oracle):
+    """EmbeddingLocation.MANAGED tables live in the operator's second weights buffer (in HBM here): the same
+    lookups as an all-DEVICE module holding the same rows."""
+    rng = np.random.default_rng(88)
+    S, L = M.SparseType, M.EmbeddingLocation
+    shapes = [("a", 120, 64, S.INT4), ("b", 80, 32, S.INT8), ("c", 60, 16, S.FP16), ("d", 90, 128, S.INT4)]
+    tables = [torch.from_numpy(rng.normal(size=(n, d)).astype(np.float32)) for _, n, d, _ in shapes]
+    mods = []
+    for locs in ([L.DEVICE] * 4, [L.MANAGED, L.DEVICE, L.MANAGED, L.DEVICE], [L.MANAGED] * 4):
+        m = M.IntNBitTableBatchedEmbeddingBagsCodegen([s + (loc,) for s, loc in zip(shapes, locs)],
+                                                      bounds_check_mode=M.BoundsCheckMode.NONE, output_dtype=S.FP32)
+        m.quantize_and_assign(tables)
+        mods.append(m)
+    assert mods[1].weights_uvm.numel() > 0 and mods[1].weights_placements.tolist() == [1, 0, 1, 0]
+    idx, off = make_inputs(rng, [s[1] for s in shapes], 11, 9, np.int64)
+    want = mods[0](cu(idx), cu(off))
+    for m in mods[1:]:
+        assert torch.equal(m(cu(idx), cu(off)), want)
+    with pytest.raises(NotImplementedError):
+        M.IntNBitTableBatchedEmbeddingBagsCodegen([shapes[0] + (L.MANAGED_CACHING,)])
