@@ -37,7 +37,8 @@ hipError_t launch_prune_gather(const void* in, int64_t rows, int64_t row_bytes, 
 hipError_t launch_compressed_indices_remap(const void* indices, bool idx64, const int32_t* mapping, int64_t mapping_numel,
                                            const void* offsets, int64_t offsets_numel, const float* weights, int64_t first,
                                            int64_t n, void* out_indices, void* out_offsets, float* out_weights,
-                                           int64_t* before, int64_t* partial, Status* status, hipStream_t stream);
+                                           int64_t* before, int64_t* partial, int32_t* mapped, Status* status,
+                                           hipStream_t stream);
 hipError_t launch_quantize_segments(const float* input, int64_t lines, int32_t T, const int32_t* d_seg_offsets,
                                     int32_t total_D, int32_t max_D, uint8_t* output, hipStream_t stream);
 hipError_t launch_calibration_copy(const void* src, void* dst, int64_t bytes, hipStream_t stream);
@@ -1121,11 +1122,13 @@ int fbgemm_amd_compressed_indices_remap(
   std::lock_guard<std::mutex> lk(g_mu);
   DeviceScratch* s;
   if (int rc = get_scratch(&s)) return rc;
-  if (int rc = grow(&s->fixed, &s->fixed_cap, n + 1, stream)) return rc;
+  // one scratch buffer: n + 1 running counts (int64), then the n mapped rows (int32)
+  if (int rc = grow(&s->fixed, &s->fixed_cap, (n + 1) + (n + 1) / 2 + 1, stream)) return rc;
   if (int rc = grow(&s->partial, &s->partial_cap, prune_partials(n + 1), stream)) return rc;
   HIP_TRY(launch_compressed_indices_remap(d_indices, index_bits == 64, d_mapping, mapping_numel, d_offsets, offsets_numel,
                                           d_weights, first, n, d_out_indices, d_out_offsets, d_out_weights, s->fixed,
-                                          s->partial, d_status ? (Status*)d_status : s->status, stream));
+                                          s->partial, reinterpret_cast<int32_t*>(s->fixed + n + 1),
+                                          d_status ? (Status*)d_status : s->status, stream));
   return 0;
 }
 

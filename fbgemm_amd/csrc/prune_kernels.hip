@@ -161,28 +161,33 @@ __global__ __launch_bounds__(256) void prune_gather_kernel(const uint8_t* in, in
 template <typename index_t>
 __global__ __launch_bounds__(PSCAN_THREADS) void remap_count_kernel(const index_t* indices, const int32_t* mapping,
                                                                     int64_t mapping_numel, int64_t first, int64_t n,
-                                                                    int64_t* partial, Status* status) {
+                                                                    int64_t* partial, int32_t* mapped, Status* status) {
   __shared__ int64_t lds[PSCAN_THREADS];
   const int64_t base = (int64_t)blockIdx.x * PSCAN_BLOCK + (int64_t)threadIdx.x * PSCAN_ITEMS;
   int64_t local = 0;
-  for (int i = 0; i < PSCAN_ITEMS; ++i)
-    if (base + i < n && mapped_row(indices, mapping, mapping_numel, first + base + i, status) != -1) ++local;
+  for (int i = 0; i < PSCAN_ITEMS; ++i) {
+    if (base + i < n) {
+      // the gather through the mapping is made once: pass 3 reads the rows back in order
+      const int32_t row = mapped_row(indices, mapping, mapping_numel, first + base + i, status);
+      mapped[base + i] = row;
+      if (row != -1) ++local;
+    }
+  }
   const int64_t incl = block_inclusive_sum(local, lds);
   if (threadIdx.x == PSCAN_THREADS - 1) partial[blockIdx.x] = incl;
 }
 
 // pass 3: move the entries; before[k] = entries that stay in front of position first + k (k = 0 .. n)
 template <typename index_t>
-__global__ __launch_bounds__(PSCAN_THREADS) void remap_move_kernel(const index_t* indices, const int32_t* mapping,
-                                                                   int64_t mapping_numel, const float* weights, int64_t first,
+__global__ __launch_bounds__(PSCAN_THREADS) void remap_move_kernel(const int32_t* mapped, const float* weights, int64_t first,
                                                                    int64_t n, const int64_t* carry_in, index_t* out_indices,
-                                                                   float* out_weights, int64_t* before_out, Status* status) {
+                                                                   float* out_weights, int64_t* before_out) {
   __shared__ int64_t lds[PSCAN_THREADS];
   const int64_t base = (int64_t)blockIdx.x * PSCAN_BLOCK + (int64_t)threadIdx.x * PSCAN_ITEMS;
   int32_t row[PSCAN_ITEMS];
   int64_t local = 0;
   for (int i = 0; i < PSCAN_ITEMS; ++i) {
-    row[i] = base + i < n ? mapped_row(indices, mapping, mapping_numel, first + base + i, status) : -1;
+    row[i] = base + i < n ? mapped[base + i] : -1;
     local += row[i] != -1 ? 1 : 0;
   }
   const int64_t incl = block_inclusive_sum(local, lds);
@@ -254,27 +259,28 @@ hipError_t launch_prune_gather(const void* in, int64_t rows, int64_t row_bytes, 
 }
 
 // n = offsets[last] - offsets[0] positions starting at `first` = offsets[0]; `before` holds n + 1 entries,
-// `partial` prune_partials(n + 1).
+// `partial` prune_partials(n + 1), `mapped` n.
 hipError_t launch_compressed_indices_remap(const void* indices, bool idx64, const int32_t* mapping, int64_t mapping_numel,
                                            const void* offsets, int64_t offsets_numel, const float* weights, int64_t first,
                                            int64_t n, void* out_indices, void* out_offsets, float* out_weights,
-                                           int64_t* before, int64_t* partial, Status* status, hipStream_t stream) {
+                                           int64_t* before, int64_t* partial, int32_t* mapped, Status* status,
+                                           hipStream_t stream) {
   const int64_t nblocks = prune_partials(n + 1);
   const unsigned oblocks = (unsigned)((offsets_numel + 255) / 256);
   if (idx64) {
     hipLaunchKernelGGL(remap_count_kernel<int64_t>, dim3((unsigned)nblocks), dim3(PSCAN_THREADS), 0, stream, (const int64_t*)indices,
-                       mapping, mapping_numel, first, n, partial, status);
+                       mapping, mapping_numel, first, n, partial, mapped, status);
     hipLaunchKernelGGL(prune_carry_kernel, dim3(1), dim3(PSCAN_THREADS), 0, stream, partial, nblocks);
-    hipLaunchKernelGGL(remap_move_kernel<int64_t>, dim3((unsigned)nblocks), dim3(PSCAN_THREADS), 0, stream, (const int64_t*)indices,
-                       mapping, mapping_numel, weights, first, n, partial, (int64_t*)out_indices, out_weights, before, status);
+    hipLaunchKernelGGL(remap_move_kernel<int64_t>, dim3((unsigned)nblocks), dim3(PSCAN_THREADS), 0, stream, (const int32_t*)mapped,
+                       weights, first, n, partial, (int64_t*)out_indices, out_weights, before);
     hipLaunchKernelGGL(remap_offsets_kernel<int64_t>, dim3(oblocks), dim3(256), 0, stream, (const int64_t*)offsets, offsets_numel,
                        first, n, before, (int64_t*)out_offsets);
   } else {
     hipLaunchKernelGGL(remap_count_kernel<int32_t>, dim3((unsigned)nblocks), dim3(PSCAN_THREADS), 0, stream, (const int32_t*)indices,
-                       mapping, mapping_numel, first, n, partial, status);
+                       mapping, mapping_numel, first, n, partial, mapped, status);
     hipLaunchKernelGGL(prune_carry_kernel, dim3(1), dim3(PSCAN_THREADS), 0, stream, partial, nblocks);
-    hipLaunchKernelGGL(remap_move_kernel<int32_t>, dim3((unsigned)nblocks), dim3(PSCAN_THREADS), 0, stream, (const int32_t*)indices,
-                       mapping, mapping_numel, weights, first, n, partial, (int32_t*)out_indices, out_weights, before, status);
+    hipLaunchKernelGGL(remap_move_kernel<int32_t>, dim3((unsigned)nblocks), dim3(PSCAN_THREADS), 0, stream, (const int32_t*)mapped,
+                       weights, first, n, partial, (int32_t*)out_indices, out_weights, before);
     hipLaunchKernelGGL(remap_offsets_kernel<int32_t>, dim3(oblocks), dim3(256), 0, stream, (const int32_t*)offsets, offsets_numel,
                        first, n, before, (int32_t*)out_offsets);
   }
