@@ -98,11 +98,19 @@ __global__ __launch_bounds__(SCAN_THREADS) void bounds_carry_kernel(int64_t* par
 // pass 3: the repaired offsets (into `fixed`), the count of bad bags, the
 // conditions a FATAL run reports
 __global__ __launch_bounds__(SCAN_THREADS) void bounds_fix_offsets_kernel(
-    const void* offsets, int is64, int64_t total_B, int64_t N, const int64_t* carry_in, int64_t* fixed,
-    int mode, int64_t* warning, Status* status) {
+    const void* offsets, int is64, int64_t total_B, int64_t N, const int64_t* carry_in, int carry_is_prefix,
+    int64_t* fixed, int mode, int64_t* warning, Status* status) {
   __shared__ int64_t lds[SCAN_THREADS];
   __shared__ int bad_count;
   if (threadIdx.x == 0) bad_count = 0;
+  // what the blocks before this one leave: either pass 2 has made it (carry_is_prefix), or, with at most
+  // SCAN_THREADS blocks, every block takes the maximum of the earlier blocks' maxima itself and pass 2 is not run
+  int64_t carry;
+  if (carry_is_prefix) {
+    carry = carry_in[blockIdx.x];
+  } else {
+    carry = block_max(threadIdx.x < blockIdx.x ? carry_in[threadIdx.x] : 0, lds);
+  }
   const int64_t base = (int64_t)blockIdx.x * SCAN_BLOCK + (int64_t)threadIdx.x * SCAN_ITEMS;
   int64_t v[SCAN_ITEMS];
   int64_t local = 0;
@@ -111,17 +119,20 @@ __global__ __launch_bounds__(SCAN_THREADS) void bounds_fix_offsets_kernel(
     v[i] = k <= total_B ? clamped_offset(offsets, is64, k, total_B, N) : 0;
     local = v[i] > local ? v[i] : local;
   }
-  // inclusive running maximum over the threads' local maxima
-  lds[threadIdx.x] = local;
-  __syncthreads();
-  for (int step = 1; step < SCAN_THREADS; step <<= 1) {
-    const int64_t o = (int)threadIdx.x >= step ? lds[threadIdx.x - step] : 0;
-    __syncthreads();
-    lds[threadIdx.x] = lds[threadIdx.x] > o ? lds[threadIdx.x] : o;
-    __syncthreads();
+  // running maximum of the threads' local maxima before this thread: inside each wave through lane
+  // shuffles, then over the 16 wave maxima (two workgroup barriers instead of twenty)
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int64_t incl = local;
+  for (int step = 1; step < 64; step <<= 1) {
+    const int64_t o = __shfl_up(incl, step, 64);
+    if (lane >= step) incl = incl > o ? incl : o;
   }
-  int64_t run = threadIdx.x > 0 ? lds[threadIdx.x - 1] : 0;
-  const int64_t carry = carry_in[blockIdx.x];
+  int64_t run = __shfl_up(incl, 1, 64); // exclusive inside the wave (values are >= 0)
+  if (lane == 0) run = 0;
+  __syncthreads(); // lds is free again (the carry above may have used it)
+  if (lane == 63) lds[wave] = incl;
+  __syncthreads();
+  for (int w = 0; w < wave; ++w) run = run > lds[w] ? run : lds[w];
   run = run > carry ? run : carry;
   int bad = 0, err = 0;
   for (int i = 0; i < SCAN_ITEMS; ++i) {
@@ -270,9 +281,10 @@ hipError_t launch_bounds_check(const int64_t* rows_per_table, int32_t T, void* i
   const int64_t nblocks = (n + SCAN_BLOCK - 1) / SCAN_BLOCK;
   hipLaunchKernelGGL(bounds_partial_max_kernel, dim3((unsigned)nblocks), dim3(SCAN_THREADS), 0, stream, offsets,
                      is64 ? 1 : 0, total_B, num_indices, partial, warning, mode);
-  hipLaunchKernelGGL(bounds_carry_kernel, dim3(1), dim3(SCAN_THREADS), 0, stream, partial, nblocks);
+  const int own_carry = nblocks <= SCAN_THREADS; // up to 4 M offsets: one launch less
+  if (!own_carry) hipLaunchKernelGGL(bounds_carry_kernel, dim3(1), dim3(SCAN_THREADS), 0, stream, partial, nblocks);
   hipLaunchKernelGGL(bounds_fix_offsets_kernel, dim3((unsigned)nblocks), dim3(SCAN_THREADS), 0, stream, offsets,
-                     is64 ? 1 : 0, total_B, num_indices, partial, fixed, mode, warning, status);
+                     is64 ? 1 : 0, total_B, num_indices, partial, own_carry ? 0 : 1, fixed, mode, warning, status);
   if (total_B > 0) {
     const int64_t per_block = 256 / BAG_LANES;
     int64_t blocks = (total_B + per_block - 1) / per_block;

@@ -142,6 +142,20 @@ def test_bounds_check_large_offsets_scan(env):
     assert got[1][5000] == idx.size and (np.diff(got[1]) >= 0).all()
 
 
+def test_bounds_check_more_scan_blocks_than_a_workgroup_has_threads(env):
+    """4.5 M bags: the running maximum then goes through the separate carry pass (with fewer blocks every
+    block takes the maximum of the earlier blocks itself)."""
+    torch, ops = env
+    rng = np.random.default_rng(105)
+    T, B = 3, 1_500_000
+    rows, idx, off = make_problem(rng, T, B, 2, np.int32)
+    off[2_000_000] = off[-1] + 1  # everything after it is raised to num_indices
+    off[7] = -1
+    idx[::1000] = 10 ** 6
+    got, want = run_bounds(torch, ops, rows, idx, off, WARNING)
+    assert (got[1] == want[1]).all() and (got[0] == want[0]).all() and got[2] == want[2]
+
+
 @pytest.mark.parametrize("idt", [np.int32, np.int64])
 @pytest.mark.parametrize("hdt", [np.int32, np.int64])
 def test_pruned_hashmap_lookup_matches_oracle(env, idt, hdt):
