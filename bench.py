@@ -49,7 +49,7 @@ def parse():
     ap.add_argument("--op", default="lookup",
                     choices=["lookup", "quantize", "dequantize", "bounds_check", "pruned_array_lookup",
                              "pruned_hashmap_lookup", "float_to_hfp8", "hfp8_to_float", "rowwise_prune",
-                             "compressed_indices_remap", "sequence", "no_bag"],
+                             "compressed_indices_remap", "sequence", "no_bag", "inplace_update"],
                     help="lookup = the table-batched forward (the metric); the others time one operator beside "
                          "the path at the shape config 4 / config 3 gives it and print the same kind of line")
     return ap.parse_args()
@@ -252,7 +252,8 @@ def side_op(a):
     columns (a table of config 2's shape), 4-bit rows in the table-batched layout;
     so do the hfp8 converters and the single-table no_bag kernel (8-bit rows);
     rowwise_prune sees 2 M x 64 fp32 with half of the rows kept; sequence
-    (PoolingMode.NONE) sees 32 int4 tables x 1 M rows x 128 with config 4's bags."""
+    (PoolingMode.NONE) sees 32 int4 tables x 1 M rows x 128 with config 4's bags;
+    inplace_update overwrites 1 M random rows of those tables."""
     import numpy as np
     import torch
 
@@ -322,6 +323,24 @@ def side_op(a):
         launch = lambda: kern(n, n, rows, table, idx, None, None, out, status=st)
         alg_bytes, units = n * (cols + 8 + cols * 4 + 8), n
         kernel, workload = "row_lookup_kernel", f"8-bit rows [{rows}, {cols}] (fp32 scale/bias last), {n} int64 indices -> fp32 rows"
+    elif a.op == "inplace_update":
+        T, D = 32, 128
+        E = max(1000, int(1_000_000 * a.scale))
+        n = max(1, int(1_000_000 * a.scale))
+        rb = ops.padded_row_size_in_bytes(D, ops.INT4, 16)
+        weights = torch.randint(0, 256, (T * E * rb,), dtype=torch.uint8, device="cuda")
+        tables = rng.integers(0, T, size=n).astype(np.int32)
+        # distinct rows per table: two updates of one row in a call race
+        rows = (rng.permutation(T * E)[:n] // T).astype(np.int64)
+        upd = torch.randint(0, 256, (n * rb,), dtype=torch.uint8, device="cuda")
+        args = (weights, torch.zeros(0, dtype=torch.uint8, device="cuda"), torch.zeros(T, dtype=torch.int32, device="cuda"),
+                (torch.arange(T, dtype=torch.int64) * (E * rb)).cuda(), torch.full((T,), ops.INT4, dtype=torch.uint8, device="cuda"),
+                torch.arange(T + 1, dtype=torch.int32, device="cuda") * D, upd, cu(tables), cu(rows),
+                cu(np.arange(n + 1, dtype=np.int64) * rb), 16)
+        st = ops.Status()
+        launch = lambda: ops.emb_inplace_update(*args, status=st)
+        alg_bytes, units = n * (2 * rb + 4 + 8 + 8), n
+        kernel, workload = "inplace_update_kernel", f"{n} rows of {rb} bytes into {T} int4 tables x {E} rows x {D} (random rows)"
     elif a.op == "sequence":
         T, B, D = 32, max(1, int(4096 * a.scale)), 128
         E = max(1000, int(1_000_000 * a.scale))

@@ -11,7 +11,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "lib", "libfbgemm_amd.so")
 
-SOURCES = ["lookup_kernels.hip", "index_ops_kernels.hip", "quantize_kernels.hip", "sequence_kernels.hip", "prune_kernels.hip", "c_api.cpp"]
+SOURCES = ["lookup_kernels.hip", "index_ops_kernels.hip", "quantize_kernels.hip", "sequence_kernels.hip", "prune_kernels.hip", "update_kernels.hip", "c_api.cpp"]
 HEADERS = ["lookup_common.h", os.path.join("..", "..", "include", "fbgemm_amd.h")]
 
 # -ffp-contract=off: the kernels spell out every fma; nothing else may be fused,

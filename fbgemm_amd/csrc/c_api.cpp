@@ -29,6 +29,12 @@ hipError_t launch_row_lookup(const TableDesc& d, const uint8_t* table, const voi
 hipError_t launch_float_to_hfp8(const float* input, int64_t n, int32_t ebits, int32_t bias, float max_pos, uint8_t* output,
                                 hipStream_t stream);
 hipError_t launch_hfp8_to_float(const uint8_t* input, int64_t n, int32_t ebits, int32_t bias, float* output, hipStream_t stream);
+hipError_t launch_inplace_update(const TableDesc* tables, int32_t T, uint8_t* w0, uint8_t* w1, const uint8_t* update,
+                                 int64_t update_bytes, const int32_t* table_idx, const void* row_idx, bool idx64,
+                                 const int64_t* update_offsets, int64_t n, int64_t max_row_bytes, Status* status,
+                                 hipStream_t stream);
+hipError_t launch_remap_row_idx(const void* rows, bool idx64, const int32_t* table_idx, const void* remap, bool remap64,
+                                const int64_t* remap_offsets, int32_t T, int64_t n, void* dense, hipStream_t stream);
 int64_t prune_partials(int64_t rows);
 hipError_t launch_prune_map(const float* indicator, int64_t rows, double threshold, int use_abs, int64_t min_rows,
                             bool idx64, void* remap, int64_t* num_kept, int64_t* partial, hipStream_t stream);
@@ -1254,6 +1260,44 @@ int fbgemm_amd_pruned_array_lookup(
   if (!d_indices || !d_offsets || !d_remap_offsets || !d_dense) return fail(FBGEMM_AMD_E_ARG, "null data pointer");
   HIP_TRY(launch_pruned_array_lookup(d_indices, d_offsets, index_bits == 64, d_remap, remap_bits == 64,
                                      d_remap_offsets, (int32_t)B, T, d_dense, (hipStream_t)stream));
+  return 0;
+}
+
+int fbgemm_amd_tbe_inplace_update(
+    fbgemm_amd_tbe_plan* plan, void* d_dev_weights, void* d_uvm_weights, const void* d_update_weights,
+    int64_t update_weights_bytes, const int32_t* d_update_table_idx, const void* d_update_row_idx,
+    int32_t row_index_bits, const int64_t* d_update_offsets, int64_t n, void* d_status, void* stream) {
+  if (!plan) return fail(FBGEMM_AMD_E_ARG, "plan is null");
+  if (row_index_bits != 32 && row_index_bits != 64) return fail(FBGEMM_AMD_E_ARG, "row_index_bits must be 32 or 64");
+  if (n < 0 || update_weights_bytes < 0) return fail(FBGEMM_AMD_E_ARG, "negative size");
+  if (n == 0) return 0;
+  if (!d_update_weights || !d_update_table_idx || !d_update_row_idx || !d_update_offsets)
+    return fail(FBGEMM_AMD_E_ARG, "null data pointer");
+  int64_t max_row_bytes = 0;
+  for (int t = 0; t < plan->T; ++t) {
+    const TableDesc& d = plan->tables[t];
+    if (d.num_rows > 0 && !(d.placement ? d_uvm_weights : d_dev_weights))
+      return fail(FBGEMM_AMD_E_ARG, "table %d lives in a weights buffer that was not passed", t);
+    max_row_bytes = std::max(max_row_bytes, d.row_stride);
+  }
+  HIP_TRY(launch_inplace_update(plan->d_tables, plan->T, (uint8_t*)d_dev_weights, (uint8_t*)d_uvm_weights,
+                                (const uint8_t*)d_update_weights, update_weights_bytes, d_update_table_idx,
+                                d_update_row_idx, row_index_bits == 64, d_update_offsets, n, max_row_bytes,
+                                (Status*)d_status, (hipStream_t)stream));
+  return 0;
+}
+
+int fbgemm_amd_pruned_array_lookup_from_row_idx(
+    const void* d_update_row_idx, int32_t index_bits, const int32_t* d_update_table_idx, int64_t n, const void* d_remap,
+    int32_t remap_bits, const int64_t* d_remap_offsets, int32_t T, void* d_dense, void* stream) {
+  if (T <= 0 || n < 0) return fail(FBGEMM_AMD_E_ARG, "bad sizes");
+  if ((index_bits != 32 && index_bits != 64) || (remap_bits != 32 && remap_bits != 64))
+    return fail(FBGEMM_AMD_E_ARG, "index_bits/remap_bits must be 32 or 64");
+  if (n == 0) return 0;
+  if (!d_update_row_idx || !d_update_table_idx || !d_remap_offsets || !d_dense)
+    return fail(FBGEMM_AMD_E_ARG, "null data pointer");
+  HIP_TRY(launch_remap_row_idx(d_update_row_idx, index_bits == 64, d_update_table_idx, d_remap, remap_bits == 64,
+                               d_remap_offsets, T, n, d_dense, (hipStream_t)stream));
   return 0;
 }
 

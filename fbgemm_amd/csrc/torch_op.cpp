@@ -208,6 +208,57 @@ Tensor pruned_array_lookup_hip(Tensor indices, Tensor offsets, Tensor index_rema
   return dense;
 }
 
+// pruned_array_lookup_from_row_idx (fbgemm_gpu/src/embedding_inplace_ops/embedding_inplace_update_cpu.cpp:199-251)
+Tensor pruned_array_lookup_from_row_idx_hip(const Tensor& update_row_indices, const Tensor& update_table_indices,
+                                            const Tensor& index_remappings, const Tensor& index_remappings_offsets) {
+  TORCH_CHECK(update_row_indices.is_cuda() && update_table_indices.is_cuda() && index_remappings.is_cuda() &&
+              index_remappings_offsets.is_cuda());
+  TORCH_CHECK(update_table_indices.scalar_type() == at::kInt, "update_table_indices must be int32");
+  TORCH_CHECK(update_table_indices.numel() == update_row_indices.numel());
+  const Tensor rows = update_row_indices.contiguous();
+  const Tensor tables = update_table_indices.contiguous();
+  const Tensor remap = index_remappings.contiguous();
+  const Tensor ro = index_remappings_offsets.to(at::kLong).contiguous();
+  Tensor dense = at::empty_like(rows);
+  const int rc = fbgemm_amd_pruned_array_lookup_from_row_idx(
+      rows.data_ptr(), rows.scalar_type() == at::kLong ? 64 : 32, tables.data_ptr<int32_t>(), rows.numel(),
+      remap.data_ptr(), remap.scalar_type() == at::kLong ? 64 : 32, ro.data_ptr<int64_t>(), (int32_t)(ro.numel() - 1),
+      dense.data_ptr(), current_stream(rows));
+  TORCH_CHECK(rc == 0, "fbgemm_amd: ", fbgemm_amd_last_error());
+  return dense;
+}
+
+// emb_inplace_update (embedding_inplace_update_cpu.cpp:72-120): rows of the weights buffers are overwritten in
+// place. Updates that name no row are skipped and recorded where lookup_status reads them.
+void emb_inplace_update_hip(Tensor dev_weights, Tensor uvm_weights, Tensor weights_placements, Tensor weights_offsets,
+                            Tensor weights_tys, Tensor D_offsets, Tensor update_weights, Tensor update_table_idx,
+                            Tensor update_row_idx, Tensor update_offsets, const int64_t row_alignment,
+                            std::optional<Tensor> /*lxu_cache_weights*/, std::optional<Tensor> lxu_cache_locations) {
+  TORCH_CHECK(dev_weights.is_cuda() && update_weights.is_cuda() && update_table_idx.is_cuda() && update_row_idx.is_cuda() &&
+                  update_offsets.is_cuda(), "fbgemm_amd: tensors must be on the GPU");
+  TORCH_CHECK(!lxu_cache_locations || lxu_cache_locations->numel() == 0,
+              "fbgemm_amd: the LXU cache is not on this path (tables are resident in HBM)");
+  TORCH_CHECK(update_weights.scalar_type() == at::kByte && update_table_idx.scalar_type() == at::kInt &&
+              update_offsets.scalar_type() == at::kLong, "update_weights is uint8, update_table_indices int32, update_offsets int64");
+  const int64_t n = update_row_idx.numel();
+  TORCH_CHECK(update_table_idx.numel() == n && update_offsets.numel() >= n);
+  if (n == 0) return;
+  update_weights = update_weights.contiguous();
+  update_table_idx = update_table_idx.contiguous();
+  update_row_idx = update_row_idx.contiguous();
+  update_offsets = update_offsets.contiguous();
+  std::lock_guard<std::mutex> lk(g_mu);
+  fbgemm_amd_tbe_plan* plan = plan_for(dev_weights, uvm_weights, weights_placements, weights_offsets, weights_tys,
+                                       D_offsets, row_alignment);
+  Tensor& st = status_block(dev_weights);
+  const int rc = fbgemm_amd_tbe_inplace_update(
+      plan, dev_weights.numel() ? dev_weights.data_ptr() : nullptr, uvm_weights.numel() ? uvm_weights.data_ptr() : nullptr,
+      update_weights.data_ptr(), update_weights.numel(), update_table_idx.data_ptr<int32_t>(), update_row_idx.data_ptr(),
+      update_row_idx.scalar_type() == at::kLong ? 64 : 32, update_offsets.data_ptr<int64_t>(), n, st.data_ptr(),
+      current_stream(dev_weights));
+  TORCH_CHECK(rc == 0, "fbgemm_amd: ", fbgemm_amd_last_error());
+}
+
 // bounds_check_indices (fbgemm_gpu/codegen/utils/embedding_bounds_check_host_cpu.cpp:76-219):
 // in place on indices / offsets / warning. WARNING and IGNORE repair on the
 // device without a synchronization. FATAL raises where the reference's CPU
@@ -451,6 +502,15 @@ TORCH_LIBRARY_FRAGMENT(fbgemm, m) {
   m.impl("pruned_array_lookup", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(pruned_array_lookup_hip)));
   m.impl("int_nbit_split_embedding_codegen_lookup_function", torch::dispatch(c10::DispatchKey::Meta, TORCH_FN(lookup_meta)));
   m.impl("pruned_array_lookup", torch::dispatch(c10::DispatchKey::Meta, TORCH_FN(same_shape_as_indices_meta)));
+#ifndef FBGEMM_AMD_IMPL_ONLY
+  // fbgemm_gpu/src/embedding_inplace_ops/embedding_inplace_update_cpu.cpp:257-260
+  m.def(
+      "emb_inplace_update(Tensor(a!) dev_weights, Tensor(b!) uvm_weights, Tensor weights_placements, Tensor weights_offsets, Tensor weights_tys, Tensor D_offsets, Tensor update_weights, Tensor update_table_indices, Tensor update_row_indices, Tensor update_offsets, int row_alignment=1, Tensor(c!)? lxu_cache_weights=None, Tensor? lxu_cache_locations=None) -> ()");
+  m.def(
+      "pruned_array_lookup_from_row_idx(Tensor update_row_indices, Tensor update_table_indices, Tensor index_remappings, Tensor index_remappings_offsets) -> Tensor");
+#endif
+  m.impl("emb_inplace_update", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(emb_inplace_update_hip)));
+  m.impl("pruned_array_lookup_from_row_idx", torch::dispatch(c10::DispatchKey::CUDA, TORCH_FN(pruned_array_lookup_from_row_idx_hip)));
 #ifndef FBGEMM_AMD_IMPL_ONLY
   // embedding_forward_quantized_host_cpu.cpp:338-341
   m.def(

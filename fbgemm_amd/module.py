@@ -275,6 +275,44 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(torch.nn.Module):
         self.index_remapping_hash_table = hash_table.to(dev)
         self.index_remapping_hash_table_offsets = hto.to(dev)
 
+    # ---- in-place updates ------------------------------------------------------
+    def _embedding_inplace_update_per_table(self, update_table_idx, update_row_indices, update_weights):
+        # split_table_batched_embeddings_ops_inference.py:2018-2041: whole padded rows, scattered by row id
+        if len(update_row_indices) == 0:
+            return
+        rows = torch.tensor(update_row_indices, device=self.current_device, dtype=torch.int64)
+        table = self.split_embedding_weights(split_scale_shifts=False)[update_table_idx][0]
+        table.scatter_(dim=0, index=rows.view(-1, 1).expand_as(update_weights), src=update_weights)
+
+    def embedding_inplace_update(self, update_table_indices, update_row_indices, update_weights):
+        """Per table: a list of rows and a [rows, padded row bytes] uint8 tensor
+        (split_table_batched_embeddings_ops_inference.py:2044-2055)."""
+        for t, rows, w in zip(update_table_indices, update_row_indices, update_weights):
+            self._embedding_inplace_update_per_table(t, rows, w)
+
+    def embedding_inplace_update_internal(self, update_table_indices, update_row_indices, update_weights):
+        """Flat form: update i overwrites row update_row_indices[i] (a logical row when the module prunes
+        through arrays) of table update_table_indices[i] with the next padded row of ``update_weights``
+        (split_table_batched_embeddings_ops_inference.py:2057-2144). One kernel for all tables."""
+        assert len(update_table_indices) == len(update_row_indices)
+        dev = self.current_device
+        sizes = [rounded_row_size_in_bytes(self.embedding_specs[t][2], self.embedding_specs[t][3], self.row_alignment,
+                                           self.scale_bias_size_in_bytes) for t in update_table_indices]
+        update_offsets = torch.tensor([0] + list(accumulate(sizes)), device=dev, dtype=torch.int64)
+        tables = torch.tensor(update_table_indices, device=dev, dtype=torch.int32)
+        rows = torch.tensor(update_row_indices, device=dev, dtype=torch.int64)
+        # only array based pruning, as in the reference
+        assert self.index_remapping_hash_table.numel() == 0
+        if self.index_remappings_array.numel() > 0:
+            rows = ops.pruned_array_lookup_from_row_idx(rows, tables, self.index_remappings_array,
+                                                        self.index_remappings_array_offsets)
+        # the operator addresses weights_offsets, which has one entry per feature: the first feature of each table
+        first_feature = [self.feature_table_map.index(t) for t in range(len(self.embedding_specs))]
+        features = torch.tensor([first_feature[t] for t in update_table_indices], device=dev, dtype=torch.int32)
+        ops.emb_inplace_update(self.weights_dev, self.weights_uvm, self.weights_placements, self.weights_offsets,
+                               self.weights_tys, self.D_offsets, update_weights.to(dev), features, rows, update_offsets,
+                               row_alignment=self.row_alignment)
+
     # ---- forward ---------------------------------------------------------------
     def forward(self, indices, offsets, per_sample_weights=None):
         assert self.weight_initialized, "weight needs to be initialized before forward function"

@@ -371,6 +371,60 @@ def pruned_array_lookup(indices, offsets, index_remappings, index_remappings_off
     return dense
 
 
+def pruned_array_lookup_from_row_idx(update_row_indices, update_table_indices, index_remappings,
+                                     index_remappings_offsets):
+    """pruned_array_lookup_from_row_idx (embedding_inplace_update_cpu.cpp:199-251, schema :259-260): the
+    logical rows of an update as physical rows; -1 for a pruned row."""
+    _require_cuda(update_row_indices, update_table_indices, index_remappings, index_remappings_offsets)
+    if update_table_indices.dtype != torch.int32:
+        raise TypeError("update_table_indices must be int32")
+    if update_table_indices.numel() != update_row_indices.numel():
+        raise ValueError("update_table_indices and update_row_indices differ in length")
+    T = index_remappings_offsets.numel() - 1
+    dense = torch.empty_like(update_row_indices)
+    ro = index_remappings_offsets.to(torch.int64).contiguous()
+    check(_lib.lib().fbgemm_amd_pruned_array_lookup_from_row_idx(
+        _ptr(update_row_indices.contiguous()), _bits(update_row_indices), _ptr(update_table_indices.contiguous()),
+        update_row_indices.numel(), _ptr(index_remappings), _bits(index_remappings), _ptr(ro), T, _ptr(dense),
+        _stream()))
+    return dense
+
+
+def emb_inplace_update(dev_weights, uvm_weights, weights_placements, weights_offsets, weights_tys, D_offsets,
+                       update_weights, update_table_indices, update_row_indices, update_offsets, row_alignment=1,
+                       lxu_cache_weights=None, lxu_cache_locations=None, status=None, plan=None):
+    """emb_inplace_update (embedding_inplace_update_cpu.cpp:257-258): overwrites rows of the weights buffers
+    in place. An update outside its table (or past ``update_weights``) raises unless ``status`` is given; a row id
+    of -1 (a pruned row) is skipped."""
+    _require_cuda(dev_weights, update_weights, update_table_indices, update_row_indices, update_offsets)
+    if lxu_cache_locations is not None and lxu_cache_locations.numel() > 0:
+        raise NotImplementedError("the LXU cache is not on this path: tables are resident in HBM")
+    if update_weights.dtype != torch.uint8 or update_table_indices.dtype != torch.int32 or update_offsets.dtype != torch.int64:
+        raise TypeError("update_weights is uint8, update_table_indices int32, update_offsets int64")
+    n = update_row_indices.numel()
+    if update_table_indices.numel() != n or update_offsets.numel() < n:
+        raise ValueError("update_table_indices / update_offsets do not cover update_row_indices")
+    if n == 0:
+        return
+    if plan is None:
+        plan = _plan_for(dev_weights, uvm_weights, weights_placements, weights_offsets, weights_tys, D_offsets,
+                         row_alignment)
+    own = status is None
+    st = Status(dev_weights.device) if own else status
+    update_weights = update_weights.contiguous()
+    check(_lib.lib().fbgemm_amd_tbe_inplace_update(
+        plan.handle, _ptr(dev_weights), _ptr(uvm_weights), _ptr(update_weights), update_weights.numel(),
+        _ptr(update_table_indices.contiguous()), _ptr(update_row_indices.contiguous()), _bits(update_row_indices),
+        _ptr(update_offsets.contiguous()), n, _ptr(st.buf), _stream()))
+    if own:
+        bits, pos = st.read()
+        if bits & ERR_INDEX_OUT_OF_RANGE:
+            raise RuntimeError(f"update {pos} names table {int(update_table_indices[pos])}, row "
+                               f"{int(update_row_indices[pos])}, which does not exist")
+        if bits:
+            raise RuntimeError("an update reads past the end of update_weights")
+
+
 def padded_row_size_in_bytes(dim, weight_ty, row_alignment, scale_bias_bytes=4):
     """nbit::padded_row_size_in_bytes (embedding_common.h:217-225)."""
     return _lib.lib().fbgemm_amd_padded_row_size_in_bytes(dim, weight_ty, row_alignment, scale_bias_bytes)

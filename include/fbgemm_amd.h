@@ -246,6 +246,38 @@ int fbgemm_amd_pruned_array_lookup(
     const int64_t* d_index_remappings_offsets, int32_t T, void* d_dense,
     void* stream);
 
+/* ---- in-place row update of a table-batched weights buffer ----------------- *
+ * Replaces emb_inplace_update
+ * (fbgemm_gpu/src/embedding_inplace_ops/embedding_inplace_update.cu:28-101,207-282,
+ * CPU form embedding_inplace_update_cpu.cpp:25-70; schema :257-258; caller
+ * embedding_inplace_update_internal,
+ * fbgemm_gpu/fbgemm_gpu/split_table_batched_embeddings_ops_inference.py:2057-2144):
+ * for update i the padded row d_update_row_idx[i] of table d_update_table_idx[i]
+ * (fbgemm_amd_tbe_plan_row_bytes bytes) is overwritten with the bytes at
+ * d_update_weights + d_update_offsets[i]. Tables, row sizes, placements and row
+ * counts come from the plan. Beyond the reference, which checks nothing: a row id
+ * of -1 (a pruned row, see below) is skipped; a table outside [0, T), another row
+ * outside its table, or an update that would read past update_weights_bytes is
+ * skipped and recorded in d_status (out-of-range / overrun bits; may be NULL:
+ * then it is only skipped). Two updates of one row in a call race, as in the
+ * reference's kernel. Asynchronous; forwards that should see the rows must be
+ * ordered after it on `stream`. */
+int fbgemm_amd_tbe_inplace_update(
+    fbgemm_amd_tbe_plan* plan, void* d_dev_weights, void* d_uvm_weights,
+    const void* d_update_weights, int64_t update_weights_bytes,
+    const int32_t* d_update_table_idx, const void* d_update_row_idx, int32_t row_index_bits,
+    const int64_t* d_update_offsets, int64_t n, void* d_status, void* stream);
+
+/* Replaces pruned_array_lookup_from_row_idx (embedding_inplace_update.cu:359-465,
+ * embedding_inplace_update_cpu.cpp:199-251): the logical rows of an update become
+ * physical rows, d_dense[i] = index_remappings[offsets[t_i] + row_i] where table
+ * t_i owns a mapping and row_i otherwise. A row outside its mapping or a table
+ * outside [0, T) yields -1 (the reference reads out of bounds). */
+int fbgemm_amd_pruned_array_lookup_from_row_idx(
+    const void* d_update_row_idx, int32_t index_bits, const int32_t* d_update_table_idx, int64_t n,
+    const void* d_index_remappings, int32_t remap_bits, const int64_t* d_index_remappings_offsets,
+    int32_t T, void* d_dense, void* stream);
+
 /* ---- index operators that run before the lookup ---------------------------- *
  *
  * bounds_check_indices (fbgemm_gpu/codegen/utils/embedding_bounds_check_host_cpu.cpp:76-219,

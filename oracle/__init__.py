@@ -311,6 +311,39 @@ def pruned_array_lookup(indices, offsets, remap, remap_offsets):
     return dense
 
 
+def pruned_array_lookup_from_row_idx(update_row_indices, update_table_indices, remap, remap_offsets):
+    rows = np.ascontiguousarray(update_row_indices)
+    tables = np.ascontiguousarray(update_table_indices, dtype=np.int32)
+    remap = np.ascontiguousarray(remap)
+    remap_offsets = np.ascontiguousarray(remap_offsets, dtype=np.int64)
+    dense = np.empty_like(rows)
+    fn = _lib("oracle").oracle_pruned_array_lookup_from_row_idx
+    fn.restype = None
+    fn.argtypes = [_c.c_int64, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p]
+    fn(len(rows), _ptr(rows), _is64(rows), _ptr(tables), _ptr(remap), _is64(remap), _ptr(remap_offsets), _ptr(dense))
+    return dense
+
+
+def emb_inplace_update(dev_weights, uvm_weights, weights_placements, weights_offsets, weights_tys, D_offsets,
+                       update_weights, update_table_indices, update_row_indices, update_offsets, row_alignment):
+    """In place on ``dev_weights`` / ``uvm_weights`` (contiguous uint8 arrays), updates applied in order."""
+    assert dev_weights.flags.c_contiguous and uvm_weights.flags.c_contiguous
+    assert dev_weights.dtype == np.uint8 and uvm_weights.dtype == np.uint8
+    wp = np.ascontiguousarray(weights_placements, dtype=np.int32)
+    wo = np.ascontiguousarray(weights_offsets, dtype=np.int64)
+    wt = np.ascontiguousarray(weights_tys, dtype=np.uint8)
+    do = np.ascontiguousarray(D_offsets, dtype=np.int32)
+    uw = np.ascontiguousarray(update_weights, dtype=np.uint8)
+    ut = np.ascontiguousarray(update_table_indices, dtype=np.int32)
+    ur = np.ascontiguousarray(update_row_indices)
+    uo = np.ascontiguousarray(update_offsets, dtype=np.int64)
+    fn = _lib("oracle").oracle_emb_inplace_update
+    fn.restype = None
+    fn.argtypes = [_c.c_void_p] * 9 + [_c.c_int, _c.c_void_p, _c.c_int64, _c.c_int64]
+    fn(_ptr(dev_weights), _ptr(uvm_weights), _ptr(wp), _ptr(wo), _ptr(wt), _ptr(do), _ptr(uw), _ptr(ut), _ptr(ur),
+       _is64(ur), _ptr(uo), len(ur), int(row_alignment))
+
+
 BOUNDS_FATAL, BOUNDS_WARNING, BOUNDS_IGNORE = 0, 1, 2
 
 

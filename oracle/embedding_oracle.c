@@ -25,6 +25,8 @@
  *   fbgemm_gpu/include/fbgemm_gpu/embedding_common.h:20-48,189-225  enums, row sizes
  *   fbgemm_gpu/codegen/inference/embedding_forward_quantized_cpu_template.cpp:208-520,605-659
  *                                        table-batched forward loop, pruned_array_lookup
+ *   fbgemm_gpu/src/embedding_inplace_ops/embedding_inplace_update_cpu.cpp:25-70,199-251
+ *                                        emb_inplace_update, pruned_array_lookup_from_row_idx
  */
 #include <math.h>
 #include <stdint.h>
@@ -295,6 +297,42 @@ void oracle_pruned_array_lookup(
       if (re - rs > 0) v = read_index(remap, remap64, rs + v);
       if (idx64) ((int64_t*)dense)[i] = v; else ((int32_t*)dense)[i] = (int32_t)v;
     }
+  }
+}
+
+/* ---- in-place row update (fbgemm_gpu/src/embedding_inplace_ops/
+ *      embedding_inplace_update_cpu.cpp:25-70) --------------------------------
+ * Update n overwrites the padded row update_row_idx[n] of table
+ * update_table_idx[n] with the bytes at update_weights + update_offsets[n];
+ * updates are applied in order (the last one of a row wins). The buffer is
+ * chosen by the table's placement: 0 = the first weights buffer. */
+void oracle_emb_inplace_update(
+    uint8_t* dev_weights, uint8_t* uvm_weights, const int32_t* weights_placements,
+    const int64_t* weights_offsets, const uint8_t* weights_tys, const int32_t* D_offsets,
+    const uint8_t* update_weights, const int32_t* update_table_idx, const void* update_row_idx,
+    int idx64, const int64_t* update_offsets, int64_t n_updates, int64_t row_alignment) {
+  for (int64_t n = 0; n < n_updates; ++n) {
+    int32_t t = update_table_idx[n];
+    int64_t row = read_index(update_row_idx, idx64, n);
+    int32_t D = D_offsets[t + 1] - D_offsets[t];
+    int32_t D_bytes = oracle_padded_row_bytes(D, weights_tys[t], (int32_t)row_alignment, 4);
+    uint8_t* base = weights_placements[t] == 0 ? dev_weights : uvm_weights;
+    memcpy(base + weights_offsets[t] + (int64_t)D_bytes * row, update_weights + update_offsets[n], (size_t)D_bytes);
+  }
+}
+
+/* pruned_array_lookup_from_row_idx (embedding_inplace_update_cpu.cpp:199-251):
+ * the rows of an update through the pruning arrays; tables without a mapping
+ * keep their rows. */
+void oracle_pruned_array_lookup_from_row_idx(
+    int64_t n, const void* update_row_idx, int idx64, const int32_t* update_table_idx,
+    const void* remap, int remap64, const int64_t* remap_offsets, void* dense) {
+  for (int64_t i = 0; i < n; ++i) {
+    int32_t t = update_table_idx[i];
+    int64_t v = read_index(update_row_idx, idx64, i);
+    int64_t rs = remap_offsets[t], re = remap_offsets[t + 1];
+    if (re - rs > 0) v = read_index(remap, remap64, rs + v);
+    if (idx64) ((int64_t*)dense)[i] = v; else ((int32_t*)dense)[i] = (int32_t)v;
   }
 }
 
