@@ -62,6 +62,28 @@ struct TableDesc {
   int32_t lanes_recip;    // ceil(65536 / lanes): j / lanes == (j * lanes_recip) >> 16 for 0 <= j <= 64
 };
 
+#if defined(__HIPCC__)
+// Streaming stores for output a kernel never reads back: marked non-temporal so
+// that the lines do not displace table rows and indices in the caches. Same
+// bytes as a plain store of the same width; `p` must be aligned to the width.
+typedef uint32_t stream_u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t stream_u32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void stream_store16(void* p, uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+  const stream_u32x4 q = {a, b, c, d};
+  __builtin_nontemporal_store(q, reinterpret_cast<stream_u32x4*>(p));
+}
+__device__ __forceinline__ void stream_store16(void* p, float a, float b, float c, float d) {
+  stream_store16(p, __float_as_uint(a), __float_as_uint(b), __float_as_uint(c), __float_as_uint(d));
+}
+__device__ __forceinline__ void stream_store8(void* p, uint32_t a, uint32_t b) {
+  const stream_u32x2 q = {a, b};
+  __builtin_nontemporal_store(q, reinterpret_cast<stream_u32x2*>(p));
+}
+__device__ __forceinline__ void stream_store4(void* p, uint32_t a) {
+  __builtin_nontemporal_store(a, reinterpret_cast<uint32_t*>(p));
+}
+#endif
+
 // Bags a wave pools side by side when `lanes` lanes share a bag. The memory
 // pipeline merges the addresses of a 16-byte-per-lane load 16 lanes at a time,
 // so a bag's lanes should not straddle a multiple of 16: with `packed` = 0 each

@@ -140,7 +140,10 @@ __global__ __launch_bounds__(256) void prune_gather_kernel(const uint8_t* in, in
     uint8_t* dst = out + to * row_bytes;
     if (vec) {
       for (int64_t b = (int64_t)sub * 16; b < row_bytes; b += (int64_t)lpr * 16)
-        *reinterpret_cast<uint4*>(dst + b) = *reinterpret_cast<const uint4*>(src + b);
+      {
+        const uint4 q = *reinterpret_cast<const uint4*>(src + b);
+        stream_store16(dst + b, q.x, q.y, q.z, q.w);
+      }
     } else {
       for (int64_t b = sub; b < row_bytes; b += lpr) dst[b] = src[b];
     }

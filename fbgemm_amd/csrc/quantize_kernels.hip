@@ -331,7 +331,7 @@ __global__ __launch_bounds__(256) void dequantize_rowwise_kernel(
     if (output_ty == ST_FP32) {
       float* op = reinterpret_cast<float*>(output) + o;
       if (n == DRUN && (reinterpret_cast<uintptr_t>(op) & 15) == 0) {
-        *reinterpret_cast<float4*>(op) = make_float4(v[0], v[1], v[2], v[3]);
+        stream_store16(op, v[0], v[1], v[2], v[3]);
       } else {
         for (int k = 0; k < DRUN; ++k) if (k < n) op[k] = v[k];
       }
@@ -340,7 +340,7 @@ __global__ __launch_bounds__(256) void dequantize_rowwise_kernel(
       for (int k = 0; k < DRUN; ++k) h[k] = output_ty == ST_FP16 ? float_to_half_bits(v[k]) : float_to_bf16_bits(v[k]);
       uint16_t* op = reinterpret_cast<uint16_t*>(output) + o;
       if (n == DRUN && (reinterpret_cast<uintptr_t>(op) & 7) == 0) {
-        *reinterpret_cast<uint2*>(op) = make_uint2(h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16));
+        stream_store8(op, h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16));
       } else {
         for (int k = 0; k < DRUN; ++k) if (k < n) op[k] = h[k];
       }
@@ -393,7 +393,7 @@ __global__ __launch_bounds__(256) void float_to_hfp8_kernel(const float* in, uin
     const float4 x = reinterpret_cast<const float4*>(in)[i];
     const uint32_t c = float_to_hfp8(x.x, ebits, bias, max_pos) | (float_to_hfp8(x.y, ebits, bias, max_pos) << 8) |
         (float_to_hfp8(x.z, ebits, bias, max_pos) << 16) | (float_to_hfp8(x.w, ebits, bias, max_pos) << 24);
-    reinterpret_cast<uint32_t*>(out)[i] = c;
+    stream_store4(reinterpret_cast<uint32_t*>(out) + i, c);
   }
   for (int64_t i = n4 * 4 + tid; i < n; i += nthreads) out[i] = (uint8_t)float_to_hfp8(in[i], ebits, bias, max_pos);
 }
@@ -405,8 +405,8 @@ __global__ __launch_bounds__(256) void hfp8_to_float_kernel(const uint8_t* in, f
   const int64_t n4 = vec ? n / 4 : 0;
   for (int64_t i = tid; i < n4; i += nthreads) {
     const uint32_t c = reinterpret_cast<const uint32_t*>(in)[i];
-    reinterpret_cast<float4*>(out)[i] = make_float4(hfp8_to_float(c & 0xffu, shift, mult), hfp8_to_float((c >> 8) & 0xffu, shift, mult),
-                                                    hfp8_to_float((c >> 16) & 0xffu, shift, mult), hfp8_to_float(c >> 24, shift, mult));
+    stream_store16(reinterpret_cast<float4*>(out) + i, hfp8_to_float(c & 0xffu, shift, mult), hfp8_to_float((c >> 8) & 0xffu, shift, mult),
+                   hfp8_to_float((c >> 16) & 0xffu, shift, mult), hfp8_to_float(c >> 24, shift, mult));
   }
   for (int64_t i = n4 * 4 + tid; i < n; i += nthreads) out[i] = hfp8_to_float(in[i], shift, mult);
 }
