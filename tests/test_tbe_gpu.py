@@ -319,6 +319,65 @@ def test_no_pooling_matches_oracle(ops, oracle, dt, D):
                     ops.POOL_NONE, None, FP16, row_alignment=row_alignment)
 
 
+def _no_pooling_case(ops, oracle, rng, specs, B, max_len, dt, row_alignment, out_ty, tag):
+    T, D = len(specs), specs[0][1]
+    tys = [s[2] for s in specs]
+    weights, wo, _ = build_weights(rng, specs, row_alignment)
+    lens = rng.integers(0, max_len + 1, size=T * B)
+    for t in range(T):
+        if rng.random() < 0.15:
+            lens[t * B:(t + 1) * B] = 0  # a table nobody asks for
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(dt)
+    idx = np.concatenate([rng.integers(0, specs[t][0], size=int(lens[t * B:(t + 1) * B].sum())) for t in range(T)]
+                         + [np.zeros(0, np.int64)]).astype(dt)
+    idx[rng.random(len(idx)) < 0.05] = -1
+    wt = np.array(tys, np.uint8)
+    D_offsets = (np.arange(T + 1) * D).astype(np.int32)
+    maxd = lambda ty: D if ty in tys else 0
+    got = ops.int_nbit_split_embedding_codegen_lookup_function(
+        cu(weights), torch.zeros(0, dtype=torch.uint8, device="cuda"), cu(np.zeros(T, np.int32)), cu(wo), cu(wt),
+        cu(D_offsets), T * D, maxd(INT2), maxd(INT4), maxd(INT8), maxd(FP16), maxd(FP32), cu(idx), cu(off),
+        ops.POOL_NONE, None, out_ty, row_alignment=row_alignment)
+    assert tuple(got.shape) == (len(idx), D)
+    ok, want = oracle.tbe_forward_nobag(weights, wo, wt, [s[0] for s in specs], D, idx, off, out_ty, row_alignment)
+    assert ok
+    g = got.cpu()
+    g = g.numpy() if out_ty == FP32 else g.view(torch.int16).numpy().view(np.uint16)
+    H.assert_same_bits(g, want, tag)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_no_pooling_random_shapes(ops, oracle, seed):
+    """Random table counts, row types, widths (narrower and wider than what the lanes of a row cover in one
+    pass), alignments and bag lengths: the positions a wave takes together then begin and end anywhere inside
+    tables, cross table boundaries and run past the end of the index array."""
+    rng = np.random.default_rng(7000 + seed)
+    for _ in range(6):
+        T = int(rng.integers(1, 7))
+        D = int(rng.choice([8, 16, 40, 64, 100, 128, 256, 520, 1024]))
+        tys = [int(rng.choice([INT4, INT8, FP16, INT2, FP32])) for _ in range(T)]
+        if any(ty == INT2 for ty in tys) and D % 4:
+            D += 4 - D % 4
+        specs = [(int(rng.integers(1, 400)), D, ty) for ty in tys]
+        B = int(rng.integers(1, 40))
+        max_len = int(rng.choice([1, 3, 9, 40]))
+        if T * B * max_len * D > 6_000_000:
+            max_len = 3
+        dt = rng.choice([np.int32, np.int64])
+        align = int(rng.choice([16, 4, 1]))
+        out_ty = int(rng.choice([FP32, FP16, BF16]))
+        _no_pooling_case(ops, oracle, rng, specs, B, max_len, dt, align, out_ty,
+                         f"seed {seed}: T={T} D={D} tys={tys} B={B} L<={max_len} align={align} out={out_ty}")
+
+
+def test_no_pooling_more_positions_than_one_pass_of_the_grid(ops, oracle):
+    """Rows of 512 columns take a whole wave; 300 K positions are more than the largest grid covers at once, so
+    every wave walks several groups and uses the indices it fetched one group ahead."""
+    rng = np.random.default_rng(31)
+    specs = [(500, 512, INT4), (300, 512, INT8), (200, 512, INT4)]
+    _no_pooling_case(ops, oracle, rng, specs, 2500, 80, np.int64, 16, FP16, "300 K positions of 512 columns")
+
+
 def test_no_pooling_with_more_tables_than_the_kernel_keeps_in_lds(ops, oracle):
     """1100 small tables (some without any index): the table boundaries no longer fit the
     workgroup's LDS and the bisection reads them from memory."""
