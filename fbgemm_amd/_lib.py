@@ -32,6 +32,8 @@ SYMBOLS = {
     "fbgemm_amd_stream_synchronize": (C.c_int, [_P]),
     "fbgemm_amd_status_read": (C.c_int, [_P, _P, C.POINTER(_I32), C.POINTER(_I64)]),
     "fbgemm_amd_spmdm_launch": (C.c_int, [C.POINTER(SpmdmConfig), _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _P, _P]),
+    "fbgemm_amd_spmdm_launch_noalloc": (C.c_int, [C.POINTER(SpmdmConfig), _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _P, _P]),
+    "fbgemm_amd_noalloc_max_bags": (_I64, []),
     "fbgemm_amd_spmdm_run": (C.c_int, [C.POINTER(SpmdmConfig), _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _P]),
     "fbgemm_amd_tbe_plan_create": (C.c_int, [C.POINTER(_P), _I32, _P, _P, _P, _P, _I64, _I64, _I64]),
     "fbgemm_amd_tbe_plan_destroy": (None, [_P]),

@@ -347,12 +347,51 @@ int32_t fbgemm_amd_padded_row_size_in_bytes(int32_t dim, int32_t ty, int32_t row
   return (int32_t)((r + a - 1) / a * a);
 }
 
-int fbgemm_amd_spmdm_launch(
+} // extern "C"
+
+namespace {
+
+// ---- scratch of the entry point that allocates nothing ------------------------
+//
+// fbgemm_amd_spmdm_launch_noalloc keeps what fbgemm_amd_spmdm_launch would put
+// into hipMalloc'ed scratch (the prefix sum of Caffe2-style lengths, the bag
+// order of the scheduler) in this array, which is part of the code object:
+// every GPU the library runs on holds its own copy from module load until the
+// process ends. Host code never uses the array's name as an address; the
+// device address is asked for once per device (noalloc_scratch_ptr).
+constexpr int64_t NOALLOC_MAX_BAGS = FBGEMM_AMD_NOALLOC_MAX_BAGS;
+constexpr size_t NOALLOC_OFFSETS_BYTES = ((size_t)(NOALLOC_MAX_BAGS + 1) * sizeof(int64_t) + 255) / 256 * 256;
+constexpr size_t NOALLOC_ORDER_BYTES = (size_t)NOALLOC_MAX_BAGS * sizeof(BagEntry);
+static __device__ __align__(256) unsigned char scratch[NOALLOC_OFFSETS_BYTES + NOALLOC_ORDER_BYTES];
+
+std::map<int, unsigned char*> g_noalloc_ptr; // per device; guarded by g_mu
+
+// Device address of the current device's copy of `scratch`. Allocates nothing:
+// the array came with the code object.
+int noalloc_scratch_ptr(unsigned char** out) {
+  int dev = 0;
+  HIP_TRY(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lk(g_mu);
+  auto it = g_noalloc_ptr.find(dev);
+  if (it == g_noalloc_ptr.end()) {
+    void* p = nullptr;
+    HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) return fail(FBGEMM_AMD_E_HIP, "hipGetSymbolAddress gave no address for the static scratch array");
+    it = g_noalloc_ptr.emplace(dev, (unsigned char*)p).first;
+  }
+  *out = it->second;
+  return 0;
+}
+
+int spmdm_launch_impl(
     const fbgemm_amd_spmdm_config* cfg, int64_t output_size, int64_t index_size,
     int64_t data_size, const void* d_input, const void* d_indices,
     const void* d_offsets_or_lengths, const float* d_weights, void* d_out,
-    const int32_t* d_remap, void* d_status, void* stream_) {
+    const int32_t* d_remap, void* d_status, void* stream_, bool noalloc) {
   if (int rc = check_cfg(cfg)) return rc;
+  if (noalloc && output_size > NOALLOC_MAX_BAGS)
+    return fail(FBGEMM_AMD_E_ARG, "fbgemm_amd_spmdm_launch_noalloc takes at most %lld bags per call (got %lld); "
+                "use fbgemm_amd_spmdm_launch", (long long)NOALLOC_MAX_BAGS, (long long)output_size);
   if (!d_status) return fail(FBGEMM_AMD_E_ARG, "d_status is null");
   if (output_size < 0 || index_size < 0 || data_size < 0) return fail(FBGEMM_AMD_E_ARG, "negative size");
   if (output_size > 0x7fffffffLL) return fail(FBGEMM_AMD_E_ARG, "output_size exceeds 2^31-1");
@@ -480,7 +519,24 @@ int fbgemm_amd_spmdm_launch(
     a.offsets = d_offsets_or_lengths;
     a.off64 = cfg->offset_bits == 64;
   }
-  if (!cfg->use_offsets || sort) {
+  if ((!cfg->use_offsets || sort) && noalloc) {
+    // the static array: offsets first, then the bag order. Both are written in
+    // full (output_size + 1 offsets, output_size entries) before they are read,
+    // so what an earlier call left there does not matter.
+    unsigned char* base;
+    if (int rc = noalloc_scratch_ptr(&base)) return rc;
+    if (!cfg->use_offsets) {
+      int64_t* offs = reinterpret_cast<int64_t*>(base);
+      HIP_TRY(launch_lengths_to_offsets(d_offsets_or_lengths, cfg->offset_bits == 64, output_size, offs, stream));
+      a.offsets = offs;
+      a.off64 = 1;
+    }
+    if (sort) {
+      BagEntry* order = reinterpret_cast<BagEntry*>(base + NOALLOC_OFFSETS_BYTES);
+      HIP_TRY(launch_bag_order(a.offsets, a.off64, (int32_t)output_size, 1, order, stream));
+      a.order = order;
+    }
+  } else if (!cfg->use_offsets || sort) {
     // library-owned scratch: calls that use it must be ordered on one stream
     std::lock_guard<std::mutex> lk(g_mu);
     DeviceScratch* s;
@@ -500,6 +556,30 @@ int fbgemm_amd_spmdm_launch(
   HIP_TRY(launch_lookup(a, cfg->index_bits == 64, stream));
   return 0;
 }
+
+} // namespace
+
+extern "C" {
+
+int fbgemm_amd_spmdm_launch(
+    const fbgemm_amd_spmdm_config* cfg, int64_t output_size, int64_t index_size,
+    int64_t data_size, const void* d_input, const void* d_indices,
+    const void* d_offsets_or_lengths, const float* d_weights, void* d_out,
+    const int32_t* d_remap, void* d_status, void* stream) {
+  return spmdm_launch_impl(cfg, output_size, index_size, data_size, d_input, d_indices, d_offsets_or_lengths,
+                           d_weights, d_out, d_remap, d_status, stream, false);
+}
+
+int fbgemm_amd_spmdm_launch_noalloc(
+    const fbgemm_amd_spmdm_config* cfg, int64_t output_size, int64_t index_size,
+    int64_t data_size, const void* d_input, const void* d_indices,
+    const void* d_offsets_or_lengths, const float* d_weights, void* d_out,
+    const int32_t* d_remap, void* d_status, void* stream) {
+  return spmdm_launch_impl(cfg, output_size, index_size, data_size, d_input, d_indices, d_offsets_or_lengths,
+                           d_weights, d_out, d_remap, d_status, stream, true);
+}
+
+int64_t fbgemm_amd_noalloc_max_bags(void) { return NOALLOC_MAX_BAGS; }
 
 int fbgemm_amd_spmdm_run(
     const fbgemm_amd_spmdm_config* cfg, int64_t output_size, int64_t index_size,

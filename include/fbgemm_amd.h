@@ -123,6 +123,31 @@ int fbgemm_amd_spmdm_launch(
     const void* d_offsets_or_lengths, const float* d_weights, void* d_out,
     const int32_t* d_compressed_indices_table, void* d_status, void* stream);
 
+/* fbgemm_amd_spmdm_launch for callers that cannot allocate device memory (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc). It has no counterpart in the reference. Same arguments, same
+ * kernels, same results bit for bit; the two pieces of scratch the call above
+ * takes from hipMalloc'ed buffers (the prefix sum of the lengths when
+ * use_offsets == 0, and the bag order of the scheduler for calls of 2^21
+ * lookups and more) live in a static device array of the library instead
+ * (about 2.5 MiB, held by every GPU the library runs on until the process
+ * ends). Limit: output_size <= FBGEMM_AMD_NOALLOC_MAX_BAGS, larger calls are
+ * rejected with FBGEMM_AMD_E_ARG. It calls no hipMalloc / hipFree and no
+ * allocating library routine; its first call on a device asks the runtime for
+ * the array's device address (no allocation, but make that call outside a
+ * graph capture). All calls on one GPU share the array: two of them that
+ * overlap in time (different streams, or host threads without ordering) race;
+ * order them on one stream. Nothing in the array has to start at zero (every
+ * call writes what it reads). */
+#define FBGEMM_AMD_NOALLOC_MAX_BAGS 65536
+int fbgemm_amd_spmdm_launch_noalloc(
+    const fbgemm_amd_spmdm_config* cfg, int64_t output_size, int64_t index_size,
+    int64_t data_size, const void* d_input, const void* d_indices,
+    const void* d_offsets_or_lengths, const float* d_weights, void* d_out,
+    const int32_t* d_compressed_indices_table, void* d_status, void* stream);
+/* The limit above, for callers that bind the library without its header. */
+int64_t fbgemm_amd_noalloc_max_bags(void);
+
 /* Same, synchronous, with the reference's return convention: 1 = true,
  * 0 = false (the inputs were rejected; output unspecified), < 0 = API error.
  * Uses a library-owned status block. */
