@@ -1,6 +1,6 @@
 #!/bin/bash
 # Collect the rocprofv3 evidence for one benchmark configuration and condense it.
-#   bash fbgemm_amd/profile_run.sh <config id> <output summary file> [extra bench.py args]
+#   bash profile_run.sh <config id> <output summary file> [extra bench.py args]
 # (extra args "--op quantize" etc. profile an operator beside the lookup; the config id is then unused)
 # Runs from the repository root on a machine with the GPU. One rocprofv3 run per
 # counter group (the hardware cannot collect them together); raw CSVs go to /tmp.
@@ -9,18 +9,18 @@ CFG=${1:-3}; OUT=${2:-profile_summary.txt}; shift; shift
 export TMPDIR=/tmp
 RAW=$(mktemp -d /tmp/fbgemm_amd_prof.XXXXXX)
 mkdir -p "$(dirname "$OUT")"
-BENCH="python3 bench.py --config $CFG --no-cpu --calibration-copy-mib 1024 $*"
+BENCH="python3 bench.py --config $CFG --no-cpu --no-also --no-check --calibration-copy-mib 1024 $*"
 {
   echo "# rocprofv3 summary, bench.py --config $CFG $*"
   echo "# commands (each its own run):"
   echo "#   rocprofv3 --kernel-trace --stats --output-format csv -d <dir> -o t -- $BENCH --steps 20 --warmup 3"
   echo "#   rocprofv3 --pmc <counters> --output-format csv -d <dir> -o p -- $BENCH --steps 3 --warmup 1"
-  echo "# condensed with: python3 -m fbgemm_amd.profile_summary <dir>"
+  echo "# condensed with: python3 profile_summary.py <dir>"
 } > "$OUT"
 echo "== kernel trace (--kernel-trace --stats), 23 launches" >> "$OUT"
 timeout -k 10 900 rocprofv3 --kernel-trace --stats --output-format csv -d $RAW/trace -o t -- $BENCH --steps 20 --warmup 3 > $RAW/trace.log 2>&1 || { echo "trace run failed" | tee -a "$OUT"; tail -5 $RAW/trace.log; exit 1; }
 grep '^{' $RAW/trace.log | tail -1 | cut -c1-1200 >> "$OUT"
-python3 -m fbgemm_amd.profile_summary $RAW/trace | grep -v '^#' >> "$OUT"
+python3 profile_summary.py $RAW/trace | grep -v '^#' >> "$OUT"
 # PROFILE_SHORT=1 keeps the byte counters only (for workloads whose set-up takes minutes)
 if [ -n "$PROFILE_SHORT" ]; then
   PASSES=("FETCH_SIZE" "WRITE_SIZE" "TCC_HIT_sum TCC_MISS_sum" "GRBM_GUI_ACTIVE")
@@ -33,8 +33,8 @@ for pass in "${PASSES[@]}"; do
   n=$(echo $pass | tr ' ' '_' | cut -c1-40)
   echo "== --pmc $pass" >> "$OUT"
   timeout -s KILL 600 rocprofv3 --pmc $pass --output-format csv -d $RAW/pmc_$n -o p -- $BENCH --steps 3 --warmup 1 > $RAW/pmc_$n.log 2>&1 || { echo "pass failed: $pass" >> "$OUT"; tail -3 $RAW/pmc_$n.log >> "$OUT"; exit 1; }
-  python3 -m fbgemm_amd.profile_summary $RAW/pmc_$n | grep -v '^#\|^launch' >> "$OUT"
+  python3 profile_summary.py $RAW/pmc_$n | grep -v '^#\|^launch' >> "$OUT"
 done
-python3 -m fbgemm_amd.profile_summary $RAW/pmc_GRBM_GUI_ACTIVE | grep '^launch' >> "$OUT"
+python3 profile_summary.py $RAW/pmc_GRBM_GUI_ACTIVE | grep '^launch' >> "$OUT"
 rm -rf $RAW
 echo "summary written to $OUT"

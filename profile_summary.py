@@ -1,11 +1,16 @@
 """Condense rocprofv3 CSV output into a few lines per kernel of this library.
 
-    python -m fbgemm_amd.profile_summary <rocprofv3 output dir> [more dirs...]
+    python3 profile_summary.py <rocprofv3 output dir> [more dirs...]
 
 Prints, for every kernel of this library (and the totals row of --stats), the call count and
 average duration, and the per-dispatch average of every hardware counter
 collected. Raw CSVs hold every torch kernel of the run and are large; this is
 the part worth keeping.
+
+The `launch` lines repeat rocprofv3's own columns. Its VGPR_Count is not the
+kernel's register allocation on this device (it reads 80 for lookup_kernel,
+whose code object allocates 157 vector registers, 3 waves per SIMD): take
+register counts from the code object's notes, not from here.
 """
 import csv
 import glob
@@ -13,7 +18,7 @@ import os
 import sys
 from collections import defaultdict
 
-OURS = ("inplace_update_kernel", "remap_row_idx_kernel", "sequence_lookup_kernel", "row_lookup_kernel", "pruned_array_lookup", "pruned_hashmap_lookup", "lookup_kernel",
+OURS = ("gather_lines_kernel", "stream_read_kernel", "remap_rank_build", "inplace_update_kernel", "remap_row_idx_kernel", "sequence_lookup_kernel", "row_lookup_kernel", "pruned_array_lookup", "pruned_hashmap_lookup", "lookup_kernel",
         "calibration_copy_kernel", "float_to_hfp8_kernel", "hfp8_to_float_kernel", "prune_count", "prune_carry", "prune_remap",
         "prune_gather", "remap_count", "remap_move", "remap_offsets",
         "bag_order_kernel", "lengths_to_offsets", "bounds_partial_max", "bounds_carry", "bounds_fix_offsets",
@@ -53,7 +58,7 @@ def summarize(d):
         for (s, c), (tot, n) in sorted(acc.items()):
             lines.append(f"pmc    {s}: {c} avg_per_dispatch={tot / n:.6g} dispatches={n}")
         for s, g in sorted(grid.items()):
-            lines.append(f"launch {s}: grid={g[0]} wg={g[1]} vgpr={g[2]} agpr={g[3]} sgpr={g[4]} lds={g[5]} scratch={g[6]}")
+            lines.append(f"launch {s}: grid={g[0]} wg={g[1]} rocprof_vgpr_column={g[2]} agpr={g[3]} sgpr={g[4]} lds={g[5]} scratch={g[6]}")
     return lines
 
 

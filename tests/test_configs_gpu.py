@@ -1,8 +1,11 @@
-"""The five benchmark configurations on the GPU. Configs 1, 2 and 4 (a table
-subset) are checked in full against the oracle; config 3 at its real size on
-sampled tables plus size-independent properties (determinism, independence of
-a bag from the rest of the batch, exact zeros for empty bags); config 5 at
-1/100 scale in full (its real size is exercised by bench.py --config 5 --check)."""
+"""The five benchmark configurations on the GPU at their real sizes. Configs 1
+and 2 in full against the oracle; config 3 with all 64 tables against the
+oracle; config 4 both ways (per-table row-wise-sparse kernels on two tables,
+and the table-batched forward with the mappings fused in, which is what the
+benchmark times) and config 5 on sampled tables; the three table-batched ones
+also through size-independent properties of the whole output (determinism,
+independence of a bag from the rest of the batch, exact zeros for empty bags).
+Config 5 once more at 1/100 scale in full."""
 import numpy as np
 import pytest
 
@@ -71,14 +74,17 @@ def tbe_forward(ops, p, indices=None, offsets=None, weights="same"):
         p.dev_weights, torch.zeros(0, dtype=torch.uint8, device="cuda"), cu(np.zeros(p.T, np.int32)),
         cu(p.weights_offsets), cu(p.tys), cu(p.D_offsets), p.total_D, 32, 256, 256, 256, 0,
         p.indices if indices is None else indices, p.offsets if offsets is None else offsets, p.pooling_mode, w,
-        p.output_dtype, row_alignment=p.row_alignment)
+        p.output_dtype, row_alignment=p.row_alignment, index_remappings=p.extra.get("remap"),
+        index_remappings_offsets=p.extra.get("remap_offsets"))
 
 
 def oracle_table(oracle, p, t):
+    """Table t's [B, D_t] block from the oracle (the physical row ids: for pruned tables the
+    oracle's own pruned_array_lookup has been compared with them by the caller)."""
     s, e = int(p.host_offsets[t * p.B]), int(p.host_offsets[(t + 1) * p.B])
     ty = int(p.tys[t])
     elem = 4 if ty == 0 else 2 if ty == 1 else 1
-    ok, want = oracle.spmdm(ty, int(p.Ds[t]), p.table_host_bytes(t), p.host_indices[s:e],
+    ok, want = oracle.spmdm(ty, int(p.Ds[t]), p.table_host_bytes(t), p.physical_indices[s:e],
                             p.host_offsets[t * p.B:(t + 1) * p.B + 1] - p.host_offsets[t * p.B],
                             weights=None if p.host_weights is None else p.host_weights[s:e],
                             normalize=p.pooling_mode == 1, out_ty=p.output_dtype,
@@ -88,36 +94,73 @@ def oracle_table(oracle, p, t):
     return want.reshape(p.B, int(p.Ds[t]))
 
 
+def check_tables(oracle, p, out, tables, what):
+    for t in tables:
+        c0, c1 = int(p.D_offsets[t]), int(p.D_offsets[t + 1])
+        got = bits_of(out[:, c0:c1].contiguous(), p.output_dtype)
+        H.assert_same_bits(got, oracle_table(oracle, p, t), f"{what} table {t}")
+
+
+def check_properties(ops, p, out):
+    """What holds at any size, on the whole output: the same bits on a second forward (the
+    scheduler's bag order may differ between runs, the sums may not); a bag's result does not
+    depend on where it sits in the batch (the bags of every table in reverse); exact zeros
+    for empty bags."""
+    assert torch.equal(out, tbe_forward(ops, p))
+    B, T = p.B, p.T
+    lens = p.lengths.reshape(T, B)
+    rev_lens = np.ascontiguousarray(lens[:, ::-1]).reshape(-1)
+    rev_off = np.concatenate([[0], np.cumsum(rev_lens)]).astype(p.host_offsets.dtype)
+    starts = np.ascontiguousarray(p.host_offsets[:-1].reshape(T, B)[:, ::-1]).reshape(-1)
+    bag_of = np.repeat(np.arange(T * B), rev_lens)
+    gather = starts[bag_of] + (np.arange(int(rev_off[-1]), dtype=np.int64) - rev_off[bag_of])
+    del bag_of
+    rev_idx = torch.from_numpy(p.host_indices[gather]).cuda()
+    rev_w = None if p.host_weights is None else torch.from_numpy(p.host_weights[gather]).cuda()
+    del gather
+    out_rev = tbe_forward(ops, p, rev_idx, torch.from_numpy(rev_off).cuda(), rev_w)
+    del rev_idx, rev_w
+    assert torch.equal(out_rev.flip(0), out)
+    del out_rev
+    for t, b in zip(*np.nonzero(lens == 0)):
+        blk = out[int(b), int(p.D_offsets[t]):int(p.D_offsets[t + 1])]
+        assert int((blk.view(torch.int16 if p.output_dtype else torch.int32) != 0).sum()) == 0
+
+
 def test_config3_full_size(ops, oracle):
+    """All 64 tables against the oracle, then the size-independent properties."""
     from fbgemm_amd import bench_configs as bc
     p = bc.config3("cuda")
     out = tbe_forward(ops, p)
-    got = bits_of(out, p.output_dtype)
-    # one table of every (type, D) combination present, against the oracle
-    seen = {}
-    for t in range(p.T):
-        seen.setdefault((int(p.tys[t]), int(p.Ds[t])), t)
-    for t in sorted(seen.values()):
-        c0, c1 = int(p.D_offsets[t]), int(p.D_offsets[t + 1])
-        H.assert_same_bits(np.ascontiguousarray(got[:, c0:c1]), oracle_table(oracle, p, t), f"config3 table {t}")
-    # determinism: the bag order inside the scheduler may differ between runs, the bits may not
-    assert torch.equal(out, tbe_forward(ops, p))
-    # a bag's result does not depend on the rest of the batch: reverse the bag order of every table
-    B, T = p.B, p.T
-    lens = p.lengths.reshape(T, B)
-    rev_lens = lens[:, ::-1].reshape(-1)
-    rev_off = np.concatenate([[0], np.cumsum(rev_lens)]).astype(np.int64)
-    starts = p.host_offsets[:-1].reshape(T, B)[:, ::-1].reshape(-1)
-    gather = np.concatenate([np.arange(s, s + l) for s, l in zip(starts, rev_lens)])
-    rev_idx = p.host_indices[gather]
-    rev_w = p.host_weights[gather]
-    cu = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
-    out_rev = tbe_forward(ops, p, cu(rev_idx), cu(rev_off), cu(rev_w))
-    assert torch.equal(out_rev.flip(0), out)
-    # empty bags are exact zeros
-    empty = np.nonzero(lens == 0)
-    for t, b in zip(*empty):
-        assert (got[b, int(p.D_offsets[t]):int(p.D_offsets[t + 1])] == 0).all()
+    check_tables(oracle, p, out, range(p.T), "config3")
+    check_properties(ops, p, out)
+
+
+def test_config4_batched_full_size(ops, oracle):
+    """Config 4 as the benchmark times it (one table-batched forward, the int32 mappings fused
+    in) at its real size: the logical -> physical mapping against the oracle's
+    pruned_array_lookup, first / middle / last tables against the oracle, properties on all."""
+    from fbgemm_amd import bench_configs as bc
+    p = bc.config4_batched("cuda")
+    dense = oracle.pruned_array_lookup(p.host_indices, p.host_offsets, p.extra["host_remap"], p.extra["host_remap_offsets"])
+    assert (dense == p.extra["host_dense"]).all()
+    frac = float((dense != -1).mean())
+    assert 0.3 < frac < 0.7  # pruned rows are hit at the base rate
+    out = tbe_forward(ops, p)
+    check_tables(oracle, p, out, [0, 1, p.T // 2, p.T - 1], "config4 batched")
+    check_properties(ops, p, out)
+
+
+def test_config5_full_size(ops, oracle):
+    """The HBM-sized workload at its real size (173 GB of rows, a grid of millions of
+    workgroups, 64-bit row offsets far beyond 2^32, 7 M offsets): the first, a middle and the
+    last 4-bit table and two of the 2-bit tables against the oracle, properties on all."""
+    from fbgemm_amd import bench_configs as bc
+    p = bc.config5("cuda")
+    assert int(p.weights_offsets[-1]) > 1 << 37
+    out = tbe_forward(ops, p)
+    check_tables(oracle, p, out, [0, 200, 399, 400, 431], "config5")
+    check_properties(ops, p, out)
 
 
 def test_config5_scaled(ops, oracle):
