@@ -48,6 +48,10 @@ def parse():
     ap.add_argument("--no-check", dest="check", action="store_false",
                     help="skip the parity gate (by default a sample of tables of the first forward is compared with "
                          "the oracle before anything is timed, and the line says \"checked\": true)")
+    ap.add_argument("--accumulate", default="exact", choices=["exact", "fast"],
+                    help="exact = the reference's sequence of fp32 roundings, bit-identical to the CPU path (the "
+                         "library's default); fast = the biases of a bag summed apart (tolerance grade: the parity "
+                         "gate then holds fp16 / bf16 output to one unit in the last place and fp32 output to 1e-5)")
     ap.add_argument("--no-also", dest="also", action="store_false",
                     help="default run only: do not append the driver-timed figures of config 5 under \"also\"")
     ap.add_argument("--op", default="lookup",
@@ -85,7 +89,7 @@ def traffic_from_profile(config_id):
         return None
 
 
-def tbe_runner(p, torch):
+def tbe_runner(p, torch, accumulate="exact"):
     """Returns (launch, out, status, plan) for a TbeProblem: launch() enqueues one forward."""
     from fbgemm_amd import _lib, ops
 
@@ -93,6 +97,7 @@ def tbe_runner(p, torch):
     dev = p.dev_weights.device
     plan = ops.TbePlan(torch.from_numpy(p.weights_offsets), torch.from_numpy(p.tys), torch.from_numpy(p.D_offsets),
                        torch.zeros(p.T, dtype=torch.int32), p.dev_weights.numel(), 0, p.row_alignment)
+    _lib.check(lib.fbgemm_amd_tbe_plan_set_accumulate(plan.handle, 1 if accumulate == "fast" else 0))
     out_dt = {0: torch.float32, 1: torch.float16, 5: torch.bfloat16}[p.output_dtype]
     out = torch.empty((p.B, p.total_D), dtype=out_dt, device=dev)
     st = ops.Status(dev)
@@ -470,13 +475,38 @@ def sample_tables(p):
     return sorted(set(seen.values()) | {0, p.T // 2, p.T - 1})
 
 
-def parity_gate(p, out, launch, torch, np):
+def ordered(bits16):
+    """16-bit float patterns as integers in value order (so that neighbours differ by one)."""
+    import numpy as np
+    b = bits16.astype(np.int32)
+    return np.where(b & 0x8000, -(b & 0x7fff), b)
+
+
+def within_grade(got, want, out_ty, np):
+    """Tolerance-grade comparison: fp16 / bf16 within one unit in the last place; fp32 within
+    1e-5 of the larger of |want| and the largest magnitude in the bag's block (a sum that
+    cancels to near zero is held to the size of what was summed). Returns (ok, worst)."""
+    if out_ty != 0:
+        d = np.abs(ordered(got) - ordered(want))
+        nan = ((want & 0x7fff) > (0x7c00 if out_ty == 1 else 0x7f80))
+        d = np.where(nan, 0, d)
+        return bool((d <= 1).all()), int(d.max(initial=0))
+    g, w = got.astype(np.float64), want.astype(np.float64)
+    scale = np.maximum(np.abs(w), np.abs(w).max(axis=1, keepdims=True))
+    rel = np.abs(g - w) / np.maximum(scale, 1e-30)
+    rel = np.where(np.isfinite(w), rel, 0.0)
+    return bool((rel <= 1e-5).all()), float(rel.max(initial=0.0))
+
+
+def parity_gate(p, out, launch, torch, np, accumulate="exact"):
     """One forward, then the sampled tables' blocks of its output against the
-    oracle on the same inputs, bit for bit. Raises before anything is timed."""
+    oracle on the same inputs: bit for bit (exact), or to the stated tolerance
+    (fast). Raises before anything is timed."""
     import oracle
     launch()
     torch.cuda.synchronize()
     tables = sample_tables(p)
+    worst = 0
     for t in tables:
         s, e = int(p.host_offsets[t * p.B]), int(p.host_offsets[(t + 1) * p.B])
         elem = 4 if int(p.tys[t]) == 0 else 2 if int(p.tys[t]) == 1 else 1
@@ -488,9 +518,17 @@ def parity_gate(p, out, launch, torch, np):
                                 data_size=int(p.rows[t]), output_size=p.B)
         got = out[:, int(p.D_offsets[t]):int(p.D_offsets[t + 1])].contiguous().cpu()
         got = got.numpy() if p.output_dtype == 0 else got.view(torch.int16).numpy().view(np.uint16)
-        if not (ok and (got.reshape(-1).view(want.dtype) == want).all()):
+        if accumulate == "exact":
+            same = ok and (got.reshape(-1).view(want.dtype) == want).all()
+        else:
+            same, w = within_grade(got.reshape(p.B, -1), want.reshape(p.B, -1), p.output_dtype, np)
+            worst = max(worst, w)
+            same = ok and same
+        if not same:
             raise AssertionError(f"parity gate: table {t} of {p.name} differs from the oracle; nothing was timed")
-    print(f"parity gate: tables {tables} of {p.name} match the oracle bit for bit", file=sys.stderr)
+    how = "bit for bit" if accumulate == "exact" else (
+        f"to tolerance (worst: {worst} {'units in the last place' if p.output_dtype else 'relative'})")
+    print(f"parity gate: tables {tables} of {p.name} match the oracle {how}", file=sys.stderr)
     return tables
 
 
@@ -498,9 +536,9 @@ def time_tbe(p, a, torch, np, steps, warmup, graph=False):
     """Parity gate, warm-up, `steps` timed forwards of one table-batched problem.
     Returns the figures of the JSON line that depend on the measurement."""
     from fbgemm_amd import _lib
-    launch, out, st, plan = tbe_runner(p, torch)
+    launch, out, st, plan = tbe_runner(p, torch, a.accumulate)
     torch.cuda.synchronize()
-    checked = parity_gate(p, out, launch, torch, np) if a.check else None
+    checked = parity_gate(p, out, launch, torch, np, a.accumulate) if a.check else None
     for _ in range(warmup):
         launch()
     torch.cuda.synchronize()
@@ -634,7 +672,8 @@ def main():
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": name, "config_id": a.config, "scale": a.scale, "lookups_per_step": lookups,
                    "useful_row_bytes_per_step": useful, "other_bytes_per_step": other,
-                   "output_dtype": dtype_out, "launches_per_step": launches_per_step, "hip_graph": bool(a.graph)},
+                   "output_dtype": dtype_out, "launches_per_step": launches_per_step, "hip_graph": bool(a.graph),
+                   "accumulate": a.accumulate},
         "checked": bool(checked), "checked_tables": checked,
         "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
         "pooled_rows_per_s": round(lookups / (ms_per_step * 1e-3), 1),

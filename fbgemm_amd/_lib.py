@@ -21,7 +21,7 @@ class SpmdmConfig(C.Structure):
         ("block_size", _I64), ("output_stride", _I64), ("input_stride", _I64),
         ("normalize_by_lengths", _I32), ("is_weight_positional", _I32),
         ("use_offsets", _I32), ("scale_bias_last", _I32),
-        ("no_bag", _I32), ("fp8_exponent_bits", _I32), ("fp8_exponent_bias", _I32), ("reserved", _I32),
+        ("no_bag", _I32), ("fp8_exponent_bits", _I32), ("fp8_exponent_bias", _I32), ("accumulate", _I32),
     ]
 
 
@@ -40,6 +40,11 @@ SYMBOLS = {
     "fbgemm_amd_tbe_forward": (C.c_int, [_P, _P, _P, _P, _P, _I32, _I64, _I64, _I32, _P, _I32, _P, _P, _P]),
     "fbgemm_amd_tbe_forward_pruned": (C.c_int, [_P, _P, _P, _P, _P, _I32, _I64, _I64, _I32, _P, _I32, _P, _P, _I32, _P, _P, _P]),
     "fbgemm_amd_tbe_plan_set_fp8": (C.c_int, [_P, _I32, _I32]),
+    "fbgemm_amd_tbe_plan_set_accumulate": (C.c_int, [_P, _I32]),
+    "fbgemm_amd_tbe_plan_trim": (C.c_int, [_P]),
+    "fbgemm_amd_tbe_plan_cached_work": (_I64, [_P]),
+    "fbgemm_amd_set_lean": (C.c_int, [_I32]),
+    "fbgemm_amd_set_narrow_below_waves": (C.c_int, [_I32]),
     "fbgemm_amd_tbe_forward_nobag": (C.c_int, [_P, _P, _P, _P, _P, _I32, _I64, _I64, _I32, _I32, _P, _P, _P]),
     "fbgemm_amd_tbe_plan_profile": (C.c_int, [_P, _I32]),
     "fbgemm_amd_tbe_plan_profile_read": (C.c_int, [_P, _P, _I32, _P]),

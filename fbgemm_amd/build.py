@@ -11,8 +11,12 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "lib", "libfbgemm_amd.so")
 
-SOURCES = ["lookup_kernels.hip", "index_ops_kernels.hip", "quantize_kernels.hip", "sequence_kernels.hip", "prune_kernels.hip", "update_kernels.hip", "c_api.cpp"]
-HEADERS = ["lookup_common.h", os.path.join("..", "..", "include", "fbgemm_amd.h")]
+# the lookup kernels compile one instance per translation unit (the slowest files first)
+SOURCES = ["lookup_lean_i64_exact.hip", "lookup_lean_i64_fast.hip", "lookup_lean_i32_exact.hip", "lookup_lean_i32_fast.hip",
+           "lookup_i64.hip", "lookup_i32.hip", "lookup_i64_general.hip", "lookup_i32_general.hip",
+           "lookup_kernels.hip", "index_ops_kernels.hip", "quantize_kernels.hip", "sequence_kernels.hip",
+           "prune_kernels.hip", "update_kernels.hip", "c_api.cpp"]
+HEADERS = ["lookup_common.h", "lookup_device.h", "lookup_general.h", "lookup_lean.h", os.path.join("..", "..", "include", "fbgemm_amd.h")]
 
 # -ffp-contract=off: the kernels spell out every fma; nothing else may be fused,
 #   or the fp32 rounding sequence would differ from the reference's.
@@ -54,7 +58,7 @@ def build_library(verbose=False, force=True):
     if verbose:
         for j in jobs:
             print(" ".join(j), flush=True)
-    with ThreadPoolExecutor(max_workers=4) as pool:
+    with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 4)) as pool:
         outs = list(pool.map(_hipcc, jobs))
     objs = [os.path.join(objdir, os.path.splitext(s)[0] + ".o") for s in SOURCES]
     outs.append(_hipcc(["hipcc", "--offload-arch=gfx950", "-fPIC", "-shared", "-o", OUT, *objs]))

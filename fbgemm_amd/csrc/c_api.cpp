@@ -16,6 +16,7 @@
 
 namespace fbgemm_amd {
 hipError_t launch_lookup(const LookupArgs& a, bool idx64, hipStream_t stream);
+hipError_t launch_lookup_lean(const LookupArgs& a, bool idx64, bool exact, hipStream_t stream);
 hipError_t launch_lengths_to_offsets(const void* lengths, bool is64, int64_t n, int64_t* offsets, hipStream_t stream);
 hipError_t launch_status_clear(Status* st, hipStream_t stream);
 hipError_t launch_bag_order(const void* offsets, bool off64, int32_t B, int32_t T, BagEntry* order, hipStream_t stream);
@@ -231,6 +232,33 @@ double row_cost(const TableDesc& d) {
   return lines + 0.35;
 }
 
+// Launches of fewer waves than this take 4-byte lanes (see plan_lanes). Read once; tests set it.
+int g_narrow_override = -1;
+int narrow_below_waves() {
+  static int v = env_int("FBGEMM_AMD_NARROW_BELOW_WAVES", 1024);
+  return g_narrow_override >= 0 ? g_narrow_override : v;
+}
+
+// 1: shapes the lean kernel takes go to it (0: everything through the general kernel, for A/B runs and tests).
+int lean_default() {
+  static int v = env_int("FBGEMM_AMD_LEAN", 1);
+  return v;
+}
+int g_lean_override = -1; // tests: fbgemm_amd_set_lean
+
+bool lean_enabled() { return g_lean_override >= 0 ? g_lean_override != 0 : lean_default() != 0; }
+
+// What lookup_lean.h pools: 4-bit / 8-bit / fp16 rows read as 16-byte chunks at 4-byte
+// alignment in one pass, every lane owning 32 columns (1 / 2 / 4 chunks), rows numbered in 31 bits.
+bool lean_shape(const TableDesc& d) {
+  const int want_c = d.ty == ST_INT4 ? 1 : d.ty == ST_INT8 ? 2 : d.ty == ST_FP16 ? 4 : 0;
+  if (!want_c || d.vb != 16 || d.passes != 1 || d.chunks != want_c) return false;
+  if (d.lanes < 2 || d.lanes > 64) return false;
+  if (d.num_rows > (1LL << 31) || d.row_stride <= 0 || d.row_stride > 0xffffffffLL) return false;
+  if (!d.inline_hdr && (int64_t)d.lanes * d.chunks * 16 != d.data_bytes) return false;
+  return true;
+}
+
 struct DeviceScratch {
   Status* status = nullptr;
   int64_t* offsets = nullptr; // lengths -> offsets
@@ -292,6 +320,8 @@ int check_cfg(const fbgemm_amd_spmdm_config* c) {
   if ((c->index_bits != 32 && c->index_bits != 64) || (c->offset_bits != 32 && c->offset_bits != 64))
     return fail(FBGEMM_AMD_E_ARG, "index_bits/offset_bits must be 32 or 64");
   if (c->block_size <= 0 || c->block_size > (1 << 24)) return fail(FBGEMM_AMD_E_ARG, "bad block_size");
+  if (c->accumulate != FBGEMM_AMD_ACC_EXACT && c->accumulate != FBGEMM_AMD_ACC_FAST)
+    return fail(FBGEMM_AMD_E_ARG, "accumulate must be FBGEMM_AMD_ACC_EXACT or FBGEMM_AMD_ACC_FAST");
   return 0;
 }
 
@@ -480,9 +510,8 @@ int spmdm_launch_impl(
   plan_lanes(d, (uintptr_t)d_input, out_stride, has_sb, false);
   {
     // a launch of fewer than four waves per compute unit: prefer narrow lanes
-    const int narrow_below = env_int("FBGEMM_AMD_NARROW_BELOW_WAVES", 1024); // read per call: tests switch it
     const int G16 = bags_per_wave(d.lanes, d.packed);
-    if (d.vb == 16 && (output_size + G16 - 1) / G16 < narrow_below) plan_lanes(d, (uintptr_t)d_input, out_stride, has_sb, false, true);
+    if (d.vb == 16 && (output_size + G16 - 1) / G16 < narrow_below_waves()) plan_lanes(d, (uintptr_t)d_input, out_stride, has_sb, false, true);
   }
   d.lanes_recip = (65536 + d.lanes - 1) / d.lanes;
 
@@ -494,7 +523,7 @@ int spmdm_launch_impl(
   a.remap = d_remap;
   a.remap_rows = data_size;
   if (d_remap) {
-    d.num_rows = INT64_MAX; // the reference does not bound the physical id (RefImplementations.cc:1789-1791)
+    d.num_rows = 1LL << 31; // the reference does not bound the physical id (RefImplementations.cc:1789-1791); the mapping's int32 entries do
     d.skip_minus_one = 0;
   }
   a.out = d_out;
@@ -553,13 +582,26 @@ int spmdm_launch_impl(
       a.order = s->order;
     }
   }
-  HIP_TRY(launch_lookup(a, cfg->index_bits == 64, stream));
+  if (lean_enabled() && !cfg->is_weight_positional && lean_shape(d))
+    HIP_TRY(launch_lookup_lean(a, cfg->index_bits == 64, cfg->accumulate != FBGEMM_AMD_ACC_FAST, stream));
+  else
+    HIP_TRY(launch_lookup(a, cfg->index_bits == 64, stream));
   return 0;
 }
 
 } // namespace
 
 extern "C" {
+
+int fbgemm_amd_set_narrow_below_waves(int32_t waves) {
+  g_narrow_override = waves < 0 ? -1 : waves;
+  return 0;
+}
+
+int fbgemm_amd_set_lean(int32_t on) {
+  g_lean_override = on < 0 ? -1 : (on != 0);
+  return 0;
+}
 
 int fbgemm_amd_spmdm_launch(
     const fbgemm_amd_spmdm_config* cfg, int64_t output_size, int64_t index_size,
@@ -624,14 +666,43 @@ struct fbgemm_amd_tbe_plan {
   std::vector<TableDesc> tables_narrow;
   TableDesc* d_tables_narrow = nullptr;
   int device = 0;
-  // per-B work lists
-  struct Work {
+  // what a forward needs beyond the tables, cached per (B, lane-shape set): the work lists of
+  // the two kernels (tables the lean kernel takes, and the rest) and the bag order the scheduler
+  // kernel rewrites on every forward. The bag order is scratch, so every stream that runs
+  // forwards of the plan gets a buffer of its own (ORDER_SLOTS of them; one is allocated ahead
+  // so that a stream met first under capture, where nothing may be allocated, finds one).
+  static constexpr int ORDER_SLOTS = 4;
+  struct WorkList {
     WaveWork* d_work = nullptr;
-    BagEntry* d_order = nullptr; // T*B bags, rewritten by every forward
     int64_t* d_xcd_start = nullptr;
     int64_t num_waves = 0;
   };
-  std::map<std::pair<int32_t, int>, Work> work; // per (B, lane-shape set)
+  struct Work {
+    WorkList lean, general;
+    BagEntry* d_order[ORDER_SLOTS] = {nullptr, nullptr, nullptr, nullptr}; // T*B bags each, rewritten by every forward
+    hipStream_t order_stream[ORDER_SLOTS] = {nullptr, nullptr, nullptr, nullptr};
+    bool order_claimed[ORDER_SLOTS] = {false, false, false, false};
+    bool pinned = false;         // used by a forward under stream capture: a graph may hold its pointers
+    uint64_t last_use = 0;
+  };
+  struct WorkKey {
+    int32_t B;
+    int variant;
+    int lean;
+    bool operator<(const WorkKey& o) const {
+      if (B != o.B) return B < o.B;
+      if (variant != o.variant) return variant < o.variant;
+      return lean < o.lean;
+    }
+  };
+  std::map<WorkKey, Work> work;
+  uint64_t use_clock = 0;
+  int32_t accumulate = FBGEMM_AMD_ACC_EXACT;
+  // lane-shape choice of the last forward, per (B, indices_numel >> 16)
+  int32_t shape_B = -1;
+  int64_t shape_bucket = -1;
+  int shape_variant = 0;
+  int shape_narrow = -1;
   std::mutex mu;
   // optional timing of the lookup kernel alone: a ring of (start, stop) event pairs
   int32_t fp8_shift = 0; // FP8 rows: set by fbgemm_amd_tbe_plan_set_fp8
@@ -640,6 +711,119 @@ struct fbgemm_amd_tbe_plan {
   std::vector<hipEvent_t> prof_ev;
   int64_t prof_count = 0;
 };
+
+namespace {
+
+void free_work(fbgemm_amd_tbe_plan::Work& w) {
+  for (fbgemm_amd_tbe_plan::WorkList* l : {&w.lean, &w.general}) {
+    if (l->d_work) (void)hipFree(l->d_work);
+    if (l->d_xcd_start) (void)hipFree(l->d_xcd_start);
+    *l = fbgemm_amd_tbe_plan::WorkList();
+  }
+  for (int k = 0; k < fbgemm_amd_tbe_plan::ORDER_SLOTS; ++k) {
+    if (w.d_order[k]) (void)hipFree(w.d_order[k]);
+    w.d_order[k] = nullptr;
+    w.order_claimed[k] = false;
+  }
+}
+
+// The per-wave work list of one kernel over the tables `members` (indices into `tables`).
+// The list is 8 runs, one per XCD (see lookup_kernel). Tables are cut into slices of waves,
+// the slices are dealt to the XCDs so that every XCD gets the same number of 128-byte line
+// requests (what the memory system charges for), and inside a run every slice advances
+// through its bag order (longest first) at the same relative pace, so that tables of
+// different row types share the CUs at all times.
+int build_work_list(const std::vector<TableDesc>& tables, const std::vector<int>& members, int32_t B,
+                    fbgemm_amd_tbe_plan::WorkList* out) {
+  *out = fbgemm_amd_tbe_plan::WorkList();
+  if (members.empty()) return 0;
+  static const int xcd_lists = env_int("FBGEMM_AMD_XCD_LISTS", 1);
+  static const int interleave = env_int("FBGEMM_AMD_INTERLEAVE", 1);
+  static const int max_parts = env_int("FBGEMM_AMD_MAX_PARTS", 8);
+  static const int by_shape = env_int("FBGEMM_AMD_GROUP_BY_SHAPE", 1);
+  struct Slice { int t, first, step, count; double cost; };
+  std::vector<Slice> slices;
+  double total_cost = 0;
+  const int T = (int)tables.size();
+  std::vector<double> wave_cost(T, 0.0);
+  std::vector<int> nwaves(T, 0);
+  for (int t : members) {
+    const TableDesc& d = tables[t];
+    const int G = bags_per_wave(d.lanes, d.packed);
+    nwaves[t] = (B + G - 1) / G;
+    wave_cost[t] = G * row_cost(d);
+    total_cost += wave_cost[t] * nwaves[t];
+  }
+  const int nx = xcd_lists ? 8 : 1;
+  for (int t : members) {
+    // slices no larger than 1/4 of an XCD's share; slice p takes waves p, p + parts, ...
+    int parts = (int)std::ceil(wave_cost[t] * nwaves[t] / (total_cost / nx / 4.0 + 1e-9));
+    parts = std::max(1, std::min(parts, std::min(nwaves[t], std::min(nx, max_parts))));
+    for (int p = 0; p < parts; ++p) {
+      const int count = (nwaves[t] - p + parts - 1) / parts;
+      slices.push_back(Slice{t, p, parts, count, wave_cost[t] * count});
+    }
+  }
+  std::stable_sort(slices.begin(), slices.end(), [](const Slice& x, const Slice& y) { return x.cost > y.cost; });
+  std::vector<std::vector<Slice>> per_x(nx);
+  std::vector<double> load(nx, 0.0);
+  for (const Slice& sl : slices) {
+    const int x = (int)(std::min_element(load.begin(), load.end()) - load.begin());
+    per_x[x].push_back(sl);
+    load[x] += sl.cost;
+  }
+  std::vector<WaveWork> list;
+  std::vector<int64_t> xcd_start(9, 0);
+  int64_t longest = 0;
+  // Inside a run the slices are walked in groups that hold one slice of every
+  // row shape (type, D) the run has; the slices of a group advance together,
+  // each through its bag order at the same relative pace, and the groups
+  // follow one another. Mixing shapes keeps waves of different cost on the
+  // CUs at all times; taking few tables at a time keeps the working set of
+  // the XCD's L2 small (hot rows of a table are reused while they are there).
+  for (int x = 0; x < nx; ++x) {
+    std::vector<std::pair<double, WaveWork>> keyed;
+    std::map<std::pair<int, int>, std::vector<Slice>> shapes; // slices of a shape, largest first (per_x order)
+    for (const Slice& sl : per_x[x]) {
+      const TableDesc& d = tables[sl.t];
+      shapes[(interleave && by_shape) ? std::make_pair((int)d.ty, (int)d.D) : std::make_pair(0, 0)].push_back(sl);
+    }
+    size_t depth = 0;
+    for (auto& kv : shapes) depth = std::max(depth, kv.second.size());
+    int gidx = 0;
+    for (size_t i = 0; i < depth; ++i) {
+      for (auto& kv : shapes) {
+        if (i >= kv.second.size()) continue;
+        const Slice& sl = kv.second[i];
+        const int G = bags_per_wave(tables[sl.t].lanes, tables[sl.t].packed);
+        // one shape only (or no interleaving asked for): slice after slice
+        const double base = (interleave && by_shape) ? (double)gidx : (interleave ? 0.0 : (double)gidx++);
+        for (int k = 0; k < sl.count; ++k)
+          keyed.push_back({base + (k + 0.5) / sl.count, WaveWork{sl.t, (sl.first + k * sl.step) * G}});
+      }
+      if (interleave && by_shape) ++gidx;
+    }
+    std::stable_sort(keyed.begin(), keyed.end(),
+                     [](const std::pair<double, WaveWork>& p, const std::pair<double, WaveWork>& q) { return p.first < q.first; });
+    for (auto& kv : keyed) list.push_back(kv.second);
+    xcd_start[x + 1] = (int64_t)list.size();
+    longest = std::max<int64_t>(longest, (int64_t)keyed.size());
+  }
+  for (int x = nx; x < 8; ++x) xcd_start[x + 1] = xcd_start[nx];
+  out->num_waves = xcd_lists ? longest : (int64_t)list.size();
+  HIP_TRY(hipMalloc((void**)&out->d_work, sizeof(WaveWork) * list.size()));
+  HIP_TRY(hipMemcpy(out->d_work, list.data(), sizeof(WaveWork) * list.size(), hipMemcpyHostToDevice));
+  if (xcd_lists) {
+    HIP_TRY(hipMalloc((void**)&out->d_xcd_start, sizeof(int64_t) * 9));
+    HIP_TRY(hipMemcpy(out->d_xcd_start, xcd_start.data(), sizeof(int64_t) * 9, hipMemcpyHostToDevice));
+  }
+  return 0;
+}
+
+// Cached work lists beyond this many: the least recently used one that no graph can hold is dropped.
+constexpr size_t MAX_CACHED_WORK = 16;
+
+} // namespace
 
 extern "C" {
 
@@ -731,12 +915,7 @@ int fbgemm_amd_tbe_plan_create(
 void fbgemm_amd_tbe_plan_destroy(fbgemm_amd_tbe_plan* plan) {
   if (!plan) return;
   (void)hipDeviceSynchronize();
-  for (auto& kv : plan->work)
-  {
-    if (kv.second.d_work) (void)hipFree(kv.second.d_work);
-    if (kv.second.d_order) (void)hipFree(kv.second.d_order);
-    if (kv.second.d_xcd_start) (void)hipFree(kv.second.d_xcd_start);
-  }
+  for (auto& kv : plan->work) free_work(kv.second);
   if (plan->d_tables) (void)hipFree(plan->d_tables);
   if (plan->d_tables_packed) (void)hipFree(plan->d_tables_packed);
   if (plan->d_tables_narrow) (void)hipFree(plan->d_tables_narrow);
@@ -837,128 +1016,102 @@ int fbgemm_amd_tbe_forward_pruned(
   static const int packed_mode = env_int("FBGEMM_AMD_PACKED", 1); // 0 never, 1 by bag length, 2 always
   // A forward of fewer than four waves per compute unit is bound by the chain of memory round
   // trips inside a wave: 4-byte lanes spread its bags over four times the waves.
-  const int narrow_below = env_int("FBGEMM_AMD_NARROW_BELOW_WAVES", 1024); // read per call: tests switch it
-  int64_t wide_waves = 0;
-  for (const TableDesc& d : plan->tables) {
-    const int G = bags_per_wave(d.lanes, d.packed);
-    wide_waves += (B + G - 1) / G;
-  }
-  const bool use_narrow = wide_waves < narrow_below;
-  const bool use_packed = !use_narrow && !plan->tables_packed.empty() &&
-      (packed_mode == 2 || (packed_mode == 1 && indices_numel >= 20 * (int64_t)plan->T * B));
-  const std::vector<TableDesc>& tables = use_narrow ? plan->tables_narrow : (use_packed ? plan->tables_packed : plan->tables);
-  const int variant = use_narrow ? 2 : (use_packed ? 1 : 0);
+  const bool lean = lean_enabled();
   fbgemm_amd_tbe_plan::Work w;
+  int variant, order_slot = 0;
   {
     std::lock_guard<std::mutex> lk(plan->mu);
-    auto it = plan->work.find({B, variant});
-    if (it == plan->work.end()) {
-      // The work list is 8 runs, one per XCD (see lookup_kernel). Tables are
-      // cut into slices of waves, the slices are dealt to the XCDs so that
-      // every XCD gets the same number of 128-byte line requests (what the
-      // memory system charges for), and inside a run every slice advances
-      // through its bag order (longest first) at the same relative pace, so
-      // that tables of different row types share the CUs at all times.
-      static const int xcd_lists = env_int("FBGEMM_AMD_XCD_LISTS", 1);
-      static const int interleave = env_int("FBGEMM_AMD_INTERLEAVE", 1);
-      static const int max_parts = env_int("FBGEMM_AMD_MAX_PARTS", 8);
-      struct Slice { int t, first, step, count; double cost; };
-      std::vector<Slice> slices;
-      double total_cost = 0;
-      std::vector<double> wave_cost(plan->T);
-      std::vector<int> nwaves(plan->T);
-      for (int t = 0; t < plan->T; ++t) {
-        const TableDesc& d = tables[t];
+    // the lane shapes depend on B and (through the average bag length) on the number of indices:
+    // remember the choice of the last forward with the same B and about the same indices
+    const int64_t bucket = indices_numel >> 16;
+    if (plan->shape_B == B && plan->shape_bucket == bucket && plan->shape_narrow == narrow_below_waves()) {
+      variant = plan->shape_variant;
+    } else {
+      int64_t wide_waves = 0;
+      for (const TableDesc& d : plan->tables) {
         const int G = bags_per_wave(d.lanes, d.packed);
-        nwaves[t] = (B + G - 1) / G;
-        wave_cost[t] = G * row_cost(d);
-        total_cost += wave_cost[t] * nwaves[t];
+        wide_waves += (B + G - 1) / G;
       }
-      const int nx = xcd_lists ? 8 : 1;
-      for (int t = 0; t < plan->T; ++t) {
-        // slices no larger than 1/4 of an XCD's share; slice p takes waves p, p + parts, ...
-        int parts = (int)std::ceil(wave_cost[t] * nwaves[t] / (total_cost / nx / 4.0 + 1e-9));
-        parts = std::max(1, std::min(parts, std::min(nwaves[t], std::min(nx, max_parts))));
-        for (int p = 0; p < parts; ++p) {
-          const int count = (nwaves[t] - p + parts - 1) / parts;
-          slices.push_back(Slice{t, p, parts, count, wave_cost[t] * count});
-        }
-      }
-      std::stable_sort(slices.begin(), slices.end(), [](const Slice& x, const Slice& y) { return x.cost > y.cost; });
-      std::vector<std::vector<Slice>> per_x(nx);
-      std::vector<double> load(nx, 0.0);
-      for (const Slice& sl : slices) {
-        const int x = (int)(std::min_element(load.begin(), load.end()) - load.begin());
-        per_x[x].push_back(sl);
-        load[x] += sl.cost;
-      }
-      std::vector<WaveWork> list;
-      std::vector<int64_t> xcd_start(9, 0);
-      int64_t longest = 0;
-      // Inside a run the slices are walked in groups that hold one slice of every
-      // row shape (type, D) the run has; the slices of a group advance together,
-      // each through its bag order at the same relative pace, and the groups
-      // follow one another. Mixing shapes keeps waves of different cost on the
-      // CUs at all times; taking few tables at a time keeps the working set of
-      // the XCD's L2 small (hot rows of a table are reused while they are there).
-      static const int by_shape = env_int("FBGEMM_AMD_GROUP_BY_SHAPE", 1);
-      for (int x = 0; x < nx; ++x) {
-        std::vector<std::pair<double, WaveWork>> keyed;
-        std::map<std::pair<int, int>, std::vector<Slice>> shapes; // slices of a shape, largest first (per_x order)
-        for (const Slice& sl : per_x[x]) {
-          const TableDesc& d = tables[sl.t];
-          shapes[(interleave && by_shape) ? std::make_pair((int)d.ty, (int)d.D) : std::make_pair(0, 0)].push_back(sl);
-        }
-        size_t depth = 0;
-        for (auto& kv : shapes) depth = std::max(depth, kv.second.size());
-        int gidx = 0;
-        for (size_t i = 0; i < depth; ++i) {
-          for (auto& kv : shapes) {
-            if (i >= kv.second.size()) continue;
-            const Slice& sl = kv.second[i];
-            const int G = bags_per_wave(tables[sl.t].lanes, tables[sl.t].packed);
-            // one shape only (or no interleaving asked for): slice after slice
-            const double base = (interleave && by_shape) ? (double)gidx : (interleave ? 0.0 : (double)gidx++);
-            for (int k = 0; k < sl.count; ++k)
-              keyed.push_back({base + (k + 0.5) / sl.count, WaveWork{sl.t, (sl.first + k * sl.step) * G}});
-          }
-          if (interleave && by_shape) ++gidx;
-        }
-        std::stable_sort(keyed.begin(), keyed.end(),
-                         [](const std::pair<double, WaveWork>& p, const std::pair<double, WaveWork>& q) { return p.first < q.first; });
-        for (auto& kv : keyed) list.push_back(kv.second);
-        xcd_start[x + 1] = (int64_t)list.size();
-        longest = std::max<int64_t>(longest, (int64_t)keyed.size());
-      }
-      for (int x = nx; x < 8; ++x) xcd_start[x + 1] = xcd_start[nx];
-      fbgemm_amd_tbe_plan::Work nw;
-      nw.num_waves = xcd_lists ? longest : (int64_t)list.size();
-      HIP_TRY(hipMalloc((void**)&nw.d_work, sizeof(WaveWork) * list.size()));
-      HIP_TRY(hipMemcpy(nw.d_work, list.data(), sizeof(WaveWork) * list.size(), hipMemcpyHostToDevice));
-      if (xcd_lists) {
-        HIP_TRY(hipMalloc((void**)&nw.d_xcd_start, sizeof(int64_t) * 9));
-        HIP_TRY(hipMemcpy(nw.d_xcd_start, xcd_start.data(), sizeof(int64_t) * 9, hipMemcpyHostToDevice));
-      }
-      HIP_TRY(hipMalloc((void**)&nw.d_order, sizeof(BagEntry) * (size_t)plan->T * (size_t)B));
-      // A caller whose batch size keeps changing would grow this cache without bound: past 16
-      // batch sizes, wait for the launches that may still read the old lists and drop them all.
-      if (plan->work.size() >= 16) {
-        HIP_TRY(hipDeviceSynchronize());
-        for (auto& kv : plan->work) {
-          if (kv.second.d_work) (void)hipFree(kv.second.d_work);
-          if (kv.second.d_order) (void)hipFree(kv.second.d_order);
-          if (kv.second.d_xcd_start) (void)hipFree(kv.second.d_xcd_start);
-        }
-        plan->work.clear();
-      }
-      it = plan->work.emplace(std::make_pair(B, variant), nw).first;
+      const bool use_narrow = wide_waves < narrow_below_waves();
+      const bool use_packed = !use_narrow && !plan->tables_packed.empty() &&
+          (packed_mode == 2 || (packed_mode == 1 && indices_numel >= 20 * (int64_t)plan->T * B));
+      variant = use_narrow ? 2 : (use_packed ? 1 : 0);
+      plan->shape_B = B;
+      plan->shape_bucket = bucket;
+      plan->shape_variant = variant;
+      plan->shape_narrow = narrow_below_waves();
     }
-    w = it->second;
+    const std::vector<TableDesc>& tables = variant == 2 ? plan->tables_narrow : (variant == 1 ? plan->tables_packed : plan->tables);
+    const fbgemm_amd_tbe_plan::WorkKey key{B, variant, lean ? 1 : 0};
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    (void)hipStreamIsCapturing(stream, &cap);
+    const bool capturing = cap != hipStreamCaptureStatusNone;
+    auto it = plan->work.find(key);
+    if (it == plan->work.end()) {
+      if (capturing)
+        return fail(FBGEMM_AMD_E_ARG, "the first forward of a plan with a new batch size allocates its work lists: "
+                    "run it once outside the stream capture");
+      std::vector<int> lean_members, general_members;
+      for (int t = 0; t < plan->T; ++t) (lean && lean_shape(tables[t]) ? lean_members : general_members).push_back(t);
+      fbgemm_amd_tbe_plan::Work nw;
+      if (int rc = build_work_list(tables, lean_members, B, &nw.lean)) return rc;
+      if (int rc = build_work_list(tables, general_members, B, &nw.general)) return rc;
+      // the bag order: one buffer for this stream, one ahead for the next stream
+      for (int k = 0; k < 2; ++k) HIP_TRY(hipMalloc((void**)&nw.d_order[k], sizeof(BagEntry) * (size_t)plan->T * (size_t)B));
+      nw.order_stream[0] = stream;
+      nw.order_claimed[0] = true;
+      // A caller whose batch size keeps changing would grow this cache without bound. Past
+      // MAX_CACHED_WORK entries the least recently used one goes, after the launches that may
+      // still read it are done. Entries a forward under stream capture has used are never
+      // dropped here: a captured graph holds their device pointers (fbgemm_amd_tbe_plan_trim
+      // drops those too, and says what that means for graphs).
+      if (plan->work.size() >= MAX_CACHED_WORK) {
+        auto victim = plan->work.end();
+        for (auto jt = plan->work.begin(); jt != plan->work.end(); ++jt)
+          if (!jt->second.pinned && (victim == plan->work.end() || jt->second.last_use < victim->second.last_use)) victim = jt;
+        if (victim != plan->work.end()) {
+          HIP_TRY(hipDeviceSynchronize());
+          free_work(victim->second);
+          plan->work.erase(victim);
+        }
+      }
+      it = plan->work.emplace(key, nw).first;
+    }
+    it->second.pinned = it->second.pinned || capturing;
+    it->second.last_use = ++plan->use_clock;
+    // this stream's bag-order buffer: the one it has, else one nobody has claimed, else (outside
+    // a capture) a new one; with all of that exhausted the first buffer is shared, and forwards
+    // of this plan on the streams that share it must not overlap
+    fbgemm_amd_tbe_plan::Work& W = it->second;
+    constexpr int NS = fbgemm_amd_tbe_plan::ORDER_SLOTS;
+    order_slot = -1;
+    for (int k = 0; k < NS && order_slot < 0; ++k)
+      if (W.order_claimed[k] && W.order_stream[k] == stream) order_slot = k;
+    for (int k = 0; k < NS && order_slot < 0; ++k)
+      if (!W.order_claimed[k] && W.d_order[k]) order_slot = k;
+    for (int k = 0; k < NS && order_slot < 0 && !capturing; ++k)
+      if (!W.d_order[k]) {
+        HIP_TRY(hipMalloc((void**)&W.d_order[k], sizeof(BagEntry) * (size_t)plan->T * (size_t)B));
+        order_slot = k;
+      }
+    if (order_slot < 0) order_slot = 0;
+    if (!W.order_claimed[order_slot]) {
+      W.order_claimed[order_slot] = true;
+      W.order_stream[order_slot] = stream;
+      // keep one buffer ahead for the next stream, when that is possible now
+      if (!capturing)
+        for (int k = 0; k < NS; ++k)
+          if (!W.d_order[k]) {
+            HIP_TRY(hipMalloc((void**)&W.d_order[k], sizeof(BagEntry) * (size_t)plan->T * (size_t)B));
+            break;
+          }
+    }
+    w = W;
   }
 
   LookupArgs a;
   memset(&a, 0, sizeof(a));
-  a.tables = use_narrow ? plan->d_tables_narrow : (use_packed ? plan->d_tables_packed : plan->d_tables);
+  a.tables = variant == 2 ? plan->d_tables_narrow : (variant == 1 ? plan->d_tables_packed : plan->d_tables);
   a.weights[0] = (const uint8_t*)d_dev_weights;
   a.weights[1] = (const uint8_t*)d_uvm_weights;
   a.indices = d_indices;
@@ -971,9 +1124,6 @@ int fbgemm_amd_tbe_forward_pruned(
   a.out = d_output;
   a.out_stride = plan->total_D;
   a.index_size = indices_numel;
-  a.work = w.d_work;
-  a.xcd_start = w.d_xcd_start;
-  a.num_waves = w.num_waves;
   a.B = B;
   a.T = plan->T;
   a.out_ty = output_ty;
@@ -984,41 +1134,51 @@ int fbgemm_amd_tbe_forward_pruned(
   a.fp8_shift = plan->fp8_shift;
   a.fp8_mult = plan->fp8_mult;
   if (sort_bags_default() && indices_numel >= (int64_t)SORT_MIN_LOOKUPS) {
-    HIP_TRY(launch_bag_order(d_offsets, index_bits == 64, B, plan->T, w.d_order, stream));
-    a.order = w.d_order;
+    HIP_TRY(launch_bag_order(d_offsets, index_bits == 64, B, plan->T, w.d_order[order_slot], stream));
+    a.order = w.d_order[order_slot];
   }
-#ifdef FBGEMM_AMD_WAVE_TRACE
-  static unsigned long long* trace_buf = nullptr;
-  static size_t trace_cap = 0;
-  const size_t trace_words = (size_t)(w.d_xcd_start ? 8 * w.num_waves : w.num_waves) * 4; // >= items
-  if (trace_cap < trace_words) {
-    if (trace_buf) (void)hipFree(trace_buf);
-    HIP_TRY(hipMalloc((void**)&trace_buf, trace_words * 8));
-    trace_cap = trace_words;
-  }
-  HIP_TRY(hipMemsetAsync(trace_buf, 0, trace_words * 8, stream));
-  a.trace = trace_buf;
-#endif
   const size_t slots = plan->prof_ev.size() / 2;
   const size_t slot = slots ? (size_t)(plan->prof_count % (int64_t)slots) : 0;
   if (slots) HIP_TRY(hipEventRecord(plan->prof_ev[2 * slot], stream));
-  HIP_TRY(launch_lookup(a, index_bits == 64, stream));
+  if (w.lean.num_waves > 0) {
+    a.work = w.lean.d_work;
+    a.xcd_start = w.lean.d_xcd_start;
+    a.num_waves = w.lean.num_waves;
+    HIP_TRY(launch_lookup_lean(a, index_bits == 64, plan->accumulate != FBGEMM_AMD_ACC_FAST, stream));
+  }
+  if (w.general.num_waves > 0) {
+    a.work = w.general.d_work;
+    a.xcd_start = w.general.d_xcd_start;
+    a.num_waves = w.general.num_waves;
+    HIP_TRY(launch_lookup(a, index_bits == 64, stream));
+  }
   if (slots) {
     HIP_TRY(hipEventRecord(plan->prof_ev[2 * slot + 1], stream));
     ++plan->prof_count;
   }
-#ifdef FBGEMM_AMD_WAVE_TRACE
-  if (const char* path = getenv("FBGEMM_AMD_TRACE_FILE")) {
-    std::vector<unsigned long long> h(trace_words);
-    HIP_TRY(hipStreamSynchronize(stream));
-    HIP_TRY(hipMemcpy(h.data(), trace_buf, trace_words * 8, hipMemcpyDeviceToHost));
-    if (FILE* f = fopen(path, "wb")) {
-      fwrite(h.data(), 8, h.size(), f);
-      fclose(f);
-    }
-  }
-#endif
   return 0;
+}
+
+int fbgemm_amd_tbe_plan_set_accumulate(fbgemm_amd_tbe_plan* plan, int32_t mode) {
+  if (!plan) return fail(FBGEMM_AMD_E_ARG, "plan is null");
+  if (mode != FBGEMM_AMD_ACC_EXACT && mode != FBGEMM_AMD_ACC_FAST)
+    return fail(FBGEMM_AMD_E_ARG, "accumulate must be FBGEMM_AMD_ACC_EXACT or FBGEMM_AMD_ACC_FAST");
+  std::lock_guard<std::mutex> lk(plan->mu);
+  plan->accumulate = mode;
+  return 0;
+}
+
+int fbgemm_amd_tbe_plan_trim(fbgemm_amd_tbe_plan* plan) {
+  if (!plan) return fail(FBGEMM_AMD_E_ARG, "plan is null");
+  std::lock_guard<std::mutex> lk(plan->mu);
+  HIP_TRY(hipDeviceSynchronize());
+  for (auto& kv : plan->work) free_work(kv.second);
+  plan->work.clear();
+  return 0;
+}
+
+int64_t fbgemm_amd_tbe_plan_cached_work(const fbgemm_amd_tbe_plan* plan) {
+  return plan ? (int64_t)plan->work.size() : -1;
 }
 
 int fbgemm_amd_tbe_forward_nobag(

@@ -1,0 +1,579 @@
+// The lean pooled-lookup kernel: the shapes that carry the traffic.
+//
+// Rows of 4-bit, 8-bit or fp16 elements whose data is a whole number of
+// 16-byte chunks at 4-byte alignment, every lane owning 32 output columns of
+// its bag (1, 2 or 4 chunks). Everything else (odd widths, unaligned tables,
+// column passes, positional weights, 2-bit / fp32 / bf16 / fp8 rows) stays with
+// the general kernel of lookup_general.h; the host decides per table
+// (lean_shape in c_api.cpp).
+//
+// Same lane mapping and the same two row layouts as the general kernel: `lanes`
+// consecutive lanes share a bag; either every lane loads data chunks and a
+// staging lane fetches the row's (scale, bias) pair, or (inline_hdr) the lanes
+// own 16-byte chunks of the whole row and the header rides in chunk 0. What is
+// different:
+//  * entries are staged 8 per bag at a time whatever the round size, so a line
+//    of indices or per-sample weights is asked for at most twice instead of
+//    once per round of 2 or 4 rows;
+//  * a block in which every bag of the wave has all 8 rows (the normal case
+//    once bags are ordered by length) runs as straight-line code of its own;
+//    blocks with holes take a second, predicated copy of the code, so neither
+//    pays for the other;
+//  * EXACT selects the arithmetic: true is the reference's sequence of
+//    roundings, acc = fma(scale, q, acc + bias) per element
+//    (src/RefImplementations.cc:1326-1333,1519-1527), bit-identical to the CPU
+//    path; false adds the biases of a bag apart, acc = fma(scale, q, acc) and
+//    one bsum += bias per row and lane, out = acc + bsum: a third fewer vector
+//    instructions per 4-bit element, results within a few fp32 roundings of the
+//    reference's (tolerance grade, selected per plan).
+//  * a wave that meets a scale too large for the pre-scaled arithmetic (scale *
+//    2^24 times a half-precision denormal) starts over in pool_lean_slow, a plain
+//    row-at-a-time loop that converts integers to float before the fma. Both
+//    round identically; the slow one only has to be correct.
+//  * what is staged per entry is the row number (32 bits), not its byte offset.
+#pragma once
+#include "lookup_device.h"
+
+namespace fbgemm_amd {
+
+constexpr int LEAN_BLOCK = 8;   // entries of every bag staged at a time
+
+struct __attribute__((aligned(16))) LeanMul {
+  float s24;  // w * scale * 2^24 (4- and 8-bit rows, pre-scaled route); w * scale (plain route); w (fp16 rows)
+  float s20;  // w * scale * 2^20 (4-bit rows, pre-scaled route)
+  float bias; // w * bias
+  float pad;
+};
+
+// ---- per-chunk arithmetic -------------------------------------------------------
+//
+// 16 bytes of a row in raw[4]. PLAIN = false: the pre-scaled route, masks leave
+// small integers in the halves of a register as half-precision denormals
+// (q * 2^-24, or q * 2^-20 for the odd nibbles), which the fma widens exactly;
+// m.s24 / m.s20 carry the matching powers of two. PLAIN = true: the same masks,
+// then one exact multiply turns the denormal into the integer as a float and
+// the fma takes the unscaled m.s24 (= w * scale): for scales whose product with
+// 2^24 would overflow. Both round like fma(scale, float(q), ...).
+
+template <bool EXACT, bool PLAIN>
+__device__ __forceinline__ float lean_fma(float s, float qd, float acc, float bias, float up) {
+  const float q = PLAIN ? qd * up : qd; // exact: a small integer times a power of two
+  return EXACT ? __builtin_fmaf(s, q, acc + bias) : __builtin_fmaf(s, q, acc);
+}
+
+template <int TY, bool EXACT, bool PLAIN>
+__device__ __forceinline__ void lean_chunk(float (&acc)[32], int base, const uint32_t (&raw)[4], const LeanMul& m) {
+  if constexpr (TY == ST_INT4) {
+    const float sa = m.s24, sb = PLAIN ? m.s24 : m.s20;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const uint32_t x = raw[w];
+      const uint32_t y = x >> 8;
+      const uint32_t a0 = x & 0x000f000fu; // nibbles 0, 4
+      const uint32_t a1 = x & 0x00f000f0u; // nibbles 1, 5 (times 16)
+      const uint32_t a2 = y & 0x000f000fu; // nibbles 2, 6
+      const uint32_t a3 = y & 0x00f000f0u; // nibbles 3, 7 (times 16)
+      float* c = acc + base + 8 * w;
+      c[0] = lean_fma<EXACT, PLAIN>(sa, half_lo(a0), c[0], m.bias, 0x1p24f);
+      c[1] = lean_fma<EXACT, PLAIN>(sb, half_lo(a1), c[1], m.bias, 0x1p20f);
+      c[2] = lean_fma<EXACT, PLAIN>(sa, half_lo(a2), c[2], m.bias, 0x1p24f);
+      c[3] = lean_fma<EXACT, PLAIN>(sb, half_lo(a3), c[3], m.bias, 0x1p20f);
+      c[4] = lean_fma<EXACT, PLAIN>(sa, half_hi(a0), c[4], m.bias, 0x1p24f);
+      c[5] = lean_fma<EXACT, PLAIN>(sb, half_hi(a1), c[5], m.bias, 0x1p20f);
+      c[6] = lean_fma<EXACT, PLAIN>(sa, half_hi(a2), c[6], m.bias, 0x1p24f);
+      c[7] = lean_fma<EXACT, PLAIN>(sb, half_hi(a3), c[7], m.bias, 0x1p20f);
+    }
+  } else if constexpr (TY == ST_INT8) {
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const uint32_t lo = __builtin_amdgcn_perm(0u, raw[w], 0x0c010c00u); // bytes 0, 1
+      const uint32_t hi = __builtin_amdgcn_perm(0u, raw[w], 0x0c030c02u); // bytes 2, 3
+      float* c = acc + base + 4 * w;
+      c[0] = lean_fma<EXACT, PLAIN>(m.s24, half_lo(lo), c[0], m.bias, 0x1p24f);
+      c[1] = lean_fma<EXACT, PLAIN>(m.s24, half_hi(lo), c[1], m.bias, 0x1p24f);
+      c[2] = lean_fma<EXACT, PLAIN>(m.s24, half_lo(hi), c[2], m.bias, 0x1p24f);
+      c[3] = lean_fma<EXACT, PLAIN>(m.s24, half_hi(hi), c[3], m.bias, 0x1p24f);
+    }
+  } else { // fp16: acc = fma(w, x, acc), the reference's own sequence in either mode
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      float* c = acc + base + 2 * w;
+      c[0] = __builtin_fmaf(m.s24, half_lo(raw[w]), c[0]);
+      c[1] = __builtin_fmaf(m.s24, half_hi(raw[w]), c[1]);
+    }
+  }
+}
+
+// What a lane knows about its bag before the first row.
+struct LeanLane {
+  int grp, sub;   // bag slot inside the wave, chunk position inside the bag's lanes
+  int lgrp;       // the bag slot whose staging area the lane reads (lanes left over shadow the last one)
+  bool bag_ok;    // the lane pools a bag
+  int bag;        // the bag's number inside its table
+  int n;          // entries of the bag
+  int64_t pos0;   // position of its first entry in the index array
+  int64_t remap_base, remap_cap; // pruned table: its slice of the remap array
+  bool remapped;
+};
+
+template <typename index_t>
+__device__ __forceinline__ LeanLane lean_lane(const LookupArgs& a, const TableDesc& d, int table, int first_slot, int lane) {
+  LeanLane L;
+  const int S = d.lanes;
+  const int G = bags_per_wave(S, d.packed);
+  bool idle;
+  const uint32_t recip = (uint32_t)d.lanes_recip; // divisions by S, exact for arguments up to 64
+  if (S <= 16 && !d.packed) {
+    // quarter q of the wave holds bags q * (16 / S) ...; its last 16 % S lanes are left over
+    const int per_q = (int)((16u * recip) >> 16);
+    const int j = lane & 15;
+    const int gq = (int)(((uint32_t)j * recip) >> 16);
+    idle = gq >= per_q;
+    L.grp = (lane >> 4) * per_q + (idle ? per_q - 1 : gq);
+    L.sub = j - gq * S;
+  } else {
+    L.grp = (int)(((uint32_t)lane * recip) >> 16);
+    L.sub = lane - L.grp * S;
+    idle = L.grp >= G;
+  }
+  const int slot = first_slot + L.grp;
+  L.lgrp = idle ? G - 1 : L.grp;
+  L.bag_ok = !idle && slot < a.B;
+  const bool reporter = L.sub == 0;
+  L.bag = slot;
+  L.pos0 = 0;
+  int64_t len = 0;
+  if (L.bag_ok) {
+    const int64_t ob = (int64_t)table * a.B;
+    int64_t o0, o1;
+    if (a.order) {
+      const BagEntry be = a.order[ob + slot];
+      L.bag = be.bag;
+      o0 = be.o0;
+      o1 = be.o1;
+    } else {
+      o0 = read_offset(a.offsets, a.off64, ob + slot);
+      o1 = read_offset(a.offsets, a.off64, ob + slot + 1);
+    }
+    int64_t base = 0;
+    if (a.check_total) base = read_offset(a.offsets, a.off64, ob);
+    L.pos0 = o0 - base; // table-batched calls index the shared array: base = 0
+    len = o1 - o0;
+    if (len < 0) {
+      if (reporter) report(a.status, ERR_NEGATIVE_LENGTH);
+      len = 0;
+    }
+    if (len > 0x7fffffffLL || L.pos0 < 0 || L.pos0 + len > a.index_size) {
+      if (reporter) report(a.status, ERR_BAG_OVERRUN);
+      len = 0;
+    }
+    if (a.check_total && L.bag == a.B - 1 && o1 - base != a.index_size && reporter) report(a.status, ERR_LENGTH_MISMATCH);
+  }
+  L.n = (int)len;
+  L.remap_base = 0;
+  L.remap_cap = 0;
+  L.remapped = false;
+  if (a.remap) {
+    L.remapped = true;
+    L.remap_cap = a.remap_rows;
+    if (a.remap_offsets) {
+      L.remap_base = a.remap_offsets[table];
+      L.remap_cap = a.remap_offsets[table + 1] - L.remap_base;
+      L.remapped = L.remap_cap > 0;
+    }
+  }
+  return L;
+}
+
+constexpr int LEAN_NO_ENTRY = INT32_MIN;  // the bag has no such entry
+constexpr int LEAN_SKIP = -1;             // an entry that adds nothing (a pruned or rejected row)
+
+// index -> row number, LEAN_SKIP for what the reference skips, reporting what it rejects.
+// `mapped` is the remap entry already fetched for a pruned table.
+__device__ __forceinline__ int lean_row(const LookupArgs& a, const TableDesc& d, const LeanLane& L, int64_t row, int64_t pos) {
+  if (!L.remapped && d.skip_minus_one && row == -1) return LEAN_SKIP;
+  if (row < 0 || row >= d.num_rows) {
+    report_index(a.status, pos);
+    return LEAN_SKIP;
+  }
+  return (int)row;
+}
+constexpr int64_t LEAN_PRUNED = INT64_MIN; // what lean_remap returns for an entry that adds nothing
+__device__ __forceinline__ int64_t lean_remap(const LookupArgs& a, const LeanLane& L, int64_t logical, int64_t pos) {
+  if (logical < 0 || logical >= L.remap_cap) {
+    report_index(a.status, pos);
+    return LEAN_PRUNED;
+  }
+  const int64_t m = a.remap64 ? reinterpret_cast<const int64_t*>(a.remap)[L.remap_base + logical]
+                              : (int64_t) reinterpret_cast<const int32_t*>(a.remap)[L.remap_base + logical];
+  return m == -1 ? LEAN_PRUNED : m;
+}
+
+template <bool EXACT, int TY, int C, bool INHDR>
+__device__ __forceinline__ void lean_write(const LookupArgs& a, const TableDesc& d, const LeanLane& L, float (&acc)[32], float bsum) {
+  constexpr bool QUANT = TY == ST_INT8 || TY == ST_INT4;
+  constexpr int E = TY == ST_INT4 ? 32 : (TY == ST_INT8 ? 16 : 8);
+  const bool vec_ok = a.out_aligned && ((d.vec_store >> (a.out_ty == ST_FP32 ? 0 : 1)) & 1);
+  if constexpr (!EXACT && QUANT) {
+#pragma unroll
+    for (int e = 0; e < 32; ++e) acc[e] += bsum;
+  }
+  if (a.normalize && L.n > 0) {
+    const float inv_len = 1.0f / (float)L.n; // the reference keeps the bag length in an int when it forms 1/len
+#pragma unroll
+    for (int e = 0; e < 32; ++e) acc[e] *= inv_len;
+  }
+  const int nchunks = INHDR ? (d.data_bytes + 4 + 15) / 16 : d.lanes * C;
+#pragma unroll
+  for (int c = 0; c < C; ++c) {
+    const int k = L.sub + c * d.lanes;
+    if (L.bag_ok && k < nchunks) {
+      float part[E];
+#pragma unroll
+      for (int e = 0; e < E; ++e) part[e] = acc[c * E + e];
+      if constexpr (INHDR) {
+        write_out_runs<E>(a, part, (int64_t)L.bag * a.out_stride + d.out_col, k * E - E / 4, d.D, vec_ok);
+      } else {
+        const int col0 = k * E;
+        write_out<E>(a, part, (int64_t)L.bag * a.out_stride + d.out_col + col0, col0, d.D, vec_ok);
+      }
+    }
+  }
+}
+
+// One wave pools bags_per_wave(lanes, packed) bags of one table.
+// C: 16-byte chunks per lane and row (32 columns per lane: 1 for 4-bit, 2 for
+// 8-bit, 4 for fp16 rows). INHDR as in the general kernel. R: entries a staging
+// lane handles per block (8 / the staging lanes of a bag: 1 for bags of 8 lanes
+// and more, 2 for 4..7 lanes, 4 for 2..3 lanes).
+// Returns false (wave-uniform, nothing written) when a scale is too large for
+// the pre-scaled arithmetic.
+template <typename index_t, bool EXACT, int TY, int C, bool INHDR, int R>
+__device__ __forceinline__ bool pool_lean(const LookupArgs& a, const TableDesc& d, int table, int first_slot, int lane,
+                                          int* stage_row, LeanMul* stage_mul) {
+  constexpr bool QUANT = TY == ST_INT8 || TY == ST_INT4;
+  constexpr int E = TY == ST_INT4 ? 32 : (TY == ST_INT8 ? 16 : 8); // columns per chunk
+  constexpr int RN = 8 / C;                                        // rows per round: 8 loads in flight per lane
+  constexpr int SL = LEAN_BLOCK / R;                               // staging lanes per bag
+  static_assert(!INHDR || QUANT, "whole-row chunks belong to rows with a header");
+
+  const LeanLane L = lean_lane<index_t>(a, d, table, first_slot, lane);
+  const int S = d.lanes;
+  const int sub = L.sub;
+  const int n = L.n;
+  const bool bag_ok = L.bag_ok;
+  const bool stager = bag_ok && sub < SL;
+  // the longest bag of the wave bounds the loop (wave-uniform)
+  int nmax = n;
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) nmax = max(nmax, __shfl_xor(nmax, o, 64));
+  nmax = __builtin_amdgcn_readfirstlane(nmax);
+
+  const index_t* idx = reinterpret_cast<const index_t*>(a.indices) + L.pos0;
+  const float* sw = a.sample_weights ? a.sample_weights + L.pos0 : nullptr;
+  const uint8_t* wbase = (d.placement ? a.weights[1] : a.weights[0]) + d.weights_offset;
+  const uint8_t* psb = wbase + d.sb_off;
+  // this lane's first chunk of row 0
+  const uint8_t* pdata = INHDR ? wbase + sub * 16 : wbase + d.data_off + sub * 16;
+  const uint32_t stride = (uint32_t)d.row_stride;
+  int* my_row = stage_row + L.lgrp * LEAN_BLOCK;
+  LeanMul* my_mul = stage_mul + L.lgrp * LEAN_BLOCK;
+  // byte offset of the lane's chunks from its first; whole-row chunks: a slot past
+  // the row's last chunk shadows it (same bytes, nothing written)
+  int rowb[C];
+  if constexpr (INHDR) {
+    const int nchunks = (d.data_bytes + 4 + 15) / 16;
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+      const int k = sub + c * S;
+      rowb[c] = ((k < nchunks ? k : nchunks - 1) - sub) * 16;
+    }
+  } else {
+#pragma unroll
+    for (int c = 0; c < C; ++c) rowb[c] = c * S * 16;
+  }
+
+  float acc[32];
+#pragma unroll
+  for (int e = 0; e < 32; ++e) acc[e] = 0.0f;
+  float bsum = -0.0f; // tolerance grade: the biases of the bag, added once at the end
+
+  // the rows in flight. Zeroed once: a slot without a row keeps what it held (finite
+  // integers for the quantized types; fp16 slots are cleared when they have no row)
+  uint32_t raw[RN][C][4];
+#pragma unroll
+  for (int e = 0; e < RN; ++e)
+#pragma unroll
+    for (int c = 0; c < C; ++c)
+#pragma unroll
+      for (int w = 0; w < 4; ++w) raw[e][c][w] = 0u;
+
+  // registers of the staging lanes: raw indices and weights of the block being fetched
+  int64_t nrow[R];
+  float nw[R];
+  bool have[R];
+  auto load_idx = [&](int blk) {
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      nrow[j] = 0;
+      nw[j] = 1.0f;
+      const int i = blk * LEAN_BLOCK + sub + j * SL;
+      have[j] = stager && i < n;
+      if (have[j]) {
+        nrow[j] = (int64_t)idx[i];
+        if (sw) nw[j] = sw[i];
+      }
+    }
+  };
+
+  load_idx(0);
+  for (int blk = 0; blk * LEAN_BLOCK < nmax; ++blk) {
+    // ---- logical -> physical rows of pruned tables (the loads of the block issued together) ----
+    if (L.remapped) {
+#pragma unroll
+      for (int j = 0; j < R; ++j)
+        if (have[j]) nrow[j] = lean_remap(a, L, nrow[j], L.pos0 + blk * LEAN_BLOCK + sub + j * SL);
+    }
+    // ---- stage the block: row numbers (or holes), the weights ----
+    int crow[R];
+    float cw[R];
+    bool hole = false, big = false;
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      crow[j] = LEAN_NO_ENTRY;
+      cw[j] = nw[j];
+      if (have[j]) crow[j] = nrow[j] == LEAN_PRUNED ? LEAN_SKIP : lean_row(a, d, L, nrow[j], L.pos0 + blk * LEAN_BLOCK + sub + j * SL);
+      if (stager) {
+        hole = hole || crow[j] < 0;
+        my_row[sub + j * SL] = crow[j];
+        if (!QUANT || INHDR || crow[j] < 0) {
+          // fp16 rows and whole-row chunks: the multiplier is the weight. A hole gets
+          // (-0, -0, -0), which leaves every accumulator exactly as it is.
+          LeanMul m;
+          m.s24 = crow[j] < 0 ? -0.0f : nw[j];
+          m.s20 = -0.0f;
+          m.bias = -0.0f;
+          m.pad = 0.0f;
+          // whole-row chunks take fp16 headers: |scale| <= 65504, so only a huge weight can overflow the pre-scaling
+          if (INHDR) big = big || !(__builtin_fabsf(nw[j]) < 0x1p60f);
+          my_mul[sub + j * SL] = m;
+        }
+      }
+    }
+    // wave-uniform: every bag slot of the wave holds a bag with 8 rows to add in this block
+    // (lanes left over shadow the last bag slot, so that one must be there too)
+    const bool full = __builtin_amdgcn_ballot_w64(hole || first_slot + L.lgrp >= a.B) == 0ull;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+    auto load_round_full = [&](int rd) {
+#pragma unroll
+      for (int e = 0; e < RN; ++e) {
+        const uint8_t* p = pdata + (uint64_t)(uint32_t)my_row[rd * RN + e] * stride;
+#pragma unroll
+        for (int c = 0; c < C; ++c) load_raw<16>(raw[e][c], p + rowb[c]);
+      }
+    };
+    auto load_round_ragged = [&](int rd) {
+#pragma unroll
+      for (int e = 0; e < RN; ++e) {
+        const int row = my_row[rd * RN + e];
+        if (bag_ok && row >= 0) {
+          const uint8_t* p = pdata + (uint64_t)(uint32_t)row * stride;
+#pragma unroll
+          for (int c = 0; c < C; ++c) load_raw<16>(raw[e][c], p + rowb[c]);
+        } else if (!QUANT || INHDR) { // fp16: no stale infinities; whole-row chunks: no stale header
+#pragma unroll
+          for (int c = 0; c < C; ++c)
+#pragma unroll
+            for (int w = 0; w < 4; ++w) raw[e][c][w] = 0u;
+        }
+      }
+    };
+    // the rows first, then what depends on them least: (scale, bias) of the staged
+    // rows, the indices of the next block. One wait covers rows and headers.
+    if (full) load_round_full(0);
+    else load_round_ragged(0);
+    uint32_t h0[R], h1[R];
+    if constexpr (QUANT && !INHDR) {
+#pragma unroll
+      for (int j = 0; j < R; ++j) {
+        h0[j] = h1[j] = 0u;
+        if (crow[j] >= 0) {
+          const uint8_t* p = psb + (uint64_t)(uint32_t)crow[j] * stride;
+          if (d.sb_fp32) {
+            const Dwordx2 v = *reinterpret_cast<const Dwordx2*>(p);
+            h0[j] = v.v[0];
+            h1[j] = v.v[1];
+          } else {
+            h0[j] = *reinterpret_cast<const uint32_t*>(p);
+          }
+        }
+      }
+    }
+    load_idx(blk + 1);
+
+    if constexpr (QUANT && !INHDR) {
+#pragma unroll
+      for (int j = 0; j < R; ++j) {
+        if (crow[j] >= 0) {
+          const float rs = d.sb_fp32 ? bits_to_float(h0[j]) : half_lo(h0[j]);
+          const float rb = d.sb_fp32 ? bits_to_float(h1[j]) : half_hi(h0[j]);
+          const float sc = cw[j] * rs;
+          big = big || !(__builtin_fabsf(sc) < 0x1p100f);
+          LeanMul m;
+          m.s24 = sc * 0x1p24f;
+          m.s20 = sc * 0x1p20f;
+          m.bias = cw[j] * rb;
+          m.pad = 0.0f;
+          my_mul[sub + j * SL] = m;
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+    if constexpr (QUANT) {
+      // wave-uniform: a scale too large for the pre-scaled route; nothing has been written yet
+      if (__builtin_amdgcn_ballot_w64(big) != 0ull) return false;
+    }
+
+#pragma unroll
+    for (int rd = 0; rd < LEAN_BLOCK / RN; ++rd) {
+      if (rd > 0) {
+        if (rd * RN >= nmax - blk * LEAN_BLOCK) break; // no bag of the wave reaches this round
+        if (full) load_round_full(rd);
+        else load_round_ragged(rd);
+      }
+#pragma unroll
+      for (int e = 0; e < RN; ++e) {
+        LeanMul m = my_mul[rd * RN + e];
+        if constexpr (INHDR) {
+          // the row header sits in the first dword of chunk 0, which the first lane
+          // of the group holds (zero for a row that is not there)
+          const uint32_t h = (uint32_t)__builtin_amdgcn_ds_bpermute((lane - sub) * 4, (int)raw[e][0][0]);
+          const float sc = m.s24 * half_lo(h);
+          m.bias = m.s24 * half_hi(h);
+          m.s24 = sc * 0x1p24f;
+          m.s20 = sc * 0x1p20f;
+        }
+        if constexpr (!EXACT && QUANT) bsum += m.bias;
+#pragma unroll
+        for (int c = 0; c < C; ++c) lean_chunk<TY, EXACT, false>(acc, c * E, raw[e][c], m);
+      }
+    }
+    __builtin_amdgcn_wave_barrier(); // the column lanes are done with the block before it is overwritten
+  }
+  lean_write<EXACT, TY, C, INHDR>(a, d, L, acc, bsum);
+  return true;
+}
+
+// The same bags, one row at a time, integers converted to float before the fma:
+// for waves that met a scale the pre-scaled arithmetic cannot take. Every lane
+// walks its bag's entries itself; nothing is staged.
+template <typename index_t, bool EXACT, int TY, int C, bool INHDR>
+__device__ __forceinline__ void pool_lean_slow(const LookupArgs& a, const TableDesc& d, int table, int first_slot, int lane) {
+  constexpr int E = TY == ST_INT4 ? 32 : 16;
+  const LeanLane L = lean_lane<index_t>(a, d, table, first_slot, lane);
+  const int S = d.lanes;
+  const index_t* idx = reinterpret_cast<const index_t*>(a.indices) + L.pos0;
+  const uint8_t* wbase = (d.placement ? a.weights[1] : a.weights[0]) + d.weights_offset;
+  const int nchunks = INHDR ? (d.data_bytes + 4 + 15) / 16 : S * C;
+  float acc[32];
+#pragma unroll
+  for (int e = 0; e < 32; ++e) acc[e] = 0.0f;
+  float bsum = -0.0f;
+  for (int i = 0; i < L.n; ++i) {
+    int64_t row = (int64_t)idx[i];
+    const float w = a.sample_weights ? a.sample_weights[L.pos0 + i] : 1.0f;
+    if (L.remapped) row = lean_remap(a, L, row, L.pos0 + i);
+    const int r = row == LEAN_PRUNED ? LEAN_SKIP : lean_row(a, d, L, row, L.pos0 + i);
+    if (r < 0) continue;
+    const uint8_t* prow = wbase + (uint64_t)(uint32_t)r * (uint32_t)d.row_stride;
+    float rs, rb;
+    load_scale_bias(prow + d.sb_off, d.sb_fp32 != 0, true, rs, rb);
+    LeanMul m;
+    m.s24 = w * rs;
+    m.s20 = m.s24;
+    m.bias = w * rb;
+    m.pad = 0.0f;
+    if constexpr (!EXACT) bsum += m.bias;
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+      const int k = L.sub + c * S;
+      uint32_t raw[4];
+      load_raw<16>(raw, prow + (INHDR ? 0 : d.data_off) + (k < nchunks ? k : nchunks - 1) * 16);
+      lean_chunk<TY, EXACT, true>(acc, c * E, raw, m);
+    }
+  }
+  lean_write<EXACT, TY, C, INHDR>(a, d, L, acc, bsum);
+}
+
+template <typename index_t, bool EXACT, int TY, int C, bool INHDR>
+__device__ __forceinline__ void run_lean(const LookupArgs& a, const TableDesc& d, int table, int first_slot, int lane,
+                                         int* stage_row, LeanMul* stage_mul) {
+  bool done;
+  if (d.lanes >= 8) done = pool_lean<index_t, EXACT, TY, C, INHDR, 1>(a, d, table, first_slot, lane, stage_row, stage_mul);
+  else if (d.lanes >= 4) done = pool_lean<index_t, EXACT, TY, C, INHDR, 2>(a, d, table, first_slot, lane, stage_row, stage_mul);
+  else done = pool_lean<index_t, EXACT, TY, C, INHDR, 4>(a, d, table, first_slot, lane, stage_row, stage_mul);
+  if constexpr (TY == ST_INT4 || TY == ST_INT8) {
+    if (!done) pool_lean_slow<index_t, EXACT, TY, C, INHDR>(a, d, table, first_slot, lane);
+  }
+}
+
+// Row types and the chunks per lane the host picks for lean shapes: 1 (4-bit), 2 (8-bit), 4 (fp16).
+template <typename index_t, bool EXACT>
+__device__ __forceinline__ void lean_dispatch(const LookupArgs& a, const TableDesc& d, int table, int first_slot, int lane,
+                                              int* stage_row, LeanMul* stage_mul) {
+  if (d.ty == ST_INT4) {
+    if (d.inline_hdr) run_lean<index_t, EXACT, ST_INT4, 1, true>(a, d, table, first_slot, lane, stage_row, stage_mul);
+    else run_lean<index_t, EXACT, ST_INT4, 1, false>(a, d, table, first_slot, lane, stage_row, stage_mul);
+  } else if (d.ty == ST_INT8) {
+    if (d.inline_hdr) run_lean<index_t, EXACT, ST_INT8, 2, true>(a, d, table, first_slot, lane, stage_row, stage_mul);
+    else run_lean<index_t, EXACT, ST_INT8, 2, false>(a, d, table, first_slot, lane, stage_row, stage_mul);
+  } else if (d.ty == ST_FP16) {
+    run_lean<index_t, EXACT, ST_FP16, 4, false>(a, d, table, first_slot, lane, stage_row, stage_mul);
+  }
+}
+
+#ifndef FBGEMM_AMD_LEAN_MIN_WAVES
+#define FBGEMM_AMD_LEAN_MIN_WAVES 3 // waves per SIMD the register allocation must leave room for
+#endif
+
+// Same work list and workgroup -> XCD mapping as lookup_kernel.
+template <typename index_t, bool EXACT>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(FBGEMM_AMD_LEAN_MIN_WAVES, 8))) void lookup_lean_kernel(const LookupArgs a) {
+  __shared__ int stage_row[MAX_GROUPS * LEAN_BLOCK];
+  __shared__ LeanMul stage_mul[MAX_GROUPS * LEAN_BLOCK];
+  const int lane = threadIdx.x;
+  int64_t wave;
+  if (a.xcd_start) {
+    const int xb = blockIdx.x & 7;
+    const int64_t w = (int64_t)(blockIdx.x >> 3);
+    const int64_t lo = a.xcd_start[xb], hi = a.xcd_start[xb + 1];
+    if (w >= hi - lo) return;
+    wave = lo + w;
+  } else {
+    wave = (int64_t)blockIdx.x;
+    if (wave >= a.num_waves) return;
+  }
+  int table = 0, first_slot;
+  if (a.work) {
+    const WaveWork ww = a.work[wave];
+    table = ww.table;
+    first_slot = ww.first_bag;
+  } else {
+    first_slot = (int)(wave * bags_per_wave(a.single.lanes, a.single.packed));
+  }
+  const TableDesc d = a.tables ? a.tables[table] : a.single;
+  lean_dispatch<index_t, EXACT>(a, d, table, first_slot, lane, stage_row, stage_mul);
+}
+
+#define FBGEMM_AMD_DEFINE_LEAN_LAUNCH(FN, INDEX_T, EXACT)                                                \
+  hipError_t FN(const LookupArgs& a, unsigned blocks, hipStream_t stream) {                              \
+    hipLaunchKernelGGL((lookup_lean_kernel<INDEX_T, EXACT>), dim3(blocks), dim3(64), 0, stream, a);      \
+    return hipGetLastError();                                                                            \
+  }
+
+} // namespace fbgemm_amd

@@ -108,8 +108,23 @@ typedef struct fbgemm_amd_spmdm_config {
                                    input_stride bytes to rows input_stride apart */
   int32_t fp8_exponent_bits;    /* weight_ty FP8 (GenerateEmbeddingSpMDMFP8WithStrides, */
   int32_t fp8_exponent_bias;    /* FbgemmEmbedding.h:185-203): the format of the rows */
-  int32_t reserved;             /* 0 */
+  int32_t accumulate;           /* FBGEMM_AMD_ACC_EXACT (0, the default) or
+                                   FBGEMM_AMD_ACC_FAST, see below */
 } fbgemm_amd_spmdm_config;
+
+/* How 4- and 8-bit rows are accumulated. No counterpart in the reference.
+ * EXACT: the reference's own sequence of fp32 roundings, acc = fma(scale, q,
+ *   acc + bias) per element in index order (src/RefImplementations.cc:1326-1333,
+ *   1519-1527): results are bit-identical to the CPU path.
+ * FAST: the biases of a bag are summed apart, acc = fma(scale, q, acc) per
+ *   element, out = acc + sum of the biases: a third fewer vector instructions
+ *   per 4-bit element. Same index order, one lane per output column, so results
+ *   are deterministic and differ from the reference's by a few fp32 roundings of
+ *   the partial sums (tests hold it to 1e-5 of the bag's sum of magnitudes for
+ *   fp32 output and to one unit in the last place of fp16 / bf16 output).
+ * Rows the lean kernel does not take (odd widths, 2-bit, fp32, ...) and fp16 /
+ * bf16 / fp32 / fp8 rows are computed the EXACT way in either mode. */
+enum { FBGEMM_AMD_ACC_EXACT = 0, FBGEMM_AMD_ACC_FAST = 1 };
 
 /* Enqueue one pooled lookup. d_weights may be NULL (unweighted).
  * d_compressed_indices_table, when non-NULL, selects the row-wise-sparse
@@ -218,6 +233,20 @@ int fbgemm_amd_tbe_forward_pruned(
     const float* d_indice_weights, int32_t output_ty, void* d_output,
     const void* d_index_remappings, int32_t remap_bits,
     const int64_t* d_index_remappings_offsets, void* d_status, void* stream);
+
+/* Select FBGEMM_AMD_ACC_EXACT (the default of a new plan) or FBGEMM_AMD_ACC_FAST
+ * for the forwards of a plan. No counterpart in the reference. */
+int fbgemm_amd_tbe_plan_set_accumulate(fbgemm_amd_tbe_plan* plan, int32_t mode);
+
+/* A plan caches, per (batch size, stream), the work lists of its forwards and the
+ * scratch of the bag scheduler; past 16 entries the least recently used one that
+ * no forward under stream capture has touched is dropped. This call drops ALL of
+ * them (after a device synchronize), including those a captured graph may hold:
+ * graphs that contain forwards of this plan must be captured again afterwards.
+ * fbgemm_amd_tbe_plan_cached_work returns the number of cached entries. No
+ * counterpart in the reference. */
+int fbgemm_amd_tbe_plan_trim(fbgemm_amd_tbe_plan* plan);
+int64_t fbgemm_amd_tbe_plan_cached_work(const fbgemm_amd_tbe_plan* plan);
 
 /* Tables of FBGEMM_AMD_FP8 rows (D bytes per row, no scale/bias) are decoded
  * with the operator's fp8_exponent_bits / fp8_exponent_bias
@@ -437,6 +466,17 @@ int fbgemm_amd_stream_synchronize(void* stream);
  * the hardware byte counters of the lookup kernel against what the same
  * counters read for this copy of known size. */
 int fbgemm_amd_calibration_copy(const void* d_src, void* d_dst, int64_t bytes, void* stream);
+
+/* Process-wide switches for A/B measurements and tests (no counterpart in the
+ * reference; results are bit-identical under every setting of both).
+ * fbgemm_amd_set_lean: 1 = shapes the lean kernel takes go to it (the default,
+ * also FBGEMM_AMD_LEAN in the environment at load time), 0 = everything goes
+ * through the general kernel, -1 = back to the default.
+ * fbgemm_amd_set_narrow_below_waves: launches of fewer waves than this take
+ * 4-byte lanes (default 1024, FBGEMM_AMD_NARROW_BELOW_WAVES at load time; -1 =
+ * back to the default). */
+int fbgemm_amd_set_lean(int32_t on);
+int fbgemm_amd_set_narrow_below_waves(int32_t waves);
 
 /* ---- row-size arithmetic (host, no GPU) ------------------------------------ *
  * embedding_common.h:189-225. */

@@ -19,10 +19,16 @@ def oracle():
     return o
 
 
-@pytest.fixture(params=["wide", "narrow"])
-def lane_shape(request, monkeypatch):
-    """Launches too small to fill the device take 4-byte lanes by default; test modules that ask for this
-    fixture run every test with that policy and with the 16-byte lanes large launches get (the library
-    reads the switch on every call)."""
-    monkeypatch.setenv("FBGEMM_AMD_NARROW_BELOW_WAVES", "0" if request.param == "wide" else "1024")
-    return request.param
+@pytest.fixture(params=["wide", "narrow", "general"])
+def lane_shape(request):
+    """The three routes a pooled lookup can take, for test modules that ask for this fixture:
+    "wide" = 16-byte lanes, the lean kernel where the shape allows it (what large launches get);
+    "narrow" = 4-byte lanes (what launches too small to fill the device get by default);
+    "general" = 16-byte lanes with the lean kernel switched off (everything through the general kernel)."""
+    import fbgemm_amd
+    lib = fbgemm_amd.lib()
+    lib.fbgemm_amd_set_narrow_below_waves(1024 if request.param == "narrow" else 0)
+    lib.fbgemm_amd_set_lean(0 if request.param == "general" else 1)
+    yield request.param
+    lib.fbgemm_amd_set_narrow_below_waves(-1)
+    lib.fbgemm_amd_set_lean(-1)
