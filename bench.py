@@ -57,7 +57,7 @@ def parse():
     ap.add_argument("--op", default="lookup",
                     choices=["lookup", "quantize", "dequantize", "bounds_check", "pruned_array_lookup",
                              "pruned_hashmap_lookup", "float_to_hfp8", "hfp8_to_float", "rowwise_prune",
-                             "compressed_indices_remap", "sequence", "no_bag", "inplace_update"],
+                             "compressed_indices_remap", "sequence", "no_bag", "inplace_update", "gather_ceiling"],
                     help="lookup = the table-batched forward (the metric); the others time one operator beside "
                          "the path at the shape config 4 / config 3 gives it and print the same kind of line")
     return ap.parse_args()
@@ -281,6 +281,82 @@ def calibration_copy(a, torch):
         C.c_void_p(src.data_ptr()), C.c_void_p(dst.data_ptr()), n,
         C.c_void_p(torch.cuda.current_stream().cuda_stream)))
     torch.cuda.synchronize()
+
+
+def gather_ceiling(a):
+    """What this GPU sustains for the access patterns of a pooled lookup, measured with
+    the library's own yardstick kernels (ceiling_kernels.hip): a streaming read, and
+    gathers of random rows with 16-byte lanes and 8 rows per lane group in flight, from a
+    table far larger than the caches. One JSON line: `value` is the rate of random
+    128-byte lines (the pattern of a cold row), the other cases are under "cases"."""
+    import numpy as np
+    import torch
+
+    from fbgemm_amd import _lib
+    lib = _lib.lib()
+    torch.cuda.set_device(0)
+    stream = lambda: C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    table_bytes = int((32 << 30) * a.scale)
+    table = torch.empty(table_bytes, dtype=torch.uint8, device="cuda")
+    table.view(torch.int32).random_(0, 1 << 30)
+    sink = torch.zeros(1 << 20, dtype=torch.int32, device="cuda")
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(99)
+    n = int((1 << 25) * a.scale)
+    ptr = lambda t: C.c_void_p(t.data_ptr())
+
+    def timed(fn):
+        for _ in range(max(1, a.warmup // 4)):
+            fn()
+        torch.cuda.synchronize()
+        steps = max(3, a.steps // 10)
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record()
+        for _ in range(steps):
+            fn()
+        ev1.record()
+        torch.cuda.synchronize()
+        return ev0.elapsed_time(ev1) / steps
+
+    cases = []
+    ms = timed(lambda: _lib.check(lib.fbgemm_amd_ceiling_stream_read(ptr(table), table_bytes, ptr(sink), stream())))
+    cases.append({"case": f"streaming read of {table_bytes >> 30} GiB, 16 bytes per lane, 8 loads in flight",
+                  "kernel": "stream_read_kernel", "ms": round(ms, 4), "GB/s": round(table_bytes / ms / 1e6, 1)})
+    # (what, row stride, lanes per row, byte offset of the first lane's load)
+    shapes = [("random 128-byte lines (aligned)", 128, 8, 0),
+              ("128 bytes at byte 4 of rows 144 bytes apart (4-bit rows of 256 columns, data after the header)", 144, 8, 4),
+              ("144-byte rows whole, as 8 aligned lanes of the first 128 bytes", 144, 8, 0),
+              ("random 64-byte half lines (aligned)", 64, 4, 0),
+              ("random 512-byte rows (fp16 rows of 256 columns)", 512, 32, 0),
+              ("32 bytes at byte 4 of rows 48 bytes apart (4-bit rows of 64 columns)", 48, 2, 4)]
+    headline = None
+    for what, stride, lanes, off in shapes:
+        rows = table_bytes // stride
+        idx = torch.randint(0, rows, (n,), dtype=torch.int32, device="cuda", generator=gen)
+        waves = 256 * 64
+        ms = timed(lambda: _lib.check(lib.fbgemm_amd_ceiling_gather(ptr(table), rows, stride, lanes, off, ptr(idx), n,
+                                                                     ptr(sink), waves, stream())))
+        useful = n * lanes * 16
+        first, last = off, off + lanes * 16 - 1
+        g = np.gcd(stride, 128)
+        starts = (np.arange(128 // g) * g) % 128
+        lines = float(np.mean((starts + last) // 128 - (starts + first) // 128 + 1))
+        rec = {"case": what, "kernel": "gather_lines_kernel", "rows": n, "ms": round(ms, 4),
+               "useful_GB/s": round(useful / ms / 1e6, 1), "lines_per_row": round(lines, 3),
+               "G_lines/s": round(n * lines / ms / 1e6, 2), "G_rows/s": round(n / ms / 1e6, 2)}
+        cases.append(rec)
+        if headline is None:
+            headline = rec
+    res = {"metric": "random 128-byte line gathers, G lines/s on 1 MI355X", "value": headline["G_lines/s"], "unit": "G lines/s",
+           "n_gpus": 1, "steps": max(3, a.steps // 10), "warmup": max(1, a.warmup // 4), "ms_per_step": headline["ms"],
+           "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+           "config": {"workload": f"yardstick kernels over a {table_bytes >> 30} GiB table, {n} random rows per launch"},
+           "roofline": {"bound": "hbm", "achieved": headline["useful_GB/s"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                        "frac": round(headline["useful_GB/s"] / HBM_PEAK_GBPS, 4), "traffic": None,
+                        "kernel": "gather_lines_kernel", "kernel_ms": headline["ms"],
+                        "algorithmic_bytes_per_launch": n * 128},
+           "cases": cases, "cpu_baseline": None}
+    print(json.dumps(res))
 
 
 def side_op(a):
@@ -584,6 +660,8 @@ def main():
         print("bench.py: this path is measured on ONE GPU (no sharding, no collectives); "
               f"--gpus {a.gpus} is not supported", file=sys.stderr)
         sys.exit(2)
+    if a.op == "gather_ceiling":
+        return gather_ceiling(a)
     if a.op != "lookup":
         return side_op(a)
     import numpy as np

@@ -64,6 +64,8 @@ SYMBOLS = {
     "fbgemm_amd_tbe_inplace_update": (C.c_int, [_P, _P, _P, _P, _I64, _P, _P, _I32, _P, _I64, _P, _P]),
     "fbgemm_amd_pruned_array_lookup_from_row_idx": (C.c_int, [_P, _I32, _P, _I64, _P, _I32, _P, _I32, _P, _P]),
     "fbgemm_amd_calibration_copy": (C.c_int, [_P, _P, _I64, _P]),
+    "fbgemm_amd_ceiling_stream_read": (C.c_int, [_P, _I64, _P, _P]),
+    "fbgemm_amd_ceiling_gather": (C.c_int, [_P, _I64, _I64, _I32, _I32, _P, _I64, _P, _I32, _P]),
     "fbgemm_amd_unpadded_row_size_in_bytes": (_I32, [_I32, _I32, _I32]),
     "fbgemm_amd_padded_row_size_in_bytes": (_I32, [_I32, _I32, _I32, _I32]),
 }

@@ -49,6 +49,9 @@ hipError_t launch_compressed_indices_remap(const void* indices, bool idx64, cons
 hipError_t launch_quantize_segments(const float* input, int64_t lines, int32_t T, const int32_t* d_seg_offsets,
                                     int32_t total_D, int32_t max_D, uint8_t* output, hipStream_t stream);
 hipError_t launch_calibration_copy(const void* src, void* dst, int64_t bytes, hipStream_t stream);
+hipError_t launch_stream_read(const void* src, int64_t bytes, uint32_t* sink, hipStream_t stream);
+hipError_t launch_gather_lines(const void* table, int64_t stride, int32_t lanes, int32_t byte_offset, const int32_t* idx,
+                               int64_t n, uint32_t* sink, int32_t waves, hipStream_t stream);
 hipError_t launch_bounds_check(const int64_t* rows_per_table, int32_t T, void* indices, void* offsets, bool is64,
                                int64_t num_indices, int64_t total_B, int64_t B, const int32_t* B_offsets, int mode,
                                int64_t* warning, int64_t* fixed, int64_t* partial, Status* status, hipStream_t stream);
@@ -359,6 +362,24 @@ int fbgemm_amd_calibration_copy(const void* d_src, void* d_dst, int64_t bytes, v
   return 0;
 }
 
+int fbgemm_amd_ceiling_stream_read(const void* d_src, int64_t bytes, void* d_sink, void* stream) {
+  if (!d_src || !d_sink || bytes < 0 || bytes % 16) return fail(FBGEMM_AMD_E_ARG, "the read needs a 16-byte multiple and a sink of 8192 dwords");
+  HIP_TRY(launch_stream_read(d_src, bytes, (uint32_t*)d_sink, (hipStream_t)stream));
+  return 0;
+}
+
+int fbgemm_amd_ceiling_gather(const void* d_table, int64_t rows, int64_t row_stride, int32_t lanes_per_row, int32_t byte_offset,
+                              const int32_t* d_rows, int64_t n, void* d_sink, int32_t waves, void* stream) {
+  if (!d_table || !d_rows || !d_sink || rows <= 0 || n < 0 || waves <= 0)
+    return fail(FBGEMM_AMD_E_ARG, "bad gather arguments");
+  if (lanes_per_row < 1 || lanes_per_row > 64 || (lanes_per_row & (lanes_per_row - 1)))
+    return fail(FBGEMM_AMD_E_ARG, "lanes_per_row must be a power of two up to 64");
+  if (byte_offset < 0 || byte_offset % 4 || row_stride % 4 || (int64_t)byte_offset + 16 * lanes_per_row > row_stride)
+    return fail(FBGEMM_AMD_E_ARG, "the bytes read must lie inside the row, at 4-byte alignment");
+  HIP_TRY(launch_gather_lines(d_table, row_stride, lanes_per_row, byte_offset, d_rows, n, (uint32_t*)d_sink, waves, (hipStream_t)stream));
+  return 0;
+}
+
 int32_t fbgemm_amd_unpadded_row_size_in_bytes(int32_t dim, int32_t ty, int32_t sb) {
   switch (ty) {
     case ST_FP32: return dim * 4;
@@ -514,6 +535,7 @@ int spmdm_launch_impl(
     if (d.vb == 16 && (output_size + G16 - 1) / G16 < narrow_below_waves()) plan_lanes(d, (uintptr_t)d_input, out_stride, has_sb, false, true);
   }
   d.lanes_recip = (65536 + d.lanes - 1) / d.lanes;
+    d.bags = bags_per_wave(d.lanes, d.packed);
 
   a.tables = nullptr;
   a.weights[0] = (const uint8_t*)d_input;
@@ -880,6 +902,7 @@ int fbgemm_amd_tbe_plan_create(
     // weights buffers come from hipMalloc / torch: at least 256-byte aligned
     plan_lanes(d, 0, plan->total_D, q, false);
     d.lanes_recip = (65536 + d.lanes - 1) / d.lanes;
+    d.bags = bags_per_wave(d.lanes, d.packed);
   }
   HIP_TRY(hipMalloc((void**)&plan->d_D_offsets, sizeof(int32_t) * (T + 1)));
   HIP_TRY(hipMemcpy(plan->d_D_offsets, D_offsets, sizeof(int32_t) * (T + 1), hipMemcpyHostToDevice));
@@ -892,6 +915,7 @@ int fbgemm_amd_tbe_plan_create(
     TableDesc& d = plan->tables_packed[t];
     plan_lanes(d, 0, plan->total_D, quantised(d.ty), true);
     d.lanes_recip = (65536 + d.lanes - 1) / d.lanes;
+    d.bags = bags_per_wave(d.lanes, d.packed);
     any_packed = any_packed || d.packed;
   }
   if (any_packed) {
@@ -905,6 +929,7 @@ int fbgemm_amd_tbe_plan_create(
     TableDesc& d = plan->tables_narrow[t];
     plan_lanes(d, 0, plan->total_D, quantised(d.ty), false, true);
     d.lanes_recip = (65536 + d.lanes - 1) / d.lanes;
+    d.bags = bags_per_wave(d.lanes, d.packed);
   }
   HIP_TRY(hipMalloc((void**)&plan->d_tables_narrow, sizeof(TableDesc) * T));
   HIP_TRY(hipMemcpy(plan->d_tables_narrow, plan->tables_narrow.data(), sizeof(TableDesc) * T, hipMemcpyHostToDevice));

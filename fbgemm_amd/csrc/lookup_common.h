@@ -60,6 +60,7 @@ struct TableDesc {
                           // and costs no request of its own; `lanes` need not divide 64
   int32_t packed;         // 1: bags lie end to end in the wave (see bags_per_wave)
   int32_t lanes_recip;    // ceil(65536 / lanes): j / lanes == (j * lanes_recip) >> 16 for 0 <= j <= 64
+  int32_t bags;           // bags_per_wave(lanes, packed), so that no kernel divides
 };
 
 #if defined(__HIPCC__)

@@ -56,7 +56,7 @@ __device__ __forceinline__ bool pool_bags(const LookupArgs& a, const TableDesc& 
 
   static_assert(!INHDR || (VB == 16 && QUANT), "whole-row chunks are 16 bytes of a quantised row");
   const int S = d.lanes;
-  const int G = bags_per_wave(S, d.packed);
+  const int G = d.bags;
   // quarter q of the wave holds bags q * (16 / S) ...; its last 16 % S lanes idle
   int grp, sub;
   bool idle;
@@ -463,7 +463,7 @@ __device__ __forceinline__ void run_item(const LookupArgs& a, int64_t wave, int 
     table = ww.table;
     first_slot = ww.first_bag;
   } else {
-    first_slot = (int)(wave * bags_per_wave(a.single.lanes, a.single.packed));
+    first_slot = (int)(wave * a.single.bags);
   }
   const TableDesc d = a.tables ? a.tables[table] : a.single;
 #ifdef FBGEMM_AMD_ONLY_TY // register-budget experiments: compile a single row type

@@ -120,12 +120,12 @@ template <typename index_t>
 __device__ __forceinline__ LeanLane lean_lane(const LookupArgs& a, const TableDesc& d, int table, int first_slot, int lane) {
   LeanLane L;
   const int S = d.lanes;
-  const int G = bags_per_wave(S, d.packed);
+  const int G = d.bags;
   bool idle;
   const uint32_t recip = (uint32_t)d.lanes_recip; // divisions by S, exact for arguments up to 64
   if (S <= 16 && !d.packed) {
     // quarter q of the wave holds bags q * (16 / S) ...; its last 16 % S lanes are left over
-    const int per_q = (int)((16u * recip) >> 16);
+    const int per_q = G >> 2;
     const int j = lane & 15;
     const int gq = (int)(((uint32_t)j * recip) >> 16);
     idle = gq >= per_q;
@@ -183,6 +183,18 @@ __device__ __forceinline__ LeanLane lean_lane(const LookupArgs& a, const TableDe
     }
   }
   return L;
+}
+
+// Largest of a non-negative value over the wave, through lane shifts inside the
+// rows of 16 and the two row broadcasts (six vector instructions, no LDS).
+__device__ __forceinline__ int lean_wave_max(int v) {
+  v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false)); // row_shr:1
+  v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false)); // row_shr:2
+  v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false)); // row_shr:4
+  v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false)); // row_shr:8: lane 15 of a row holds the row's largest
+  v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false)); // row_bcast:15 into rows 1 and 3
+  v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false)); // row_bcast:31 into rows 2 and 3
+  return __builtin_amdgcn_readlane(v, 63);
 }
 
 constexpr int LEAN_NO_ENTRY = INT32_MIN;  // the bag has no such entry
@@ -264,10 +276,7 @@ __device__ __forceinline__ bool pool_lean(const LookupArgs& a, const TableDesc& 
   const bool bag_ok = L.bag_ok;
   const bool stager = bag_ok && sub < SL;
   // the longest bag of the wave bounds the loop (wave-uniform)
-  int nmax = n;
-#pragma unroll
-  for (int o = 32; o >= 1; o >>= 1) nmax = max(nmax, __shfl_xor(nmax, o, 64));
-  nmax = __builtin_amdgcn_readfirstlane(nmax);
+  const int nmax = lean_wave_max(n);
 
   const index_t* idx = reinterpret_cast<const index_t*>(a.indices) + L.pos0;
   const float* sw = a.sample_weights ? a.sample_weights + L.pos0 : nullptr;
@@ -297,16 +306,6 @@ __device__ __forceinline__ bool pool_lean(const LookupArgs& a, const TableDesc& 
 #pragma unroll
   for (int e = 0; e < 32; ++e) acc[e] = 0.0f;
   float bsum = -0.0f; // tolerance grade: the biases of the bag, added once at the end
-
-  // the rows in flight. Zeroed once: a slot without a row keeps what it held (finite
-  // integers for the quantized types; fp16 slots are cleared when they have no row)
-  uint32_t raw[RN][C][4];
-#pragma unroll
-  for (int e = 0; e < RN; ++e)
-#pragma unroll
-    for (int c = 0; c < C; ++c)
-#pragma unroll
-      for (int w = 0; w < 4; ++w) raw[e][c][w] = 0u;
 
   // registers of the staging lanes: raw indices and weights of the block being fetched
   int64_t nrow[R];
@@ -367,6 +366,7 @@ __device__ __forceinline__ bool pool_lean(const LookupArgs& a, const TableDesc& 
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
+    uint32_t raw[RN][C][4]; // the rows in flight; a slot without a row reads as zeros
     auto load_round_full = [&](int rd) {
 #pragma unroll
       for (int e = 0; e < RN; ++e) {
@@ -383,7 +383,7 @@ __device__ __forceinline__ bool pool_lean(const LookupArgs& a, const TableDesc& 
           const uint8_t* p = pdata + (uint64_t)(uint32_t)row * stride;
 #pragma unroll
           for (int c = 0; c < C; ++c) load_raw<16>(raw[e][c], p + rowb[c]);
-        } else if (!QUANT || INHDR) { // fp16: no stale infinities; whole-row chunks: no stale header
+        } else {
 #pragma unroll
           for (int c = 0; c < C; ++c)
 #pragma unroll
@@ -564,7 +564,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(FBGEMM_AMD_L
     table = ww.table;
     first_slot = ww.first_bag;
   } else {
-    first_slot = (int)(wave * bags_per_wave(a.single.lanes, a.single.packed));
+    first_slot = (int)(wave * a.single.bags);
   }
   const TableDesc d = a.tables ? a.tables[table] : a.single;
   lean_dispatch<index_t, EXACT>(a, d, table, first_slot, lane, stage_row, stage_mul);

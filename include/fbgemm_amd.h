@@ -467,6 +467,21 @@ int fbgemm_amd_stream_synchronize(void* stream);
  * counters read for this copy of known size. */
 int fbgemm_amd_calibration_copy(const void* d_src, void* d_dst, int64_t bytes, void* stream);
 
+/* Two more yardsticks (no counterpart in the reference, not on the product path):
+ * what this GPU sustains for the access patterns a pooled lookup is made of.
+ * _stream_read: every lane reads 16 bytes per load, 8 loads in flight, through
+ *   `bytes` of d_src once (kernel stream_read_kernel); d_sink: 8192 dwords.
+ * _gather: `n` rows d_rows[i] (int32, each < rows) of a table whose rows are
+ *   row_stride bytes apart; lanes_per_row consecutive lanes read 16 bytes each
+ *   from byte_offset on (4 = what rows with a 4-byte header in front of their
+ *   data give: loads at 4-byte alignment), 8 rows per lane group in flight, as
+ *   the lookup kernels do (kernel gather_lines_kernel, `waves` workgroups of one
+ *   wave each); d_sink: `waves` dwords. */
+int fbgemm_amd_ceiling_stream_read(const void* d_src, int64_t bytes, void* d_sink, void* stream);
+int fbgemm_amd_ceiling_gather(const void* d_table, int64_t rows, int64_t row_stride, int32_t lanes_per_row,
+                              int32_t byte_offset, const int32_t* d_rows, int64_t n, void* d_sink, int32_t waves,
+                              void* stream);
+
 /* Process-wide switches for A/B measurements and tests (no counterpart in the
  * reference; results are bit-identical under every setting of both).
  * fbgemm_amd_set_lean: 1 = shapes the lean kernel takes go to it (the default,
