@@ -52,6 +52,9 @@ def parse():
                     help="exact = the reference's sequence of fp32 roundings, bit-identical to the CPU path (the "
                          "library's default); fast = the biases of a bag summed apart (tolerance grade: the parity "
                          "gate then holds fp16 / bf16 output to one unit in the last place and fp32 output to 1e-5)")
+    ap.add_argument("--no-rank-records", action="store_true",
+                    help="config 4 only: read the int32 mapping arrays in the forward instead of the compact "
+                         "bitmap-and-rank form of the (order-preserving) mappings")
     ap.add_argument("--no-also", dest="also", action="store_false",
                     help="default run only: do not append the driver-timed figures of config 5 under \"also\"")
     ap.add_argument("--op", default="lookup",
@@ -89,7 +92,7 @@ def traffic_from_profile(config_id):
         return None
 
 
-def tbe_runner(p, torch, accumulate="exact"):
+def tbe_runner(p, torch, accumulate="exact", rank_records=True):
     """Returns (launch, out, status, plan) for a TbeProblem: launch() enqueues one forward."""
     from fbgemm_amd import _lib, ops
 
@@ -109,7 +112,10 @@ def tbe_runner(p, torch, accumulate="exact"):
             p.output_dtype, C.c_void_p(out.data_ptr()),
             C.c_void_p(p.extra["remap"].data_ptr()) if "remap" in p.extra else None, 32,
             C.c_void_p(p.extra["remap_offsets"].data_ptr()) if "remap" in p.extra else None,
+            p.extra["remap_offsets"].numel() if "remap" in p.extra else 0,
             C.c_void_p(st.buf.data_ptr()), stream)
+    if "remap" in p.extra and rank_records:
+        plan.set_index_remappings(p.extra["remap"], p.extra["remap_offsets"])
 
     def launch():
         # the stream of the moment: under graph capture it is the capturing stream
@@ -612,7 +618,7 @@ def time_tbe(p, a, torch, np, steps, warmup, graph=False):
     """Parity gate, warm-up, `steps` timed forwards of one table-batched problem.
     Returns the figures of the JSON line that depend on the measurement."""
     from fbgemm_amd import _lib
-    launch, out, st, plan = tbe_runner(p, torch, a.accumulate)
+    launch, out, st, plan = tbe_runner(p, torch, a.accumulate, not a.no_rank_records)
     torch.cuda.synchronize()
     checked = parity_gate(p, out, launch, torch, np, a.accumulate) if a.check else None
     for _ in range(warmup):

@@ -38,7 +38,9 @@ SYMBOLS = {
     "fbgemm_amd_tbe_plan_create": (C.c_int, [C.POINTER(_P), _I32, _P, _P, _P, _P, _I64, _I64, _I64]),
     "fbgemm_amd_tbe_plan_destroy": (None, [_P]),
     "fbgemm_amd_tbe_forward": (C.c_int, [_P, _P, _P, _P, _P, _I32, _I64, _I64, _I32, _P, _I32, _P, _P, _P]),
-    "fbgemm_amd_tbe_forward_pruned": (C.c_int, [_P, _P, _P, _P, _P, _I32, _I64, _I64, _I32, _P, _I32, _P, _P, _I32, _P, _P, _P]),
+    "fbgemm_amd_tbe_forward_pruned": (C.c_int, [_P, _P, _P, _P, _P, _I32, _I64, _I64, _I32, _P, _I32, _P, _P, _I32, _P, _I64, _P, _P]),
+    "fbgemm_amd_tbe_plan_set_index_remappings": (C.c_int, [_P, _P, _I32, _P, _I64, _P]),
+    "fbgemm_amd_tbe_plan_rank_tables": (_I32, [_P]),
     "fbgemm_amd_tbe_plan_set_fp8": (C.c_int, [_P, _I32, _I32]),
     "fbgemm_amd_tbe_plan_set_accumulate": (C.c_int, [_P, _I32]),
     "fbgemm_amd_tbe_plan_trim": (C.c_int, [_P]),

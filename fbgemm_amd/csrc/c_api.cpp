@@ -37,6 +37,10 @@ hipError_t launch_inplace_update(const TableDesc* tables, int32_t T, uint8_t* w0
 hipError_t launch_remap_row_idx(const void* rows, bool idx64, const int32_t* table_idx, const void* remap, bool remap64,
                                 const int64_t* remap_offsets, int32_t T, int64_t n, void* dense, hipStream_t stream);
 int64_t prune_partials(int64_t rows);
+int64_t remap_rank_words(int64_t rows);
+int64_t remap_rank_partials(int64_t rows);
+hipError_t launch_remap_rank_build(const void* mapping, bool remap64, int64_t rows, RankRecord* records, int64_t* partial,
+                                   int32_t* not_monotone, hipStream_t stream);
 hipError_t launch_prune_map(const float* indicator, int64_t rows, double threshold, int use_abs, int64_t min_rows,
                             bool idx64, void* remap, int64_t* num_kept, int64_t* partial, hipStream_t stream);
 hipError_t launch_prune_gather(const void* in, int64_t rows, int64_t row_bytes, const void* remap, bool idx64, void* out,
@@ -720,6 +724,12 @@ struct fbgemm_amd_tbe_plan {
   std::map<WorkKey, Work> work;
   uint64_t use_clock = 0;
   int32_t accumulate = FBGEMM_AMD_ACC_EXACT;
+  // compact form of the pruned-row mappings (fbgemm_amd_tbe_plan_set_index_remappings)
+  RankRecord* d_rank_records = nullptr;
+  int64_t* d_rank_offsets = nullptr; // T entries: first record of the table, or -1
+  const void* rank_source = nullptr; // the mapping array the records were made from
+  int32_t rank_bits = 0;
+  int32_t rank_tables = 0;           // tables that use the records
   // lane-shape choice of the last forward, per (B, indices_numel >> 16)
   int32_t shape_B = -1;
   int64_t shape_bucket = -1;
@@ -946,6 +956,8 @@ void fbgemm_amd_tbe_plan_destroy(fbgemm_amd_tbe_plan* plan) {
   if (plan->d_tables_narrow) (void)hipFree(plan->d_tables_narrow);
   if (plan->d_D_offsets) (void)hipFree(plan->d_D_offsets);
   if (plan->pooled_tmp) (void)hipFree(plan->pooled_tmp);
+  if (plan->d_rank_records) (void)hipFree(plan->d_rank_records);
+  if (plan->d_rank_offsets) (void)hipFree(plan->d_rank_offsets);
   for (hipEvent_t e : plan->prof_ev) (void)hipEventDestroy(e);
   delete plan;
 }
@@ -977,7 +989,7 @@ int fbgemm_amd_tbe_forward(
     void* stream_) {
   return fbgemm_amd_tbe_forward_pruned(plan, d_dev_weights, d_uvm_weights, d_indices, d_offsets, index_bits,
                                        indices_numel, offsets_numel, pooling_mode, d_indice_weights, output_ty,
-                                       d_output, nullptr, 32, nullptr, d_status, stream_);
+                                       d_output, nullptr, 32, nullptr, 0, d_status, stream_);
 }
 
 int fbgemm_amd_tbe_forward_pruned(
@@ -986,10 +998,14 @@ int fbgemm_amd_tbe_forward_pruned(
     int64_t indices_numel, int64_t offsets_numel, int32_t pooling_mode,
     const float* d_indice_weights, int32_t output_ty, void* d_output,
     const void* d_index_remappings, int32_t remap_bits, const int64_t* d_index_remappings_offsets,
-    void* d_status, void* stream_) {
+    int64_t index_remappings_offsets_numel, void* d_status, void* stream_) {
   if (!plan) return fail(FBGEMM_AMD_E_ARG, "plan is null");
   if (d_index_remappings && (!d_index_remappings_offsets || (remap_bits != 32 && remap_bits != 64)))
     return fail(FBGEMM_AMD_E_ARG, "a remap array needs its T+1 offsets and 32- or 64-bit entries");
+  // the kernels read offsets[t] and offsets[t + 1] for every t the plan has (one per FEATURE of the operator)
+  if (d_index_remappings && index_remappings_offsets_numel != (int64_t)plan->T + 1)
+    return fail(FBGEMM_AMD_E_ARG, "index_remappings_offsets holds %lld entries, the plan's %d tables need %d",
+                (long long)index_remappings_offsets_numel, plan->T, plan->T + 1);
   if (index_bits != 32 && index_bits != 64) return fail(FBGEMM_AMD_E_ARG, "index_bits must be 32 or 64");
   if (output_ty == ST_INT8) {
     // The reference's GPU operator quantizes every table's pooled vector row-wise to 8 bits in its
@@ -1008,7 +1024,8 @@ int fbgemm_amd_tbe_forward_pruned(
     }
     if (int rc = fbgemm_amd_tbe_forward_pruned(plan, d_dev_weights, d_uvm_weights, d_indices, d_offsets, index_bits,
                                                indices_numel, offsets_numel, pooling_mode, d_indice_weights, ST_FP32, tmp,
-                                               d_index_remappings, remap_bits, d_index_remappings_offsets, d_status, stream_))
+                                               d_index_remappings, remap_bits, d_index_remappings_offsets,
+                                               index_remappings_offsets_numel, d_status, stream_))
       return rc;
     HIP_TRY(launch_quantize_segments(tmp, B, plan->T, plan->d_D_offsets, (int32_t)plan->total_D, plan->max_D,
                                      (uint8_t*)d_output, (hipStream_t)stream_));
@@ -1146,6 +1163,10 @@ int fbgemm_amd_tbe_forward_pruned(
   a.remap = d_index_remappings;
   a.remap_offsets = d_index_remappings ? d_index_remappings_offsets : nullptr;
   a.remap64 = remap_bits == 64;
+  if (d_index_remappings && plan->d_rank_records && plan->rank_source == d_index_remappings && plan->rank_bits == remap_bits) {
+    a.rank_records = plan->d_rank_records;
+    a.rank_offsets = plan->d_rank_offsets;
+  }
   a.out = d_output;
   a.out_stride = plan->total_D;
   a.index_size = indices_numel;
@@ -1192,6 +1213,96 @@ int fbgemm_amd_tbe_plan_set_accumulate(fbgemm_amd_tbe_plan* plan, int32_t mode) 
   plan->accumulate = mode;
   return 0;
 }
+
+int fbgemm_amd_tbe_plan_set_index_remappings(
+    fbgemm_amd_tbe_plan* plan, const void* d_index_remappings, int32_t remap_bits,
+    const int64_t* index_remappings_offsets, int64_t index_remappings_offsets_numel, void* stream_) {
+  if (!plan) return fail(FBGEMM_AMD_E_ARG, "plan is null");
+  hipStream_t stream = (hipStream_t)stream_;
+  std::lock_guard<std::mutex> lk(plan->mu);
+  // forget what was made from an earlier array (after the forwards that may still read it)
+  if (plan->d_rank_records || plan->d_rank_offsets) {
+    HIP_TRY(hipDeviceSynchronize());
+    if (plan->d_rank_records) (void)hipFree(plan->d_rank_records);
+    if (plan->d_rank_offsets) (void)hipFree(plan->d_rank_offsets);
+    plan->d_rank_records = nullptr;
+    plan->d_rank_offsets = nullptr;
+  }
+  plan->rank_source = nullptr;
+  plan->rank_tables = 0;
+  if (!d_index_remappings) return 0;
+  if (remap_bits != 32 && remap_bits != 64) return fail(FBGEMM_AMD_E_ARG, "remap entries are 32 or 64 bits wide");
+  if (!index_remappings_offsets || index_remappings_offsets_numel != (int64_t)plan->T + 1)
+    return fail(FBGEMM_AMD_E_ARG, "index_remappings_offsets must hold T+1 = %d entries (on the host)", plan->T + 1);
+  const int T = plan->T;
+  std::vector<int64_t> first(T, -1);
+  int64_t words = 0, max_partials = 1;
+  for (int t = 0; t < T; ++t) {
+    const int64_t rows = index_remappings_offsets[t + 1] - index_remappings_offsets[t];
+    if (rows < 0) return fail(FBGEMM_AMD_E_ARG, "index_remappings_offsets must not decrease");
+    if (rows == 0) continue;
+    first[t] = words;
+    words += remap_rank_words(rows);
+    max_partials = std::max(max_partials, remap_rank_partials(rows));
+  }
+  if (words == 0) return 0;
+  RankRecord* records = nullptr;
+  int64_t* partial = nullptr;
+  int32_t* flags = nullptr;
+  auto drop = [&]() {
+    if (records) (void)hipFree(records);
+    if (partial) (void)hipFree(partial);
+    if (flags) (void)hipFree(flags);
+  };
+#define HIP_TRY_DROP(expr)                                                              \
+  do {                                                                                  \
+    hipError_t e_ = (expr);                                                             \
+    if (e_ != hipSuccess) {                                                             \
+      drop();                                                                           \
+      return fail(FBGEMM_AMD_E_HIP, "%s: %s", #expr, hipGetErrorString(e_));            \
+    }                                                                                   \
+  } while (0)
+  HIP_TRY_DROP(hipMalloc((void**)&records, sizeof(RankRecord) * (size_t)words));
+  HIP_TRY_DROP(hipMalloc((void**)&partial, sizeof(int64_t) * (size_t)max_partials));
+  HIP_TRY_DROP(hipMalloc((void**)&flags, sizeof(int32_t) * (size_t)T));
+  HIP_TRY_DROP(hipMemsetAsync(flags, 0, sizeof(int32_t) * (size_t)T, stream));
+  const size_t esz = remap_bits / 8;
+  for (int t = 0; t < T; ++t) {
+    if (first[t] < 0) continue;
+    const int64_t rows = index_remappings_offsets[t + 1] - index_remappings_offsets[t];
+    HIP_TRY_DROP(launch_remap_rank_build((const char*)d_index_remappings + (size_t)index_remappings_offsets[t] * esz,
+                                         remap_bits == 64, rows, records + first[t], partial, flags + t, stream));
+  }
+  std::vector<int32_t> h_flags(T, 0);
+  HIP_TRY_DROP(hipMemcpyAsync(h_flags.data(), flags, sizeof(int32_t) * (size_t)T, hipMemcpyDeviceToHost, stream));
+  HIP_TRY_DROP(hipStreamSynchronize(stream));
+  int used = 0;
+  for (int t = 0; t < T; ++t) {
+    if (first[t] >= 0 && h_flags[t] != 0) first[t] = -1; // not order-preserving: the forward reads the array
+    used += first[t] >= 0;
+  }
+  int64_t* d_first = nullptr;
+  if (used > 0) {
+    hipError_t e = hipMalloc((void**)&d_first, sizeof(int64_t) * (size_t)T);
+    if (e == hipSuccess) e = hipMemcpy(d_first, first.data(), sizeof(int64_t) * (size_t)T, hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+      if (d_first) (void)hipFree(d_first);
+      drop();
+      return fail(FBGEMM_AMD_E_HIP, "rank offsets: %s", hipGetErrorString(e));
+    }
+    plan->d_rank_records = records;
+    records = nullptr;
+    plan->d_rank_offsets = d_first;
+    plan->rank_source = d_index_remappings;
+    plan->rank_bits = remap_bits;
+    plan->rank_tables = used;
+  }
+  drop();
+#undef HIP_TRY_DROP
+  return 0;
+}
+
+int32_t fbgemm_amd_tbe_plan_rank_tables(const fbgemm_amd_tbe_plan* plan) { return plan ? plan->rank_tables : -1; }
 
 int fbgemm_amd_tbe_plan_trim(fbgemm_amd_tbe_plan* plan) {
   if (!plan) return fail(FBGEMM_AMD_E_ARG, "plan is null");

@@ -107,6 +107,13 @@ struct __attribute__((aligned(16))) BagEntry {
   int64_t pad1;
 };
 
+// The pruned-row mapping of an order-preserving table, 32 logical rows per record
+// (remap_rank_kernels.hip): physical row = before + popcount(bits below the row's bit).
+struct __attribute__((aligned(8))) RankRecord {
+  uint32_t before; // kept rows in front of the record's first logical row
+  uint32_t bits;   // bit b: logical row 32 * record + b is kept
+};
+
 // One entry per wave: which table and which first position of the bag order.
 struct WaveWork {
   int32_t table;
@@ -125,6 +132,8 @@ struct LookupArgs {
                              // into `remap`, an empty range meaning "this table is not pruned"
   int64_t remap_rows;        // bound for logical ids when remap_offsets == nullptr
   int32_t remap64;           // remap entries are int64 (else int32)
+  const RankRecord* rank_records; // nullptr, or the compact form of the mappings of order-preserving tables
+  const int64_t* rank_offsets;    // T entries: first record of table t, or -1: the table's mapping is read from `remap`
   void* out;
   int64_t out_stride;        // elements between consecutive bags' outputs
   int64_t index_size;        // entries the index array holds for this call

@@ -123,7 +123,7 @@ __device__ __forceinline__ bool pool_bags(const LookupArgs& a, const TableDesc& 
   const int n = (int)len; // same for every lane of the bag
 
   // pruned tables: logical ids go through the table's slice of the remap array
-  int64_t remap_base = 0, remap_cap = 0;
+  int64_t remap_base = 0, remap_cap = 0, rank_base = -1;
   bool remapped = false;
   if (GENERAL && a.remap) {
     remapped = true;
@@ -132,6 +132,7 @@ __device__ __forceinline__ bool pool_bags(const LookupArgs& a, const TableDesc& 
       remap_base = a.remap_offsets[table];
       remap_cap = a.remap_offsets[table + 1] - remap_base;
       remapped = remap_cap > 0;
+      if (a.rank_records) rank_base = a.rank_offsets[table];
     }
   }
 
@@ -208,8 +209,14 @@ __device__ __forceinline__ bool pool_bags(const LookupArgs& a, const TableDesc& 
               if (pass == 0) report_index(a.status, pos);
               ok = false;
             } else {
-              row = a.remap64 ? reinterpret_cast<const int64_t*>(a.remap)[remap_base + row]
-                              : (int64_t) reinterpret_cast<const int32_t*>(a.remap)[remap_base + row];
+              if (rank_base >= 0) { // order-preserving mapping: the rank among the kept rows (remap_rank_kernels.hip)
+                const RankRecord rr = a.rank_records[rank_base + (row >> 5)];
+                const uint32_t bit = (uint32_t)row & 31u;
+                row = ((rr.bits >> bit) & 1u) ? (int64_t)(rr.before + (uint32_t)__builtin_popcount(rr.bits & ((1u << bit) - 1u))) : -1;
+              } else {
+                row = a.remap64 ? reinterpret_cast<const int64_t*>(a.remap)[remap_base + row]
+                                : (int64_t) reinterpret_cast<const int32_t*>(a.remap)[remap_base + row];
+              }
               ok = row != -1;
               if (ok && (row < 0 || row >= d.num_rows)) {
                 if (pass == 0) report_index(a.status, pos);

@@ -113,6 +113,7 @@ struct LeanLane {
   int n;          // entries of the bag
   int64_t pos0;   // position of its first entry in the index array
   int64_t remap_base, remap_cap; // pruned table: its slice of the remap array
+  int64_t rank_base;             // >= 0: the table's first rank record (its mapping is order-preserving)
   bool remapped;
 };
 
@@ -172,6 +173,7 @@ __device__ __forceinline__ LeanLane lean_lane(const LookupArgs& a, const TableDe
   L.n = (int)len;
   L.remap_base = 0;
   L.remap_cap = 0;
+  L.rank_base = -1;
   L.remapped = false;
   if (a.remap) {
     L.remapped = true;
@@ -180,6 +182,7 @@ __device__ __forceinline__ LeanLane lean_lane(const LookupArgs& a, const TableDe
       L.remap_base = a.remap_offsets[table];
       L.remap_cap = a.remap_offsets[table + 1] - L.remap_base;
       L.remapped = L.remap_cap > 0;
+      if (a.rank_records) L.rank_base = a.rank_offsets[table];
     }
   }
   return L;
@@ -215,6 +218,12 @@ __device__ __forceinline__ int64_t lean_remap(const LookupArgs& a, const LeanLan
   if (logical < 0 || logical >= L.remap_cap) {
     report_index(a.status, pos);
     return LEAN_PRUNED;
+  }
+  if (L.rank_base >= 0) { // order-preserving mapping: the physical row is the rank among the kept rows
+    const RankRecord r = a.rank_records[L.rank_base + (logical >> 5)];
+    const uint32_t bit = (uint32_t)logical & 31u;
+    if (!((r.bits >> bit) & 1u)) return LEAN_PRUNED;
+    return (int64_t)(r.before + (uint32_t)__builtin_popcount(r.bits & ((1u << bit) - 1u)));
   }
   const int64_t m = a.remap64 ? reinterpret_cast<const int64_t*>(a.remap)[L.remap_base + logical]
                               : (int64_t) reinterpret_cast<const int32_t*>(a.remap)[L.remap_base + logical];

@@ -255,6 +255,23 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(torch.nn.Module):
         kept = [m for m in index_remapping if m is not None]
         self.index_remappings_array = (torch.cat(kept).to(dtype=self.indices_dtype, device=dev) if kept
                                        else torch.empty(0, dtype=self.indices_dtype, device=dev))
+        # The lookups address a mapping slice per FEATURE (offsets[f], offsets[f + 1]), the arrays above hold
+        # one per TABLE, as the reference's do (its own pruned_array_lookup derives the batch size from them and
+        # so does not support features that share a pruned table). With shared tables the forward gets a
+        # per-feature copy of the slices; without, the very same tensors.
+        ftm = list(self.feature_table_map)
+        if ftm == list(range(len(self.embedding_specs))) or not kept:
+            self._feature_remap_array = self.index_remappings_array
+            self._feature_remap_offsets = (self.index_remappings_array_offsets if kept else
+                                           torch.zeros(len(ftm) + 1, device=dev, dtype=torch.int64))
+        else:
+            parts, foffs = [], [0]
+            for t in ftm:
+                if index_remapping[t] is not None:
+                    parts.append(index_remapping[t].to(dtype=self.indices_dtype, device=dev))
+                foffs.append(foffs[-1] + (index_remapping[t].numel() if index_remapping[t] is not None else 0))
+            self._feature_remap_array = torch.cat(parts)
+            self._feature_remap_offsets = torch.tensor(foffs, device=dev, dtype=torch.int64)
 
     def set_index_remappings(self, index_remapping, pruning_hash_load_factor=0.5, use_array_for_index_remapping=True):
         if use_array_for_index_remapping:
@@ -334,8 +351,7 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(torch.nn.Module):
             indices = ops.pruned_hashmap_lookup(indices, offsets, self.index_remapping_hash_table,
                                                 self.index_remapping_hash_table_offsets)
         elif arrayed and not fuse_remap:
-            indices = ops.pruned_array_lookup(indices, offsets, self.index_remappings_array,
-                                              self.index_remappings_array_offsets)
+            indices = ops.pruned_array_lookup(indices, offsets, self._feature_remap_array, self._feature_remap_offsets)
         if check:
             ops.bounds_check_indices(self.rows_per_table, indices, offsets, self.bounds_check_mode_int,
                                      self.bounds_check_warning, per_sample_weights)
@@ -345,5 +361,5 @@ class IntNBitTableBatchedEmbeddingBagsCodegen(torch.nn.Module):
             self.max_float32_D, indices, offsets, int(self.pooling_mode), per_sample_weights, self.output_dtype,
             row_alignment=self.row_alignment, max_float8_D=self.max_float8_D,
             fp8_exponent_bits=self.fp8_exponent_bits, fp8_exponent_bias=self.fp8_exponent_bias,
-            index_remappings=self.index_remappings_array if fuse_remap else None,
-            index_remappings_offsets=self.index_remappings_array_offsets if fuse_remap else None)
+            index_remappings=self._feature_remap_array if fuse_remap else None,
+            index_remappings_offsets=self._feature_remap_offsets if fuse_remap else None)

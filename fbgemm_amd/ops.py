@@ -20,6 +20,7 @@ from ._lib import SpmdmConfig, check
 
 FP32, FP16, INT8, INT4, INT2, BF16, FP8 = 0, 1, 2, 3, 4, 5, 6
 POOL_SUM, POOL_MEAN, POOL_NONE = 0, 1, 2
+ACC_EXACT, ACC_FAST = 0, 1  # how 4- and 8-bit rows are accumulated (include/fbgemm_amd.h)
 
 _OUT_TORCH = {FP32: torch.float32, FP16: torch.float16, BF16: torch.bfloat16}
 _TORCH_OUT = {v: k for k, v in _OUT_TORCH.items()}
@@ -212,6 +213,28 @@ class TbePlan:
     def num_rows(self, t):
         return _lib.lib().fbgemm_amd_tbe_plan_num_rows(self.handle, t)
 
+    def set_accumulate(self, mode):
+        """ACC_EXACT (the reference's sequence of roundings, the default) or ACC_FAST (tolerance grade)."""
+        check(_lib.lib().fbgemm_amd_tbe_plan_set_accumulate(self.handle, int(mode)))
+
+    def set_index_remappings(self, index_remappings, index_remappings_offsets):
+        """Build the compact form of order-preserving pruned-row mappings (2 bits per logical
+        row) that the fused remap of the forward then uses whenever it is passed this very
+        array. Made again when the array or its contents change (tensor version)."""
+        if index_remappings is None or index_remappings.numel() == 0:
+            check(_lib.lib().fbgemm_amd_tbe_plan_set_index_remappings(self.handle, None, 32, None, 0, _stream()))
+            self._rank_key = None
+            return 0
+        ro = index_remappings_offsets.detach().to("cpu", torch.int64).contiguous()
+        check(_lib.lib().fbgemm_amd_tbe_plan_set_index_remappings(
+            self.handle, _ptr(index_remappings), _bits(index_remappings), _ptr(ro), ro.numel(), _stream()))
+        self._rank_key = (index_remappings.data_ptr(), index_remappings._version, index_remappings.numel())
+        self._rank_keepalive = index_remappings
+        return self.rank_tables()
+
+    def rank_tables(self):
+        return _lib.lib().fbgemm_amd_tbe_plan_rank_tables(self.handle)
+
     def row_bytes(self, t):
         return _lib.lib().fbgemm_amd_tbe_plan_row_bytes(self.handle, t)
 
@@ -324,12 +347,20 @@ def int_nbit_split_embedding_codegen_lookup_function(
     ro = None
     if index_remappings is not None:
         _require_cuda(index_remappings, index_remappings_offsets)
+        if index_remappings_offsets.numel() != T + 1:
+            raise ValueError(f"index_remappings_offsets holds {index_remappings_offsets.numel()} entries; the operator's "
+                             f"{T} features need {T + 1} (one mapping slice per feature)")
         ro = index_remappings_offsets.to(torch.int64).contiguous()
+        # the compact form of order-preserving mappings, made once per array (and again when it changes)
+        key = (index_remappings.data_ptr(), index_remappings._version, index_remappings.numel())
+        if getattr(plan, "_rank_key", None) != key and not torch.cuda.is_current_stream_capturing():
+            plan.set_index_remappings(index_remappings, ro)
     check(_lib.lib().fbgemm_amd_tbe_forward_pruned(
         plan.handle, _ptr(dev_weights), _ptr(uvm_weights), _ptr(indices.contiguous()),
         _ptr(offsets.contiguous()), _bits(indices), indices.numel(), offsets.numel(), pooling_mode,
         _ptr(indice_weights), output_dtype, _ptr(out), _ptr(index_remappings),
-        32 if index_remappings is None else _bits(index_remappings), _ptr(ro), _ptr(st.buf), _stream()))
+        32 if index_remappings is None else _bits(index_remappings), _ptr(ro), 0 if ro is None else ro.numel(),
+        _ptr(st.buf), _stream()))
     if own:
         bits, pos = st.read()
         if bits:

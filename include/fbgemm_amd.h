@@ -224,15 +224,35 @@ int fbgemm_amd_tbe_forward(
  * fbgemm_amd_pruned_array_lookup followed by fbgemm_amd_tbe_forward (the order
  * of split_table_batched_embeddings_ops_inference.py:1067-1152) without the
  * round trip of the dense indices through HBM. A logical id outside its
- * mapping is reported as out of range. No counterpart as one call in the
- * reference. */
+ * mapping is reported as out of range. index_remappings_offsets_numel must be
+ * T + 1 with T the plan's tables (the operator's features). No counterpart as
+ * one call in the reference. */
 int fbgemm_amd_tbe_forward_pruned(
     fbgemm_amd_tbe_plan* plan, const void* d_dev_weights, const void* d_uvm_weights,
     const void* d_indices, const void* d_offsets, int32_t index_bits,
     int64_t indices_numel, int64_t offsets_numel, int32_t pooling_mode,
     const float* d_indice_weights, int32_t output_ty, void* d_output,
     const void* d_index_remappings, int32_t remap_bits,
-    const int64_t* d_index_remappings_offsets, void* d_status, void* stream);
+    const int64_t* d_index_remappings_offsets, int64_t index_remappings_offsets_numel,
+    void* d_status, void* stream);
+
+/* A compact form of the mappings for the call above. No counterpart in the
+ * reference. For every table whose mapping is order-preserving (its kept rows
+ * are numbered 0, 1, 2, ... in logical order: what embedding_bag_rowwise_prune
+ * and the inference converter produce) the plan builds, on the device, 2 bits per
+ * logical row (a kept-row bitmap with a running count per 32 rows) and the
+ * forwards compute the physical row from that instead of fetching a 4- or 8-byte
+ * entry of a table-sized array: the same integers, from a structure that fits
+ * the caches. Tables whose mapping is anything else keep reading the array.
+ * d_index_remappings / remap_bits as in the forward; index_remappings_offsets is
+ * the HOST copy of the T+1 offsets. The forwards use the records whenever they
+ * are passed the same d_index_remappings pointer; call this again after the
+ * array's contents change (NULL array = drop the records). Allocates; synchronizes
+ * `stream`. fbgemm_amd_tbe_plan_rank_tables returns how many tables use records. */
+int fbgemm_amd_tbe_plan_set_index_remappings(
+    fbgemm_amd_tbe_plan* plan, const void* d_index_remappings, int32_t remap_bits,
+    const int64_t* index_remappings_offsets, int64_t index_remappings_offsets_numel, void* stream);
+int32_t fbgemm_amd_tbe_plan_rank_tables(const fbgemm_amd_tbe_plan* plan);
 
 /* Select FBGEMM_AMD_ACC_EXACT (the default of a new plan) or FBGEMM_AMD_ACC_FAST
  * for the forwards of a plan. No counterpart in the reference. */

@@ -96,3 +96,4 @@ def test_workload_generators_are_seeded():
     assert p2.row_bytes() == 68 and np.diff(p2.host_offsets).min() >= 1 and np.diff(p2.host_offsets).max() <= 40
     p4 = bc.config4("cpu", 0.001, tables=2)
     assert p4[0].row_bytes() == 36 and abs((p4[0].host_remap == -1).mean() - 0.5) < 0.1
+

@@ -226,3 +226,41 @@ def test_module_with_managed_tables(M, oracle):
         assert torch.equal(m(cu(idx), cu(off)), want)
     with pytest.raises(NotImplementedError):
         M.IntNBitTableBatchedEmbeddingBagsCodegen([shapes[0] + (L.MANAGED_CACHING,)])
+
+
+@pytest.mark.parametrize("mode", ["NONE", "WARNING"])
+def test_module_pruned_tables_shared_by_features(M, oracle, mode):
+    """Features that share a pruned table: every feature's lookups go through its table's mapping
+    (fused into the forward without bounds check, as a separate pruned_array_lookup with one)."""
+    rng = np.random.default_rng(401)
+    S, L = M.SparseType, M.EmbeddingLocation.DEVICE
+    logical = [400, 250, 320]
+    ftm = [0, 1, 0, 2, 2, 1]
+    remaps, phys = [], []
+    for t, n in enumerate(logical):
+        if t == 1:
+            remaps.append(None)
+            phys.append(n)
+            continue
+        keep = rng.random(n) < 0.6
+        r = np.full(n, -1, np.int32)
+        r[keep] = np.arange(int(keep.sum()))
+        remaps.append(torch.from_numpy(r))
+        phys.append(int(keep.sum()))
+    specs = [(f"t{t}", phys[t], [64, 128, 32][t], S.INT4, L) for t in range(3)]
+    m = M.IntNBitTableBatchedEmbeddingBagsCodegen(
+        specs, feature_table_map=ftm, index_remapping=remaps, pooling_mode=M.PoolingMode.SUM,
+        bounds_check_mode=M.BoundsCheckMode[mode], output_dtype=S.FP16, indices_dtype=torch.int64)
+    m.quantize_and_assign([torch.from_numpy(rng.normal(0, 1, size=(n, d)).astype(np.float32))
+                           for n, (_, _, d, _, _) in zip(phys, specs)])
+    B = 17
+    idx, off = make_inputs(rng, [logical[t] for t in ftm], B, 12, np.int64)
+    got = m(cu(idx), cu(off))
+    dense = idx.copy()
+    for f, t in enumerate(ftm):
+        s, e = int(off[f * B]), int(off[(f + 1) * B])
+        if remaps[t] is not None:
+            dense[s:e] = remaps[t].numpy()[idx[s:e]]
+    rc, want = oracle_forward(oracle, m, dense, off, 0, None, FP16)
+    assert rc == 0
+    H.assert_same_bits(bits_of(got, FP16), want, f"shared pruned tables, mode={mode}")

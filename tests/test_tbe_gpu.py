@@ -610,3 +610,85 @@ def test_special_values_in_the_table_batched_forward(ops, oracle, long_bags):
                 rc, want = oracle.tbe_forward(weights, wo, tys, D_offsets, total_D, idx, off, pooling, w, out_ty, 16)
                 assert rc == 0
                 same_bits_or_both_nan(got, want, f"special values weighted={w is not None} pooling={pooling} {name}")
+
+
+def _monotone_mapping(rng, logical, keep_frac, dt):
+    keep = rng.random(logical) < keep_frac
+    m = np.full(logical, -1, dt)
+    m[keep] = np.arange(int(keep.sum()), dtype=dt)
+    return m, int(keep.sum())
+
+
+@pytest.mark.parametrize("rdt", [np.int32, np.int64])
+def test_rank_records_replace_order_preserving_mappings(ops, oracle, rdt):
+    """The compact form of the pruned-row mappings (a kept-row bitmap with running counts): taken
+    for the tables whose mapping numbers the kept rows in logical order, not for a table whose
+    mapping does anything else, and never a different result than the array gives (integers)."""
+    rng = np.random.default_rng(77)
+    logical = [1000, 37, 5000, 64, 2049, 300]
+    maps, specs = [], []
+    for t, n in enumerate(logical):
+        if t == 3:
+            maps.append(np.zeros(0, rdt))  # this table is not pruned
+            specs.append((n, 64, INT4))
+            continue
+        m, kept = _monotone_mapping(rng, n, [0.5, 1.0, 0.3, 0, 0.0, 0.7][t], rdt)
+        if t == 5:  # two kept rows swapped: a valid mapping, but not order-preserving
+            k = np.nonzero(m >= 0)[0]
+            m[k[3]], m[k[9]] = m[k[9]], m[k[3]]
+        maps.append(m)
+        specs.append((max(kept, 1), [64, 128, 256, 64, 32, 128][t], [INT4, INT8, INT4, INT4, FP16, INT4][t]))
+    T, B = len(specs), 33
+    weights, wo, _ = build_weights(rng, specs, 16)
+    remap = np.concatenate(maps)
+    remap_off = np.concatenate([[0], np.cumsum([len(m) for m in maps])]).astype(np.int64)
+    lens = rng.integers(0, 25, size=T * B)
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    idx = np.concatenate([rng.integers(0, logical[t], size=int(lens[t * B:(t + 1) * B].sum())) for t in range(T)]).astype(np.int64)
+    dense = oracle.pruned_array_lookup(idx, off, remap, remap_off)
+    tys = np.array([s[2] for s in specs], np.uint8)
+    D_offsets = np.concatenate([[0], np.cumsum([s[1] for s in specs])]).astype(np.int32)
+    total_D = int(D_offsets[-1])
+    meta = (cu(weights), torch.zeros(0, dtype=torch.uint8, device="cuda"), cu(np.zeros(T, np.int32)), cu(wo), cu(tys), cu(D_offsets))
+    plan = ops.TbePlan(torch.from_numpy(wo), torch.from_numpy(tys), torch.from_numpy(D_offsets), torch.zeros(T, dtype=torch.int32),
+                       len(weights), 0, 16)
+    d_remap, d_remap_off = cu(remap), cu(remap_off)
+    assert plan.set_index_remappings(d_remap, d_remap_off) == 4  # tables 0, 1, 2, 4; not 3 (none) and 5 (swapped)
+    call = lambda: ops.int_nbit_split_embedding_codegen_lookup_function(
+        *meta, total_D, 0, 256, 128, 32, 0, cu(idx), cu(off), 1, None, FP32, row_alignment=16, plan=plan,
+        index_remappings=d_remap, index_remappings_offsets=d_remap_off).cpu().numpy()
+    with_records = call()
+    rc, want = oracle.tbe_forward(weights, wo, tys, D_offsets, total_D, dense, off, 1, None, FP32, 16)
+    assert rc == 0
+    H.assert_same_bits(with_records, want, "rank records")
+    plan.set_index_remappings(None, None)
+    plan._rank_key = (d_remap.data_ptr(), d_remap._version, d_remap.numel())  # keep the wrapper from rebuilding them
+    assert plan.rank_tables() == 0
+    H.assert_same_bits(call(), want, "mapping arrays")
+
+
+def test_remap_offsets_must_cover_every_feature(ops):
+    rng = np.random.default_rng(78)
+    specs = [(50, 64, INT4), (60, 64, INT4), (70, 64, INT4)]
+    weights, wo, _ = build_weights(rng, specs, 16)
+    tys = np.array([s[2] for s in specs], np.uint8)
+    D_offsets = (np.arange(4) * 64).astype(np.int32)
+    off = (np.arange(3 * 4 + 1) * 2).astype(np.int64)
+    idx = rng.integers(0, 50, size=24).astype(np.int64)
+    remap = np.arange(100, dtype=np.int32)
+    with pytest.raises(ValueError, match="features need 4"):
+        ops.int_nbit_split_embedding_codegen_lookup_function(
+            cu(weights), torch.zeros(0, dtype=torch.uint8, device="cuda"), cu(np.zeros(3, np.int32)), cu(wo), cu(tys),
+            cu(D_offsets), 192, 0, 64, 0, 0, 0, cu(idx), cu(off), 0, None, FP32, row_alignment=16,
+            index_remappings=cu(remap), index_remappings_offsets=cu(np.array([0, 50, 100], np.int64)))
+    # and the C entry point itself refuses it (callers that bind the library directly)
+    import ctypes as C
+    from fbgemm_amd import _lib
+    plan = ops.TbePlan(torch.from_numpy(wo), torch.from_numpy(tys), torch.from_numpy(D_offsets), torch.zeros(3, dtype=torch.int32),
+                       len(weights), 0, 16)
+    d = [cu(weights), cu(idx), cu(off), cu(remap), cu(np.array([0, 50, 100], np.int64)), torch.empty(4, 192, device="cuda")]
+    st = ops.Status()
+    p = lambda t: C.c_void_p(t.data_ptr())
+    rc = _lib.lib().fbgemm_amd_tbe_forward_pruned(plan.handle, p(d[0]), None, p(d[1]), p(d[2]), 64, 24, 13, 0, None, 0, p(d[5]),
+                                                  p(d[3]), 32, p(d[4]), 3, p(st.buf), None)
+    assert rc == -1 and b"need 4" in _lib.lib().fbgemm_amd_last_error()
