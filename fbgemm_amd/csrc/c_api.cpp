@@ -37,6 +37,11 @@ hipError_t launch_inplace_update(const TableDesc* tables, int32_t T, uint8_t* w0
 hipError_t launch_remap_row_idx(const void* rows, bool idx64, const int32_t* table_idx, const void* remap, bool remap64,
                                 const int64_t* remap_offsets, int32_t T, int64_t n, void* dense, hipStream_t stream);
 int64_t prune_partials(int64_t rows);
+hipError_t launch_split_offsets(const void* offsets, bool off64, int64_t bags, int32_t K, bool relative, int64_t index_size,
+                                int64_t* voff, Status* status, hipStream_t stream);
+hipError_t launch_combine_segments(const float* partial, int64_t partial_stride, int32_t B, int32_t K, int32_t T,
+                                   const int32_t* D_offsets, int32_t single_D, const void* offsets, bool off64, bool normalize,
+                                   void* out, int32_t out_ty, int64_t out_stride, hipStream_t stream);
 int64_t remap_rank_words(int64_t rows);
 int64_t remap_rank_partials(int64_t rows);
 hipError_t launch_remap_rank_build(const void* mapping, bool remap64, int64_t rows, RankRecord* records, int64_t* partial,
@@ -276,7 +281,22 @@ struct DeviceScratch {
   int64_t fixed_cap = 0;
   int64_t* partial = nullptr; // bounds check: per-block maxima of the offset scan
   int64_t partial_cap = 0;
+  int64_t* seg_offsets = nullptr; // split bags: where every segment starts
+  int64_t seg_offsets_cap = 0;
+  float* seg_partial = nullptr;   // split bags: the segments' fp32 sums
+  int64_t seg_partial_cap = 0;
 };
+
+// Few, long bags (tolerance-grade accumulate only): the number of segments a bag is cut into so that
+// the launch has enough waves to fill the device. `waves` = what the launch would have, `avg_len` =
+// entries per bag on average. 1 = no split.
+int split_factor(int64_t waves, int64_t avg_len) {
+  static const int enabled = env_int("FBGEMM_AMD_SPLIT_BAGS", 1);
+  if (!enabled || waves >= 256 || avg_len < 32) return 1;
+  int K = 2;
+  while (K < 32 && K * 2 * 8 <= avg_len && waves * K < 1024) K *= 2; // segments of 8 rows at least
+  return K;
+}
 
 // Grow-only device buffer; the old one may still be read by an enqueued kernel.
 template <typename T>
@@ -533,10 +553,19 @@ int spmdm_launch_impl(
     return 0;
   }
   plan_lanes(d, (uintptr_t)d_input, out_stride, has_sb, false);
+  // few, long bags, and the caller accepts sums in another order: cut every bag into K segments
+  int K = 1;
+  if (!noalloc && cfg->accumulate == FBGEMM_AMD_ACC_FAST && !cfg->is_weight_positional && output_size * 32 <= 0x7fffffffLL) {
+    const int G16 = bags_per_wave(d.lanes, d.packed);
+    K = split_factor((output_size + G16 - 1) / G16, index_size / output_size);
+  }
+  const int64_t pooled_bags = output_size * K;       // what the lookup kernel sees as bags
+  const int64_t pooled_stride = K > 1 ? D : out_stride; // segments' sums are rows of D floats
+  if (K > 1) plan_lanes(d, (uintptr_t)d_input, pooled_stride, has_sb, false);
   {
     // a launch of fewer than four waves per compute unit: prefer narrow lanes
     const int G16 = bags_per_wave(d.lanes, d.packed);
-    if (d.vb == 16 && (output_size + G16 - 1) / G16 < narrow_below_waves()) plan_lanes(d, (uintptr_t)d_input, out_stride, has_sb, false, true);
+    if (d.vb == 16 && (pooled_bags + G16 - 1) / G16 < narrow_below_waves()) plan_lanes(d, (uintptr_t)d_input, pooled_stride, has_sb, false, true);
   }
   d.lanes_recip = (65536 + d.lanes - 1) / d.lanes;
     d.bags = bags_per_wave(d.lanes, d.packed);
@@ -569,7 +598,7 @@ int spmdm_launch_impl(
 
   // Ordering the bags pays once several waves' worth of bags and enough lookups exist
   // (the scheduler launch costs 6-8 us and buys ~5 % of the lookup: it pays from a few million lookups on)
-  const bool sort = sort_bags_default() && output_size > 2 * G && index_size >= (int64_t)SORT_MIN_LOOKUPS;
+  const bool sort = K == 1 && sort_bags_default() && output_size > 2 * G && index_size >= (int64_t)SORT_MIN_LOOKUPS;
   if (cfg->use_offsets) {
     a.offsets = d_offsets_or_lengths;
     a.off64 = cfg->offset_bits == 64;
@@ -607,6 +636,31 @@ int spmdm_launch_impl(
       HIP_TRY(launch_bag_order(a.offsets, a.off64, (int32_t)output_size, 1, s->order, stream));
       a.order = s->order;
     }
+  }
+  if (K > 1) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    DeviceScratch* s;
+    if (int rc = get_scratch(&s)) return rc;
+    if (int rc = grow(&s->seg_offsets, &s->seg_offsets_cap, pooled_bags + 1, stream)) return rc;
+    if (int rc = grow(&s->seg_partial, &s->seg_partial_cap, pooled_bags * D, stream)) return rc;
+    HIP_TRY(launch_split_offsets(a.offsets, a.off64, output_size, K, true, index_size, s->seg_offsets, (Status*)d_status, stream));
+    LookupArgs v = a;
+    v.offsets = s->seg_offsets;
+    v.off64 = 1;
+    v.order = nullptr;
+    v.B = (int32_t)pooled_bags;
+    v.out = s->seg_partial;
+    v.out_stride = D;
+    v.out_ty = ST_FP32;
+    v.normalize = 0;
+    v.check_total = 0;
+    v.out_aligned = 1;
+    v.num_waves = (pooled_bags + G - 1) / G;
+    if (lean_enabled() && lean_shape(d)) HIP_TRY(launch_lookup_lean(v, cfg->index_bits == 64, false, stream));
+    else HIP_TRY(launch_lookup(v, cfg->index_bits == 64, stream));
+    HIP_TRY(launch_combine_segments(s->seg_partial, D, (int32_t)output_size, K, 1, nullptr, (int32_t)D, a.offsets, a.off64 != 0,
+                                    cfg->normalize_by_lengths != 0, d_out, cfg->output_ty, out_stride, stream));
+    return 0;
   }
   if (lean_enabled() && !cfg->is_weight_positional && lean_shape(d))
     HIP_TRY(launch_lookup_lean(a, cfg->index_bits == 64, cfg->accumulate != FBGEMM_AMD_ACC_FAST, stream));
@@ -684,6 +738,10 @@ struct fbgemm_amd_tbe_plan {
   int32_t max_D = 0;
   float* pooled_tmp = nullptr;    // fp32 [B, total_D] the 8-bit pooled output is quantized from
   int64_t pooled_tmp_cap = 0;
+  int64_t* seg_offsets = nullptr; // split bags: where every segment starts (T*B*K + 1)
+  int64_t seg_offsets_cap = 0;
+  float* seg_partial = nullptr;   // split bags: the segments' fp32 sums [B*K, total_D]
+  int64_t seg_partial_cap = 0;
   // the same tables with bags laid end to end where that saves a request per row
   // (see bags_per_wave); empty when no table has such a shape. Used for long bags.
   std::vector<TableDesc> tables_packed;
@@ -956,6 +1014,8 @@ void fbgemm_amd_tbe_plan_destroy(fbgemm_amd_tbe_plan* plan) {
   if (plan->d_tables_narrow) (void)hipFree(plan->d_tables_narrow);
   if (plan->d_D_offsets) (void)hipFree(plan->d_D_offsets);
   if (plan->pooled_tmp) (void)hipFree(plan->pooled_tmp);
+  if (plan->seg_offsets) (void)hipFree(plan->seg_offsets);
+  if (plan->seg_partial) (void)hipFree(plan->seg_partial);
   if (plan->d_rank_records) (void)hipFree(plan->d_rank_records);
   if (plan->d_rank_offsets) (void)hipFree(plan->d_rank_offsets);
   for (hipEvent_t e : plan->prof_ev) (void)hipEventDestroy(e);
@@ -992,13 +1052,18 @@ int fbgemm_amd_tbe_forward(
                                        d_output, nullptr, 32, nullptr, 0, d_status, stream_);
 }
 
-int fbgemm_amd_tbe_forward_pruned(
+} // extern "C"
+
+namespace {
+// The forward behind fbgemm_amd_tbe_forward[_pruned]. offset_bits: the width of d_offsets (the
+// operator's offsets have the width of its indices; the segment offsets of split bags are int64).
+int tbe_forward_impl(
     fbgemm_amd_tbe_plan* plan, const void* d_dev_weights, const void* d_uvm_weights,
-    const void* d_indices, const void* d_offsets, int32_t index_bits,
+    const void* d_indices, const void* d_offsets, int32_t index_bits, int32_t offset_bits,
     int64_t indices_numel, int64_t offsets_numel, int32_t pooling_mode,
     const float* d_indice_weights, int32_t output_ty, void* d_output,
     const void* d_index_remappings, int32_t remap_bits, const int64_t* d_index_remappings_offsets,
-    int64_t index_remappings_offsets_numel, void* d_status, void* stream_) {
+    int64_t index_remappings_offsets_numel, void* d_status, void* stream_, bool allow_split) {
   if (!plan) return fail(FBGEMM_AMD_E_ARG, "plan is null");
   if (d_index_remappings && (!d_index_remappings_offsets || (remap_bits != 32 && remap_bits != 64)))
     return fail(FBGEMM_AMD_E_ARG, "a remap array needs its T+1 offsets and 32- or 64-bit entries");
@@ -1022,10 +1087,10 @@ int fbgemm_amd_tbe_forward_pruned(
       if (int rc = grow(&plan->pooled_tmp, &plan->pooled_tmp_cap, B * plan->total_D, (hipStream_t)stream_)) return rc;
       tmp = plan->pooled_tmp;
     }
-    if (int rc = fbgemm_amd_tbe_forward_pruned(plan, d_dev_weights, d_uvm_weights, d_indices, d_offsets, index_bits,
-                                               indices_numel, offsets_numel, pooling_mode, d_indice_weights, ST_FP32, tmp,
-                                               d_index_remappings, remap_bits, d_index_remappings_offsets,
-                                               index_remappings_offsets_numel, d_status, stream_))
+    if (int rc = tbe_forward_impl(plan, d_dev_weights, d_uvm_weights, d_indices, d_offsets, index_bits, offset_bits,
+                                  indices_numel, offsets_numel, pooling_mode, d_indice_weights, ST_FP32, tmp,
+                                  d_index_remappings, remap_bits, d_index_remappings_offsets,
+                                  index_remappings_offsets_numel, d_status, stream_, allow_split))
       return rc;
     HIP_TRY(launch_quantize_segments(tmp, B, plan->T, plan->d_D_offsets, (int32_t)plan->total_D, plan->max_D,
                                      (uint8_t*)d_output, (hipStream_t)stream_));
@@ -1050,6 +1115,39 @@ int fbgemm_amd_tbe_forward_pruned(
   hipStream_t stream = (hipStream_t)stream_;
   if (plan->has_fp8 && plan->fp8_shift == 0)
     return fail(FBGEMM_AMD_E_ARG, "the plan holds FP8 tables: set their exponent bits and bias first (fbgemm_amd_tbe_plan_set_fp8)");
+
+  // Few, long bags, and the plan accepts sums in another order: every bag is cut into K segments that
+  // are pooled as bags of their own into fp32 partial sums, which a second launch adds up in order.
+  if (allow_split && plan->accumulate == FBGEMM_AMD_ACC_FAST && (int64_t)B * 32 <= 0x7fffffffLL) {
+    int64_t wide_waves = 0;
+    for (const TableDesc& d : plan->tables) wide_waves += (B + d.bags - 1) / d.bags;
+    const int K = split_factor(wide_waves, indices_numel / ((int64_t)plan->T * B));
+    if (K > 1) {
+      hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+      (void)hipStreamIsCapturing(stream, &cap);
+      const int64_t vbags = (int64_t)plan->T * B * K;
+      int64_t* voff;
+      float* partial;
+      {
+        std::lock_guard<std::mutex> lk(plan->mu);
+        const bool fits = plan->seg_offsets_cap >= vbags + 1 && plan->seg_partial_cap >= (int64_t)B * K * plan->total_D;
+        if (!fits && cap != hipStreamCaptureStatusNone)
+          return fail(FBGEMM_AMD_E_ARG, "the first forward of this size allocates the scratch of split bags: run it once outside the stream capture");
+        if (int rc = grow(&plan->seg_offsets, &plan->seg_offsets_cap, vbags + 1, stream)) return rc;
+        if (int rc = grow(&plan->seg_partial, &plan->seg_partial_cap, (int64_t)B * K * plan->total_D, stream)) return rc;
+        voff = plan->seg_offsets;
+        partial = plan->seg_partial;
+      }
+      HIP_TRY(launch_split_offsets(d_offsets, offset_bits == 64, (int64_t)plan->T * B, K, false, indices_numel, voff, (Status*)d_status, stream));
+      if (int rc = tbe_forward_impl(plan, d_dev_weights, d_uvm_weights, d_indices, voff, index_bits, 64, indices_numel, vbags + 1,
+                                    FBGEMM_AMD_POOL_SUM, d_indice_weights, ST_FP32, partial, d_index_remappings, remap_bits,
+                                    d_index_remappings_offsets, index_remappings_offsets_numel, d_status, stream_, false))
+        return rc;
+      HIP_TRY(launch_combine_segments(partial, plan->total_D, B, K, plan->T, plan->d_D_offsets, 0, d_offsets, offset_bits == 64,
+                                      pooling_mode == FBGEMM_AMD_POOL_MEAN, d_output, output_ty, plan->total_D, stream));
+      return 0;
+    }
+  }
 
   // Bags laid end to end save a line request per row and cost about a fifth more
   // arithmetic on the tables they apply to. With short bags the per-bag work
@@ -1158,7 +1256,7 @@ int fbgemm_amd_tbe_forward_pruned(
   a.weights[1] = (const uint8_t*)d_uvm_weights;
   a.indices = d_indices;
   a.offsets = d_offsets;
-  a.off64 = index_bits == 64;
+  a.off64 = offset_bits == 64;
   a.sample_weights = d_indice_weights;
   a.remap = d_index_remappings;
   a.remap_offsets = d_index_remappings ? d_index_remappings_offsets : nullptr;
@@ -1180,7 +1278,7 @@ int fbgemm_amd_tbe_forward_pruned(
   a.fp8_shift = plan->fp8_shift;
   a.fp8_mult = plan->fp8_mult;
   if (sort_bags_default() && indices_numel >= (int64_t)SORT_MIN_LOOKUPS) {
-    HIP_TRY(launch_bag_order(d_offsets, index_bits == 64, B, plan->T, w.d_order[order_slot], stream));
+    HIP_TRY(launch_bag_order(d_offsets, offset_bits == 64, B, plan->T, w.d_order[order_slot], stream));
     a.order = w.d_order[order_slot];
   }
   const size_t slots = plan->prof_ev.size() / 2;
@@ -1204,6 +1302,21 @@ int fbgemm_amd_tbe_forward_pruned(
   }
   return 0;
 }
+} // namespace
+
+extern "C" {
+
+int fbgemm_amd_tbe_forward_pruned(
+    fbgemm_amd_tbe_plan* plan, const void* d_dev_weights, const void* d_uvm_weights,
+    const void* d_indices, const void* d_offsets, int32_t index_bits,
+    int64_t indices_numel, int64_t offsets_numel, int32_t pooling_mode,
+    const float* d_indice_weights, int32_t output_ty, void* d_output,
+    const void* d_index_remappings, int32_t remap_bits, const int64_t* d_index_remappings_offsets,
+    int64_t index_remappings_offsets_numel, void* d_status, void* stream) {
+  return tbe_forward_impl(plan, d_dev_weights, d_uvm_weights, d_indices, d_offsets, index_bits, index_bits, indices_numel,
+                          offsets_numel, pooling_mode, d_indice_weights, output_ty, d_output, d_index_remappings, remap_bits,
+                          d_index_remappings_offsets, index_remappings_offsets_numel, d_status, stream, true);
+}
 
 int fbgemm_amd_tbe_plan_set_accumulate(fbgemm_amd_tbe_plan* plan, int32_t mode) {
   if (!plan) return fail(FBGEMM_AMD_E_ARG, "plan is null");
@@ -1223,7 +1336,9 @@ int fbgemm_amd_tbe_plan_set_index_remappings(
   // forget what was made from an earlier array (after the forwards that may still read it)
   if (plan->d_rank_records || plan->d_rank_offsets) {
     HIP_TRY(hipDeviceSynchronize());
-    if (plan->d_rank_records) (void)hipFree(plan->d_rank_records);
+    if (plan->seg_offsets) (void)hipFree(plan->seg_offsets);
+  if (plan->seg_partial) (void)hipFree(plan->seg_partial);
+  if (plan->d_rank_records) (void)hipFree(plan->d_rank_records);
     if (plan->d_rank_offsets) (void)hipFree(plan->d_rank_offsets);
     plan->d_rank_records = nullptr;
     plan->d_rank_offsets = nullptr;

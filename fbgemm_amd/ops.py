@@ -71,7 +71,7 @@ def _make_kernel(weight_ty, block_size, normalize_by_lengths, is_weight_position
                  output_stride, input_stride, scale_bias_last, output_ty, has_weight, sparse, no_bag=False,
                  fp8=(0, 0)):
     def kernel(output_size, index_size, data_size, input, indices, offsets_or_lengths, weights, out,
-               compressed_indices_table=None, status=None):
+               compressed_indices_table=None, status=None, accumulate=ACC_EXACT):
         _require_cuda(input, indices, offsets_or_lengths, weights, out, compressed_indices_table)
         if sparse and compressed_indices_table is None:
             raise ValueError("row-wise-sparse kernels need compressed_indices_table")
@@ -89,7 +89,7 @@ def _make_kernel(weight_ty, block_size, normalize_by_lengths, is_weight_position
             normalize_by_lengths=int(normalize_by_lengths),
             is_weight_positional=int(is_weight_positional), use_offsets=int(use_offsets),
             scale_bias_last=int(scale_bias_last), no_bag=int(no_bag), fp8_exponent_bits=fp8[0],
-            fp8_exponent_bias=fp8[1])
+            fp8_exponent_bias=fp8[1], accumulate=int(accumulate))
         lib = _lib.lib()
         if status is not None:
             check(lib.fbgemm_amd_spmdm_launch(
@@ -275,7 +275,7 @@ def int_nbit_split_embedding_codegen_lookup_function(
         offsets, pooling_mode, indice_weights=None, output_dtype=FP16, lxu_cache_weights=None,
         lxu_cache_locations=None, row_alignment=None, max_float8_D=0, fp8_exponent_bits=-1,
         fp8_exponent_bias=-1, status=None, plan=None, index_remappings=None,
-        index_remappings_offsets=None):
+        index_remappings_offsets=None, accumulate=None):
     """Same arguments, in the same order, as the reference operator
     (embedding_forward_quantized_host_cpu.cpp:316-318). Returns [B, total_D].
 
@@ -284,7 +284,10 @@ def int_nbit_split_embedding_codegen_lookup_function(
 
     ``index_remappings`` / ``index_remappings_offsets`` (the arguments of
     ``pruned_array_lookup``) fuse the pruned-row remap into the forward:
-    ``indices`` are then logical ids."""
+    ``indices`` are then logical ids.
+
+    ``accumulate`` = ACC_EXACT / ACC_FAST sets the plan's arithmetic for this and
+    later forwards (None leaves it as it is; a new plan is exact)."""
     _require_cuda(dev_weights, indices, offsets, indice_weights)
     if lxu_cache_locations is not None and lxu_cache_locations.numel() > 0:
         raise NotImplementedError("the LXU cache is not on this path: tables are resident in HBM")
@@ -331,6 +334,8 @@ def int_nbit_split_embedding_codegen_lookup_function(
         plan = _plan_for(dev_weights, uvm_weights, weights_placements, weights_offsets, weights_tys,
                          D_offsets, row_alignment)
     _set_fp8(plan, max_float8_D, fp8_exponent_bits, fp8_exponent_bias)
+    if accumulate is not None:
+        plan.set_accumulate(accumulate)
     T = plan.T
     if total_D != plan.total_D:
         raise ValueError(f"total_D {total_D} does not match D_offsets[-1] {plan.total_D}")

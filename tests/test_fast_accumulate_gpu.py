@@ -1,0 +1,203 @@
+"""The tolerance-grade accumulate mode (FBGEMM_AMD_ACC_FAST) against the oracle.
+
+In this mode the biases of a bag are summed apart from the scaled elements and
+bags of a launch too small to fill the device are cut into segments whose
+partial sums are added afterwards, so the fp32 roundings are not the
+reference's. The stated bound of the path: fp32 output within 1e-5 relative,
+fp16 / bf16 output within one unit in the last place. "Relative" is taken
+against the larger of |expected| and the largest magnitude in the bag's output
+row: a sum that cancels to nearly zero is held to the size of what was summed
+(for 16-bit outputs too: an element a thousand times smaller than its row may
+be off by more than one of ITS last places and still within 1e-5 of the row).
+Each test prints the worst error it met. The default mode stays bit-exact and
+is what every other test file checks."""
+import numpy as np
+import pytest
+
+import helpers as H
+from helpers import BF16, FP16, FP32, INT2, INT4, INT8
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    assert torch.cuda.is_available()
+    import fbgemm_amd.ops as o
+    return o
+
+
+@pytest.fixture(autouse=True, params=["wide", "default"])
+def lanes(request):
+    """Test-sized launches would take 4-byte lanes (the general kernel, which is exact in either
+    mode): "wide" gives them the 16-byte lanes and the lean kernel that large launches get."""
+    import fbgemm_amd
+    lib = fbgemm_amd.lib()
+    if request.param == "wide":
+        lib.fbgemm_amd_set_narrow_below_waves(0)
+    yield request.param
+    lib.fbgemm_amd_set_narrow_below_waves(-1)
+
+
+def cu(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def ordered(bits16):
+    b = bits16.astype(np.int32)
+    return np.where(b & 0x8000, -(b & 0x7fff), b)
+
+
+def as_float(bits16, out_ty):
+    if out_ty == FP16:
+        return bits16.view(np.float16).astype(np.float64)
+    return (bits16.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+
+
+def check_grade(got, want, out_ty, rows, what):
+    """got / want: fp32 arrays or uint16 bit patterns, reshaped to [rows, -1]. fp32: within 1e-5 of
+    the larger of |want| and the largest magnitude of the bag's row. fp16 / bf16: within one unit
+    in the last place, or (elements that nearly cancel) within that same 1e-5 of the row's
+    magnitude. Returns the worst error: relative (fp32) or units in the last place."""
+    got, want = got.reshape(rows, -1), want.reshape(rows, -1)
+    if out_ty == FP32:
+        g, w = got.astype(np.float64), want.astype(np.float64)
+    else:
+        g, w = as_float(got, out_ty), as_float(want, out_ty)
+    scale = np.maximum(np.abs(w), np.abs(w).max(axis=1, keepdims=True))
+    rel = np.where(np.isfinite(w), np.abs(g - w) / np.maximum(scale, 1e-30), 0.0)
+    if out_ty == FP32:
+        worst = float(rel.max(initial=0.0))
+        assert worst <= 1e-5, f"{what}: relative error {worst:.3g} exceeds 1e-5"
+        return worst
+    d = np.where(rel <= 1e-5, np.minimum(np.abs(ordered(got) - ordered(want)), 1), np.abs(ordered(got) - ordered(want)))
+    worst = int(d.max(initial=0))
+    assert worst <= 1, f"{what}: {worst} units in the last place"
+    return worst
+
+
+def bits_of(t, out_ty):
+    t = t.cpu()
+    return t.numpy() if out_ty == FP32 else t.view(torch.int16).numpy().view(np.uint16)
+
+
+@pytest.mark.parametrize("ty", [INT4, INT8])
+@pytest.mark.parametrize("shape", [(300, 5000, 128, 20), (40, 300, 256, 10), (64, 2000, 64, 33), (3, 1000, 128, 300),
+                                   (10, 4000, 256, 100), (1, 500, 64, 400), (20, 1000, 48, 50)])
+def test_single_table_fast_mode(ops, oracle, ty, shape):
+    """Regular shapes (the lean kernel, biases summed apart), few long bags (split into
+    segments) and a width the lean kernel does not take (D = 48: the general kernel, exact)."""
+    nb, rows, D, avg = shape
+    rng = np.random.default_rng(hash((ty, shape)) % 2**32)
+    worst = {}
+    for sbl in (True, False):
+        for out_ty in (FP32, FP16, BF16):
+            for weighted in (False, True):
+                for normalize in (False, True):
+                    table, _ = H.make_table(rng, ty, rows, D, sbl)
+                    idx, off, _ = H.make_bags(rng, rows, nb, avg, np.int64, np.int32, empty_frac=0.1)
+                    if not sbl and len(idx) > 3:
+                        idx[3] = -1  # a pruned row
+                    w = rng.uniform(0, 1, len(idx)).astype(np.float32) if weighted else None  # as the configurations draw them
+                    kern = (ops.generate_embedding_spmdm_nbit_with_strides(4, D, weighted, normalize, 16, False, True, -1, -1, sbl, out_ty=out_ty)
+                            if ty == INT4 else
+                            ops.generate_embedding_spmdm_with_strides(INT8, D, weighted, normalize, 16, False, True, -1, -1, sbl, out_ty=out_ty))
+                    out = torch.full((nb * D,), 7.0, dtype={FP32: torch.float32, FP16: torch.float16, BF16: torch.bfloat16}[out_ty], device="cuda")
+                    ok = kern(nb, len(idx), rows, cu(table), cu(idx), cu(off), None if w is None else cu(w), out,
+                              accumulate=ops.ACC_FAST)
+                    ok_o, want = oracle.spmdm(ty, D, table, idx, off, weights=w, normalize=normalize, out_ty=out_ty,
+                                              scale_bias_last=sbl, data_size=rows)
+                    assert ok and ok_o
+                    e = check_grade(bits_of(out, out_ty), want, out_ty, nb, f"ty={ty} {shape} sbl={sbl} out={out_ty} w={weighted} norm={normalize}")
+                    worst[out_ty] = max(worst.get(out_ty, 0), e)
+    print(f"worst error, ty={ty} shape={shape}: fp32 relative {worst[FP32]:.3g}, fp16 {worst[FP16]} ulp, bf16 {worst[BF16]} ulp")
+
+
+def test_cancellation_heavy_bags(ops, oracle):
+    """Bags whose terms cancel: the same rows with weights +w and -w, and biases that sum to
+    nearly nothing. The error stays within 1e-5 of the magnitude of what was summed."""
+    rng = np.random.default_rng(5)
+    rows, D, nb, L = 400, 128, 50, 24
+    for ty in (INT4, INT8):
+        table, _ = H.make_table(rng, ty, rows, D, False, scale_range=(0.5, 2.0), bias_range=(-100.0, 100.0))
+        half = rng.integers(0, rows, size=(nb, L // 2))
+        idx = np.concatenate([half, half], axis=1).reshape(-1).astype(np.int64)
+        w = rng.uniform(0.5, 1.5, size=(nb, L // 2)).astype(np.float32)
+        w = np.concatenate([w, -w], axis=1).reshape(-1)
+        off = (np.arange(nb + 1) * L).astype(np.int32)
+        kern = (ops.generate_embedding_spmdm_nbit_with_strides(4, D, True, False, 16, False, True, -1, -1, False) if ty == INT4 else
+                ops.generate_embedding_spmdm_with_strides(INT8, D, True, False, 16, False, True, -1, -1, False))
+        out = torch.empty(nb * D, dtype=torch.float32, device="cuda")
+        assert kern(nb, len(idx), rows, cu(table), cu(idx), cu(off), cu(w), out, accumulate=ops.ACC_FAST)
+        ok, want = oracle.spmdm(ty, D, table, idx, off, weights=w, scale_bias_last=False, data_size=rows)
+        assert ok
+        got = out.cpu().numpy().astype(np.float64).reshape(nb, D)
+        # what was summed per bag: |w| * (|scale| * 15 or 255 + |bias|) is of the order of 100
+        err = np.abs(got - want.reshape(nb, D).astype(np.float64)).max()
+        assert err <= 1e-5 * 100.0 * L, f"ty={ty}: absolute error {err}"
+        print(f"cancelling bags, ty={ty}: largest absolute error {err:.3g} against terms of magnitude ~100")
+
+
+def tbe_problem(rng, specs, B, max_L, row_alignment, weighted):
+    from test_tbe_gpu import build_weights
+    weights, wo, _ = build_weights(rng, specs, row_alignment)
+    T = len(specs)
+    lens = rng.integers(0, max_L, size=T * B)
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    idx = np.concatenate([rng.integers(0, specs[t][0], size=int(lens[t * B:(t + 1) * B].sum())) for t in range(T)] + [np.zeros(0, np.int64)]).astype(np.int64)
+    idx[rng.random(len(idx)) < 0.05] = -1
+    psw = rng.uniform(0, 1, len(idx)).astype(np.float32) if weighted else None
+    tys = np.array([s[2] for s in specs], np.uint8)
+    D_offsets = np.concatenate([[0], np.cumsum([s[1] for s in specs])]).astype(np.int32)
+    return weights, wo, tys, D_offsets, idx, off, psw
+
+
+@pytest.mark.parametrize("B,max_L", [(257, 40), (3, 900), (1, 2000)])
+def test_table_batched_fast_mode(ops, oracle, B, max_L):
+    """Mixed tables (lean and general shapes together) in the tolerance-grade mode; with few, long
+    bags the forward cuts them into segments."""
+    rng = np.random.default_rng(1000 + B)
+    specs = [(500, 64, INT4), (300, 128, INT8), (200, 256, FP16), (100, 32, INT2), (400, 256, INT4), (64, 48, INT4),
+             (150, 16, FP32), (700, 128, INT4), (90, 256, INT8)]
+    for row_alignment in (16, 4):
+        for weighted in (False, True):
+            weights, wo, tys, D_offsets, idx, off, psw = tbe_problem(rng, specs, B, max_L, row_alignment, weighted)
+            T, total_D = len(specs), int(D_offsets[-1])
+            for pooling in (0, 1):
+                for out_ty in (FP32, FP16, BF16):
+                    got = ops.int_nbit_split_embedding_codegen_lookup_function(
+                        cu(weights), torch.zeros(0, dtype=torch.uint8, device="cuda"), cu(np.zeros(T, np.int32)), cu(wo), cu(tys),
+                        cu(D_offsets), total_D, 32, 256, 256, 256, 16, cu(idx), cu(off), pooling, None if psw is None else cu(psw),
+                        out_ty, row_alignment=row_alignment, accumulate=ops.ACC_FAST)
+                    rc, want = oracle.tbe_forward(weights, wo, tys, D_offsets, total_D, idx, off, pooling, psw, out_ty, row_alignment)
+                    assert rc == 0
+                    # per table, so that a table of small values is not held to another table's magnitudes
+                    g = bits_of(got, out_ty).reshape(B, total_D)
+                    for t in range(T):
+                        c0, c1 = int(D_offsets[t]), int(D_offsets[t + 1])
+                        check_grade(np.ascontiguousarray(g[:, c0:c1]), np.ascontiguousarray(want.reshape(B, total_D)[:, c0:c1]), out_ty, B,
+                                    f"B={B} L<{max_L} align={row_alignment} w={weighted} pool={pooling} out={out_ty} table={t}")
+
+
+def test_configs_scaled_fast_mode(ops, oracle):
+    """Configs 3, 4 (batched, pruned) and 5 at reduced size, in full, in the tolerance-grade mode."""
+    from fbgemm_amd import bench_configs as bc
+    for name, p in (("config3", bc.config3("cuda", scale=0.05)), ("config4", bc.config4_batched("cuda", scale=0.05)),
+                    ("config5", bc.config5("cuda", scale=0.01, tables_int4=6, tables_int2=3))):
+        got = ops.int_nbit_split_embedding_codegen_lookup_function(
+            p.dev_weights, torch.zeros(0, dtype=torch.uint8, device="cuda"), cu(np.zeros(p.T, np.int32)), cu(p.weights_offsets),
+            cu(p.tys), cu(p.D_offsets), p.total_D, 32, 256, 256, 256, 0, p.indices, p.offsets, p.pooling_mode, p.indice_weights,
+            p.output_dtype, row_alignment=p.row_alignment, index_remappings=p.extra.get("remap"),
+            index_remappings_offsets=p.extra.get("remap_offsets"), accumulate=ops.ACC_FAST)
+        rc, want = oracle.tbe_forward(p.dev_weights.cpu().numpy(), p.weights_offsets, p.tys, p.D_offsets, p.total_D,
+                                      p.physical_indices, p.host_offsets, p.pooling_mode, p.host_weights, p.output_dtype,
+                                      p.row_alignment)
+        assert rc == 0
+        g = bits_of(got, p.output_dtype).reshape(p.B, p.total_D)
+        worst = 0
+        for t in range(p.T):
+            c0, c1 = int(p.D_offsets[t]), int(p.D_offsets[t + 1])
+            worst = max(worst, check_grade(np.ascontiguousarray(g[:, c0:c1]), np.ascontiguousarray(want.reshape(p.B, p.total_D)[:, c0:c1]),
+                                           p.output_dtype, p.B, f"{name} table {t}"))
+        print(f"{name} (scaled) in the tolerance-grade mode: worst error {worst}")
