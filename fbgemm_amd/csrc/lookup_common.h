@@ -156,11 +156,6 @@ struct LookupArgs {
   int32_t fp8_shift;         // FP8 rows: 16 + exponent bits (moves the 7 low bits to fp32's exponent/mantissa)
   float fp8_mult;            // FP8 rows: 2^(127 - exponent bias)
   Status* status;
-#ifdef FBGEMM_AMD_WAVE_TRACE
-  // diagnostic build only: 4 words per workgroup (start, end of the wave on the
-  // 100 MHz wall clock; hardware id | XCC id << 32; work-list position)
-  unsigned long long* trace;
-#endif
 };
 
 } // namespace fbgemm_amd

@@ -473,9 +473,6 @@ __device__ __forceinline__ void run_item(const LookupArgs& a, int64_t wave, int 
     first_slot = (int)(wave * a.single.bags);
   }
   const TableDesc d = a.tables ? a.tables[table] : a.single;
-#ifdef FBGEMM_AMD_ONLY_TY // register-budget experiments: compile a single row type
-  if (d.ty == FBGEMM_AMD_ONLY_TY) pool_dispatch_vb<index_t, GENERAL, FBGEMM_AMD_ONLY_TY>(a, d, table, first_slot, lane, stage_row, stage_mul);
-#else
   switch (d.ty) {
     case ST_INT4: pool_dispatch_vb<index_t, GENERAL, ST_INT4>(a, d, table, first_slot, lane, stage_row, stage_mul); break;
     case ST_INT8: pool_dispatch_vb<index_t, GENERAL, ST_INT8>(a, d, table, first_slot, lane, stage_row, stage_mul); break;
@@ -486,22 +483,8 @@ __device__ __forceinline__ void run_item(const LookupArgs& a, int64_t wave, int 
     case ST_FP8: pool_dispatch_vb<index_t, GENERAL, ST_FP8>(a, d, table, first_slot, lane, stage_row, stage_mul); break;
     default: break;
   }
-#endif
 }
 
-#ifdef FBGEMM_AMD_WAVE_TRACE
-__device__ __forceinline__ void trace_item(const LookupArgs& a, int64_t wave, int lane, unsigned long long t0) {
-  if (a.trace && lane == 0) {
-    unsigned long long* t = a.trace + (size_t)wave * 4;
-    const unsigned hw = __builtin_amdgcn_s_getreg((31 << 11) | 4);   // HW_ID
-    const unsigned xcc = __builtin_amdgcn_s_getreg((3 << 11) | 20);  // XCC_ID
-    t[0] = t0;
-    t[1] = wall_clock64();
-    t[2] = (unsigned long long)hw | ((unsigned long long)xcc << 32);
-    t[3] = (unsigned long long)blockIdx.x | ((unsigned long long)(a.work ? a.work[wave].table : 0) << 32);
-  }
-}
-#endif
 
 // One wave per workgroup: waves come and go independently, and a workgroup
 // needs no more than its own 4 KB of LDS.
@@ -528,13 +511,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(FBGEMM_AMD_M
     wave = (int64_t)blockIdx.x;
     if (wave >= a.num_waves) return;
   }
-#ifdef FBGEMM_AMD_WAVE_TRACE
-  const unsigned long long trace_t0 = wall_clock64();
-#endif
   run_item<index_t, GENERAL>(a, wave, lane, stage_row, stage_mul);
-#ifdef FBGEMM_AMD_WAVE_TRACE
-  trace_item(a, wave, lane, trace_t0);
-#endif
 }
 
 

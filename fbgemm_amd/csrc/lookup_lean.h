@@ -37,6 +37,7 @@
 namespace fbgemm_amd {
 
 constexpr int LEAN_BLOCK = 8;   // entries of every bag staged at a time
+constexpr int LEAN_LDS_WORDS = 2048; // LDS of a wave: 64 lanes * 32 columns of fp32 output
 
 struct __attribute__((aligned(16))) LeanMul {
   float s24;  // w * scale * 2^24 (4- and 8-bit rows, pre-scaled route); w * scale (plain route); w (fp16 rows)
@@ -61,8 +62,8 @@ __device__ __forceinline__ float lean_fma(float s, float qd, float acc, float bi
   return EXACT ? __builtin_fmaf(s, q, acc + bias) : __builtin_fmaf(s, q, acc);
 }
 
-template <int TY, bool EXACT, bool PLAIN>
-__device__ __forceinline__ void lean_chunk(float (&acc)[32], int base, const uint32_t (&raw)[4], const LeanMul& m) {
+template <int TY, bool EXACT, bool PLAIN, int NACC>
+__device__ __forceinline__ void lean_chunk(float (&acc)[NACC], int base, const uint32_t (&raw)[4], const LeanMul& m) {
   if constexpr (TY == ST_INT4) {
     const float sa = m.s24, sb = PLAIN ? m.s24 : m.s20;
 #pragma unroll
@@ -230,19 +231,100 @@ __device__ __forceinline__ int64_t lean_remap(const LookupArgs& a, const LeanLan
   return m == -1 ? LEAN_PRUNED : m;
 }
 
+// The output of a wave through LDS, so that every store instruction writes runs
+// of consecutive bytes: a lane holds 32 consecutive columns of its bag (64 or 128
+// bytes of output), and storing them lane by lane would put the lanes of one
+// instruction 64 or 128 bytes apart, four or eight partial writes to every line.
+// Here the lanes of a bag first leave their 16-byte pieces in LDS in column order
+// and then take them back interleaved: piece sub, sub + lanes, sub + 2 lanes, ...,
+// which makes each instruction write lanes * 16 consecutive bytes per bag.
+// ESZ: bytes per output element. `lds` must hold the wave's whole output (at most
+// 64 lanes * 32 columns * 4 bytes) and is free once the last block is pooled.
+template <int TY, int C, bool INHDR, int ESZ>
+__device__ __forceinline__ void lean_store_interleaved(const LookupArgs& a, const TableDesc& d, const LeanLane& L,
+                                                       const float (&acc)[C * (TY == ST_INT4 ? 32 : (TY == ST_INT8 ? 16 : 8))],
+                                                       uint32_t* lds) {
+  constexpr int E = TY == ST_INT4 ? 32 : (TY == ST_INT8 ? 16 : 8);
+  // whole-row chunks start E / 4 columns before a multiple of E: pieces of 8 bytes where that is not 16 bytes
+  constexpr int PB = (INHDR && (E / 4 * ESZ) % 16 != 0) ? 8 : 16;
+  constexpr int WP = PB / 4;           // words per piece
+  constexpr int NP = E * ESZ / PB;     // pieces per chunk
+  constexpr int SHIFT = INHDR ? (E / 4 * ESZ) / PB : 0;
+  const int S = d.lanes;
+  const int npb = d.D * ESZ / PB;      // pieces of a bag's block of the output
+  uint32_t* mine = lds + (size_t)L.grp * npb * WP;
+  const bool bf = a.out_ty == ST_BF16;
+#pragma unroll
+  for (int c = 0; c < C; ++c) {
+    uint32_t w[E * ESZ / 4];
+    if constexpr (ESZ == 4) {
+#pragma unroll
+      for (int e = 0; e < E; ++e) w[e] = float_to_bits(acc[c * E + e]);
+    } else {
+      if (bf) {
+#pragma unroll
+        for (int e = 0; e < E; e += 2) w[e / 2] = pack_bf16x2(acc[c * E + e], acc[c * E + e + 1]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < E; e += 2) w[e / 2] = pack_half2(acc[c * E + e], acc[c * E + e + 1]);
+      }
+    }
+    const int g0 = (L.sub + c * S) * NP - SHIFT;
+#pragma unroll
+    for (int q = 0; q < NP; ++q) {
+      const int gq = g0 + q;
+      if (L.bag_ok && gq >= 0 && gq < npb) {
+        if constexpr (WP == 4) *reinterpret_cast<uint4*>(mine + gq * 4) = make_uint4(w[4 * q], w[4 * q + 1], w[4 * q + 2], w[4 * q + 3]);
+        else *reinterpret_cast<uint2*>(mine + gq * 2) = make_uint2(w[2 * q], w[2 * q + 1]);
+      }
+    }
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  uint8_t* block = reinterpret_cast<uint8_t*>(a.out) + ((int64_t)L.bag * a.out_stride + d.out_col) * ESZ;
+#pragma unroll
+  for (int it = 0; it < C * NP; ++it) {
+    const int gq = L.sub + it * S;
+    if (L.bag_ok && gq < npb) {
+      // streaming stores: whole runs of the output, written once and never read back here
+      if constexpr (WP == 4) {
+        const uint4 v = *reinterpret_cast<const uint4*>(mine + gq * 4);
+        stream_store16(block + (size_t)gq * 16, v.x, v.y, v.z, v.w);
+      } else {
+        const uint2 v = *reinterpret_cast<const uint2*>(mine + gq * 2);
+        stream_store8(block + (size_t)gq * 8, v.x, v.y);
+      }
+    }
+  }
+}
+
 template <bool EXACT, int TY, int C, bool INHDR>
-__device__ __forceinline__ void lean_write(const LookupArgs& a, const TableDesc& d, const LeanLane& L, float (&acc)[32], float bsum) {
+__device__ __forceinline__ void lean_write(const LookupArgs& a, const TableDesc& d, const LeanLane& L, float (&acc)[C * (TY == ST_INT4 ? 32 : (TY == ST_INT8 ? 16 : 8))], float bsum, uint32_t* lds) {
   constexpr bool QUANT = TY == ST_INT8 || TY == ST_INT4;
   constexpr int E = TY == ST_INT4 ? 32 : (TY == ST_INT8 ? 16 : 8);
+  constexpr int NACC = C * E;
   const bool vec_ok = a.out_aligned && ((d.vec_store >> (a.out_ty == ST_FP32 ? 0 : 1)) & 1);
   if constexpr (!EXACT && QUANT) {
 #pragma unroll
-    for (int e = 0; e < 32; ++e) acc[e] += bsum;
+    for (int e = 0; e < NACC; ++e) acc[e] += bsum;
   }
   if (a.normalize && L.n > 0) {
     const float inv_len = 1.0f / (float)L.n; // the reference keeps the bag length in an int when it forms 1/len
 #pragma unroll
-    for (int e = 0; e < 32; ++e) acc[e] *= inv_len;
+    for (int e = 0; e < NACC; ++e) acc[e] *= inv_len;
+  }
+  // whole 16-byte (8-byte) pieces at aligned places: through LDS, interleaved
+  if (lds && vec_ok) {
+    if (a.out_ty == ST_FP32) {
+      if ((d.D * 4) % 16 == 0) {
+        lean_store_interleaved<TY, C, INHDR, 4>(a, d, L, acc, lds);
+        return;
+      }
+    } else if ((d.D * 2) % 16 == 0) {
+      lean_store_interleaved<TY, C, INHDR, 2>(a, d, L, acc, lds);
+      return;
+    }
   }
   const int nchunks = INHDR ? (d.data_bytes + 4 + 15) / 16 : d.lanes * C;
 #pragma unroll
@@ -311,9 +393,9 @@ __device__ __forceinline__ bool pool_lean(const LookupArgs& a, const TableDesc& 
     for (int c = 0; c < C; ++c) rowb[c] = c * S * 16;
   }
 
-  float acc[32];
+  float acc[C * E];
 #pragma unroll
-  for (int e = 0; e < 32; ++e) acc[e] = 0.0f;
+  for (int e = 0; e < C * E; ++e) acc[e] = 0.0f;
   float bsum = -0.0f; // tolerance grade: the biases of the bag, added once at the end
 
   // registers of the staging lanes: raw indices and weights of the block being fetched
@@ -469,12 +551,12 @@ __device__ __forceinline__ bool pool_lean(const LookupArgs& a, const TableDesc& 
         }
         if constexpr (!EXACT && QUANT) bsum += m.bias;
 #pragma unroll
-        for (int c = 0; c < C; ++c) lean_chunk<TY, EXACT, false>(acc, c * E, raw[e][c], m);
+        for (int c = 0; c < C; ++c) lean_chunk<TY, EXACT, false, C * E>(acc, c * E, raw[e][c], m);
       }
     }
     __builtin_amdgcn_wave_barrier(); // the column lanes are done with the block before it is overwritten
   }
-  lean_write<EXACT, TY, C, INHDR>(a, d, L, acc, bsum);
+  lean_write<EXACT, TY, C, INHDR>(a, d, L, acc, bsum, reinterpret_cast<uint32_t*>(stage_row));
   return true;
 }
 
@@ -489,9 +571,9 @@ __device__ __forceinline__ void pool_lean_slow(const LookupArgs& a, const TableD
   const index_t* idx = reinterpret_cast<const index_t*>(a.indices) + L.pos0;
   const uint8_t* wbase = (d.placement ? a.weights[1] : a.weights[0]) + d.weights_offset;
   const int nchunks = INHDR ? (d.data_bytes + 4 + 15) / 16 : S * C;
-  float acc[32];
+  float acc[C * E];
 #pragma unroll
-  for (int e = 0; e < 32; ++e) acc[e] = 0.0f;
+  for (int e = 0; e < C * E; ++e) acc[e] = 0.0f;
   float bsum = -0.0f;
   for (int i = 0; i < L.n; ++i) {
     int64_t row = (int64_t)idx[i];
@@ -513,10 +595,10 @@ __device__ __forceinline__ void pool_lean_slow(const LookupArgs& a, const TableD
       const int k = L.sub + c * S;
       uint32_t raw[4];
       load_raw<16>(raw, prow + (INHDR ? 0 : d.data_off) + (k < nchunks ? k : nchunks - 1) * 16);
-      lean_chunk<TY, EXACT, true>(acc, c * E, raw, m);
+      lean_chunk<TY, EXACT, true, C * E>(acc, c * E, raw, m);
     }
   }
-  lean_write<EXACT, TY, C, INHDR>(a, d, L, acc, bsum);
+  lean_write<EXACT, TY, C, INHDR>(a, d, L, acc, bsum, nullptr);
 }
 
 template <typename index_t, bool EXACT, int TY, int C, bool INHDR>
@@ -553,8 +635,10 @@ __device__ __forceinline__ void lean_dispatch(const LookupArgs& a, const TableDe
 // Same work list and workgroup -> XCD mapping as lookup_kernel.
 template <typename index_t, bool EXACT>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(FBGEMM_AMD_LEAN_MIN_WAVES, 8))) void lookup_lean_kernel(const LookupArgs a) {
-  __shared__ int stage_row[MAX_GROUPS * LEAN_BLOCK];
-  __shared__ LeanMul stage_mul[MAX_GROUPS * LEAN_BLOCK];
+  // 8 KB: while a bag is pooled, the staged rows (1 KB) and multipliers (4 KB); at the end, the wave's output
+  __shared__ __attribute__((aligned(16))) uint32_t lds[LEAN_LDS_WORDS];
+  int* stage_row = reinterpret_cast<int*>(lds);
+  LeanMul* stage_mul = reinterpret_cast<LeanMul*>(lds + MAX_GROUPS * LEAN_BLOCK);
   const int lane = threadIdx.x;
   int64_t wave;
   if (a.xcd_start) {

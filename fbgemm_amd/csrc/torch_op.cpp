@@ -12,6 +12,7 @@
 
 #include <algorithm>
 #include <map>
+#include <memory>
 #include <mutex>
 #include <tuple>
 
@@ -27,24 +28,37 @@ void* current_stream(const Tensor& t) {
 
 // One plan per distinct set of metadata tensors (the operator receives them as
 // device tensors on every call; the host copy a plan needs is made once).
+// A plan is cached per set of metadata tensors: their addresses AND versions (an in-place edit of
+// weights_offsets / weights_tys / D_offsets makes a new plan), sizes and the row alignment.
 struct PlanKey {
   const void *wo, *wt, *dofs, *wp;
+  int64_t v_wo, v_wt, v_dofs, v_wp;
   int64_t T, dev_bytes, uvm_bytes, row_alignment;
   bool operator<(const PlanKey& o) const {
-    return std::tie(wo, wt, dofs, wp, T, dev_bytes, uvm_bytes, row_alignment) <
-        std::tie(o.wo, o.wt, o.dofs, o.wp, o.T, o.dev_bytes, o.uvm_bytes, o.row_alignment);
+    return std::tie(wo, wt, dofs, wp, v_wo, v_wt, v_dofs, v_wp, T, dev_bytes, uvm_bytes, row_alignment) <
+        std::tie(o.wo, o.wt, o.dofs, o.wp, o.v_wo, o.v_wt, o.v_dofs, o.v_wp, o.T, o.dev_bytes, o.uvm_bytes, o.row_alignment);
   }
 };
-std::mutex g_mu;
-struct PlanEntry {
-  fbgemm_amd_tbe_plan* plan;
+// Owner of a plan handle. Forwards hold a reference while they launch, so a plan that the cache
+// drops is destroyed only after the last of them has returned (the destructor waits for the device).
+struct PlanHolder {
+  fbgemm_amd_tbe_plan* plan = nullptr;
   Tensor keep[4]; // the key's tensors: alive while cached, so their addresses are not handed to other tensors
+  ~PlanHolder() { fbgemm_amd_tbe_plan_destroy(plan); }
 };
+struct PlanEntry {
+  std::shared_ptr<PlanHolder> holder;
+  uint64_t last_use;
+};
+constexpr size_t MAX_CACHED_PLANS = 64; // beyond: the least recently used plan goes
+std::mutex g_mu;                        // guards the two maps below, never held across a launch
 std::map<PlanKey, PlanEntry> g_plans;
+uint64_t g_use_clock = 0;
 std::map<int, Tensor> g_status; // one status block per device, never freed
 
-Tensor& status_block(const Tensor& like) {
+Tensor status_block(const Tensor& like) {
   const int dev = like.device().index();
+  std::lock_guard<std::mutex> lk(g_mu);
   auto it = g_status.find(dev);
   if (it == g_status.end()) {
     Tensor st = at::zeros({4}, like.options().dtype(at::kInt));
@@ -54,24 +68,52 @@ Tensor& status_block(const Tensor& like) {
   return it->second;
 }
 
-fbgemm_amd_tbe_plan* plan_for(const Tensor& dev_weights, const Tensor& uvm_weights, const Tensor& placements,
-                              const Tensor& weights_offsets, const Tensor& weights_tys, const Tensor& D_offsets,
-                              int64_t row_alignment) {
-  PlanKey key{weights_offsets.data_ptr(), weights_tys.data_ptr(), D_offsets.data_ptr(), placements.data_ptr(),
-              D_offsets.numel() - 1, dev_weights.numel(), uvm_weights.numel(), row_alignment};
-  auto it = g_plans.find(key);
-  if (it != g_plans.end()) return it->second.plan;
+std::shared_ptr<PlanHolder> plan_for(const Tensor& dev_weights, const Tensor& uvm_weights, const Tensor& placements,
+                                     const Tensor& weights_offsets, const Tensor& weights_tys, const Tensor& D_offsets,
+                                     int64_t row_alignment) {
+  const PlanKey key{weights_offsets.data_ptr(), weights_tys.data_ptr(), D_offsets.data_ptr(), placements.data_ptr(),
+                    (int64_t)weights_offsets._version(), (int64_t)weights_tys._version(), (int64_t)D_offsets._version(),
+                    (int64_t)placements._version(), D_offsets.numel() - 1, dev_weights.numel(), uvm_weights.numel(),
+                    row_alignment};
+  {
+    std::lock_guard<std::mutex> lk(g_mu);
+    auto it = g_plans.find(key);
+    if (it != g_plans.end()) {
+      it->second.last_use = ++g_use_clock;
+      return it->second.holder;
+    }
+  }
   const Tensor wo = weights_offsets.to(at::kCPU, at::kLong).contiguous();
   const Tensor wt = weights_tys.to(at::kCPU, at::kByte).contiguous();
   const Tensor dofs = D_offsets.to(at::kCPU, at::kInt).contiguous();
   const Tensor wp = placements.to(at::kCPU, at::kInt).contiguous();
-  fbgemm_amd_tbe_plan* plan = nullptr;
+  auto holder = std::make_shared<PlanHolder>();
   const int rc = fbgemm_amd_tbe_plan_create(
-      &plan, (int32_t)(dofs.numel() - 1), wo.data_ptr<int64_t>(), wt.data_ptr<uint8_t>(), dofs.data_ptr<int32_t>(),
+      &holder->plan, (int32_t)(dofs.numel() - 1), wo.data_ptr<int64_t>(), wt.data_ptr<uint8_t>(), dofs.data_ptr<int32_t>(),
       wp.data_ptr<int32_t>(), dev_weights.numel(), uvm_weights.numel(), row_alignment);
   TORCH_CHECK(rc == 0, "fbgemm_amd: ", fbgemm_amd_last_error());
-  g_plans.emplace(key, PlanEntry{plan, {weights_offsets, weights_tys, D_offsets, placements}});
-  return plan;
+  holder->keep[0] = weights_offsets;
+  holder->keep[1] = weights_tys;
+  holder->keep[2] = D_offsets;
+  holder->keep[3] = placements;
+  std::shared_ptr<PlanHolder> evicted; // destroyed (device synchronize) after the lock is released
+  {
+    std::lock_guard<std::mutex> lk(g_mu);
+    auto it = g_plans.find(key); // another thread may have made the same plan meanwhile
+    if (it != g_plans.end()) {
+      it->second.last_use = ++g_use_clock;
+      return it->second.holder;
+    }
+    if (g_plans.size() >= MAX_CACHED_PLANS) {
+      auto victim = g_plans.begin();
+      for (auto jt = g_plans.begin(); jt != g_plans.end(); ++jt)
+        if (jt->second.last_use < victim->second.last_use) victim = jt;
+      evicted = victim->second.holder;
+      g_plans.erase(victim);
+    }
+    g_plans.emplace(key, PlanEntry{holder, ++g_use_clock});
+  }
+  return holder;
 }
 
 at::ScalarType out_scalar_type(int64_t output_dtype) {
@@ -106,9 +148,9 @@ Tensor int_nbit_split_embedding_codegen_lookup_function_hip(
     w = indice_weights->to(at::kFloat).contiguous(); // embedding_forward_quantized_host.cpp:345
   }
   const int64_t align = row_alignment ? *row_alignment : 16; // embedding_forward_quantized_host.cpp:310
-  std::lock_guard<std::mutex> lk(g_mu);
-  fbgemm_amd_tbe_plan* plan = plan_for(dev_weights, uvm_weights, weights_placements, weights_offsets, weights_tys,
-                                       D_offsets, align);
+  const std::shared_ptr<PlanHolder> holder = plan_for(dev_weights, uvm_weights, weights_placements, weights_offsets,
+                                                      weights_tys, D_offsets, align);
+  fbgemm_amd_tbe_plan* plan = holder->plan;
   if (max_float8_D && *max_float8_D > 0) {
     TORCH_CHECK(fp8_exponent_bits && fp8_exponent_bias && *fp8_exponent_bits > 0 && *fp8_exponent_bias >= 0,
                 "FP8 tables need fp8_exponent_bits and fp8_exponent_bias");
@@ -129,7 +171,7 @@ Tensor int_nbit_split_embedding_codegen_lookup_function_hip(
     else
       out = at::empty({total_L, D}, dev_weights.options().dtype(out_scalar_type(output_dtype)));
     if (total_L == 0 || B == 0) return out.zero_();
-    Tensor& st = status_block(dev_weights);
+    Tensor st = status_block(dev_weights);
     const int rc = fbgemm_amd_tbe_forward_nobag(
         plan, dev_weights.data_ptr(), uvm_weights.numel() ? uvm_weights.data_ptr() : nullptr, indices.data_ptr(),
         offsets.data_ptr(), indices.scalar_type() == at::kLong ? 64 : 32, indices.numel(), offsets.numel(), (int32_t)D,
@@ -143,7 +185,7 @@ Tensor int_nbit_split_embedding_codegen_lookup_function_hip(
       ? at::empty({B, total_D + 8 * T}, dev_weights.options().dtype(at::kByte))
       : at::empty({B, total_D}, dev_weights.options().dtype(out_scalar_type(output_dtype)));
   if (B == 0) return out;
-  Tensor& st = status_block(dev_weights);
+  Tensor st = status_block(dev_weights);
   const int rc = fbgemm_amd_tbe_forward(
       plan, dev_weights.data_ptr(), uvm_weights.numel() ? uvm_weights.data_ptr() : nullptr, indices.data_ptr(),
       offsets.data_ptr(), indices.scalar_type() == at::kLong ? 64 : 32, indices.numel(), offsets.numel(),
@@ -182,8 +224,7 @@ Tensor int_nbit_split_embedding_uvm_caching_codegen_lookup_function_hip(
 // raises). This reads the record: synchronizes, returns the FBGEMM_AMD_ERR_*
 // bits seen since the last call and clears them.
 int64_t lookup_status(Tensor like) {
-  std::lock_guard<std::mutex> lk(g_mu);
-  Tensor& st = status_block(like);
+  Tensor st = status_block(like);
   int32_t bits = 0;
   int64_t pos = -1;
   TORCH_CHECK(fbgemm_amd_status_read(st.data_ptr(), current_stream(like), &bits, &pos) == 0, fbgemm_amd_last_error());
@@ -247,10 +288,10 @@ void emb_inplace_update_hip(Tensor dev_weights, Tensor uvm_weights, Tensor weigh
   update_table_idx = update_table_idx.contiguous();
   update_row_idx = update_row_idx.contiguous();
   update_offsets = update_offsets.contiguous();
-  std::lock_guard<std::mutex> lk(g_mu);
-  fbgemm_amd_tbe_plan* plan = plan_for(dev_weights, uvm_weights, weights_placements, weights_offsets, weights_tys,
-                                       D_offsets, row_alignment);
-  Tensor& st = status_block(dev_weights);
+  const std::shared_ptr<PlanHolder> holder = plan_for(dev_weights, uvm_weights, weights_placements, weights_offsets,
+                                                      weights_tys, D_offsets, row_alignment);
+  fbgemm_amd_tbe_plan* plan = holder->plan;
+  Tensor st = status_block(dev_weights);
   const int rc = fbgemm_amd_tbe_inplace_update(
       plan, dev_weights.numel() ? dev_weights.data_ptr() : nullptr, uvm_weights.numel() ? uvm_weights.data_ptr() : nullptr,
       update_weights.data_ptr(), update_weights.numel(), update_table_idx.data_ptr<int32_t>(), update_row_idx.data_ptr(),
