@@ -54,6 +54,7 @@ SYMBOLS = {
     "fbgemm_amd_pruned_hashmap_lookup": (C.c_int, [_P, _P, _I32, _I64, _P, _I32, _P, _I32, _P, _P]),
     "fbgemm_amd_pruned_hashmap_insert_host": (C.c_int, [_P, _P, _P, _I32, _I64, _P, _I32, _P, _I32]),
     "fbgemm_amd_quantize_rowwise": (C.c_int, [_P, _I32, _I64, _I32, _I32, _I32, _I32, _I64, _P, _P]),
+    "fbgemm_amd_quantize_rowwise_min_max": (C.c_int, [_P, _I32, _I64, _I32, _I32, _I32, _I32, _I64, _P, _P, _P]),
     "fbgemm_amd_dequantize_rowwise": (C.c_int, [_P, _I64, _I64, _I32, _I32, _I32, _I32, _I32, _P, _P]),
     "fbgemm_amd_float_to_hfp8": (C.c_int, [_P, _I64, _I32, _I32, C.c_float, _P, _P]),
     "fbgemm_amd_hfp8_to_float": (C.c_int, [_P, _I64, _I32, _I32, _P, _P]),

@@ -8,6 +8,7 @@
 #include <cstdio>
 #include <cstring>
 #include <map>
+#include <memory>
 #include <mutex>
 #include <vector>
 
@@ -67,7 +68,7 @@ hipError_t launch_bounds_check(const int64_t* rows_per_table, int32_t T, void* i
 int64_t bounds_check_partials(int64_t total_B);
 hipError_t launch_quantize_rowwise(const void* input, bool half_in, int64_t rows, int32_t cols, int32_t bits,
                                    int32_t sb_float, int32_t layout, int64_t out_stride, void* output,
-                                   hipStream_t stream);
+                                   const void* min_max, hipStream_t stream);
 hipError_t launch_dequantize_rowwise(const void* input, int64_t rows, int64_t in_stride, int32_t cols, int32_t bits,
                                      int32_t sb_float, int32_t layout, int32_t output_ty, void* output,
                                      hipStream_t stream);
@@ -924,7 +925,9 @@ int fbgemm_amd_tbe_plan_create(
   if (!out || T <= 0 || !weights_offsets || !weights_tys || !D_offsets)
     return fail(FBGEMM_AMD_E_ARG, "bad plan arguments");
   if (row_alignment <= 0) row_alignment = 1;
-  auto plan = new fbgemm_amd_tbe_plan();
+  // owned here until it is handed out: every early return below frees the plan and what it holds
+  std::unique_ptr<fbgemm_amd_tbe_plan, void (*)(fbgemm_amd_tbe_plan*)> owner(new fbgemm_amd_tbe_plan(), fbgemm_amd_tbe_plan_destroy);
+  fbgemm_amd_tbe_plan* plan = owner.get();
   plan->T = T;
   plan->total_D = D_offsets[T];
   plan->row_alignment = row_alignment;
@@ -945,12 +948,10 @@ int fbgemm_amd_tbe_plan_create(
     memset(&d, 0, sizeof(d));
     d.ty = weights_tys[t];
     if (type_bits(d.ty) == 0) {
-      delete plan;
       return fail(FBGEMM_AMD_E_UNSUPPORTED, "table %d: weight type %d is not supported", t, d.ty);
     }
     d.D = D_offsets[t + 1] - D_offsets[t];
     if (d.D <= 0) {
-      delete plan;
       return fail(FBGEMM_AMD_E_ARG, "table %d: D_offsets must increase", t);
     }
     d.out_col = D_offsets[t];
@@ -1001,7 +1002,7 @@ int fbgemm_amd_tbe_plan_create(
   }
   HIP_TRY(hipMalloc((void**)&plan->d_tables_narrow, sizeof(TableDesc) * T));
   HIP_TRY(hipMemcpy(plan->d_tables_narrow, plan->tables_narrow.data(), sizeof(TableDesc) * T, hipMemcpyHostToDevice));
-  *out = plan;
+  *out = owner.release();
   return 0;
 }
 
@@ -1509,17 +1510,24 @@ int check_quant_format(int32_t bit_rate, int32_t sb_float, int32_t layout, int32
 }
 } // namespace
 
-int fbgemm_amd_quantize_rowwise(
+int fbgemm_amd_quantize_rowwise_min_max(
     const void* d_input, int32_t input_ty, int64_t rows, int32_t cols, int32_t bit_rate, int32_t sb_float,
-    int32_t layout, int64_t out_row_stride, void* d_output, void* stream) {
+    int32_t layout, int64_t out_row_stride, void* d_output, const void* d_rowwise_min_max, void* stream) {
   if (input_ty != ST_FP32 && input_ty != ST_FP16) return fail(FBGEMM_AMD_E_ARG, "input must be fp32 or fp16");
   if (rows < 0) return fail(FBGEMM_AMD_E_ARG, "rows must not be negative");
   if (int rc = check_quant_format(bit_rate, sb_float, layout, cols, out_row_stride)) return rc;
   if (rows == 0) return 0;
   if (!d_input || !d_output) return fail(FBGEMM_AMD_E_ARG, "null data pointer");
   HIP_TRY(launch_quantize_rowwise(d_input, input_ty == ST_FP16, rows, cols, bit_rate, sb_float, layout, out_row_stride,
-                                  d_output, (hipStream_t)stream));
+                                  d_output, d_rowwise_min_max, (hipStream_t)stream));
   return 0;
+}
+
+int fbgemm_amd_quantize_rowwise(
+    const void* d_input, int32_t input_ty, int64_t rows, int32_t cols, int32_t bit_rate, int32_t sb_float,
+    int32_t layout, int64_t out_row_stride, void* d_output, void* stream) {
+  return fbgemm_amd_quantize_rowwise_min_max(d_input, input_ty, rows, cols, bit_rate, sb_float, layout, out_row_stride,
+                                             d_output, nullptr, stream);
 }
 
 int fbgemm_amd_dequantize_rowwise(

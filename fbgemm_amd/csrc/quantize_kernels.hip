@@ -116,7 +116,8 @@ __device__ __forceinline__ void store_run(uint8_t* p, uint64_t v, int nbytes) {
 template <bool HALF_IN, int BITS>
 __global__ __launch_bounds__(256) void quantize_rowwise_kernel(
     const void* input, int64_t rows, int32_t cols_arg, int32_t sb_float, int32_t layout,
-    int64_t out_stride, uint8_t* output, int32_t lpr, const int32_t* seg_offsets, int32_t seg_T, int64_t seg_in_stride) {
+    int64_t out_stride, uint8_t* output, int32_t lpr, const int32_t* seg_offsets, int32_t seg_T, int64_t seg_in_stride,
+    const void* min_max) {
   constexpr int bits = BITS;
   const int lane = threadIdx.x & 63;
   const int sub = lane & (lpr - 1);
@@ -195,7 +196,20 @@ __global__ __launch_bounds__(256) void quantize_rowwise_kernel(
     }
   }
   float minimum = mn.v;
-  const float maximum = mx.v;
+  float maximum = mx.v;
+  // Extremes the caller brings (two input-typed values per row, minimum then maximum) take the
+  // place of the ones found (src/QuantUtilsAvx2.cc:1605-1628, :1831-1853).
+  if (min_max) {
+    if (HALF_IN) {
+      const uint16_t* mm = reinterpret_cast<const uint16_t*>(min_max) + row * 2;
+      minimum = half_bits_to_float(mm[0]);
+      maximum = half_bits_to_float(mm[1]);
+    } else {
+      const float* mm = reinterpret_cast<const float*>(min_max) + row * 2;
+      minimum = mm[0];
+      maximum = mm[1];
+    }
+  }
 
   const int epb = 8 / bits;
   const int data_bytes = (cols + epb - 1) / epb;
@@ -242,6 +256,7 @@ __global__ __launch_bounds__(256) void quantize_rowwise_kernel(
     else store_run(sb, (uint64_t)(sb0 & 0xffffu) | ((uint64_t)(sb1 & 0xffffu) << 16), 4);
   }
   const int run_bytes = RUN / epb;
+  const int wrap_from = cols & ~31;
   for (int j0 = sub * RUN; j0 < cols; j0 += lpr * RUN) {
     float xs[RUN];
     int n;
@@ -255,7 +270,25 @@ __global__ __launch_bounds__(256) void quantize_rowwise_kernel(
     for (int k = 0; k < RUN; ++k) {
       if (k < n) {
         float r = __builtin_rintf((xs[k] - minimum) * inverse_scale); // lrintf: to nearest, ties to even
-        if (clamp) r = r < 0.0f ? 0.0f : (r > (float)maxq ? (float)maxq : r);
+        // Only elements outside extremes that the caller brought can leave 0 .. maxq in the 8-bit
+        // float-pair format. The reference's vector code then saturates the leading whole groups
+        // of 32 columns and keeps the low byte of the rounded integer in the columns behind them;
+        // a value that does not fit 32 bits converts to 0x80000000 there, which both rules turn
+        // into 0 (src/QuantUtilsAvx2.cc:1912-1950).
+        if (clamp) {
+          // fp16-pair formats clamp the rounded value as a 32-bit integer. Beyond 32 bits (extremes
+          // from the caller only) that integer is 0x80000000 in the whole groups of 32 columns of
+          // the 2- and 4-bit formats and the low half of the 64-bit integer in the other columns
+          // (src/QuantUtilsAvx2.cc:1697-1722, :1768-1773).
+          if (min_max && !(__builtin_fabsf(r) < 2147483648.0f)) {
+            if ((bits < 8 && j0 + k < wrap_from) || !(__builtin_fabsf(r) < 9223372036854775808.0f)) r = 0.0f;
+            else r = (float)(int32_t)(uint32_t)(uint64_t)(int64_t)r;
+          }
+          r = r < 0.0f ? 0.0f : (r > (float)maxq ? (float)maxq : r);
+        } else if (min_max) {
+          if (!(__builtin_fabsf(r) < 2147483648.0f)) r = 0.0f;
+          else if (j0 + k < wrap_from) r = r < 0.0f ? 0.0f : (r > 255.0f ? 255.0f : r);
+        }
         const uint32_t q = (uint32_t)(int)r & 0xffu;
         if (bits == 8 && k >= 4) w1 |= q << ((k - 4) * 8);
         else w0 |= q << (k * bits);
@@ -428,7 +461,7 @@ int lanes_per_row(int32_t cols, int run) {
 
 hipError_t launch_quantize_rowwise(const void* input, bool half_in, int64_t rows, int32_t cols, int32_t bits,
                                    int32_t sb_float, int32_t layout, int64_t out_stride, void* output,
-                                   hipStream_t stream) {
+                                   const void* min_max, hipStream_t stream) {
   if (rows <= 0 || cols <= 0) return hipSuccess;
   const int lpr = lanes_per_row(cols, RUN);
   const int64_t rows_per_block = 4 * (64 / lpr);
@@ -436,7 +469,7 @@ hipError_t launch_quantize_rowwise(const void* input, bool half_in, int64_t rows
   const dim3 grid(stream_blocks(blocks)), block(256);
 #define FBGEMM_AMD_LAUNCH_Q(H, B) \
   hipLaunchKernelGGL((quantize_rowwise_kernel<H, B>), grid, block, 0, stream, input, rows, cols, sb_float, layout, \
-                     out_stride, (uint8_t*)output, lpr, (const int32_t*)nullptr, 0, (int64_t)0)
+                     out_stride, (uint8_t*)output, lpr, (const int32_t*)nullptr, 0, (int64_t)0, min_max)
   if (half_in) {
     if (bits == 2) FBGEMM_AMD_LAUNCH_Q(true, 2);
     else if (bits == 4) FBGEMM_AMD_LAUNCH_Q(true, 4);
@@ -461,7 +494,8 @@ hipError_t launch_quantize_segments(const float* input, int64_t lines, int32_t T
   const int64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
   const dim3 grid(stream_blocks(blocks)), block(256);
   hipLaunchKernelGGL((quantize_rowwise_kernel<false, 8>), grid, block, 0, stream, (const void*)input, rows, max_D, 1, 0,
-                     (int64_t)total_D + 8 * (int64_t)T, output, lpr, d_seg_offsets, T, (int64_t)total_D);
+                     (int64_t)total_D + 8 * (int64_t)T, output, lpr, d_seg_offsets, T, (int64_t)total_D,
+                     (const void*)nullptr);
   return hipGetLastError();
 }
 

@@ -531,13 +531,15 @@ def quantized_row_bytes(cols, bit_rate, sb_float=False, layout=QLAYOUT_TRAILER):
     return (cols + epb - 1) // epb + (8 if (sb_float and layout == QLAYOUT_TRAILER) else 4)
 
 
-def quantize_rowwise(input, bit_rate, sb_float=False, layout=QLAYOUT_TRAILER, out=None):
+def quantize_rowwise(input, bit_rate, sb_float=False, layout=QLAYOUT_TRAILER, out=None, rowwise_min_max=None):
     """fp32 / fp16 ``[rows, cols]`` -> fused quantized rows, uint8 ``[rows, stride]``
     (FloatOrHalfToFusedNBitRowwiseQuantizedSBHalf, src/QuantUtils.cc:534-611;
     FloatOrHalfToFused8BitRowwiseQuantizedSBFloat, :677-718; TBE re-layout as
     fbgemm_gpu/fbgemm_gpu/tbe/utils/quantize.py:47-70). ``out`` may be a wider
-    (padded) row buffer; bytes beyond the row's own are left alone."""
-    _require_cuda(input, out)
+    (padded) row buffer; bytes beyond the row's own are left alone.
+    ``rowwise_min_max`` (``[rows, 2]``, the input's dtype: minimum, maximum) takes the
+    place of each row's own extremes (src/QuantUtilsAvx2.cc:1605-1628, :1831-1853)."""
+    _require_cuda(input, out, rowwise_min_max)
     if input.dim() != 2 or input.dtype not in (torch.float32, torch.float16):
         raise TypeError("input must be a 2-D fp32 or fp16 tensor")
     input = input.contiguous()
@@ -547,9 +549,14 @@ def quantize_rowwise(input, bit_rate, sb_float=False, layout=QLAYOUT_TRAILER, ou
                           device=input.device)
     if out.dtype != torch.uint8 or out.dim() != 2 or out.size(0) != rows or out.stride(1) != 1:
         raise ValueError("out must be uint8 [rows, stride] with unit column stride")
-    check(_lib.lib().fbgemm_amd_quantize_rowwise(
+    if rowwise_min_max is not None:
+        if rowwise_min_max.dtype != input.dtype or tuple(rowwise_min_max.shape) != (rows, 2):
+            raise ValueError("rowwise_min_max must be [rows, 2] of the input's dtype")
+        rowwise_min_max = rowwise_min_max.contiguous()
+    check(_lib.lib().fbgemm_amd_quantize_rowwise_min_max(
         _ptr(input), _TORCH_OUT[input.dtype], rows, cols, bit_rate, int(sb_float), layout,
-        out.stride(0) if rows > 1 else out.size(1), _ptr(out), _stream()))
+        out.stride(0) if rows > 1 else out.size(1), _ptr(out),
+        _ptr(rowwise_min_max) if rowwise_min_max is not None else None, _stream()))
     return out
 
 

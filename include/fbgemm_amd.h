@@ -421,6 +421,20 @@ int fbgemm_amd_quantize_rowwise(
     const void* d_input, int32_t input_ty, int64_t rows, int32_t cols, int32_t bit_rate, int32_t sb_float,
     int32_t layout, int64_t out_row_stride, void* d_output, void* stream);
 
+/* The same with extremes the caller brings: the `rowwise_min_max` argument of
+ * FloatOrHalfToFusedNBitRowwiseQuantizedSBHalf / FloatOrHalfToFused8BitRowwiseQuantizedSBFloat
+ * (include/fbgemm/QuantUtils.h:277-283, :311-317; src/QuantUtilsAvx2.cc:1605-1628, :1831-1853).
+ * d_rowwise_min_max holds [rows][2] values of the input's type, minimum then
+ * maximum, which take the place of the row's own extremes; null means "find
+ * them", as the call above. Elements outside the extremes given: the 2 / 4 / 8
+ * bit fp16-pair formats saturate to 0 .. 2^bit_rate - 1; the 8-bit fp32-pair
+ * format does what the reference's vector code does, saturate in the leading
+ * whole groups of 32 columns and keep the low byte of the rounded integer in
+ * the columns behind them. */
+int fbgemm_amd_quantize_rowwise_min_max(
+    const void* d_input, int32_t input_ty, int64_t rows, int32_t cols, int32_t bit_rate, int32_t sb_float,
+    int32_t layout, int64_t out_row_stride, void* d_output, const void* d_rowwise_min_max, void* stream);
+
 /* The inverses (src/QuantUtils.cc:743-789 FusedNBitRowwiseQuantizedSBHalfToFloatOrHalf,
  * :847-892 Fused8BitRowwiseQuantizedSBFloatToFloatOrHalf): element =
  * float(double(scale) * q + double(bias)), written as fp32, fp16 (round to

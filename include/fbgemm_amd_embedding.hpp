@@ -268,8 +268,9 @@ GenerateEmbeddingSpMDMNBitRowWiseSparse(int bit_rate, const std::int64_t block_s
 
 // ---- row-wise quantizers (include/fbgemm/QuantUtils.h:276-334 of the reference) ----
 // Same names and argument lists; every pointer is a DEVICE pointer; the call
-// returns when the work is done. `rowwise_min_max` (precomputed extremes) is
-// not supported and must be null.
+// returns when the work is done. `rowwise_min_max`, when given, is a device
+// array of [input_rows][2] values (minimum, maximum) that take the place of
+// each row's own extremes.
 
 namespace detail {
 template <typename T>
@@ -302,11 +303,11 @@ void FloatOrHalfToFusedNBitRowwiseQuantizedSBHalf(int bit_rate, const InputType*
                                                   int input_columns, std::uint8_t* output,
                                                   const InputType* rowwise_min_max = nullptr) {
   static_assert(!std::is_same_v<InputType, bfloat16>, "input is float or float16");
-  if (rowwise_min_max) throw std::invalid_argument("fbgemm_amd: rowwise_min_max is not supported");
   const int epb = 8 / bit_rate;
-  detail::done(fbgemm_amd_quantize_rowwise(input, detail::float_ty<InputType>(), (std::int64_t)input_rows, input_columns,
-                                           bit_rate, 0, FBGEMM_AMD_QLAYOUT_TRAILER, (input_columns + epb - 1) / epb + 4,
-                                           output, stream_ref()));
+  detail::done(fbgemm_amd_quantize_rowwise_min_max(input, detail::float_ty<InputType>(), (std::int64_t)input_rows,
+                                                   input_columns, bit_rate, 0, FBGEMM_AMD_QLAYOUT_TRAILER,
+                                                   (input_columns + epb - 1) / epb + 4, output, rowwise_min_max,
+                                                   stream_ref()));
 }
 
 template <typename OutputType>
@@ -323,9 +324,9 @@ template <typename InputType>
 void FloatOrHalfToFused8BitRowwiseQuantizedSBFloat(const InputType* input, std::size_t input_rows, int input_columns,
                                                    std::uint8_t* output, const InputType* rowwise_min_max = nullptr) {
   static_assert(!std::is_same_v<InputType, bfloat16>, "input is float or float16");
-  if (rowwise_min_max) throw std::invalid_argument("fbgemm_amd: rowwise_min_max is not supported");
-  detail::done(fbgemm_amd_quantize_rowwise(input, detail::float_ty<InputType>(), (std::int64_t)input_rows, input_columns,
-                                           8, 1, FBGEMM_AMD_QLAYOUT_TRAILER, input_columns + 8, output, stream_ref()));
+  detail::done(fbgemm_amd_quantize_rowwise_min_max(input, detail::float_ty<InputType>(), (std::int64_t)input_rows,
+                                                   input_columns, 8, 1, FBGEMM_AMD_QLAYOUT_TRAILER, input_columns + 8,
+                                                   output, rowwise_min_max, stream_ref()));
 }
 
 template <typename OutputType>

@@ -85,6 +85,8 @@ def _lib(impl):
         lib.oracle_quantize_rowwise.argtypes = [
             _c.c_void_p, _c.c_int, _c.c_int64, _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int64, _c.c_void_p]
         lib.oracle_quantize_rowwise.restype = None
+        lib.oracle_quantize_rowwise_min_max.argtypes = lib.oracle_quantize_rowwise.argtypes + [_c.c_void_p]
+        lib.oracle_quantize_rowwise_min_max.restype = None
         lib.oracle_dequantize_rowwise.argtypes = [
             _c.c_void_p, _c.c_int64, _c.c_int64, _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32, _c.c_int32, _c.c_void_p]
         lib.oracle_dequantize_rowwise.restype = None
@@ -99,14 +101,17 @@ def _lib(impl):
     elif impl == "refquant":
         if not os.path.exists(REF_QUANT_SO):
             raise FileNotFoundError(REF_QUANT_SO)
-        # lazy binding: the reference's vector translation units are not part of
-        # this build, and nothing that is called here reaches them
+        # lazy binding: of the reference's vector translation units only the AVX2 quantizers
+        # are part of this build, and nothing that is called here reaches the others
         lib = _c.CDLL(REF_QUANT_SO, mode=os.RTLD_LAZY)
         lib.ref_quantize_nbit.argtypes = [_c.c_int, _c.c_void_p, _c.c_int, _c.c_int64, _c.c_int, _c.c_void_p]
         lib.ref_quantize_8bit.argtypes = [_c.c_void_p, _c.c_int, _c.c_int64, _c.c_int, _c.c_void_p]
         lib.ref_dequantize_nbit.argtypes = [_c.c_int, _c.c_void_p, _c.c_int64, _c.c_int, _c.c_int, _c.c_void_p]
         lib.ref_dequantize_8bit.argtypes = [_c.c_void_p, _c.c_int64, _c.c_int, _c.c_int, _c.c_void_p]
-        for f in (lib.ref_quantize_nbit, lib.ref_quantize_8bit, lib.ref_dequantize_nbit, lib.ref_dequantize_8bit):
+        lib.ref_quantize_nbit_avx2.argtypes = lib.ref_quantize_nbit.argtypes + [_c.c_void_p]
+        lib.ref_quantize_8bit_avx2.argtypes = lib.ref_quantize_8bit.argtypes + [_c.c_void_p]
+        for f in (lib.ref_quantize_nbit, lib.ref_quantize_8bit, lib.ref_dequantize_nbit, lib.ref_dequantize_8bit,
+                  lib.ref_quantize_nbit_avx2, lib.ref_quantize_8bit_avx2):
             f.restype = None
     else:
         raise ValueError(impl)
@@ -418,21 +423,35 @@ def quantized_row_bytes(cols, bit_rate, sb_float, layout):
     return (cols + epb - 1) // epb + (8 if (sb_float and layout == LAYOUT_TRAILER) else 4)
 
 
-def quantize_rowwise(x, bit_rate, sb_float=False, layout=LAYOUT_TRAILER, out_stride=None, impl="oracle", fill=0):
+def quantize_rowwise(x, bit_rate, sb_float=False, layout=LAYOUT_TRAILER, out_stride=None, impl="oracle", fill=0,
+                     min_max=None):
     """x: [rows, cols] float32 or float16 (numpy). Returns uint8 [rows, out_stride].
-    impl: "oracle" or "ref" (the reference's scalar routine, trailer layout only)."""
+    impl: "oracle", "ref" (the reference's scalar routine, trailer layout only) or "ref_avx2"
+    (the reference's AVX2 routine, trailer layout only). min_max: [rows, 2] of x's dtype, the
+    extremes to use in place of each row's own ("oracle" and "ref_avx2" only)."""
     x = np.ascontiguousarray(x)
     assert x.ndim == 2 and x.dtype in (np.float32, np.float16)
     rows, cols = x.shape
+    if min_max is not None:
+        min_max = np.ascontiguousarray(min_max)
+        assert min_max.dtype == x.dtype and min_max.shape == (rows, 2)
     need = quantized_row_bytes(cols, bit_rate, sb_float, layout)
     out_stride = need if out_stride is None else out_stride
     out = np.full((rows, out_stride), fill, np.uint8)
     half = int(x.dtype == np.float16)
     if impl == "oracle":
-        _lib("oracle").oracle_quantize_rowwise(_ptr(x), half, rows, cols, bit_rate, int(sb_float), layout,
-                                               out_stride, _ptr(out))
-    else:
+        _lib("oracle").oracle_quantize_rowwise_min_max(_ptr(x), half, rows, cols, bit_rate, int(sb_float), layout,
+                                                       out_stride, _ptr(out),
+                                                       None if min_max is None else _ptr(min_max))
+    elif impl == "ref_avx2":
         assert layout == LAYOUT_TRAILER and out_stride == need
+        mm = None if min_max is None else _ptr(min_max)
+        if sb_float:
+            _lib("refquant").ref_quantize_8bit_avx2(_ptr(x), half, rows, cols, _ptr(out), mm)
+        else:
+            _lib("refquant").ref_quantize_nbit_avx2(bit_rate, _ptr(x), half, rows, cols, _ptr(out), mm)
+    else:
+        assert layout == LAYOUT_TRAILER and out_stride == need and min_max is None
         if sb_float:
             _lib("refquant").ref_quantize_8bit(_ptr(x), half, rows, cols, _ptr(out))
         else:

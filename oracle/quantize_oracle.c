@@ -56,8 +56,32 @@ static void row_extremes(const void* in, int half_in, int64_t base, int cols, fl
  *   elements (an fp32 pair is rounded to fp16 on the way, as quantize_embs does).
  * Bytes of a row beyond what the format defines are left alone.
  */
+void oracle_quantize_rowwise_min_max(const void* input, int half_in, int64_t rows, int32_t cols, int32_t bit_rate,
+                                     int32_t sb_float, int32_t layout, int64_t out_stride, uint8_t* output,
+                                     const void* min_max);
+
 void oracle_quantize_rowwise(const void* input, int half_in, int64_t rows, int32_t cols, int32_t bit_rate,
                              int32_t sb_float, int32_t layout, int64_t out_stride, uint8_t* output) {
+  oracle_quantize_rowwise_min_max(input, half_in, rows, cols, bit_rate, sb_float, layout, out_stride, output, 0);
+}
+
+/*
+ * min_max, when not null: [rows][2] values of the input's type, (minimum, maximum), used in place
+ * of the row's own extremes (src/QuantUtilsAvx2.cc:1605-1628, :1831-1853 -- only the reference's
+ * vector routines take them, its scalar *Ref routines do not). An element outside them:
+ *   fp16-pair formats: clamped to 0 .. 2^bit_rate - 1 at every column (:1719-1722 for whole groups
+ *     of 32 columns, :1768-1773 for the rest); what is clamped is the rounded value as a 32-bit
+ *     integer, which for a value beyond 32 bits is 0x80000000 in the whole groups of 32 columns
+ *     of the 2- and 4-bit formats and the low half of the 64-bit integer in the other columns;
+ *   8-bit fp32-pair format: columns in the leading whole groups of 32 saturate to 0 .. 255 (the
+ *     signed 32->16 and unsigned 16->8 packs, :1930-1932); the columns behind keep the low byte
+ *     of the rounded 32-bit integer (:1938-1945 byte shuffle, :1947-1950 lrintf to uint8_t). A
+ *     value that does not fit 32 bits (or a NaN) converts to 0x80000000, which both rules turn
+ *     into 0.
+ */
+void oracle_quantize_rowwise_min_max(const void* input, int half_in, int64_t rows, int32_t cols, int32_t bit_rate,
+                                     int32_t sb_float, int32_t layout, int64_t out_stride, uint8_t* output,
+                                     const void* min_max) {
   const int epb = 8 / bit_rate;
   const int data_bytes = (cols + epb - 1) / epb;
   const int maxq = (1 << bit_rate) - 1;
@@ -67,6 +91,10 @@ void oracle_quantize_rowwise(const void* input, int half_in, int64_t rows, int32
     uint8_t* sb = layout == LAYOUT_TBE ? out_row : out_row + data_bytes;
     float minimum, maximum;
     row_extremes(input, half_in, r * (int64_t)cols, cols, &minimum, &maximum);
+    if (min_max) {
+      minimum = in_elem(min_max, half_in, 2 * r);
+      maximum = in_elem(min_max, half_in, 2 * r + 1);
+    }
     if (sb_float) {
       const float range = maximum - minimum;
       const float scale = range / 255.0f;
@@ -79,8 +107,18 @@ void oracle_quantize_rowwise(const void* input, int half_in, int64_t rows, int32
         memcpy(sb, &scale, 4);
         memcpy(sb + 4, &minimum, 4);
       }
-      for (int j = 0; j < cols; ++j)
-        data[j] = (uint8_t)lrintf((in_elem(input, half_in, r * (int64_t)cols + j) - minimum) * inverse_scale);
+      for (int j = 0; j < cols; ++j) {
+        const float v = rintf((in_elem(input, half_in, r * (int64_t)cols + j) - minimum) * inverse_scale);
+        if (!min_max) {
+          data[j] = (uint8_t)lrintf(v);
+        } else if (!(fabsf(v) < 2147483648.0f)) {
+          data[j] = 0; /* the conversion yields 0x80000000: saturates to 0, and its low byte is 0 */
+        } else if (j < cols / 32 * 32) {
+          data[j] = (uint8_t)(v > 0.0f ? (v > 255.0f ? 255.0f : v) : 0.0f);
+        } else {
+          data[j] = (uint8_t)(int32_t)v;
+        }
+      }
     } else {
       const uint16_t min16 = oracle_float2half_rn(minimum);
       minimum = oracle_half2float(min16);
@@ -98,8 +136,20 @@ void oracle_quantize_rowwise(const void* input, int half_in, int64_t rows, int32
       memcpy(sb + 2, &min16, 2);
       for (int j = 0; j < cols; ++j) {
         const float x = in_elem(input, half_in, r * (int64_t)cols + j);
-        long q = lrintf((x - minimum) * inverse_scale);
-        int qi = (int)q < maxq ? (int)q : maxq;
+        const float v = rintf((x - minimum) * inverse_scale);
+        int32_t q;
+        if (!min_max) {
+          q = (int32_t)lrintf(v);
+        } else if (bit_rate < 8 && j < cols / 32 * 32) {
+          /* whole groups of 32 columns, 2 and 4 bits: the 32-bit conversion yields 0x80000000 for
+           * what does not fit (a NaN too), which the packs saturate to 0 (:1697-1722) */
+          q = fabsf(v) < 2147483648.0f ? (int32_t)v : INT32_MIN;
+        } else {
+          /* the other columns: lrintf's 64-bit result cut to its low 32 bits by std::min<int>
+           * (:1768-1773); 0x8000000000000000 for what does not fit 64 bits */
+          q = fabsf(v) < 9223372036854775808.0f ? (int32_t)(uint32_t)(uint64_t)(int64_t)v : 0;
+        }
+        int qi = q < maxq ? q : maxq;
         qi = qi > 0 ? qi : 0;
         if (j % epb == 0) data[j / epb] = (uint8_t)qi;
         else data[j / epb] |= (uint8_t)(qi << ((j % epb) * bit_rate));

@@ -32,6 +32,9 @@ extern "C" int oracle_embedding_spmdm_fp8(
     int64_t output_stride, int64_t input_stride, int exponent_bits, int exponent_bias, int skip_minus_one);
 extern "C" void oracle_quantize_rowwise(const void* input, int half_in, int64_t rows, int32_t cols, int32_t bit_rate,
                                         int32_t sb_float, int32_t layout, int64_t out_stride, uint8_t* output);
+extern "C" void oracle_quantize_rowwise_min_max(const void* input, int half_in, int64_t rows, int32_t cols,
+                                                int32_t bit_rate, int32_t sb_float, int32_t layout, int64_t out_stride,
+                                                uint8_t* output, const void* min_max);
 extern "C" void oracle_dequantize_rowwise(const uint8_t* input, int64_t rows, int64_t in_stride, int32_t cols,
                                           int32_t bit_rate, int32_t sb_float, int32_t layout, int32_t output_ty,
                                           void* output);
@@ -297,6 +300,52 @@ void run_quantizers(int rows, int cols, unsigned seed) {
   Dev<uint16_t> d_half(half_init);
   fbgemm_amd::Fused8BitRowwiseQuantizedSBFloatToFloatOrHalf<std::uint16_t>(d_q8.p, rows, stride8, d_half.p);
   CHECK(d_half.host() == half_want, "8-bit rows dequantize to fp16 differently");
+
+  // extremes from the caller, narrower than the rows' own, so that the clamping rules show
+  std::vector<float> mm((size_t)rows * 2);
+  for (int r = 0; r < rows; ++r) {
+    mm[2 * r] = -4.f + (float)(rng() % 1000) / 500.f;
+    mm[2 * r + 1] = 2.f + (float)(rng() % 1000) / 500.f;
+  }
+  Dev<float> d_mm(mm);
+  for (int bit_rate : {2, 4, 8}) {
+    const int epb = 8 / bit_rate;
+    if (cols % epb) continue;
+    const int stride = cols / epb + 4;
+    std::vector<uint8_t> want((size_t)rows * stride), zero((size_t)rows * stride, 0);
+    oracle_quantize_rowwise_min_max(x.data(), 0, rows, cols, bit_rate, 0, 0, stride, want.data(), mm.data());
+    Dev<uint8_t> d_q(zero);
+    fbgemm_amd::FloatOrHalfToFusedNBitRowwiseQuantizedSBHalf<float>(bit_rate, d_x.p, rows, cols, d_q.p, d_mm.p);
+    CHECK(d_q.host() == want, "%d-bit rows with the caller's extremes differ (%d x %d)", bit_rate, rows, cols);
+  }
+  oracle_quantize_rowwise_min_max(x.data(), 0, rows, cols, 8, 1, 0, stride8, want8.data(), mm.data());
+  Dev<uint8_t> d_q8m(zero8);
+  fbgemm_amd::FloatOrHalfToFused8BitRowwiseQuantizedSBFloat<float>(d_x.p, rows, cols, d_q8m.p, d_mm.p);
+  CHECK(d_q8m.host() == want8, "8-bit rows with the caller's extremes differ (%d x %d)", rows, cols);
+}
+
+// The reference's fixed-number case (test/QuantUtilsTest.cc:547-611, :851-945): two rows of four,
+// their extremes handed in, and the bytes its authors worked out by hand.
+void run_fixed_numbers() {
+  const std::vector<float> x = {1, 1, 1, 1, -64, -2.75f, 61.625f, 191};
+  const std::vector<float> mm = {1, 1, -64, 191};
+  Dev<float> d_x(x), d_mm(mm);
+  const std::vector<uint8_t> want8h = {0, 0, 0, 0, 0x00, 0x3c, 0x00, 0x3c, 0, 61, 126, 255, 0x00, 0x3c, 0x00, 0xd4};
+  const std::vector<uint8_t> want4 = {0x00, 0x00, 0x00, 0x3c, 0x00, 0x3c, 0x40, 0xf7, 0x40, 0x4c, 0x00, 0xd4};
+  const std::vector<uint8_t> want2 = {0x00, 0x00, 0x3c, 0x00, 0x3c, 0xd4, 0x50, 0x55, 0x00, 0xd4};
+  const std::vector<uint8_t> want8f = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0x80, 0x3f, 0, 61, 126, 255, 0, 0, 0x80, 0x3f, 0, 0, 0x80, 0xc2};
+  for (int with = 0; with < 2; ++with) {
+    const float* extremes = with ? d_mm.p : nullptr;
+    for (int bit_rate : {2, 4, 8}) {
+      const auto& want = bit_rate == 2 ? want2 : bit_rate == 4 ? want4 : want8h;
+      Dev<uint8_t> d_q(std::vector<uint8_t>(want.size(), 0));
+      fbgemm_amd::FloatOrHalfToFusedNBitRowwiseQuantizedSBHalf<float>(bit_rate, d_x.p, 2, 4, d_q.p, extremes);
+      CHECK(d_q.host() == want, "fixed numbers, %d bits, extremes %s", bit_rate, with ? "given" : "found");
+    }
+    Dev<uint8_t> d_q(std::vector<uint8_t>(want8f.size(), 0));
+    fbgemm_amd::FloatOrHalfToFused8BitRowwiseQuantizedSBFloat<float>(d_x.p, 2, 4, d_q.p, extremes);
+    CHECK(d_q.host() == want8f, "fixed numbers, 8 bits with fp32 pair, extremes %s", with ? "given" : "found");
+  }
 }
 
 int main() {
@@ -333,6 +382,7 @@ int main() {
   }
   for (int cols : {4, 8, 64, 100, 128, 260})
     for (int rows : {1, 7, 130}) run_quantizers(rows, cols, ++seed);
+  run_fixed_numbers();
   printf("%s: %d failure(s)\n", failures ? "FAILED" : "PASSED", failures);
   return failures ? 1 : 0;
 }

@@ -220,6 +220,43 @@ def test_quantize_matches_oracle(env, dtype, bit_rate, sb_float, layout):
             assert (got.cpu().numpy() == want).all(), (kind, cols)
 
 
+def caller_extremes(rng, x, mode):
+    lo, hi = x.astype(np.float32).min(1), x.astype(np.float32).max(1)
+    if mode == "wider":
+        lo, hi = lo - rng.uniform(0, 2, lo.shape), hi + rng.uniform(0, 2, hi.shape)
+    elif mode == "narrower":  # elements outside the extremes: the clamping / wrapping rules show
+        mid, half = (lo + hi) / 2, (hi - lo) / 2
+        lo, hi = mid - half * rng.uniform(0.1, 0.9, lo.shape), mid + half * rng.uniform(0.1, 0.9, hi.shape)
+    elif mode == "far":  # no range at all under spread-out values: beyond the 32-bit integers
+        lo, hi = lo + 1e-3, lo + 1e-3
+    elif mode == "steep":  # a tiny step: beyond 32 bits, and for the "large" rows beyond 64
+        lo, hi = np.zeros_like(lo), np.full_like(hi, 1e-6)
+    return np.stack([lo, hi], 1).astype(x.dtype)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("bit_rate,sb_float", [(2, False), (4, False), (8, False), (8, True)])
+@pytest.mark.parametrize("layout", [LAYOUT_TRAILER, LAYOUT_TBE])
+def test_quantize_with_caller_extremes_matches_oracle(env, dtype, bit_rate, sb_float, layout):
+    # rowwise_min_max of the reference's quantizers (include/fbgemm/QuantUtils.h:277-283, :311-317)
+    torch, ops = env
+    rng = np.random.default_rng(108)
+    for kind in ("normal", "uniform", "constant", "large"):
+        for cols in (1, 4, 8, 12, 31, 32, 36, 40, 63, 64, 72, 100, 128, 260, 1024):
+            x = rows_of(rng, kind, 9, cols, dtype)
+            for mode in ("true", "wider", "narrower", "far", "steep"):
+                if mode in ("far", "steep") and dtype == np.float16:
+                    continue
+                if mode == "steep" and kind != "large":
+                    x = (x * 1e4).astype(dtype)
+                mm = caller_extremes(rng, x, mode)
+                want = oracle.quantize_rowwise(x, bit_rate, sb_float, layout, min_max=mm)
+                got = ops.quantize_rowwise(dev(torch, x), bit_rate, sb_float, layout, rowwise_min_max=dev(torch, mm))
+                assert (got.cpu().numpy() == want).all(), (kind, cols, mode)
+    with pytest.raises(ValueError):
+        ops.quantize_rowwise(dev(torch, x), bit_rate, sb_float, layout, rowwise_min_max=dev(torch, mm[:-1]))
+
+
 def test_quantize_into_padded_rows_leaves_padding_alone(env):
     torch, ops = env
     rng = np.random.default_rng(107)

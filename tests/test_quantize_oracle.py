@@ -1,7 +1,9 @@
 """Pins oracle/quantize_oracle.c without the GPU: bit for bit against the
 reference's own scalar row-wise quantizers compiled from its sources (the *Ref
 routines its test/QuantUtilsTest.cc holds the vector code to), and against
-what the arithmetic fixes."""
+what the arithmetic fixes. Caller-supplied extremes (rowwise_min_max), which only the
+reference's AVX2 routines take, are pinned against those routines compiled from its
+sources and against the known answers of its test/QuantUtilsTest.cc:547-611."""
 import numpy as np
 import pytest
 
@@ -134,3 +136,76 @@ def test_tbe_layout_is_the_trailer_layout_rearranged(bit_rate, sb_float):
     back = oracle.dequantize_rowwise(tbe, cols, bit_rate, False, LAYOUT_TBE)
     want = oracle.dequantize_rowwise(np.concatenate([tr[:, :nb], want_sb], 1), cols, bit_rate, False, LAYOUT_TRAILER)
     assert (back == want).all()
+
+
+# ---- caller-supplied extremes (rowwise_min_max) -------------------------------------------
+
+# test/QuantUtilsTest.cc:551-598: two rows of four, their true extremes, and the bytes the
+# reference's authors worked out by hand for every format
+FIXED_INPUT = np.array([[1, 1, 1, 1], [-64, -2.75, 61.625, 191]], np.float32)
+FIXED_MIN_MAX = np.array([[1, 1], [-64, 191]], np.float32)
+FIXED_EXPECTED = {
+    (8, False): [[0, 0, 0, 0, 0x00, 0x3c, 0x00, 0x3c], [0, 61, 126, 255, 0x00, 0x3c, 0x00, 0xd4]],
+    (4, False): [[0x00, 0x00, 0x00, 0x3c, 0x00, 0x3c], [0x40, 0xf7, 0x40, 0x4c, 0x00, 0xd4]],
+    (2, False): [[0b00000000, 0x00, 0x3c, 0x00, 0x3c], [0b11010100, 0x50, 0x55, 0x00, 0xd4]],
+    (8, True): [[0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0x80, 0x3f], [0, 61, 126, 255, 0, 0, 0x80, 0x3f, 0, 0, 0x80, 0xc2]],
+}
+
+
+@pytest.mark.parametrize("bit_rate,sb_float", list(FIXED_EXPECTED))
+def test_min_max_known_answers(bit_rate, sb_float):
+    want = np.array(FIXED_EXPECTED[(bit_rate, sb_float)], np.uint8)
+    for dtype in (np.float32, np.float16):
+        x, mm = FIXED_INPUT.astype(dtype), FIXED_MIN_MAX.astype(dtype)
+        assert (oracle.quantize_rowwise(x, bit_rate, sb_float, min_max=mm) == want).all()
+        assert (oracle.quantize_rowwise(x, bit_rate, sb_float) == want).all()
+    # other extremes give other rows (QuantUtilsTest.cc:880-909)
+    wrong = np.array([[10, 15], [-14, 1]], np.float32)
+    assert (oracle.quantize_rowwise(FIXED_INPUT, bit_rate, sb_float, min_max=wrong) != want).any()
+
+
+def bracketing(rng, x, mode):
+    lo, hi = x.astype(np.float32).min(1), x.astype(np.float32).max(1)
+    if mode == "true":
+        pass
+    elif mode == "wider":
+        lo, hi = lo - rng.uniform(0, 2, lo.shape), hi + rng.uniform(0, 2, hi.shape)
+    elif mode == "narrower":  # elements fall outside: clamping / wrapping rules show
+        mid, half = (lo + hi) / 2, (hi - lo) / 2
+        lo, hi = mid - half * rng.uniform(0.1, 0.9, lo.shape), mid + half * rng.uniform(0.1, 0.9, hi.shape)
+    elif mode == "far":  # (x - min) * inverse_scale beyond the 32-bit integers
+        lo, hi = lo + 1e-3, lo + 1e-3 + 1e-12
+    elif mode == "steep":  # a tiny step under values spread widely: beyond 32 bits, within 64
+        lo, hi = np.zeros_like(lo), np.full_like(hi, 1e-6)
+    return np.stack([lo, hi], 1).astype(x.dtype)
+
+
+@needs_ref
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("bit_rate,sb_float", [(2, False), (4, False), (8, False), (8, True)])
+def test_min_max_matches_reference_avx2(dtype, bit_rate, sb_float):
+    rng = np.random.default_rng(24)
+    for kind in ("normal", "uniform", "constant", "large"):
+        for cols in (4, 8, 12, 31, 32, 36, 40, 63, 64, 72, 100, 128, 260):
+            if cols % (8 // bit_rate):
+                continue
+            x = rows_of(rng, kind, 9, cols, dtype)
+            for mode in ("true", "wider", "narrower", "far", "steep"):
+                if mode == "steep":
+                    x = (x * (1e4 if kind != "large" else 1)).astype(dtype)
+                if mode in ("far", "steep") and dtype == np.float16:
+                    continue
+                mm = bracketing(rng, x, mode)
+                want = oracle.quantize_rowwise(x, bit_rate, sb_float, impl="ref_avx2", min_max=mm)
+                got = oracle.quantize_rowwise(x, bit_rate, sb_float, min_max=mm)
+                assert (got == want).all(), (kind, cols, mode)
+
+
+@pytest.mark.parametrize("bit_rate,sb_float", [(2, False), (4, False), (8, False), (8, True)])
+def test_true_extremes_change_nothing(bit_rate, sb_float):
+    rng = np.random.default_rng(25)
+    for dtype in (np.float32, np.float16):
+        x = rows_of(rng, "normal", 13, 96, dtype)
+        mm = np.stack([x.min(1), x.max(1)], 1)
+        assert (oracle.quantize_rowwise(x, bit_rate, sb_float, min_max=mm) ==
+                oracle.quantize_rowwise(x, bit_rate, sb_float)).all()
