@@ -304,13 +304,41 @@ template <typename T>
 int grow(T** buf, int64_t* cap, int64_t need, hipStream_t stream);
 
 std::mutex g_mu;
-std::map<int, DeviceScratch> g_scratch;
 
+// The status block and scratch buffers behind the calls that own their scratch
+// (fbgemm_amd_spmdm_run, the lengths / bag-order / split-bag buffers of fbgemm_amd_spmdm_launch,
+// bounds checks, pruning): one set per host thread and device, so that threads calling
+// concurrently, each on a stream of its own, neither read each other's status bits nor free a
+// buffer another thread's enqueued kernel still uses. A thread that ends hands its sets to
+// g_idle_scratch (no HIP call at thread exit); the next new thread adopts one after a device-wide
+// synchronize. Calls of ONE thread share its set: those must be ordered on one stream.
+std::map<int, std::vector<DeviceScratch>> g_idle_scratch; // guarded by g_mu
+
+struct ThreadScratch {
+  std::map<int, DeviceScratch> by_device;
+  ~ThreadScratch() {
+    std::lock_guard<std::mutex> lk(g_mu);
+    for (auto& kv : by_device)
+      if (kv.second.status) g_idle_scratch[kv.first].push_back(kv.second);
+  }
+};
+thread_local ThreadScratch t_scratch;
+
+// call with g_mu held
 int get_scratch(DeviceScratch** out) {
   int dev = 0;
   HIP_TRY(hipGetDevice(&dev));
-  DeviceScratch& s = g_scratch[dev];
-  if (!s.status) HIP_TRY(hipMalloc((void**)&s.status, sizeof(Status)));
+  DeviceScratch& s = t_scratch.by_device[dev];
+  if (!s.status) {
+    std::vector<DeviceScratch>& idle = g_idle_scratch[dev];
+    if (!idle.empty()) {
+      HIP_TRY(hipDeviceSynchronize()); // what its last owner enqueued has finished
+      s = idle.back();
+      idle.pop_back();
+    } else {
+      HIP_TRY(hipMalloc((void**)&s.status, sizeof(Status)));
+    }
+  }
   *out = &s;
   return 0;
 }

@@ -131,7 +131,11 @@ enum { FBGEMM_AMD_ACC_EXACT = 0, FBGEMM_AMD_ACC_FAST = 1 };
  * variant: data_size then bounds the LOGICAL ids and the table maps them to
  * physical rows (-1 = pruned). d_status must be a cleared status block.
  * With use_offsets == 0 the call makes a prefix sum of the lengths into a
- * library-owned scratch buffer first (grown with hipMalloc when too small). */
+ * library-owned scratch buffer first (grown with hipMalloc when too small).
+ * The library keeps one set of scratch buffers (and one status block for
+ * fbgemm_amd_spmdm_run) per host thread and device: host threads may call
+ * concurrently, each on its own stream; the calls of one thread that use
+ * scratch must be ordered on one stream. */
 int fbgemm_amd_spmdm_launch(
     const fbgemm_amd_spmdm_config* cfg, int64_t output_size, int64_t index_size,
     int64_t data_size, const void* d_input, const void* d_indices,

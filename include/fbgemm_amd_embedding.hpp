@@ -8,7 +8,10 @@
 //     stream otherwise) and, like the reference, returns only when done, with
 //     the reference's bool;
 //   * `prefetch` and THREAD_LOCAL are accepted and ignored (they tune the CPU
-//     code generator).
+//     code generator). Kernels may be called from several host threads at once,
+//     as the reference's may: every thread has its own stream setting, status
+//     block and scratch buffers inside the library. Calls of one thread run one
+//     after the other (each returns when its work is done);
 // Header-only; link against libfbgemm_amd.so.
 #pragma once
 

@@ -8,9 +8,11 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cstdio>
 #include <cstring>
 #include <random>
+#include <thread>
 #include <vector>
 
 #include "../../include/fbgemm_amd_embedding.hpp"
@@ -57,7 +59,7 @@ struct Dev {
   }
 };
 
-static int failures = 0;
+static std::atomic<int> failures{0};
 #define CHECK(cond, ...) do { if (!(cond)) { ++failures; printf("FAIL %s:%d: ", __FILE__, __LINE__); printf(__VA_ARGS__); printf("\n"); } } while (0)
 
 template <typename IndexType, typename OffsetType, typename OutType>
@@ -363,8 +365,9 @@ int main() {
           for (int corner = 0; corner < 4; ++corner) {
             if (bit_rate == 2 && s[2] % 4) continue;
             run_nbit<int64_t, int32_t, float>(bit_rate, s[2], s[0], s[1], s[3], weighted, normalize, true, corner, ++seed);
+            const bool offsets_form = corner != 3 && (seed & 1);
             run_nbit<int32_t, int64_t, fbgemm_amd::float16>(bit_rate, s[2], s[0], s[1], s[3], weighted, normalize,
-                                                            corner != 3 && (seed & 1), corner, ++seed);
+                                                            offsets_form, corner, ++seed);
           }
   for (auto& s : shapes)
     for (int weighted = 0; weighted < 2; ++weighted)
@@ -383,6 +386,29 @@ int main() {
   for (int cols : {4, 8, 64, 100, 128, 260})
     for (int rows : {1, 7, 130}) run_quantizers(rows, cols, ++seed);
   run_fixed_numbers();
-  printf("%s: %d failure(s)\n", failures ? "FAILED" : "PASSED", failures);
+  // Kernels called from several host threads at once, each on a stream of its own, as the
+  // reference's generated kernels may be: every thread mixes calls that succeed with calls
+  // that must return false (out-of-range index, unmatched lengths), lengths as well as offsets.
+  {
+    std::vector<std::thread> threads;
+    for (int th = 0; th < 4; ++th)
+      threads.emplace_back([th] {
+        hipStream_t stream;
+        if (hipStreamCreate(&stream) != hipSuccess) { ++failures; return; }
+        fbgemm_amd::set_stream(stream);
+        unsigned seed = 5000 + 1000 * th;
+        for (int it = 0; it < 12; ++it)
+          for (int corner = 0; corner < 4; ++corner) {
+            run_nbit<int64_t, int32_t, float>(4, 128, 10 + th, 400, 5, it & 1, it & 2, (it + th) & 1 || corner == 3 ? true : false,
+                                              corner, ++seed);
+            run_8bit<int32_t, int64_t>(64, 20, 300, 6, it & 1, it & 2, ++seed);
+          }
+        fbgemm_amd::set_stream(nullptr);
+        (void)hipStreamSynchronize(stream);
+        (void)hipStreamDestroy(stream);
+      });
+    for (auto& t : threads) t.join();
+  }
+  printf("%s: %d failure(s)\n", failures ? "FAILED" : "PASSED", failures.load());
   return failures ? 1 : 0;
 }
