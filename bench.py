@@ -48,10 +48,15 @@ def parse():
     ap.add_argument("--no-check", dest="check", action="store_false",
                     help="skip the parity gate (by default a sample of tables of the first forward is compared with "
                          "the oracle before anything is timed, and the line says \"checked\": true)")
-    ap.add_argument("--accumulate", default="exact", choices=["exact", "fast"],
-                    help="exact = the reference's sequence of fp32 roundings, bit-identical to the CPU path (the "
-                         "library's default); fast = the biases of a bag summed apart (tolerance grade: the parity "
-                         "gate then holds fp16 / bf16 output to one unit in the last place and fp32 output to 1e-5)")
+    ap.add_argument("--accumulate", default="fast", choices=["exact", "fast"],
+                    help="fast = the biases of a bag summed apart, the mode a plan is switched to for throughput "
+                         "(tolerance grade: the parity gate holds fp16 / bf16 output to one unit in the last place and "
+                         "fp32 output to 1e-5, the bound the path states); exact = the reference's sequence of fp32 "
+                         "roundings, bit-identical to the CPU path (the library's default). A table-batched run in "
+                         "fast mode also times the exact mode on the same inputs and prints it under "
+                         "\"exact_accumulate\" (--no-exact skips that)")
+    ap.add_argument("--no-exact", dest="exact_too", action="store_false",
+                    help="fast-mode runs only: do not also time the exact mode")
     ap.add_argument("--no-rank-records", action="store_true",
                     help="config 4 only: read the int32 mapping arrays in the forward instead of the compact "
                          "bitmap-and-rank form of the (order-preserving) mappings")
@@ -67,7 +72,8 @@ def parse():
 
 
 def traffic_from_profile(config_id):
-    """HBM bytes one lookup_kernel launch moves, from the committed hardware-counter
+    """HBM bytes the lookup kernels of one forward move (lookup_lean_kernel, and lookup_kernel for
+    the tables the lean kernel does not take), from the committed hardware-counter
     summary of this configuration (profiles/lookup_kernel_config<N>.txt): FETCH_SIZE
     and WRITE_SIZE (KiB per dispatch), each scaled by what the same counter read
     for the plain copy of known size that ran in the same process. None when the
@@ -86,7 +92,10 @@ def traffic_from_profile(config_id):
         total = 0.0
         for ctr in ("FETCH_SIZE", "WRITE_SIZE"):
             factor = copy_bytes / (vals[("calibration_copy_kernel", ctr)] * 1024.0)
-            total += vals[("lookup_kernel", ctr)] * 1024.0 * factor
+            kib = [vals[(k, ctr)] for k in ("lookup_lean_kernel", "lookup_kernel") if (k, ctr) in vals]
+            if not kib:
+                return None
+            total += sum(kib) * 1024.0 * factor
         return int(total)
     except (AttributeError, KeyError, ZeroDivisionError):
         return None
@@ -708,13 +717,14 @@ def parity_gate(p, out, launch, torch, np, accumulate="exact"):
     return tables
 
 
-def time_tbe(p, a, torch, np, steps, warmup, graph=False):
+def time_tbe(p, a, torch, np, steps, warmup, graph=False, accumulate=None):
     """Parity gate, warm-up, `steps` timed forwards of one table-batched problem.
     Returns the figures of the JSON line that depend on the measurement."""
     from fbgemm_amd import _lib
-    launch, out, st, plan = tbe_runner(p, torch, a.accumulate, not a.no_rank_records)
+    accumulate = accumulate or a.accumulate
+    launch, out, st, plan = tbe_runner(p, torch, accumulate, not a.no_rank_records)
     torch.cuda.synchronize()
-    checked = parity_gate(p, out, launch, torch, np, a.accumulate) if a.check else None
+    checked = parity_gate(p, out, launch, torch, np, accumulate) if a.check else None
     for _ in range(warmup):
         launch()
     torch.cuda.synchronize()
@@ -743,15 +753,25 @@ def time_tbe(p, a, torch, np, steps, warmup, graph=False):
     assert bits == 0, f"the lookup rejected its inputs: status {bits:#x} at {pos}"
     ms_per_step = wall * 1e3 / steps
     forward_ms = ev0.elapsed_time(ev1) / steps  # events on the launch stream, back-to-back forwards
-    kernel_ms, kernel_name = forward_ms, "lookup_kernel (+ bag_order_kernel), per graph replay"
+    kernel_ms, kernel_name = forward_ms, "lookup_lean_kernel / lookup_kernel (+ bag_order_kernel), per graph replay"
     if not graph:
         ms = (C.c_float * steps)()
         n = C.c_int32(0)
         _lib.check(_lib.lib().fbgemm_amd_tbe_plan_profile_read(plan.handle, ms, steps, C.byref(n)))
         assert n.value == steps
-        kernel_ms, kernel_name = sum(ms[:n.value]) / n.value, "lookup_kernel"
+        kernel_ms, kernel_name = sum(ms[:n.value]) / n.value, "lookup_lean_kernel (+ lookup_kernel for tables of other shapes)"
     return {"ms_per_step": ms_per_step, "forward_ms": forward_ms, "kernel_ms": kernel_ms, "kernel": kernel_name,
             "checked": checked}
+
+
+def exact_leg(p, a, torch, np, useful, steps, warmup):
+    """The same problem in the exact accumulate mode (gate: bit for bit), for the line of a fast-mode run."""
+    m = time_tbe(p, a, torch, np, steps, warmup, False, "exact")
+    return {"steps": steps, "warmup": warmup, "ms_per_step": round(m["ms_per_step"], 5),
+            "value": round(useful / (m["ms_per_step"] * 1e-3) / 1e9, 2), "kernel_ms": round(m["kernel_ms"], 5),
+            "forward_ms": round(m["forward_ms"], 5),
+            "roofline_frac": round(useful / (m["kernel_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+            "checked": bool(m["checked"])}
 
 
 def main():
@@ -866,6 +886,8 @@ def main():
                      "algorithmic_bytes_per_launch": useful // launches_per_step},
         "setup_s": round(build_s, 1),
     }
+    if p is not None and a.accumulate == "fast" and a.exact_too and not a.graph:
+        res["exact_accumulate"] = exact_leg(p, a, torch, np, useful, max(5, min(a.steps, 50)), max(1, min(a.warmup, 5)))
     if not a.no_cpu and p is not None:
         res["cpu_baseline"] = cpu_baseline_tbe(p, a.cpu_seconds, torch)
     elif not a.no_cpu:
@@ -896,6 +918,8 @@ def main():
                          "kernel_ms": round(m5["kernel_ms"], 5), "forward_ms": round(m5["forward_ms"], 5),
                          "algorithmic_bytes_per_launch": useful5},
             "setup_s": round(setup5, 1)}}
+        if a.accumulate == "fast" and a.exact_too:
+            res["also"]["config5"]["exact_accumulate"] = exact_leg(p5, a, torch, np, useful5, steps5, warm5)
     print(json.dumps(res))
 
 

@@ -143,21 +143,18 @@ void plan_lanes(TableDesc& d, uintptr_t base_addr, int64_t out_stride, bool has_
   const bool a4 = base_addr % 4 == 0 && d.weights_offset % 4 == 0 && d.row_stride % 4 == 0 &&
       d.data_off % 4 == 0 && (!has_sb || d.sb_off % 4 == 0);
   const int min_vb = bits >= 16 ? bits / 8 : 1;
-  static const int force_vb = env_int("FBGEMM_AMD_FORCE_VB", 0);
   int vb = min_vb;
   if (a4 && d.data_bytes % 16 == 0 && d.ty != ST_INT2) vb = 16;
   else if (a4 && d.data_bytes % 4 == 0) vb = 4;
-  if ((force_vb == 4 || narrow) && vb == 16) vb = 4;
-  if (force_vb == 1) vb = min_vb;
+  if (narrow && vb == 16) vb = 4;
   d.vb = vb;
   const int chunks = (d.data_bytes + vb - 1) / vb;
   // Wide rows: give a lane several 16-byte chunks (up to 32 accumulators), so
   // that the per-row bookkeeping is shared by more elements.
-  static const int max_chunks = env_int("FBGEMM_AMD_MAX_CHUNKS", 4);
   const int type_c = bits >= 16 ? 4 : (bits == 8 ? 2 : 1);
   int C = 1;
   if (vb == 16)
-    for (int c = std::min(type_c, max_chunks); c > 1; c >>= 1)
+    for (int c = type_c; c > 1; c >>= 1)
       if (chunks % c == 0 && chunks / c >= 2) { C = c; break; }
   d.chunks = C;
   d.lanes = std::max(2, std::min(64, chunks / C)); // >= 2: a wave stages at most 32 bags
@@ -166,12 +163,11 @@ void plan_lanes(TableDesc& d, uintptr_t base_addr, int64_t out_stride, bool has_
   // stride that is a multiple of 16: the header rides in chunk 0 and costs no
   // memory request of its own. Needs every 16-byte load of a row to stay
   // inside the row's stride and a single pass.
-  static const int inline_hdr = env_int("FBGEMM_AMD_INLINE_HDR", 1);
   d.inline_hdr = 0;
-  if (inline_hdr && has_sb && (d.ty == ST_INT4 || d.ty == ST_INT8) && !d.sb_fp32 && d.sb_off == 0 && d.data_off == 4 &&
-      base_addr % 16 == 0 && d.weights_offset % 16 == 0 && d.row_stride % 16 == 0 && force_vb == 0 && !narrow) {
+  if (has_sb && (d.ty == ST_INT4 || d.ty == ST_INT8) && !d.sb_fp32 && d.sb_off == 0 && d.data_off == 4 &&
+      base_addr % 16 == 0 && d.weights_offset % 16 == 0 && d.row_stride % 16 == 0 && !narrow) {
     const int nchunks = (d.data_bytes + 4 + 15) / 16;
-    const int Ci = (d.ty == ST_INT8 && max_chunks >= 2 && nchunks >= 4) ? 2 : 1;
+    const int Ci = (d.ty == ST_INT8 && nchunks >= 4) ? 2 : 1;
     const int lanes = std::max(2, (nchunks + Ci - 1) / Ci);
     // lanes that would idle because a bag may not straddle a quarter of the wave:
     // too many (9 lanes per bag) and the bags are laid end to end instead
@@ -856,10 +852,6 @@ int build_work_list(const std::vector<TableDesc>& tables, const std::vector<int>
                     fbgemm_amd_tbe_plan::WorkList* out) {
   *out = fbgemm_amd_tbe_plan::WorkList();
   if (members.empty()) return 0;
-  static const int xcd_lists = env_int("FBGEMM_AMD_XCD_LISTS", 1);
-  static const int interleave = env_int("FBGEMM_AMD_INTERLEAVE", 1);
-  static const int max_parts = env_int("FBGEMM_AMD_MAX_PARTS", 8);
-  static const int by_shape = env_int("FBGEMM_AMD_GROUP_BY_SHAPE", 1);
   struct Slice { int t, first, step, count; double cost; };
   std::vector<Slice> slices;
   double total_cost = 0;
@@ -873,11 +865,11 @@ int build_work_list(const std::vector<TableDesc>& tables, const std::vector<int>
     wave_cost[t] = G * row_cost(d);
     total_cost += wave_cost[t] * nwaves[t];
   }
-  const int nx = xcd_lists ? 8 : 1;
+  const int nx = 8;
   for (int t : members) {
     // slices no larger than 1/4 of an XCD's share; slice p takes waves p, p + parts, ...
     int parts = (int)std::ceil(wave_cost[t] * nwaves[t] / (total_cost / nx / 4.0 + 1e-9));
-    parts = std::max(1, std::min(parts, std::min(nwaves[t], std::min(nx, max_parts))));
+    parts = std::max(1, std::min(parts, std::min(nwaves[t], nx)));
     for (int p = 0; p < parts; ++p) {
       const int count = (nwaves[t] - p + parts - 1) / parts;
       slices.push_back(Slice{t, p, parts, count, wave_cost[t] * count});
@@ -905,7 +897,7 @@ int build_work_list(const std::vector<TableDesc>& tables, const std::vector<int>
     std::map<std::pair<int, int>, std::vector<Slice>> shapes; // slices of a shape, largest first (per_x order)
     for (const Slice& sl : per_x[x]) {
       const TableDesc& d = tables[sl.t];
-      shapes[(interleave && by_shape) ? std::make_pair((int)d.ty, (int)d.D) : std::make_pair(0, 0)].push_back(sl);
+      shapes[std::make_pair((int)d.ty, (int)d.D)].push_back(sl);
     }
     size_t depth = 0;
     for (auto& kv : shapes) depth = std::max(depth, kv.second.size());
@@ -915,12 +907,10 @@ int build_work_list(const std::vector<TableDesc>& tables, const std::vector<int>
         if (i >= kv.second.size()) continue;
         const Slice& sl = kv.second[i];
         const int G = bags_per_wave(tables[sl.t].lanes, tables[sl.t].packed);
-        // one shape only (or no interleaving asked for): slice after slice
-        const double base = (interleave && by_shape) ? (double)gidx : (interleave ? 0.0 : (double)gidx++);
         for (int k = 0; k < sl.count; ++k)
-          keyed.push_back({base + (k + 0.5) / sl.count, WaveWork{sl.t, (sl.first + k * sl.step) * G}});
+          keyed.push_back({(double)gidx + (k + 0.5) / sl.count, WaveWork{sl.t, (sl.first + k * sl.step) * G}});
       }
-      if (interleave && by_shape) ++gidx;
+      ++gidx;
     }
     std::stable_sort(keyed.begin(), keyed.end(),
                      [](const std::pair<double, WaveWork>& p, const std::pair<double, WaveWork>& q) { return p.first < q.first; });
@@ -928,14 +918,11 @@ int build_work_list(const std::vector<TableDesc>& tables, const std::vector<int>
     xcd_start[x + 1] = (int64_t)list.size();
     longest = std::max<int64_t>(longest, (int64_t)keyed.size());
   }
-  for (int x = nx; x < 8; ++x) xcd_start[x + 1] = xcd_start[nx];
-  out->num_waves = xcd_lists ? longest : (int64_t)list.size();
+  out->num_waves = longest;
   HIP_TRY(hipMalloc((void**)&out->d_work, sizeof(WaveWork) * list.size()));
   HIP_TRY(hipMemcpy(out->d_work, list.data(), sizeof(WaveWork) * list.size(), hipMemcpyHostToDevice));
-  if (xcd_lists) {
-    HIP_TRY(hipMalloc((void**)&out->d_xcd_start, sizeof(int64_t) * 9));
-    HIP_TRY(hipMemcpy(out->d_xcd_start, xcd_start.data(), sizeof(int64_t) * 9, hipMemcpyHostToDevice));
-  }
+  HIP_TRY(hipMalloc((void**)&out->d_xcd_start, sizeof(int64_t) * 9));
+  HIP_TRY(hipMemcpy(out->d_xcd_start, xcd_start.data(), sizeof(int64_t) * 9, hipMemcpyHostToDevice));
   return 0;
 }
 

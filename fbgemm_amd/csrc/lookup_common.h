@@ -101,10 +101,9 @@ inline int bags_per_wave(int lanes, int packed) { return (lanes <= 16 && !packed
 // What the bag scheduler leaves per bag, in the order waves take the bags.
 struct __attribute__((aligned(16))) BagEntry {
   int64_t o0;  // offsets[bag]
-  int64_t o1;  // offsets[bag + 1]
+  int32_t len; // offsets[bag + 1] - offsets[bag]; -1 when that is negative or beyond 31 bits: the
+               // lookup then reads the two offsets itself and reports what it finds
   int32_t bag; // bag id inside its table
-  int32_t pad0;
-  int64_t pad1;
 };
 
 // The pruned-row mapping of an order-preserving table, 32 logical rows per record

@@ -100,7 +100,11 @@ __device__ __forceinline__ bool pool_bags(const LookupArgs& a, const TableDesc& 
       const BagEntry be = a.order[ob + slot];
       bag = be.bag;
       o0 = be.o0;
-      o1 = be.o1;
+      o1 = o0 + be.len;
+      if (be.len < 0) { // a length the entry cannot hold: judge the offsets themselves
+        o0 = read_offset(a.offsets, a.off64, ob + be.bag);
+        o1 = read_offset(a.offsets, a.off64, ob + be.bag + 1);
+      }
     } else {
       o0 = read_offset(a.offsets, a.off64, ob + bag);
       o1 = read_offset(a.offsets, a.off64, ob + bag + 1);

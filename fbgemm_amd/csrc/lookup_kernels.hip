@@ -8,20 +8,29 @@ namespace fbgemm_amd {
 
 // ---- bag scheduler -------------------------------------------------------------
 //
-// One workgroup per table orders the table's bags by length, longest first
-// (counting sort over lengths, lengths >= SORT_BINS - 1 share the first bin).
-// Waves then take consecutive runs of the order, so the bags a wave pools side
-// by side need the same number of rounds and no lane idles behind a long
-// neighbour. Ties are placed in arrival order of the LDS atomics: the order
-// may differ between runs, the results cannot (each bag is summed on its own).
+// One workgroup per window of SORT_WINDOW consecutive bags of a table orders them
+// by length, longest first (counting sort over lengths, lengths >= SORT_BINS - 1
+// share the first bin). Waves then take consecutive runs of the order, so the
+// bags a wave pools side by side need the same number of rounds and no lane
+// idles behind a long neighbour. Ties are placed in arrival order of the LDS
+// atomics: the order may differ between runs, the results cannot (each bag is
+// summed on its own). Windows instead of whole tables: the lookup runs as fast
+// over bags ordered inside windows of a few thousand as over a table ordered as a
+// whole, and a table of many bags is ordered by many workgroups at once.
 constexpr int SORT_BINS = 1024;
+constexpr int SORT_WINDOW = 2048;
 
-__global__ __launch_bounds__(1024) void bag_order_kernel(const void* offsets, int off64, int32_t B, BagEntry* order) {
+__global__ __launch_bounds__(1024) void bag_order_kernel(const void* offsets, int off64, int32_t B_table, int32_t window,
+                                                         BagEntry* order) {
   __shared__ int bins[SORT_BINS];
   __shared__ int partial[1024];
-  const int t = blockIdx.x;
+  // workgroup t * windows + w orders bags w * window .. of table t among themselves
+  const int windows = (B_table + window - 1) / window;
+  const int t = blockIdx.x / windows;
   const int tid = threadIdx.x;
-  const int64_t ob = (int64_t)t * B;
+  const int first = (blockIdx.x - t * windows) * window;
+  const int B = B_table - first < window ? B_table - first : window;
+  const int64_t ob = (int64_t)t * B_table + first;
   for (int i = tid; i < SORT_BINS; i += 1024) bins[i] = 0;
   __syncthreads();
   // bin of a bag: SORT_BINS - 1 - min(length, SORT_BINS - 1), so that the longest come first
@@ -57,23 +66,24 @@ __global__ __launch_bounds__(1024) void bag_order_kernel(const void* offsets, in
   bins[tid] = before + incl - mine;
   __syncthreads();
   for (int b = tid, it = 0; b < B; b += 1024, ++it) {
-    BagEntry be;
+    int64_t o0, o1;
     if (it == 0) {
-      be.o0 = a0;
-      be.o1 = a1;
+      o0 = a0;
+      o1 = a1;
     } else if (it == 1) {
-      be.o0 = b0;
-      be.o1 = b1;
+      o0 = b0;
+      o1 = b1;
     } else {
-      be.o0 = read_offset(offsets, off64, ob + b);
-      be.o1 = read_offset(offsets, off64, ob + b + 1);
+      o0 = read_offset(offsets, off64, ob + b);
+      o1 = read_offset(offsets, off64, ob + b + 1);
     }
-    int64_t len = be.o1 - be.o0;
-    len = len < 0 ? 0 : (len > SORT_BINS - 1 ? SORT_BINS - 1 : len);
+    const int64_t exact = o1 - o0;
+    const int64_t len = exact < 0 ? 0 : (exact > SORT_BINS - 1 ? SORT_BINS - 1 : exact);
     const int p = atomicAdd(&bins[SORT_BINS - 1 - (int)len], 1);
-    be.bag = b;
-    be.pad0 = 0;
-    be.pad1 = 0;
+    BagEntry be;
+    be.o0 = o0;
+    be.len = (exact < 0 || exact > 0x7fffffffLL) ? -1 : (int32_t)exact;
+    be.bag = first + b;
     order[ob + p] = be;
   }
 }
@@ -178,7 +188,10 @@ hipError_t launch_lookup(const LookupArgs& a, bool idx64, hipStream_t stream) {
 
 hipError_t launch_bag_order(const void* offsets, bool off64, int32_t B, int32_t T, BagEntry* order, hipStream_t stream) {
   if (T <= 0 || B <= 0) return hipSuccess;
-  hipLaunchKernelGGL(bag_order_kernel, dim3((unsigned)T), dim3(1024), 0, stream, offsets, off64 ? 1 : 0, B, order);
+  const int64_t blocks = (int64_t)((B + SORT_WINDOW - 1) / SORT_WINDOW) * T;
+  if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(bag_order_kernel, dim3((unsigned)blocks), dim3(1024), 0, stream, offsets, off64 ? 1 : 0, B, SORT_WINDOW,
+                     order);
   return hipGetLastError();
 }
 

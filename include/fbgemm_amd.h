@@ -149,7 +149,7 @@ int fbgemm_amd_spmdm_launch(
  * takes from hipMalloc'ed buffers (the prefix sum of the lengths when
  * use_offsets == 0, and the bag order of the scheduler for calls of 2^21
  * lookups and more) live in a static device array of the library instead
- * (about 2.5 MiB, held by every GPU the library runs on until the process
+ * (about 1.5 MiB, held by every GPU the library runs on until the process
  * ends). Limit: output_size <= FBGEMM_AMD_NOALLOC_MAX_BAGS, larger calls are
  * rejected with FBGEMM_AMD_E_ARG. It calls no hipMalloc / hipFree and no
  * allocating library routine; its first call on a device asks the runtime for

@@ -9,7 +9,7 @@ CFG=${1:-3}; OUT=${2:-profile_summary.txt}; shift; shift
 export TMPDIR=/tmp
 RAW=$(mktemp -d /tmp/fbgemm_amd_prof.XXXXXX)
 mkdir -p "$(dirname "$OUT")"
-BENCH="python3 bench.py --config $CFG --no-cpu --no-also --no-check --calibration-copy-mib 1024 $*"
+BENCH="python3 bench.py --config $CFG --no-cpu --no-also --no-exact --no-check --calibration-copy-mib 1024 $*"
 {
   echo "# rocprofv3 summary, bench.py --config $CFG $*"
   echo "# commands (each its own run):"
@@ -18,8 +18,9 @@ BENCH="python3 bench.py --config $CFG --no-cpu --no-also --no-check --calibratio
   echo "# condensed with: python3 profile_summary.py <dir>"
 } > "$OUT"
 echo "== kernel trace (--kernel-trace --stats), 23 launches" >> "$OUT"
+echo "pass: kernel trace ($(date +%T))"
 timeout -k 10 900 rocprofv3 --kernel-trace --stats --output-format csv -d $RAW/trace -o t -- $BENCH --steps 20 --warmup 3 > $RAW/trace.log 2>&1 || { echo "trace run failed" | tee -a "$OUT"; tail -5 $RAW/trace.log; exit 1; }
-grep '^{' $RAW/trace.log | tail -1 | cut -c1-1200 >> "$OUT"
+grep '^{' $RAW/trace.log | tail -1 | cut -c1-3000 >> "$OUT"
 python3 profile_summary.py $RAW/trace | grep -v '^#' >> "$OUT"
 # PROFILE_SHORT=1 keeps the byte counters only (for workloads whose set-up takes minutes)
 if [ -n "$PROFILE_SHORT" ]; then
@@ -27,10 +28,12 @@ if [ -n "$PROFILE_SHORT" ]; then
 else
   PASSES=("FETCH_SIZE" "WRITE_SIZE" "TCC_HIT_sum TCC_MISS_sum" "TCC_EA0_RDREQ_sum"
           "SQ_WAVES SQ_INSTS_VALU SQ_INSTS_VMEM_RD SQ_INSTS_LDS SQ_INSTS_SALU SQ_WAVE_CYCLES SQ_WAIT_INST_ANY SQ_ACTIVE_INST_VALU"
-          "TCP_TCC_READ_REQ_sum TCP_TOTAL_CACHE_ACCESSES_sum TCP_TCC_READ_REQ_LATENCY_sum" "GRBM_GUI_ACTIVE")
+          "TCP_TCC_READ_REQ_sum TCP_TOTAL_CACHE_ACCESSES_sum TCP_TCC_READ_REQ_LATENCY_sum TCP_PENDING_STALL_CYCLES_sum"
+          "TCP_UTCL1_REQUEST_sum TCP_UTCL1_TRANSLATION_MISS_sum TCP_UTCL1_TRANSLATION_HIT_sum" "GRBM_GUI_ACTIVE")
 fi
 for pass in "${PASSES[@]}"; do
   n=$(echo $pass | tr ' ' '_' | cut -c1-40)
+  echo "pass: $pass ($(date +%T))"
   echo "== --pmc $pass" >> "$OUT"
   timeout -s KILL 600 rocprofv3 --pmc $pass --output-format csv -d $RAW/pmc_$n -o p -- $BENCH --steps 3 --warmup 1 > $RAW/pmc_$n.log 2>&1 || { echo "pass failed: $pass" >> "$OUT"; tail -3 $RAW/pmc_$n.log >> "$OUT"; exit 1; }
   python3 profile_summary.py $RAW/pmc_$n | grep -v '^#\|^launch' >> "$OUT"

@@ -248,8 +248,20 @@ def test_large_call_takes_the_ordered_path(ops, oracle):
     off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
     idx = rng.integers(0, rows, size=int(off[-1])).astype(np.int32)
     assert len(idx) > (1 << 21)
-    check_case(ops, oracle, ty=INT4, D=D, table=table, idx=idx, off_or_len=off, normalize=True, out_ty=FP16,
-               data_size=rows, output_size=nb, what="2.6 M lookups, ordered bags")
+    kw = dict(ty=INT4, D=D, table=table, normalize=True, out_ty=FP16, data_size=rows, output_size=nb)
+    assert check_case(ops, oracle, idx=idx, off_or_len=off, what="2.6 M lookups, ordered bags", **kw)
+    # what the reference rejects is rejected on this path too
+    assert not check_case(ops, oracle, idx=idx, off_or_len=off, index_size=len(idx) - 1, what="ordered, short", **kw)
+    longer = np.concatenate([idx, idx[:1]])
+    assert not check_case(ops, oracle, idx=longer, off_or_len=off, index_size=len(idx) + 1, what="ordered, long", **kw)
+    bad = idx.copy(); bad[len(bad) // 3] = rows
+    assert not check_case(ops, oracle, idx=bad, off_or_len=off, what="ordered, idx == rows", **kw)
+    # offsets that step back once: a bag of negative length, which the scheduler's entry cannot hold
+    # (the reference's result for it is unspecified; the library always rejects it)
+    back = off.copy(); back[nb // 2] = back[nb // 2 - 1] - 3
+    ok, _, _ = run_gpu(ops, idx=idx, off_or_len=back, w=None, positional=False, use_offsets=True, output_stride=-1,
+                       input_stride=-1, sbl=True, remap=None, **kw)
+    assert not ok
 
 
 def same_bits_or_both_nan(got, want, what):
