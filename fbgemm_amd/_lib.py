@@ -45,6 +45,7 @@ SYMBOLS = {
     "fbgemm_amd_tbe_plan_set_accumulate": (C.c_int, [_P, _I32]),
     "fbgemm_amd_tbe_plan_trim": (C.c_int, [_P]),
     "fbgemm_amd_tbe_plan_cached_work": (_I64, [_P]),
+    "fbgemm_amd_tbe_plan_pinned_work": (C.c_int64, [_P]),
     "fbgemm_amd_set_lean": (C.c_int, [_I32]),
     "fbgemm_amd_set_narrow_below_waves": (C.c_int, [_I32]),
     "fbgemm_amd_tbe_forward_nobag": (C.c_int, [_P, _P, _P, _P, _P, _I32, _I64, _I64, _I32, _I32, _P, _P, _P]),

@@ -1448,6 +1448,14 @@ int64_t fbgemm_amd_tbe_plan_cached_work(const fbgemm_amd_tbe_plan* plan) {
   return plan ? (int64_t)plan->work.size() : -1;
 }
 
+int64_t fbgemm_amd_tbe_plan_pinned_work(fbgemm_amd_tbe_plan* plan) {
+  if (!plan) return -1;
+  std::lock_guard<std::mutex> lk(plan->mu);
+  int64_t n = 0;
+  for (const auto& kv : plan->work) n += kv.second.pinned ? 1 : 0;
+  return n;
+}
+
 int fbgemm_amd_tbe_forward_nobag(
     fbgemm_amd_tbe_plan* plan, const void* d_dev_weights, const void* d_uvm_weights,
     const void* d_indices, const void* d_offsets, int32_t index_bits,

@@ -50,7 +50,7 @@ struct PlanEntry {
   std::shared_ptr<PlanHolder> holder;
   uint64_t last_use;
 };
-constexpr size_t MAX_CACHED_PLANS = 64; // beyond: the least recently used plan goes
+constexpr size_t MAX_CACHED_PLANS = 64; // beyond: the least recently used plan that no graph can hold goes
 std::mutex g_mu;                        // guards the two maps below, never held across a launch
 std::map<PlanKey, PlanEntry> g_plans;
 uint64_t g_use_clock = 0;
@@ -105,11 +105,17 @@ std::shared_ptr<PlanHolder> plan_for(const Tensor& dev_weights, const Tensor& uv
       return it->second.holder;
     }
     if (g_plans.size() >= MAX_CACHED_PLANS) {
-      auto victim = g_plans.begin();
+      // the least recently used plan that no captured graph can hold (a forward under stream
+      // capture pins what it touches); when every plan is pinned the cache grows instead
+      auto victim = g_plans.end();
       for (auto jt = g_plans.begin(); jt != g_plans.end(); ++jt)
-        if (jt->second.last_use < victim->second.last_use) victim = jt;
-      evicted = victim->second.holder;
-      g_plans.erase(victim);
+        if (fbgemm_amd_tbe_plan_pinned_work(jt->second.holder->plan) == 0 &&
+            (victim == g_plans.end() || jt->second.last_use < victim->second.last_use))
+          victim = jt;
+      if (victim != g_plans.end()) {
+        evicted = victim->second.holder;
+        g_plans.erase(victim);
+      }
     }
     g_plans.emplace(key, PlanEntry{holder, ++g_use_clock});
   }

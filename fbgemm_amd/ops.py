@@ -11,6 +11,7 @@
 All tensors are device tensors (torch is only the owner of HBM and streams).
 Everything runs in the HIP library; nothing here computes.
 """
+import collections
 import ctypes as C
 
 import torch
@@ -238,6 +239,19 @@ class TbePlan:
     def row_bytes(self, t):
         return _lib.lib().fbgemm_amd_tbe_plan_row_bytes(self.handle, t)
 
+    def cached_work(self):
+        """Work lists (one per batch size) the plan keeps."""
+        return _lib.lib().fbgemm_amd_tbe_plan_cached_work(self.handle)
+
+    def pinned_work(self):
+        """How many of them a forward under stream capture has touched (a graph may hold them)."""
+        return _lib.lib().fbgemm_amd_tbe_plan_pinned_work(self.handle)
+
+    def trim(self):
+        """Drop every cached work list, pinned ones included: graphs that contain forwards of this
+        plan must be captured again afterwards."""
+        check(_lib.lib().fbgemm_amd_tbe_plan_trim(self.handle))
+
     def __del__(self):
         h, self.handle = getattr(self, "handle", None), None
         if h:
@@ -247,7 +261,8 @@ class TbePlan:
                 pass
 
 
-_plans = {}
+_plans = collections.OrderedDict()  # least recently used first
+MAX_CACHED_PLANS = 64
 
 
 def _plan_for(dev_weights, uvm_weights, weights_placements, weights_offsets, weights_tys, D_offsets,
@@ -262,10 +277,17 @@ def _plan_for(dev_weights, uvm_weights, weights_placements, weights_offsets, wei
     if entry is None:
         plan = TbePlan(weights_offsets, weights_tys, D_offsets, weights_placements,
                        dev_weights.numel(), uvm_weights.numel(), row_alignment)
-        if len(_plans) > 64:
-            _plans.clear()
+        if len(_plans) >= MAX_CACHED_PLANS:
+            # the least recently used plan goes, but never one whose work lists a captured graph may hold
+            # (a forward under stream capture pins them); when every plan is pinned the cache grows
+            for old_key, (old, _) in _plans.items():
+                if old.pinned_work() == 0:
+                    del _plans[old_key]
+                    break
         # the entry keeps the tensors alive: while it is cached their addresses cannot be handed to other tensors
         entry = _plans[key] = (plan, (weights_offsets, weights_tys, D_offsets, weights_placements))
+    else:
+        _plans.move_to_end(key)
     return entry[0]
 
 

@@ -271,6 +271,10 @@ int fbgemm_amd_tbe_plan_set_accumulate(fbgemm_amd_tbe_plan* plan, int32_t mode);
  * counterpart in the reference. */
 int fbgemm_amd_tbe_plan_trim(fbgemm_amd_tbe_plan* plan);
 int64_t fbgemm_amd_tbe_plan_cached_work(const fbgemm_amd_tbe_plan* plan);
+/* How many of the cached entries a forward under stream capture has touched (a
+ * graph may hold their addresses): a cache of plans must not destroy a plan
+ * while this is not 0 unless its owner knows the graphs are gone. */
+int64_t fbgemm_amd_tbe_plan_pinned_work(fbgemm_amd_tbe_plan* plan);
 
 /* Tables of FBGEMM_AMD_FP8 rows (D bytes per row, no scale/bias) are decoded
  * with the operator's fp8_exponent_bits / fp8_exponent_bias
