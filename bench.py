@@ -60,6 +60,9 @@ def parse():
     ap.add_argument("--no-rank-records", action="store_true",
                     help="config 4 only: read the int32 mapping arrays in the forward instead of the compact "
                          "bitmap-and-rank form of the (order-preserving) mappings")
+    ap.add_argument("--no-kernel-events", dest="kernel_events", action="store_false",
+                    help="skip the second timed region, the one with a pair of HIP events around the lookup kernels of "
+                         "every forward (roofline.kernel_ms is then the forward time)")
     ap.add_argument("--no-also", dest="also", action="store_false",
                     help="default run only: do not append the driver-timed figures of config 5 under \"also\"")
     ap.add_argument("--op", default="lookup",
@@ -739,8 +742,6 @@ def time_tbe(p, a, torch, np, steps, warmup, graph=False, accumulate=None):
         step = g.replay
         step()
         torch.cuda.synchronize()
-    else:  # HIP events around every lookup_kernel launch of the timed region, on its stream
-        _lib.check(_lib.lib().fbgemm_amd_tbe_plan_profile(plan.handle, steps))
     ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     ev0.record()
@@ -754,14 +755,26 @@ def time_tbe(p, a, torch, np, steps, warmup, graph=False, accumulate=None):
     ms_per_step = wall * 1e3 / steps
     forward_ms = ev0.elapsed_time(ev1) / steps  # events on the launch stream, back-to-back forwards
     kernel_ms, kernel_name = forward_ms, "lookup_lean_kernel / lookup_kernel (+ bag_order_kernel), per graph replay"
-    if not graph:
+    with_events_ms = None
+    if not graph and a.kernel_events:
+        # The kernels' own duration: a second timed region of the same `steps` forwards with a pair of
+        # HIP events around the lookup kernels of every forward, on the stream they are launched on.
+        # It is a region of its own because the events are not free: each pair costs a forward of
+        # config 3 about 6 us (4 %), which would otherwise sit in `value`.
+        _lib.check(_lib.lib().fbgemm_amd_tbe_plan_profile(plan.handle, steps))
+        t1 = time.perf_counter()
+        for _ in range(steps):
+            launch()
+        torch.cuda.synchronize()
+        with_events_ms = (time.perf_counter() - t1) * 1e3 / steps
         ms = (C.c_float * steps)()
         n = C.c_int32(0)
         _lib.check(_lib.lib().fbgemm_amd_tbe_plan_profile_read(plan.handle, ms, steps, C.byref(n)))
         assert n.value == steps
+        _lib.check(_lib.lib().fbgemm_amd_tbe_plan_profile(plan.handle, 0))
         kernel_ms, kernel_name = sum(ms[:n.value]) / n.value, "lookup_lean_kernel (+ lookup_kernel for tables of other shapes)"
     return {"ms_per_step": ms_per_step, "forward_ms": forward_ms, "kernel_ms": kernel_ms, "kernel": kernel_name,
-            "checked": checked}
+            "checked": checked, "ms_per_step_with_kernel_events": with_events_ms}
 
 
 def exact_leg(p, a, torch, np, useful, steps, warmup):
@@ -883,6 +896,8 @@ def main():
                                                                    and a.only_type is None) else None,
                      "kernel": kernel_name, "kernel_ms": round(kernel_ms / launches_per_step, 5),
                      "forward_ms": round(forward_ms, 5),
+                     "ms_per_step_with_kernel_events": None if not tbe or m["ms_per_step_with_kernel_events"] is None
+                     else round(m["ms_per_step_with_kernel_events"], 5),
                      "algorithmic_bytes_per_launch": useful // launches_per_step},
         "setup_s": round(build_s, 1),
     }
@@ -916,6 +931,8 @@ def main():
                          "frac": round(useful5 / (m5["kernel_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
                          "traffic": traffic_from_profile(5), "kernel": m5["kernel"],
                          "kernel_ms": round(m5["kernel_ms"], 5), "forward_ms": round(m5["forward_ms"], 5),
+                         "ms_per_step_with_kernel_events": None if m5["ms_per_step_with_kernel_events"] is None
+                         else round(m5["ms_per_step_with_kernel_events"], 5),
                          "algorithmic_bytes_per_launch": useful5},
             "setup_s": round(setup5, 1)}}
         if a.accumulate == "fast" and a.exact_too:

@@ -14,11 +14,12 @@ namespace fbgemm_amd {
 // bags a wave pools side by side need the same number of rounds and no lane
 // idles behind a long neighbour. Ties are placed in arrival order of the LDS
 // atomics: the order may differ between runs, the results cannot (each bag is
-// summed on its own). Windows instead of whole tables: the lookup runs as fast
-// over bags ordered inside windows of a few thousand as over a table ordered as a
-// whole, and a table of many bags is ordered by many workgroups at once.
+// summed on its own). Windows for tables of many bags: a launch of many rounds of
+// waves runs as fast over bags ordered inside windows of a few thousand as over
+// tables ordered as a whole, and many workgroups order a table at once.
 constexpr int SORT_BINS = 1024;
 constexpr int SORT_WINDOW = 2048;
+constexpr int SORT_WHOLE_TABLE = 8192;
 
 __global__ __launch_bounds__(1024) void bag_order_kernel(const void* offsets, int off64, int32_t B_table, int32_t window,
                                                          BagEntry* order) {
@@ -188,10 +189,13 @@ hipError_t launch_lookup(const LookupArgs& a, bool idx64, hipStream_t stream) {
 
 hipError_t launch_bag_order(const void* offsets, bool off64, int32_t B, int32_t T, BagEntry* order, hipStream_t stream) {
   if (T <= 0 || B <= 0) return hipSuccess;
-  const int64_t blocks = (int64_t)((B + SORT_WINDOW - 1) / SORT_WINDOW) * T;
+  // Tables of up to SORT_WHOLE_TABLE bags are ordered as a whole: their launches are a few rounds of
+  // waves, and longest-first over the whole table is what keeps the drain of such a launch short
+  // (32 tables x 4 096 bags of 5..50 rows: 88 us ordered whole, 100 us in windows of 2 048).
+  const int window = B <= SORT_WHOLE_TABLE ? B : SORT_WINDOW;
+  const int64_t blocks = (int64_t)((B + window - 1) / window) * T;
   if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
-  hipLaunchKernelGGL(bag_order_kernel, dim3((unsigned)blocks), dim3(1024), 0, stream, offsets, off64 ? 1 : 0, B, SORT_WINDOW,
-                     order);
+  hipLaunchKernelGGL(bag_order_kernel, dim3((unsigned)blocks), dim3(1024), 0, stream, offsets, off64 ? 1 : 0, B, window, order);
   return hipGetLastError();
 }
 
