@@ -17,7 +17,10 @@ BENCH="python3 bench.py --config $CFG --no-cpu --no-also --no-exact --no-check -
   echo "#   rocprofv3 --pmc <counters> --output-format csv -d <dir> -o p -- $BENCH --steps 3 --warmup 1"
   echo "# condensed with: python3 profile_summary.py <dir>"
 } > "$OUT"
-echo "== kernel trace (--kernel-trace --stats), 23 launches" >> "$OUT"
+case "$*" in
+  *--op*) echo "== kernel trace (--kernel-trace --stats)" >> "$OUT";;
+  *) echo "== kernel trace (--kernel-trace --stats): 3 warm-up forwards, 20 timed, 20 more with the lookup kernels between HIP events" >> "$OUT";;
+esac
 echo "pass: kernel trace ($(date +%T))"
 timeout -k 10 900 rocprofv3 --kernel-trace --stats --output-format csv -d $RAW/trace -o t -- $BENCH --steps 20 --warmup 3 > $RAW/trace.log 2>&1 || { echo "trace run failed" | tee -a "$OUT"; tail -5 $RAW/trace.log; exit 1; }
 grep '^{' $RAW/trace.log | tail -1 | cut -c1-3000 >> "$OUT"
