@@ -13,6 +13,7 @@
 #include <vector>
 
 #include "../../include/fbgemm_amd.h"
+#include "cache_policy.h"
 #include "lookup_common.h"
 
 namespace fbgemm_amd {
@@ -1222,9 +1223,9 @@ int tbe_forward_impl(
       // dropped here: a captured graph holds their device pointers (fbgemm_amd_tbe_plan_trim
       // drops those too, and says what that means for graphs).
       if (plan->work.size() >= MAX_CACHED_WORK) {
-        auto victim = plan->work.end();
-        for (auto jt = plan->work.begin(); jt != plan->work.end(); ++jt)
-          if (!jt->second.pinned && (victim == plan->work.end() || jt->second.last_use < victim->second.last_use)) victim = jt;
+        auto victim = least_recently_used_not_held(
+            plan->work, [](const fbgemm_amd_tbe_plan::Work& e) { return e.pinned; },
+            [](const fbgemm_amd_tbe_plan::Work& e) { return e.last_use; });
         if (victim != plan->work.end()) {
           HIP_TRY(hipDeviceSynchronize());
           free_work(victim->second);

@@ -17,6 +17,7 @@
 #include <tuple>
 
 #include "../../include/fbgemm_amd.h"
+#include "cache_policy.h"
 
 namespace {
 
@@ -107,11 +108,9 @@ std::shared_ptr<PlanHolder> plan_for(const Tensor& dev_weights, const Tensor& uv
     if (g_plans.size() >= MAX_CACHED_PLANS) {
       // the least recently used plan that no captured graph can hold (a forward under stream
       // capture pins what it touches); when every plan is pinned the cache grows instead
-      auto victim = g_plans.end();
-      for (auto jt = g_plans.begin(); jt != g_plans.end(); ++jt)
-        if (fbgemm_amd_tbe_plan_pinned_work(jt->second.holder->plan) == 0 &&
-            (victim == g_plans.end() || jt->second.last_use < victim->second.last_use))
-          victim = jt;
+      auto victim = fbgemm_amd::least_recently_used_not_held(
+          g_plans, [](const PlanEntry& e) { return fbgemm_amd_tbe_plan_pinned_work(e.holder->plan) != 0; },
+          [](const PlanEntry& e) { return e.last_use; });
       if (victim != g_plans.end()) {
         evicted = victim->second.holder;
         g_plans.erase(victim);
