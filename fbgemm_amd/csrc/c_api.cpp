@@ -1211,6 +1211,11 @@ int tbe_forward_impl(
       std::vector<int> lean_members, general_members;
       for (int t = 0; t < plan->T; ++t) (lean && lean_shape(tables[t]) ? lean_members : general_members).push_back(t);
       fbgemm_amd_tbe_plan::Work nw;
+      // what is allocated below goes back when a later step fails
+      struct Undo {
+        fbgemm_amd_tbe_plan::Work* w;
+        ~Undo() { if (w) free_work(*w); }
+      } undo{&nw};
       if (int rc = build_work_list(tables, lean_members, B, &nw.lean)) return rc;
       if (int rc = build_work_list(tables, general_members, B, &nw.general)) return rc;
       // the bag order: one buffer for this stream, one ahead for the next stream
@@ -1233,6 +1238,7 @@ int tbe_forward_impl(
         }
       }
       it = plan->work.emplace(key, nw).first;
+      undo.w = nullptr; // the cache owns it now
     }
     it->second.pinned = it->second.pinned || capturing;
     it->second.last_use = ++plan->use_clock;
