@@ -1359,9 +1359,7 @@ int fbgemm_amd_tbe_plan_set_index_remappings(
   // forget what was made from an earlier array (after the forwards that may still read it)
   if (plan->d_rank_records || plan->d_rank_offsets) {
     HIP_TRY(hipDeviceSynchronize());
-    if (plan->seg_offsets) (void)hipFree(plan->seg_offsets);
-  if (plan->seg_partial) (void)hipFree(plan->seg_partial);
-  if (plan->d_rank_records) (void)hipFree(plan->d_rank_records);
+    if (plan->d_rank_records) (void)hipFree(plan->d_rank_records);
     if (plan->d_rank_offsets) (void)hipFree(plan->d_rank_offsets);
     plan->d_rank_records = nullptr;
     plan->d_rank_offsets = nullptr;

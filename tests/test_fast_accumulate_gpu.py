@@ -180,6 +180,50 @@ def test_table_batched_fast_mode(ops, oracle, B, max_L):
                                     f"B={B} L<{max_L} align={row_alignment} w={weighted} pool={pooling} out={out_ty} table={t}")
 
 
+def test_rebuilding_rank_records_leaves_the_split_bag_scratch_alone(ops, oracle):
+    """A plan that has cut long bags into segments (plan-owned scratch) and is then given its
+    pruned-row mappings twice: building the compact mappings again replaces only what was made
+    from the mappings, and the next forward of long bags gives the same bits as the first."""
+    rng = np.random.default_rng(4242)
+    logical = [900, 700]
+    specs, maps = [], []
+    for n in logical:
+        keep = rng.random(n) < 0.6
+        m = np.full(n, -1, np.int32)
+        m[keep] = np.arange(int(keep.sum()), dtype=np.int32)
+        maps.append(m)
+        specs.append((int(keep.sum()), 128, INT4))
+    T, B = len(specs), 2
+    from test_tbe_gpu import build_weights
+    weights, wo, _ = build_weights(rng, specs, 16)
+    tys = np.array([s[2] for s in specs], np.uint8)
+    D_offsets = np.concatenate([[0], np.cumsum([s[1] for s in specs])]).astype(np.int32)
+    total_D = int(D_offsets[-1])
+    lens = rng.integers(600, 900, size=T * B)
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    idx = np.concatenate([rng.integers(0, logical[t], size=int(lens[t * B:(t + 1) * B].sum())) for t in range(T)]).astype(np.int64)
+    remap = np.concatenate(maps)
+    remap_off = np.concatenate([[0], np.cumsum([len(m) for m in maps])]).astype(np.int64)
+    plan = ops.TbePlan(torch.from_numpy(wo), torch.from_numpy(tys), torch.from_numpy(D_offsets), torch.zeros(T, dtype=torch.int32),
+                       len(weights), 0, 16)
+    plan.set_accumulate(ops.ACC_FAST)
+    d_remap, d_remap_off = cu(remap), cu(remap_off)
+    meta = (cu(weights), torch.zeros(0, dtype=torch.uint8, device="cuda"), cu(np.zeros(T, np.int32)), cu(wo), cu(tys), cu(D_offsets))
+    call = lambda: ops.int_nbit_split_embedding_codegen_lookup_function(
+        *meta, total_D, 0, 128, 0, 0, 0, cu(idx), cu(off), 0, None, FP32, row_alignment=16, plan=plan,
+        index_remappings=d_remap, index_remappings_offsets=d_remap_off).cpu().numpy()
+    assert plan.set_index_remappings(d_remap, d_remap_off) == 2
+    first = call()
+    dense = oracle.pruned_array_lookup(idx, off, remap, remap_off)
+    rc, want = oracle.tbe_forward(weights, wo, tys, D_offsets, total_D, dense, off, 0, None, FP32, 16)
+    assert rc == 0
+    check_grade(first, want, FP32, B, "long bags, first forward")
+    assert plan.set_index_remappings(d_remap, d_remap_off) == 2  # the records are made again
+    again = call()
+    assert (again.view(np.uint32) == first.view(np.uint32)).all()
+    del plan  # and the plan frees its scratch once
+
+
 def test_configs_scaled_fast_mode(ops, oracle):
     """Configs 3, 4 (batched, pruned) and 5 at reduced size, in full, in the tolerance-grade mode."""
     from fbgemm_amd import bench_configs as bc
