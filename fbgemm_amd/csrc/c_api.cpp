@@ -594,7 +594,7 @@ int spmdm_launch_impl(
     if (d.vb == 16 && (pooled_bags + G16 - 1) / G16 < narrow_below_waves()) plan_lanes(d, (uintptr_t)d_input, pooled_stride, has_sb, false, true);
   }
   d.lanes_recip = (65536 + d.lanes - 1) / d.lanes;
-    d.bags = bags_per_wave(d.lanes, d.packed);
+  d.bags = bags_per_wave(d.lanes, d.packed);
 
   a.tables = nullptr;
   a.weights[0] = (const uint8_t*)d_input;
@@ -1176,6 +1176,11 @@ int tbe_forward_impl(
   const bool lean = lean_enabled();
   fbgemm_amd_tbe_plan::Work w;
   int variant, order_slot = 0;
+  // what the launches below take from the plan, read under its lock
+  bool exact = true;
+  const RankRecord* rank_records = nullptr;
+  const int64_t* rank_offsets = nullptr;
+  hipEvent_t prof_begin = nullptr, prof_end = nullptr;
   {
     std::lock_guard<std::mutex> lk(plan->mu);
     // the lane shapes depend on B and (through the average bag length) on the number of indices:
@@ -1270,6 +1275,18 @@ int tbe_forward_impl(
           }
     }
     w = W;
+    exact = plan->accumulate != FBGEMM_AMD_ACC_FAST;
+    if (d_index_remappings && plan->d_rank_records && plan->rank_source == d_index_remappings && plan->rank_bits == remap_bits) {
+      rank_records = plan->d_rank_records;
+      rank_offsets = plan->d_rank_offsets;
+    }
+    // bench-only: a pair of events around the lookup kernels of this forward
+    const size_t slots = plan->prof_ev.size() / 2;
+    if (slots) {
+      const size_t slot = (size_t)(plan->prof_count++ % (int64_t)slots);
+      prof_begin = plan->prof_ev[2 * slot];
+      prof_end = plan->prof_ev[2 * slot + 1];
+    }
   }
 
   LookupArgs a;
@@ -1284,10 +1301,8 @@ int tbe_forward_impl(
   a.remap = d_index_remappings;
   a.remap_offsets = d_index_remappings ? d_index_remappings_offsets : nullptr;
   a.remap64 = remap_bits == 64;
-  if (d_index_remappings && plan->d_rank_records && plan->rank_source == d_index_remappings && plan->rank_bits == remap_bits) {
-    a.rank_records = plan->d_rank_records;
-    a.rank_offsets = plan->d_rank_offsets;
-  }
+  a.rank_records = rank_records;
+  a.rank_offsets = rank_offsets;
   a.out = d_output;
   a.out_stride = plan->total_D;
   a.index_size = indices_numel;
@@ -1304,14 +1319,12 @@ int tbe_forward_impl(
     HIP_TRY(launch_bag_order(d_offsets, offset_bits == 64, B, plan->T, w.d_order[order_slot], stream));
     a.order = w.d_order[order_slot];
   }
-  const size_t slots = plan->prof_ev.size() / 2;
-  const size_t slot = slots ? (size_t)(plan->prof_count % (int64_t)slots) : 0;
-  if (slots) HIP_TRY(hipEventRecord(plan->prof_ev[2 * slot], stream));
+  if (prof_begin) HIP_TRY(hipEventRecord(prof_begin, stream));
   if (w.lean.num_waves > 0) {
     a.work = w.lean.d_work;
     a.xcd_start = w.lean.d_xcd_start;
     a.num_waves = w.lean.num_waves;
-    HIP_TRY(launch_lookup_lean(a, index_bits == 64, plan->accumulate != FBGEMM_AMD_ACC_FAST, stream));
+    HIP_TRY(launch_lookup_lean(a, index_bits == 64, exact, stream));
   }
   if (w.general.num_waves > 0) {
     a.work = w.general.d_work;
@@ -1319,10 +1332,7 @@ int tbe_forward_impl(
     a.num_waves = w.general.num_waves;
     HIP_TRY(launch_lookup(a, index_bits == 64, stream));
   }
-  if (slots) {
-    HIP_TRY(hipEventRecord(plan->prof_ev[2 * slot + 1], stream));
-    ++plan->prof_count;
-  }
+  if (prof_end) HIP_TRY(hipEventRecord(prof_end, stream));
   return 0;
 }
 } // namespace
