@@ -27,8 +27,8 @@ HBM_PEAK_GBPS = 8000.0
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--config", type=int, default=3, choices=[1, 2, 3, 4, 5])
     ap.add_argument("--scale", type=float, default=1.0, help="shrink rows and batch (1.0 = the real configuration)")
     ap.add_argument("--rows-scale", type=float, default=None,
