@@ -811,6 +811,9 @@ struct fbgemm_amd_tbe_plan {
   // compact form of the pruned-row mappings (fbgemm_amd_tbe_plan_set_index_remappings)
   RankRecord* d_rank_records = nullptr;
   int64_t* d_rank_offsets = nullptr; // T entries: first record of the table, or -1
+  // the T + 1 mapping offsets the records were built for (device copy): forwards that use the
+  // records bound and slice the mappings with these, whatever offsets they are handed
+  int64_t* d_rank_remap_offsets = nullptr;
   const void* rank_source = nullptr; // the mapping array the records were made from
   int32_t rank_bits = 0;
   int32_t rank_tables = 0;           // tables that use the records
@@ -1035,6 +1038,7 @@ void fbgemm_amd_tbe_plan_destroy(fbgemm_amd_tbe_plan* plan) {
   if (plan->seg_partial) (void)hipFree(plan->seg_partial);
   if (plan->d_rank_records) (void)hipFree(plan->d_rank_records);
   if (plan->d_rank_offsets) (void)hipFree(plan->d_rank_offsets);
+  if (plan->d_rank_remap_offsets) (void)hipFree(plan->d_rank_remap_offsets);
   for (hipEvent_t e : plan->prof_ev) (void)hipEventDestroy(e);
   delete plan;
 }
@@ -1279,6 +1283,7 @@ int tbe_forward_impl(
     if (d_index_remappings && plan->d_rank_records && plan->rank_source == d_index_remappings && plan->rank_bits == remap_bits) {
       rank_records = plan->d_rank_records;
       rank_offsets = plan->d_rank_offsets;
+      d_index_remappings_offsets = plan->d_rank_remap_offsets;
     }
     // bench-only: a pair of events around the lookup kernels of this forward
     const size_t slots = plan->prof_ev.size() / 2;
@@ -1367,12 +1372,14 @@ int fbgemm_amd_tbe_plan_set_index_remappings(
   hipStream_t stream = (hipStream_t)stream_;
   std::lock_guard<std::mutex> lk(plan->mu);
   // forget what was made from an earlier array (after the forwards that may still read it)
-  if (plan->d_rank_records || plan->d_rank_offsets) {
+  if (plan->d_rank_records || plan->d_rank_offsets || plan->d_rank_remap_offsets) {
     HIP_TRY(hipDeviceSynchronize());
     if (plan->d_rank_records) (void)hipFree(plan->d_rank_records);
     if (plan->d_rank_offsets) (void)hipFree(plan->d_rank_offsets);
+    if (plan->d_rank_remap_offsets) (void)hipFree(plan->d_rank_remap_offsets);
     plan->d_rank_records = nullptr;
     plan->d_rank_offsets = nullptr;
+    plan->d_rank_remap_offsets = nullptr;
   }
   plan->rank_source = nullptr;
   plan->rank_tables = 0;
@@ -1428,17 +1435,22 @@ int fbgemm_amd_tbe_plan_set_index_remappings(
     used += first[t] >= 0;
   }
   int64_t* d_first = nullptr;
+  int64_t* d_offs = nullptr;
   if (used > 0) {
     hipError_t e = hipMalloc((void**)&d_first, sizeof(int64_t) * (size_t)T);
     if (e == hipSuccess) e = hipMemcpy(d_first, first.data(), sizeof(int64_t) * (size_t)T, hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMalloc((void**)&d_offs, sizeof(int64_t) * (size_t)(T + 1));
+    if (e == hipSuccess) e = hipMemcpy(d_offs, index_remappings_offsets, sizeof(int64_t) * (size_t)(T + 1), hipMemcpyHostToDevice);
     if (e != hipSuccess) {
       if (d_first) (void)hipFree(d_first);
+      if (d_offs) (void)hipFree(d_offs);
       drop();
       return fail(FBGEMM_AMD_E_HIP, "rank offsets: %s", hipGetErrorString(e));
     }
     plan->d_rank_records = records;
     records = nullptr;
     plan->d_rank_offsets = d_first;
+    plan->d_rank_remap_offsets = d_offs;
     plan->rank_source = d_index_remappings;
     plan->rank_bits = remap_bits;
     plan->rank_tables = used;

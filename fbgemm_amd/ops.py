@@ -229,9 +229,15 @@ class TbePlan:
         ro = index_remappings_offsets.detach().to("cpu", torch.int64).contiguous()
         check(_lib.lib().fbgemm_amd_tbe_plan_set_index_remappings(
             self.handle, _ptr(index_remappings), _bits(index_remappings), _ptr(ro), ro.numel(), _stream()))
-        self._rank_key = (index_remappings.data_ptr(), index_remappings._version, index_remappings.numel())
-        self._rank_keepalive = index_remappings
+        self._rank_key = self.rank_key(index_remappings, index_remappings_offsets)
+        self._rank_keepalive = (index_remappings, index_remappings_offsets)
         return self.rank_tables()
+
+    @staticmethod
+    def rank_key(index_remappings, index_remappings_offsets):
+        """What the compact mappings were made from: the array and its offsets, by address and version."""
+        return (index_remappings.data_ptr(), index_remappings._version, index_remappings.numel(),
+                index_remappings_offsets.data_ptr(), index_remappings_offsets._version)
 
     def rank_tables(self):
         return _lib.lib().fbgemm_amd_tbe_plan_rank_tables(self.handle)
@@ -378,10 +384,10 @@ def int_nbit_split_embedding_codegen_lookup_function(
             raise ValueError(f"index_remappings_offsets holds {index_remappings_offsets.numel()} entries; the operator's "
                              f"{T} features need {T + 1} (one mapping slice per feature)")
         ro = index_remappings_offsets.to(torch.int64).contiguous()
-        # the compact form of order-preserving mappings, made once per array (and again when it changes)
-        key = (index_remappings.data_ptr(), index_remappings._version, index_remappings.numel())
+        # the compact form of order-preserving mappings, made once per array and offsets (and again when either changes)
+        key = TbePlan.rank_key(index_remappings, index_remappings_offsets)
         if getattr(plan, "_rank_key", None) != key and not torch.cuda.is_current_stream_capturing():
-            plan.set_index_remappings(index_remappings, ro)
+            plan.set_index_remappings(index_remappings, index_remappings_offsets)
     check(_lib.lib().fbgemm_amd_tbe_forward_pruned(
         plan.handle, _ptr(dev_weights), _ptr(uvm_weights), _ptr(indices.contiguous()),
         _ptr(offsets.contiguous()), _bits(indices), indices.numel(), offsets.numel(), pooling_mode,

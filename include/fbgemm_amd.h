@@ -250,8 +250,10 @@ int fbgemm_amd_tbe_forward_pruned(
  * the caches. Tables whose mapping is anything else keep reading the array.
  * d_index_remappings / remap_bits as in the forward; index_remappings_offsets is
  * the HOST copy of the T+1 offsets. The forwards use the records whenever they
- * are passed the same d_index_remappings pointer; call this again after the
- * array's contents change (NULL array = drop the records). Allocates; synchronizes
+ * are passed the same d_index_remappings pointer, and then bound and slice the
+ * mappings with the offsets given HERE (the plan keeps a device copy), whatever
+ * offsets the forward is handed; call this again after the array's contents or
+ * its offsets change (NULL array = drop the records). Allocates; synchronizes
  * `stream`. fbgemm_amd_tbe_plan_rank_tables returns how many tables use records. */
 int fbgemm_amd_tbe_plan_set_index_remappings(
     fbgemm_amd_tbe_plan* plan, const void* d_index_remappings, int32_t remap_bits,

@@ -661,8 +661,16 @@ def test_rank_records_replace_order_preserving_mappings(ops, oracle, rdt):
     rc, want = oracle.tbe_forward(weights, wo, tys, D_offsets, total_D, dense, off, 1, None, FP32, 16)
     assert rc == 0
     H.assert_same_bits(with_records, want, "rank records")
+    # a forward that uses the records slices the mappings with the offsets the records were built
+    # for, not with whatever offsets it is handed (here: zeros, which would switch the remap off)
+    stale = torch.zeros_like(d_remap_off)
+    plan._rank_key = ops.TbePlan.rank_key(d_remap, stale)  # keep the wrapper from rebuilding the records
+    got = ops.int_nbit_split_embedding_codegen_lookup_function(
+        *meta, total_D, 0, 256, 128, 32, 0, cu(idx), cu(off), 1, None, FP32, row_alignment=16, plan=plan,
+        index_remappings=d_remap, index_remappings_offsets=stale).cpu().numpy()
+    H.assert_same_bits(got, want, "rank records, other offsets handed to the forward")
     plan.set_index_remappings(None, None)
-    plan._rank_key = (d_remap.data_ptr(), d_remap._version, d_remap.numel())  # keep the wrapper from rebuilding them
+    plan._rank_key = ops.TbePlan.rank_key(d_remap, d_remap_off)  # keep the wrapper from rebuilding them
     assert plan.rank_tables() == 0
     H.assert_same_bits(call(), want, "mapping arrays")
 
