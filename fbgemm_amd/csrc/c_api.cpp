@@ -792,6 +792,12 @@ struct fbgemm_amd_tbe_plan {
     BagEntry* d_order[ORDER_SLOTS] = {nullptr, nullptr, nullptr, nullptr}; // T*B bags each, rewritten by every forward
     hipStream_t order_stream[ORDER_SLOTS] = {nullptr, nullptr, nullptr, nullptr};
     bool order_claimed[ORDER_SLOTS] = {false, false, false, false};
+    // A second stream per slot, with the two events of the fork and the join: a forward with tables
+    // for both lookup kernels runs the general kernel there, beside the lean one (made with the
+    // slot's first forward outside a capture; without them the two kernels run one after the other)
+    hipStream_t side_stream[ORDER_SLOTS] = {nullptr, nullptr, nullptr, nullptr};
+    hipEvent_t side_fork[ORDER_SLOTS] = {nullptr, nullptr, nullptr, nullptr};
+    hipEvent_t side_join[ORDER_SLOTS] = {nullptr, nullptr, nullptr, nullptr};
     bool pinned = false;         // used by a forward under stream capture: a graph may hold its pointers
     uint64_t last_use = 0;
   };
@@ -843,6 +849,11 @@ void free_work(fbgemm_amd_tbe_plan::Work& w) {
     if (w.d_order[k]) (void)hipFree(w.d_order[k]);
     w.d_order[k] = nullptr;
     w.order_claimed[k] = false;
+    if (w.side_fork[k]) (void)hipEventDestroy(w.side_fork[k]);
+    if (w.side_join[k]) (void)hipEventDestroy(w.side_join[k]);
+    if (w.side_stream[k]) (void)hipStreamDestroy(w.side_stream[k]);
+    w.side_fork[k] = w.side_join[k] = nullptr;
+    w.side_stream[k] = nullptr;
   }
 }
 
@@ -1278,6 +1289,23 @@ int tbe_forward_impl(
             break;
           }
     }
+    // the slot's side stream (default priority, like every stream here) and its two events
+    if (!capturing && !W.side_stream[order_slot] && W.lean.num_waves > 0 && W.general.num_waves > 0) {
+      hipStream_t s2 = nullptr;
+      hipEvent_t e1 = nullptr, e2 = nullptr;
+      if (hipStreamCreateWithFlags(&s2, hipStreamNonBlocking) == hipSuccess &&
+          hipEventCreateWithFlags(&e1, hipEventDisableTiming) == hipSuccess &&
+          hipEventCreateWithFlags(&e2, hipEventDisableTiming) == hipSuccess) {
+        W.side_stream[order_slot] = s2;
+        W.side_fork[order_slot] = e1;
+        W.side_join[order_slot] = e2;
+      } else { // the forward works without them
+        if (e1) (void)hipEventDestroy(e1);
+        if (e2) (void)hipEventDestroy(e2);
+        if (s2) (void)hipStreamDestroy(s2);
+        (void)hipGetLastError();
+      }
+    }
     w = W;
     exact = plan->accumulate != FBGEMM_AMD_ACC_FAST;
     if (d_index_remappings && plan->d_rank_records && plan->rank_source == d_index_remappings && plan->rank_bits == remap_bits) {
@@ -1325,17 +1353,32 @@ int tbe_forward_impl(
     a.order = w.d_order[order_slot];
   }
   if (prof_begin) HIP_TRY(hipEventRecord(prof_begin, stream));
-  if (w.lean.num_waves > 0) {
-    a.work = w.lean.d_work;
-    a.xcd_start = w.lean.d_xcd_start;
-    a.num_waves = w.lean.num_waves;
-    HIP_TRY(launch_lookup_lean(a, index_bits == 64, exact, stream));
-  }
+  // Tables for both kernels, and a forward long enough not to notice two events (the size from
+  // which the bags are ordered): the general kernel runs on the slot's side stream, beside the
+  // lean one, forked off behind the scheduler and joined before the forward's stream goes on.
+  static const int side_enabled = env_int("FBGEMM_AMD_SIDE_STREAM", 1);
+  hipStream_t side = (side_enabled && w.lean.num_waves > 0 && w.general.num_waves > 0 && a.order) ? w.side_stream[order_slot] : nullptr;
   if (w.general.num_waves > 0) {
     a.work = w.general.d_work;
     a.xcd_start = w.general.d_xcd_start;
     a.num_waves = w.general.num_waves;
-    HIP_TRY(launch_lookup(a, index_bits == 64, stream));
+    if (side) {
+      HIP_TRY(hipEventRecord(w.side_fork[order_slot], stream));
+      HIP_TRY(hipStreamWaitEvent(side, w.side_fork[order_slot], 0));
+      HIP_TRY(launch_lookup(a, index_bits == 64, side));
+      HIP_TRY(hipEventRecord(w.side_join[order_slot], side));
+    }
+  }
+  if (w.lean.num_waves > 0) {
+    LookupArgs l = a;
+    l.work = w.lean.d_work;
+    l.xcd_start = w.lean.d_xcd_start;
+    l.num_waves = w.lean.num_waves;
+    HIP_TRY(launch_lookup_lean(l, index_bits == 64, exact, stream));
+  }
+  if (w.general.num_waves > 0) {
+    if (side) HIP_TRY(hipStreamWaitEvent(stream, w.side_join[order_slot], 0));
+    else HIP_TRY(launch_lookup(a, index_bits == 64, stream));
   }
   if (prof_end) HIP_TRY(hipEventRecord(prof_end, stream));
   return 0;

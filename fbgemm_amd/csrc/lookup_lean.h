@@ -43,7 +43,7 @@ struct __attribute__((aligned(16))) LeanMul {
   float s24;  // w * scale * 2^24 (4- and 8-bit rows, pre-scaled route); w * scale (plain route); w (fp16 rows)
   float s20;  // w * scale * 2^20 (4-bit rows, pre-scaled route)
   float bias; // w * bias
-  float pad;
+  uint32_t hole; // 1: nothing to add (the entry is absent, pruned or rejected): s24 = s20 = bias = -0
 };
 
 // ---- per-chunk arithmetic -------------------------------------------------------
@@ -110,6 +110,7 @@ struct LeanLane {
   int grp, sub;   // bag slot inside the wave, chunk position inside the bag's lanes
   int lgrp;       // the bag slot whose staging area the lane reads (lanes left over shadow the last one)
   bool bag_ok;    // the lane pools a bag
+  bool idle;      // the lane is left over (no bag slot of its own)
   int bag;        // the bag's number inside its table
   int n;          // entries of the bag
   int64_t pos0;   // position of its first entry in the index array
@@ -140,6 +141,7 @@ __device__ __forceinline__ LeanLane lean_lane(const LookupArgs& a, const TableDe
   }
   const int slot = first_slot + L.grp;
   L.lgrp = idle ? G - 1 : L.grp;
+  L.idle = idle;
   L.bag_ok = !idle && slot < a.B;
   const bool reporter = L.sub == 0;
   L.bag = slot;
@@ -208,20 +210,23 @@ __device__ __forceinline__ int lean_wave_max(int v) {
 constexpr int LEAN_NO_ENTRY = INT32_MIN;  // the bag has no such entry
 constexpr int LEAN_SKIP = -1;             // an entry that adds nothing (a pruned or rejected row)
 
-// index -> row number, LEAN_SKIP for what the reference skips, reporting what it rejects.
-// `mapped` is the remap entry already fetched for a pruned table.
-__device__ __forceinline__ int lean_row(const LookupArgs& a, const TableDesc& d, const LeanLane& L, int64_t row, int64_t pos) {
+// index -> row number, LEAN_SKIP for what the reference skips or rejects. A rejected index
+// leaves its position in `bad_pos` (the smallest wins); the caller reports it once its loop is
+// over (lean_report_bad): an atomic inside the loop would count as a store in flight, and with
+// loads and stores in flight together every wait of the loop becomes a wait for everything.
+constexpr int64_t LEAN_NO_BAD_POS = INT64_MAX;
+__device__ __forceinline__ int lean_row(const TableDesc& d, const LeanLane& L, int64_t row, int64_t pos, int64_t& bad_pos) {
   if (!L.remapped && d.skip_minus_one && row == -1) return LEAN_SKIP;
   if (row < 0 || row >= d.num_rows) {
-    report_index(a.status, pos);
+    bad_pos = pos < bad_pos ? pos : bad_pos;
     return LEAN_SKIP;
   }
   return (int)row;
 }
 constexpr int64_t LEAN_PRUNED = INT64_MIN; // what lean_remap returns for an entry that adds nothing
-__device__ __forceinline__ int64_t lean_remap(const LookupArgs& a, const LeanLane& L, int64_t logical, int64_t pos) {
+__device__ __forceinline__ int64_t lean_remap(const LookupArgs& a, const LeanLane& L, int64_t logical, int64_t pos, int64_t& bad_pos) {
   if (logical < 0 || logical >= L.remap_cap) {
-    report_index(a.status, pos);
+    bad_pos = pos < bad_pos ? pos : bad_pos;
     return LEAN_PRUNED;
   }
   if (L.rank_base >= 0) { // order-preserving mapping: the physical row is the rank among the kept rows
@@ -234,6 +239,9 @@ __device__ __forceinline__ int64_t lean_remap(const LookupArgs& a, const LeanLan
                               : (int64_t) reinterpret_cast<const int32_t*>(a.remap)[L.remap_base + logical];
   return m == -1 ? LEAN_PRUNED : m;
 }
+__device__ __forceinline__ void lean_report_bad(const LookupArgs& a, int64_t bad_pos) {
+  if (bad_pos != LEAN_NO_BAD_POS) report_index(a.status, bad_pos);
+}
 
 // The output of a wave through LDS, so that every store instruction writes runs
 // of consecutive bytes: a lane holds 32 consecutive columns of its bag (64 or 128
@@ -243,7 +251,8 @@ __device__ __forceinline__ int64_t lean_remap(const LookupArgs& a, const LeanLan
 // and then take them back interleaved: piece sub, sub + lanes, sub + 2 lanes, ...,
 // which makes each instruction write lanes * 16 consecutive bytes per bag.
 // ESZ: bytes per output element. `lds` must hold the wave's whole output (at most
-// 64 lanes * 32 columns * 4 bytes) and is free once the last block is pooled.
+// 64 lanes * 32 columns * 4 bytes = LEAN_LDS_WORDS) and MAX_GROUPS words behind it, and is
+// free once the last block is pooled.
 template <int TY, int C, bool INHDR, int ESZ>
 __device__ __forceinline__ void lean_store_interleaved(const LookupArgs& a, const TableDesc& d, const LeanLane& L,
                                                        const float (&acc)[C * (TY == ST_INT4 ? 32 : (TY == ST_INT8 ? 16 : 8))],
@@ -283,15 +292,51 @@ __device__ __forceinline__ void lean_store_interleaved(const LookupArgs& a, cons
       }
     }
   }
+  // the bag every group of the wave writes for (-1: none), behind the pieces
+  int* bag_of = reinterpret_cast<int*>(lds + LEAN_LDS_WORDS);
+  if (L.sub == 0 && !L.idle) bag_of[L.grp] = L.bag_ok ? L.bag : -1;
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-  uint8_t* block = reinterpret_cast<uint8_t*>(a.out) + ((int64_t)L.bag * a.out_stride + d.out_col) * ESZ;
+  const int64_t row_bytes = a.out_stride * ESZ;
+  uint8_t* out0 = reinterpret_cast<uint8_t*>(a.out) + (int64_t)d.out_col * ESZ;
+  if ((npb & (npb - 1)) == 0 && S < 8) {
+    // The pieces of the whole wave, bag after bag, dealt to the lanes in that order: consecutive
+    // lanes write consecutive pieces of one bag, so a store instruction covers whole runs of a
+    // bag's block (all of it when the block has no more than 64 pieces) instead of `lanes` pieces
+    // of every bag, which for bags of 2..4 lanes are fragments of 32..64 bytes that reach memory
+    // as partial writes of their lines. (Bags of 8 lanes and more write runs of 128 bytes either
+    // way and keep the mapping below, which needs no look-up of the bag: 2.5 % on the HBM-sized
+    // configuration.)
+    const int shift = __builtin_ctz((unsigned)npb);
+    const int total = d.bags << shift;
+#pragma unroll
+    for (int it = 0; it < C * NP; ++it) {
+      const int f = (int)threadIdx.x + it * 64;
+      if (f < total) {
+        const int g = f >> shift;
+        const int piece = f & (npb - 1);
+        const int bag = bag_of[g];
+        if (bag >= 0) {
+          uint8_t* dst = out0 + (int64_t)bag * row_bytes + (size_t)piece * PB;
+          // streaming stores: whole runs of the output, written once and never read back here
+          if constexpr (WP == 4) {
+            const uint4 v = *reinterpret_cast<const uint4*>(lds + (size_t)f * 4);
+            stream_store16(dst, v.x, v.y, v.z, v.w);
+          } else {
+            const uint2 v = *reinterpret_cast<const uint2*>(lds + (size_t)f * 2);
+            stream_store8(dst, v.x, v.y);
+          }
+        }
+      }
+    }
+    return;
+  }
+  uint8_t* block = out0 + (int64_t)L.bag * row_bytes;
 #pragma unroll
   for (int it = 0; it < C * NP; ++it) {
     const int gq = L.sub + it * S;
     if (L.bag_ok && gq < npb) {
-      // streaming stores: whole runs of the output, written once and never read back here
       if constexpr (WP == 4) {
         const uint4 v = *reinterpret_cast<const uint4*>(mine + gq * 4);
         stream_store16(block + (size_t)gq * 16, v.x, v.y, v.z, v.w);
@@ -353,48 +398,77 @@ __device__ __forceinline__ void lean_write(const LookupArgs& a, const TableDesc&
 // 8-bit, 4 for fp16 rows). INHDR as in the general kernel. R: entries a staging
 // lane handles per block (8 / the staging lanes of a bag: 1 for bags of 8 lanes
 // and more, 2 for 4..7 lanes, 4 for 2..3 lanes).
+//
+// The rows of a bag are fetched in units of 4 loads of 16 bytes per lane (4, 2 or
+// 1 rows) into two register sets that take turns: while one unit is added up the
+// other is in flight, and as soon as a set is free the unit after the next is
+// asked for, so a lane has 4 to 8 loads outstanding at all times instead of 8
+// while it waits and none while it computes. Units cross block boundaries: the
+// rows of block k + 1 are staged (in the second of two LDS buffers) before the
+// arithmetic of block k starts, its indices having been fetched a block earlier.
+// Loads return in the order they were issued, so everything a step waits for is
+// issued before what should stay in flight behind it:
+//   iteration k:  multipliers of block k    <- headers(k), issued in iteration k - 1
+//                 rows, weights of block k+1 <- indices(k+1), issued in iteration k - 1
+//                 issue indices(k+2); stage the rows of block k+1; issue headers(k+1)
+//                 for every unit of block k: add it up, issue the unit two further on
+// An entry that adds nothing (absent, pruned, rejected) is staged as a row the
+// wave has seen to be valid with the multiplier (-0, -0, -0), which leaves every
+// accumulator as it is: the loads need no predicate. (Until the wave has seen a
+// valid row its units are not loaded at all.)
 // Returns false (wave-uniform, nothing written) when a scale is too large for
 // the pre-scaled arithmetic.
 template <typename index_t, bool EXACT, int TY, int C, bool INHDR, int R>
 __device__ __forceinline__ bool pool_lean(const LookupArgs& a, const TableDesc& d, int table, int first_slot, int lane,
-                                          int* stage_row, LeanMul* stage_mul) {
+                                          uint32_t* lds) {
   constexpr bool QUANT = TY == ST_INT8 || TY == ST_INT4;
   constexpr int E = TY == ST_INT4 ? 32 : (TY == ST_INT8 ? 16 : 8); // columns per chunk
-  constexpr int RN = 8 / C;                                        // rows per round: 8 loads in flight per lane
+  // 16-byte loads per lane and unit. 4 for fp16 rows (one row). Quantised rows: 2 with the exact
+  // arithmetic, which is bound by the vector units and gains nothing from more loads in flight
+  // (HBM-sized configuration: 2.97 ms with 2, 3.10 ms with 4); 4 with the tolerance-grade
+  // arithmetic (2.71 against 2.76 ms), except where the staging lanes hold 4 entries each and
+  // fetch the row headers: their registers and 4-load units together do not fit the 168
+  // registers that 3 waves per SIMD leave a lane.
+  constexpr int UL = !QUANT ? 4 : (EXACT || (R == 4 && !INHDR)) ? 2 : 4;
+  constexpr int HALF = UL / C;                                     // rows per unit
+  constexpr int U = LEAN_BLOCK / HALF;                             // units per block
   constexpr int SL = LEAN_BLOCK / R;                               // staging lanes per bag
+  constexpr int ROWS_BUF = MAX_GROUPS * LEAN_BLOCK;                // one buffer of staged rows
   static_assert(!INHDR || QUANT, "whole-row chunks belong to rows with a header");
+
+  int* stage_row = reinterpret_cast<int*>(lds);                               // [2][MAX_GROUPS][LEAN_BLOCK]
+  LeanMul* stage_mul = reinterpret_cast<LeanMul*>(lds + 2 * ROWS_BUF);        // [MAX_GROUPS][LEAN_BLOCK]
 
   const LeanLane L = lean_lane<index_t>(a, d, table, first_slot, lane);
   const int S = d.lanes;
   const int sub = L.sub;
   const int n = L.n;
-  const bool bag_ok = L.bag_ok;
-  const bool stager = bag_ok && sub < SL;
+  // every bag slot of the wave stages, also one past the table's last bag (its entries are all absent)
+  const bool stager = !L.idle && sub < SL;
   // the longest bag of the wave bounds the loop (wave-uniform)
   const int nmax = lean_wave_max(n);
+  const int units = (int)(((uint32_t)nmax + HALF - 1) / HALF);
 
   const index_t* idx = reinterpret_cast<const index_t*>(a.indices) + L.pos0;
   const float* sw = a.sample_weights ? a.sample_weights + L.pos0 : nullptr;
   const uint8_t* wbase = (d.placement ? a.weights[1] : a.weights[0]) + d.weights_offset;
   const uint8_t* psb = wbase + d.sb_off;
-  // this lane's first chunk of row 0
-  const uint8_t* pdata = INHDR ? wbase + sub * 16 : wbase + d.data_off + sub * 16;
   const uint32_t stride = (uint32_t)d.row_stride;
-  int* my_row = stage_row + L.lgrp * LEAN_BLOCK;
+  int* my_rows = stage_row + L.lgrp * LEAN_BLOCK;
   LeanMul* my_mul = stage_mul + L.lgrp * LEAN_BLOCK;
-  // byte offset of the lane's chunks from its first; whole-row chunks: a slot past
-  // the row's last chunk shadows it (same bytes, nothing written)
-  int rowb[C];
+  // this lane's chunks of row 0; whole-row chunks: a slot past the row's last chunk
+  // shadows it (same bytes, nothing written)
+  const uint8_t* pchunk[C];
   if constexpr (INHDR) {
     const int nchunks = (d.data_bytes + 4 + 15) / 16;
 #pragma unroll
     for (int c = 0; c < C; ++c) {
       const int k = sub + c * S;
-      rowb[c] = ((k < nchunks ? k : nchunks - 1) - sub) * 16;
+      pchunk[c] = wbase + (k < nchunks ? k : nchunks - 1) * 16;
     }
   } else {
 #pragma unroll
-    for (int c = 0; c < C; ++c) rowb[c] = c * S * 16;
+    for (int c = 0; c < C; ++c) pchunk[c] = wbase + d.data_off + (sub + c * S) * 16;
   }
 
   float acc[C * E];
@@ -402,11 +476,29 @@ __device__ __forceinline__ bool pool_lean(const LookupArgs& a, const TableDesc& 
   for (int e = 0; e < C * E; ++e) acc[e] = 0.0f;
   float bsum = -0.0f; // tolerance grade: the biases of the bag, added once at the end
 
-  // registers of the staging lanes: raw indices and weights of the block being fetched
+  // the two register sets of rows in flight
+  uint32_t raw_a[HALF][C][4], raw_b[HALF][C][4];
+#pragma unroll
+  for (int e = 0; e < HALF; ++e)
+#pragma unroll
+    for (int c = 0; c < C; ++c)
+#pragma unroll
+      for (int w = 0; w < 4; ++w) raw_a[e][c][w] = raw_b[e][c][w] = 0u;
+
+  // registers of the staging lanes: the indices and weights on their way, the rows
+  // and weights of the block staged last, its headers on their way
   int64_t nrow[R];
   float nw[R];
   bool have[R];
-  auto load_idx = [&](int blk) {
+  int crow[R];
+  float cw[R];
+  uint32_t h0[R], h1[R];
+  int64_t bad_pos = LEAN_NO_BAD_POS; // the first rejected index this lane has met
+  int safe = -1;         // a row of the table that can be loaded (wave-uniform); -1: none seen yet
+  uint32_t loadable = 0; // bit p: the rows staged in buffer p can be loaded (wave-uniform)
+  uint32_t holey = 0;    // bit p: some entry staged in buffer p adds nothing (wave-uniform; fp16 rows only)
+
+  auto issue_idx = [&](int blk) {
 #pragma unroll
     for (int j = 0; j < R; ++j) {
       nrow[j] = 0;
@@ -419,148 +511,214 @@ __device__ __forceinline__ bool pool_lean(const LookupArgs& a, const TableDesc& 
       }
     }
   };
-
-  load_idx(0);
-  for (int blk = 0; blk * LEAN_BLOCK < nmax; ++blk) {
-    // ---- logical -> physical rows of pruned tables (the loads of the block issued together) ----
+  // indices that have arrived -> row numbers (negative: nothing to add), weights
+  auto take_idx = [&](int blk) {
     if (L.remapped) {
 #pragma unroll
       for (int j = 0; j < R; ++j)
-        if (have[j]) nrow[j] = lean_remap(a, L, nrow[j], L.pos0 + blk * LEAN_BLOCK + sub + j * SL);
+        if (have[j]) nrow[j] = lean_remap(a, L, nrow[j], L.pos0 + blk * LEAN_BLOCK + sub + j * SL, bad_pos);
     }
-    // ---- stage the block: row numbers (or holes), the weights ----
-    int crow[R];
-    float cw[R];
-    bool hole = false, big = false;
 #pragma unroll
     for (int j = 0; j < R; ++j) {
       crow[j] = LEAN_NO_ENTRY;
-      cw[j] = nw[j];
-      if (have[j]) crow[j] = nrow[j] == LEAN_PRUNED ? LEAN_SKIP : lean_row(a, d, L, nrow[j], L.pos0 + blk * LEAN_BLOCK + sub + j * SL);
-      if (stager) {
-        hole = hole || crow[j] < 0;
-        my_row[sub + j * SL] = crow[j];
-        if (!QUANT || INHDR || crow[j] < 0) {
-          // fp16 rows and whole-row chunks: the multiplier is the weight. A hole gets
-          // (-0, -0, -0), which leaves every accumulator exactly as it is.
-          LeanMul m;
-          m.s24 = crow[j] < 0 ? -0.0f : nw[j];
-          m.s20 = -0.0f;
-          m.bias = -0.0f;
-          m.pad = 0.0f;
-          // whole-row chunks take fp16 headers: |scale| <= 65504, so only a huge weight can overflow the pre-scaling
-          if (INHDR) big = big || !(__builtin_fabsf(nw[j]) < 0x1p60f);
-          my_mul[sub + j * SL] = m;
+      // a copy made here and now: left to itself the compiler keeps the weight where it was
+      // loaded, loads the next block's weight elsewhere and moves both at the end of the loop,
+      // which waits for that load and for everything issued before it
+      asm volatile("v_mov_b32 %0, %1" : "=v"(cw[j]) : "v"(nw[j]));
+      if (have[j]) crow[j] = nrow[j] == LEAN_PRUNED ? LEAN_SKIP : lean_row(d, L, nrow[j], L.pos0 + blk * LEAN_BLOCK + sub + j * SL, bad_pos);
+    }
+  };
+  // the rows of block blk into buffer blk & 1; the headers of its rows asked for
+  auto stage_rows = [&](int blk) {
+    int cand = -1;
+#pragma unroll
+    for (int j = 0; j < R; ++j)
+      if (crow[j] >= 0) cand = crow[j];
+    const uint64_t seen = __builtin_amdgcn_ballot_w64(cand >= 0);
+    if (seen != 0ull) safe = __builtin_amdgcn_readlane(cand, (int)__builtin_ctzll(seen));
+    const int p = blk & 1;
+    loadable = safe >= 0 ? (loadable | (1u << p)) : (loadable & ~(1u << p));
+    if constexpr (!QUANT) {
+      bool hole = false;
+#pragma unroll
+      for (int j = 0; j < R; ++j) hole = hole || crow[j] < 0;
+      holey = __builtin_amdgcn_ballot_w64(stager && hole) != 0ull ? (holey | (1u << p)) : (holey & ~(1u << p));
+    }
+    if (stager) {
+#pragma unroll
+      for (int j = 0; j < R; ++j) my_rows[p * ROWS_BUF + sub + j * SL] = crow[j] >= 0 ? crow[j] : safe;
+    }
+    if constexpr (QUANT && !INHDR) {
+#pragma unroll
+      for (int j = 0; j < R; ++j) {
+        h0[j] = h1[j] = 0u;
+        if (crow[j] >= 0) {
+          const uint8_t* ph = psb + (uint64_t)(uint32_t)crow[j] * stride;
+          if (TY == ST_INT8 && d.sb_fp32) { // two floats behind the data: 8-bit rows of the single-table layout only
+            const Dwordx2 v = *reinterpret_cast<const Dwordx2*>(ph);
+            h0[j] = v.v[0];
+            h1[j] = v.v[1];
+          } else {
+            h0[j] = *reinterpret_cast<const uint32_t*>(ph);
+          }
         }
       }
     }
-    // wave-uniform: every bag slot of the wave holds a bag with 8 rows to add in this block
-    // (lanes left over shadow the last bag slot, so that one must be there too)
-    const bool full = __builtin_amdgcn_ballot_w64(hole || first_slot + L.lgrp >= a.B) == 0ull;
+  };
+  // the multipliers of the block whose rows were staged last; true: a scale too large for the pre-scaled route
+  auto stage_muls = [&]() {
+    bool big = false;
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      LeanMul m;
+      m.s24 = -0.0f;
+      m.s20 = -0.0f;
+      m.bias = -0.0f;
+      m.hole = 1u;
+      if (crow[j] >= 0) {
+        m.hole = 0u;
+        if constexpr (QUANT && !INHDR) {
+          const bool pair32 = TY == ST_INT8 && d.sb_fp32;
+          const float rs = pair32 ? bits_to_float(h0[j]) : half_lo(h0[j]);
+          const float rb = pair32 ? bits_to_float(h1[j]) : half_hi(h0[j]);
+          const float sc = cw[j] * rs;
+          big = big || !(__builtin_fabsf(sc) < 0x1p100f);
+          m.s24 = sc * 0x1p24f;
+          m.s20 = sc * 0x1p20f;
+          m.bias = cw[j] * rb;
+        } else {
+          // fp16 rows and whole-row chunks: the multiplier is the weight. Whole-row chunks take fp16
+          // headers: |scale| <= 65504, so only a huge weight can overflow the pre-scaling
+          m.s24 = cw[j];
+          if constexpr (INHDR) big = big || !(__builtin_fabsf(cw[j]) < 0x1p60f);
+        }
+      }
+      if (stager) my_mul[sub + j * SL] = m;
+    }
+    return big;
+  };
+  auto lds_sync = [&]() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-
-    uint32_t raw[RN][C][4]; // the rows in flight; a slot without a row reads as zeros
-    auto load_round_full = [&](int rd) {
+  };
+  // unit g (counted from the bag's first row) into one of the register sets
+  auto issue_unit = [&](uint32_t (&raw)[HALF][C][4], int g) {
+    const int* rows = my_rows + ((g / U) & 1) * ROWS_BUF + (g % U) * HALF;
 #pragma unroll
-      for (int e = 0; e < RN; ++e) {
-        const uint8_t* p = pdata + (uint64_t)(uint32_t)my_row[rd * RN + e] * stride;
+    for (int e = 0; e < HALF; ++e) {
+      const uint64_t off = (uint64_t)(uint32_t)rows[e] * stride;
 #pragma unroll
-        for (int c = 0; c < C; ++c) load_raw<16>(raw[e][c], p + rowb[c]);
+      for (int c = 0; c < C; ++c) load_raw<16>(raw[e][c], pchunk[c] + off);
+    }
+  };
+  // unit u of the block whose multipliers are staged: added to the accumulators.
+  // `holes`: the block may hold entries that add nothing (fp16 rows only: see below)
+  auto add_unit = [&](uint32_t (&raw)[HALF][C][4], int u, bool holes) {
+#pragma unroll
+    for (int e = 0; e < HALF; ++e) {
+      LeanMul m = my_mul[u * HALF + e];
+      if constexpr (INHDR) {
+        // the row header sits in the first dword of chunk 0, which the first lane of the group
+        // holds; an entry that adds nothing has loaded some other row: its header does not count
+        uint32_t h = (uint32_t)__builtin_amdgcn_ds_bpermute((lane - sub) * 4, (int)raw[e][0][0]);
+        h = m.hole ? 0u : h;
+        const float sc = m.s24 * half_lo(h);
+        m.bias = m.s24 * half_hi(h);
+        m.s24 = sc * 0x1p24f;
+        m.s20 = sc * 0x1p20f;
       }
-    };
-    auto load_round_ragged = [&](int rd) {
-#pragma unroll
-      for (int e = 0; e < RN; ++e) {
-        const int row = my_row[rd * RN + e];
-        if (bag_ok && row >= 0) {
-          const uint8_t* p = pdata + (uint64_t)(uint32_t)row * stride;
-#pragma unroll
-          for (int c = 0; c < C; ++c) load_raw<16>(raw[e][c], p + rowb[c]);
-        } else {
+      if constexpr (!QUANT) {
+        // the row an absent entry has loaded may hold infinities: -0 times them is not nothing
+        if (holes && m.hole) {
 #pragma unroll
           for (int c = 0; c < C; ++c)
 #pragma unroll
             for (int w = 0; w < 4; ++w) raw[e][c][w] = 0u;
         }
       }
-    };
-    // the rows first, then what depends on them least: (scale, bias) of the staged
-    // rows, the indices of the next block. One wait covers rows and headers.
-    if (full) load_round_full(0);
-    else load_round_ragged(0);
-    uint32_t h0[R], h1[R];
-    if constexpr (QUANT && !INHDR) {
+      if constexpr (!EXACT && QUANT) bsum += m.bias;
 #pragma unroll
-      for (int j = 0; j < R; ++j) {
-        h0[j] = h1[j] = 0u;
-        if (crow[j] >= 0) {
-          const uint8_t* p = psb + (uint64_t)(uint32_t)crow[j] * stride;
-          if (d.sb_fp32) {
-            const Dwordx2 v = *reinterpret_cast<const Dwordx2*>(p);
-            h0[j] = v.v[0];
-            h1[j] = v.v[1];
+      for (int c = 0; c < C; ++c) lean_chunk<TY, EXACT, false, C * E>(acc, c * E, raw[e][c], m);
+    }
+  };
+  auto can_load = [&](int g) { return g < units && ((loadable >> ((g / U) & 1)) & 1u) != 0u; };
+
+  // A scale too large for the pre-scaled route (any lane, any block): remembered, and acted on
+  // once the loops are over; nothing is written before that. (Leaving the loop where the scale
+  // is met costs every wave of the kernel: with that exit in it the compiler makes every wait
+  // of the loop a wait for all loads in flight.)
+  bool big = false;
+  // the top of iteration blk (see above)
+  auto block_top = [&](int blk) {
+    big = stage_muls() || big;
+    take_idx(blk + 1);
+    issue_idx(blk + 2);
+    stage_rows(blk + 1);
+    lds_sync();
+  };
+
+  if (units > 0) {
+    issue_idx(0);
+    take_idx(0);
+    issue_idx(1);
+    stage_rows(0);
+    lds_sync();
+    // Iterations in which every unit exists and can be loaded run a copy of the loop without
+    // conditions around its loads: the compiler places its waits by counting the loads behind
+    // the one it waits for, and a load that may or may not have been issued counts as not
+    // issued, which would turn every wait of the loop into a wait for everything.
+    const bool steady = (loadable & 1u) != 0u && units >= 2;
+    int blk = 0;
+    if (steady) {
+      issue_unit(raw_a, 0);
+      issue_unit(raw_b, 1);
+      const int steady_blocks = (units - 2) / U; // blocks whose last unit has two units behind it
+      // (fp16 rows: and only blocks in which every entry adds a row; the first block with an
+      // absent entry and all after it take the loop below, which clears what such entries load)
+      for (; blk < steady_blocks && (QUANT || ((holey >> (blk & 1)) & 1u) == 0u); ++blk) {
+        block_top(blk);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          if (u & 1) {
+            add_unit(raw_b, u, false);
+            issue_unit(raw_b, blk * U + u + 2);
           } else {
-            h0[j] = *reinterpret_cast<const uint32_t*>(p);
+            add_unit(raw_a, u, false);
+            issue_unit(raw_a, blk * U + u + 2);
           }
+          // units stay in this order: moved ahead of the arithmetic of earlier units, the loads
+          // of later ones would need registers of their own
+          __builtin_amdgcn_sched_barrier(0);
         }
+        __builtin_amdgcn_wave_barrier(); // the column lanes are done with the block before it is overwritten
       }
+    } else {
+      if (can_load(0)) issue_unit(raw_a, 0);
+      if (can_load(1)) issue_unit(raw_b, 1);
     }
-    load_idx(blk + 1);
-
-    if constexpr (QUANT && !INHDR) {
+    for (; blk * U < units; ++blk) {
+      block_top(blk);
 #pragma unroll
-      for (int j = 0; j < R; ++j) {
-        if (crow[j] >= 0) {
-          const float rs = d.sb_fp32 ? bits_to_float(h0[j]) : half_lo(h0[j]);
-          const float rb = d.sb_fp32 ? bits_to_float(h1[j]) : half_hi(h0[j]);
-          const float sc = cw[j] * rs;
-          big = big || !(__builtin_fabsf(sc) < 0x1p100f);
-          LeanMul m;
-          m.s24 = sc * 0x1p24f;
-          m.s20 = sc * 0x1p20f;
-          m.bias = cw[j] * rb;
-          m.pad = 0.0f;
-          my_mul[sub + j * SL] = m;
+      for (int u = 0; u < U; ++u) {
+        const int g = blk * U + u;
+        if (g >= units) break; // no bag of the wave reaches this unit
+        if (u & 1) {
+          add_unit(raw_b, u, true);
+          if (can_load(g + 2)) issue_unit(raw_b, g + 2);
+        } else {
+          add_unit(raw_a, u, true);
+          if (can_load(g + 2)) issue_unit(raw_a, g + 2);
         }
       }
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     }
-    if constexpr (QUANT) {
-      // wave-uniform: a scale too large for the pre-scaled route; nothing has been written yet
-      if (__builtin_amdgcn_ballot_w64(big) != 0ull) return false;
-    }
-
-#pragma unroll
-    for (int rd = 0; rd < LEAN_BLOCK / RN; ++rd) {
-      if (rd > 0) {
-        if (rd * RN >= nmax - blk * LEAN_BLOCK) break; // no bag of the wave reaches this round
-        if (full) load_round_full(rd);
-        else load_round_ragged(rd);
-      }
-#pragma unroll
-      for (int e = 0; e < RN; ++e) {
-        LeanMul m = my_mul[rd * RN + e];
-        if constexpr (INHDR) {
-          // the row header sits in the first dword of chunk 0, which the first lane
-          // of the group holds (zero for a row that is not there)
-          const uint32_t h = (uint32_t)__builtin_amdgcn_ds_bpermute((lane - sub) * 4, (int)raw[e][0][0]);
-          const float sc = m.s24 * half_lo(h);
-          m.bias = m.s24 * half_hi(h);
-          m.s24 = sc * 0x1p24f;
-          m.s20 = sc * 0x1p20f;
-        }
-        if constexpr (!EXACT && QUANT) bsum += m.bias;
-#pragma unroll
-        for (int c = 0; c < C; ++c) lean_chunk<TY, EXACT, false, C * E>(acc, c * E, raw[e][c], m);
-      }
-    }
-    __builtin_amdgcn_wave_barrier(); // the column lanes are done with the block before it is overwritten
   }
-  lean_write<EXACT, TY, C, INHDR>(a, d, L, acc, bsum, reinterpret_cast<uint32_t*>(stage_row));
+  if constexpr (QUANT) {
+    if (__builtin_amdgcn_ballot_w64(big) != 0ull) return false; // wave-uniform
+  }
+  lean_report_bad(a, bad_pos);
+  lean_write<EXACT, TY, C, INHDR>(a, d, L, acc, bsum, lds);
   return true;
 }
 
@@ -579,11 +737,12 @@ __device__ __forceinline__ void pool_lean_slow(const LookupArgs& a, const TableD
 #pragma unroll
   for (int e = 0; e < C * E; ++e) acc[e] = 0.0f;
   float bsum = -0.0f;
+  int64_t bad_pos = LEAN_NO_BAD_POS;
   for (int i = 0; i < L.n; ++i) {
     int64_t row = (int64_t)idx[i];
     const float w = a.sample_weights ? a.sample_weights[L.pos0 + i] : 1.0f;
-    if (L.remapped) row = lean_remap(a, L, row, L.pos0 + i);
-    const int r = row == LEAN_PRUNED ? LEAN_SKIP : lean_row(a, d, L, row, L.pos0 + i);
+    if (L.remapped) row = lean_remap(a, L, row, L.pos0 + i, bad_pos);
+    const int r = row == LEAN_PRUNED ? LEAN_SKIP : lean_row(d, L, row, L.pos0 + i, bad_pos);
     if (r < 0) continue;
     const uint8_t* prow = wbase + (uint64_t)(uint32_t)r * (uint32_t)d.row_stride;
     float rs, rb;
@@ -592,7 +751,7 @@ __device__ __forceinline__ void pool_lean_slow(const LookupArgs& a, const TableD
     m.s24 = w * rs;
     m.s20 = m.s24;
     m.bias = w * rb;
-    m.pad = 0.0f;
+    m.hole = 0u;
     if constexpr (!EXACT) bsum += m.bias;
 #pragma unroll
     for (int c = 0; c < C; ++c) {
@@ -602,16 +761,17 @@ __device__ __forceinline__ void pool_lean_slow(const LookupArgs& a, const TableD
       lean_chunk<TY, EXACT, true, C * E>(acc, c * E, raw, m);
     }
   }
+  lean_report_bad(a, bad_pos);
   lean_write<EXACT, TY, C, INHDR>(a, d, L, acc, bsum, nullptr);
 }
 
 template <typename index_t, bool EXACT, int TY, int C, bool INHDR>
 __device__ __forceinline__ void run_lean(const LookupArgs& a, const TableDesc& d, int table, int first_slot, int lane,
-                                         int* stage_row, LeanMul* stage_mul) {
+                                         uint32_t* lds) {
   bool done;
-  if (d.lanes >= 8) done = pool_lean<index_t, EXACT, TY, C, INHDR, 1>(a, d, table, first_slot, lane, stage_row, stage_mul);
-  else if (d.lanes >= 4) done = pool_lean<index_t, EXACT, TY, C, INHDR, 2>(a, d, table, first_slot, lane, stage_row, stage_mul);
-  else done = pool_lean<index_t, EXACT, TY, C, INHDR, 4>(a, d, table, first_slot, lane, stage_row, stage_mul);
+  if (d.lanes >= 8) done = pool_lean<index_t, EXACT, TY, C, INHDR, 1>(a, d, table, first_slot, lane, lds);
+  else if (d.lanes >= 4) done = pool_lean<index_t, EXACT, TY, C, INHDR, 2>(a, d, table, first_slot, lane, lds);
+  else done = pool_lean<index_t, EXACT, TY, C, INHDR, 4>(a, d, table, first_slot, lane, lds);
   if constexpr (TY == ST_INT4 || TY == ST_INT8) {
     if (!done) pool_lean_slow<index_t, EXACT, TY, C, INHDR>(a, d, table, first_slot, lane);
   }
@@ -620,15 +780,15 @@ __device__ __forceinline__ void run_lean(const LookupArgs& a, const TableDesc& d
 // Row types and the chunks per lane the host picks for lean shapes: 1 (4-bit), 2 (8-bit), 4 (fp16).
 template <typename index_t, bool EXACT>
 __device__ __forceinline__ void lean_dispatch(const LookupArgs& a, const TableDesc& d, int table, int first_slot, int lane,
-                                              int* stage_row, LeanMul* stage_mul) {
+                                              uint32_t* lds) {
   if (d.ty == ST_INT4) {
-    if (d.inline_hdr) run_lean<index_t, EXACT, ST_INT4, 1, true>(a, d, table, first_slot, lane, stage_row, stage_mul);
-    else run_lean<index_t, EXACT, ST_INT4, 1, false>(a, d, table, first_slot, lane, stage_row, stage_mul);
+    if (d.inline_hdr) run_lean<index_t, EXACT, ST_INT4, 1, true>(a, d, table, first_slot, lane, lds);
+    else run_lean<index_t, EXACT, ST_INT4, 1, false>(a, d, table, first_slot, lane, lds);
   } else if (d.ty == ST_INT8) {
-    if (d.inline_hdr) run_lean<index_t, EXACT, ST_INT8, 2, true>(a, d, table, first_slot, lane, stage_row, stage_mul);
-    else run_lean<index_t, EXACT, ST_INT8, 2, false>(a, d, table, first_slot, lane, stage_row, stage_mul);
+    if (d.inline_hdr) run_lean<index_t, EXACT, ST_INT8, 2, true>(a, d, table, first_slot, lane, lds);
+    else run_lean<index_t, EXACT, ST_INT8, 2, false>(a, d, table, first_slot, lane, lds);
   } else if (d.ty == ST_FP16) {
-    run_lean<index_t, EXACT, ST_FP16, 4, false>(a, d, table, first_slot, lane, stage_row, stage_mul);
+    run_lean<index_t, EXACT, ST_FP16, 4, false>(a, d, table, first_slot, lane, lds);
   }
 }
 
@@ -639,10 +799,8 @@ __device__ __forceinline__ void lean_dispatch(const LookupArgs& a, const TableDe
 // Same work list and workgroup -> XCD mapping as lookup_kernel.
 template <typename index_t, bool EXACT>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(FBGEMM_AMD_LEAN_MIN_WAVES, 8))) void lookup_lean_kernel(const LookupArgs a) {
-  // 8 KB: while a bag is pooled, the staged rows (1 KB) and multipliers (4 KB); at the end, the wave's output
-  __shared__ __attribute__((aligned(16))) uint32_t lds[LEAN_LDS_WORDS];
-  int* stage_row = reinterpret_cast<int*>(lds);
-  LeanMul* stage_mul = reinterpret_cast<LeanMul*>(lds + MAX_GROUPS * LEAN_BLOCK);
+  // 8 KB: while a bag is pooled, two buffers of staged rows (2 KB) and the multipliers (4 KB); at the end, the wave's output
+  __shared__ __attribute__((aligned(16))) uint32_t lds[LEAN_LDS_WORDS + MAX_GROUPS];
   const int lane = threadIdx.x;
   int64_t wave;
   if (a.xcd_start) {
@@ -664,7 +822,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(FBGEMM_AMD_L
     first_slot = (int)(wave * a.single.bags);
   }
   const TableDesc d = a.tables ? a.tables[table] : a.single;
-  lean_dispatch<index_t, EXACT>(a, d, table, first_slot, lane, stage_row, stage_mul);
+  lean_dispatch<index_t, EXACT>(a, d, table, first_slot, lane, lds);
 }
 
 #define FBGEMM_AMD_DEFINE_LEAN_LAUNCH(FN, INDEX_T, EXACT)                                                \
