@@ -14,9 +14,10 @@ OUT = os.path.join(HERE, "lib", "libfbgemm_amd.so")
 # the lookup kernels compile one instance per translation unit (the slowest files first)
 SOURCES = ["lookup_lean_i64_exact.hip", "lookup_lean_i64_fast.hip", "lookup_lean_i32_exact.hip", "lookup_lean_i32_fast.hip",
            "lookup_i64.hip", "lookup_i32.hip", "lookup_i64_general.hip", "lookup_i32_general.hip",
-           "lookup_kernels.hip", "ceiling_kernels.hip", "index_ops_kernels.hip", "quantize_kernels.hip", "sequence_kernels.hip",
+           "lookup_kernels.hip", "index_ops_kernels.hip", "quantize_kernels.hip", "sequence_kernels.hip",
            "prune_kernels.hip", "remap_rank_kernels.hip", "split_bag_kernels.hip", "update_kernels.hip", "c_api.cpp"]
-HEADERS = ["cache_policy.h", "lookup_common.h", "lookup_device.h", "lookup_general.h", "lookup_lean.h", os.path.join("..", "..", "include", "fbgemm_amd.h")]
+HEADERS = ["cache_policy.h", "lookup_common.h", "lookup_device.h", "lookup_general.h", "lookup_lean.h", os.path.join("..", "..", "include", "fbgemm_amd.h"),
+           os.path.join("..", "..", "include", "fbgemm_amd_bench.h")]
 
 # -ffp-contract=off: the kernels spell out every fma; nothing else may be fused,
 #   or the fp32 rounding sequence would differ from the reference's.
@@ -69,8 +70,24 @@ def build_library(verbose=False, force=True):
     return OUT
 
 
+BENCH_OUT = os.path.join(HERE, "lib", "libfbgemm_amd_bench.so")
+
+
+def build_bench_library(verbose=False):
+    """The benchmark-only library: yardstick kernels for profiles (include/fbgemm_amd_bench.h).
+    Not linked into the product library and not loaded by it."""
+    cmd = ["hipcc", "-x", "hip", "-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-shared",
+           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           "-o", BENCH_OUT, os.path.join(CSRC, "bench_kernels.hip")]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    out = _hipcc(cmd)
+    if verbose and out.strip():
+        print(out)
+    return BENCH_OUT
+
+
 TORCH_OP_OUT = os.path.join(HERE, "lib", "libfbgemm_amd_torch.so")
-CPP_TEST_OUT = os.path.join(os.path.dirname(HERE), "tests", "cpp", "_build", "test_factories")
 
 
 def _run(cmd, verbose):
@@ -97,21 +114,8 @@ def build_torch_op(verbose=False):
     return TORCH_OP_OUT
 
 
-def build_cpp_test(verbose=False):
-    """tests/cpp/test_factories: the C++ factory templates against the C oracle."""
-    root = os.path.dirname(HERE)
-    os.makedirs(os.path.dirname(CPP_TEST_OUT), exist_ok=True)
-    subprocess.check_call(["make", "-s", "-C", os.path.join(root, "oracle"), "oracle"])
-    obuild = os.path.join(root, "oracle", "_build")
-    cmd = ["hipcc", "-x", "hip", "-O2", "--offload-arch=gfx950", "-std=c++17", "-o", CPP_TEST_OUT,
-           os.path.join(root, "tests", "cpp", "test_factories.cpp"), f"-L{os.path.dirname(OUT)}", "-lfbgemm_amd",
-           f"-L{obuild}", "-lembedding_oracle", f"-Wl,-rpath,{os.path.dirname(OUT)}", f"-Wl,-rpath,{obuild}"]
-    _run(cmd, verbose)
-    return CPP_TEST_OUT
-
-
 if __name__ == "__main__":
     print(build_library(verbose=True, force="--incremental" not in sys.argv))
+    print(build_bench_library(verbose=True))
     print(build_torch_op(verbose=True))
-    print(build_cpp_test(verbose=True))
     sys.exit(0)

@@ -13,6 +13,7 @@
 #include <vector>
 
 #include "../../include/fbgemm_amd.h"
+#include "../../include/fbgemm_amd_bench.h"
 #include "cache_policy.h"
 #include "lookup_common.h"
 
@@ -59,10 +60,6 @@ hipError_t launch_compressed_indices_remap(const void* indices, bool idx64, cons
                                            hipStream_t stream);
 hipError_t launch_quantize_segments(const float* input, int64_t lines, int32_t T, const int32_t* d_seg_offsets,
                                     int32_t total_D, int32_t max_D, uint8_t* output, hipStream_t stream);
-hipError_t launch_calibration_copy(const void* src, void* dst, int64_t bytes, hipStream_t stream);
-hipError_t launch_stream_read(const void* src, int64_t bytes, uint32_t* sink, hipStream_t stream);
-hipError_t launch_gather_lines(const void* table, int64_t stride, int32_t lanes, int32_t byte_offset, const int32_t* idx,
-                               int64_t n, uint32_t* sink, int32_t waves, hipStream_t stream);
 hipError_t launch_bounds_check(const int64_t* rows_per_table, int32_t T, void* indices, void* offsets, bool is64,
                                int64_t num_indices, int64_t total_B, int64_t B, const int32_t* B_offsets, int mode,
                                int64_t* warning, int64_t* fixed, int64_t* partial, Status* status, hipStream_t stream);
@@ -403,30 +400,6 @@ int fbgemm_amd_status_read(const void* d_status, void* stream, int32_t* bits, in
 
 int fbgemm_amd_stream_synchronize(void* stream) {
   HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
-  return 0;
-}
-
-int fbgemm_amd_calibration_copy(const void* d_src, void* d_dst, int64_t bytes, void* stream) {
-  if (!d_src || !d_dst || bytes < 0 || bytes % 16) return fail(FBGEMM_AMD_E_ARG, "copy needs 16-byte multiples");
-  HIP_TRY(launch_calibration_copy(d_src, d_dst, bytes, (hipStream_t)stream));
-  return 0;
-}
-
-int fbgemm_amd_ceiling_stream_read(const void* d_src, int64_t bytes, void* d_sink, void* stream) {
-  if (!d_src || !d_sink || bytes < 0 || bytes % 16) return fail(FBGEMM_AMD_E_ARG, "the read needs a 16-byte multiple and a sink of 8192 dwords");
-  HIP_TRY(launch_stream_read(d_src, bytes, (uint32_t*)d_sink, (hipStream_t)stream));
-  return 0;
-}
-
-int fbgemm_amd_ceiling_gather(const void* d_table, int64_t rows, int64_t row_stride, int32_t lanes_per_row, int32_t byte_offset,
-                              const int32_t* d_rows, int64_t n, void* d_sink, int32_t waves, void* stream) {
-  if (!d_table || !d_rows || !d_sink || rows <= 0 || n < 0 || waves <= 0)
-    return fail(FBGEMM_AMD_E_ARG, "bad gather arguments");
-  if (lanes_per_row < 1 || lanes_per_row > 64 || (lanes_per_row & (lanes_per_row - 1)))
-    return fail(FBGEMM_AMD_E_ARG, "lanes_per_row must be a power of two up to 64");
-  if (byte_offset < 0 || byte_offset % 4 || row_stride % 4 || (int64_t)byte_offset + 16 * lanes_per_row > row_stride)
-    return fail(FBGEMM_AMD_E_ARG, "the bytes read must lie inside the row, at 4-byte alignment");
-  HIP_TRY(launch_gather_lines(d_table, row_stride, lanes_per_row, byte_offset, d_rows, n, (uint32_t*)d_sink, waves, (hipStream_t)stream));
   return 0;
 }
 
@@ -833,8 +806,7 @@ struct fbgemm_amd_tbe_plan {
   int32_t fp8_shift = 0; // FP8 rows: set by fbgemm_amd_tbe_plan_set_fp8
   float fp8_mult = 0.0f;
   bool has_fp8 = false;
-  std::vector<hipEvent_t> prof_ev;
-  int64_t prof_count = 0;
+  bool reuse_order = false; // benchmarks: forwards skip the scheduler and take the last bag order of their stream
 };
 
 namespace {
@@ -1050,7 +1022,6 @@ void fbgemm_amd_tbe_plan_destroy(fbgemm_amd_tbe_plan* plan) {
   if (plan->d_rank_records) (void)hipFree(plan->d_rank_records);
   if (plan->d_rank_offsets) (void)hipFree(plan->d_rank_offsets);
   if (plan->d_rank_remap_offsets) (void)hipFree(plan->d_rank_remap_offsets);
-  for (hipEvent_t e : plan->prof_ev) (void)hipEventDestroy(e);
   delete plan;
 }
 
@@ -1195,7 +1166,7 @@ int tbe_forward_impl(
   bool exact = true;
   const RankRecord* rank_records = nullptr;
   const int64_t* rank_offsets = nullptr;
-  hipEvent_t prof_begin = nullptr, prof_end = nullptr;
+  bool reuse_order = false;
   {
     std::lock_guard<std::mutex> lk(plan->mu);
     // the lane shapes depend on B and (through the average bag length) on the number of indices:
@@ -1313,13 +1284,7 @@ int tbe_forward_impl(
       rank_offsets = plan->d_rank_offsets;
       d_index_remappings_offsets = plan->d_rank_remap_offsets;
     }
-    // bench-only: a pair of events around the lookup kernels of this forward
-    const size_t slots = plan->prof_ev.size() / 2;
-    if (slots) {
-      const size_t slot = (size_t)(plan->prof_count++ % (int64_t)slots);
-      prof_begin = plan->prof_ev[2 * slot];
-      prof_end = plan->prof_ev[2 * slot + 1];
-    }
+    reuse_order = plan->reuse_order;
   }
 
   LookupArgs a;
@@ -1349,10 +1314,9 @@ int tbe_forward_impl(
   a.fp8_shift = plan->fp8_shift;
   a.fp8_mult = plan->fp8_mult;
   if (sort_bags_default() && indices_numel >= (int64_t)SORT_MIN_LOOKUPS) {
-    HIP_TRY(launch_bag_order(d_offsets, offset_bits == 64, B, plan->T, w.d_order[order_slot], stream));
+    if (!reuse_order) HIP_TRY(launch_bag_order(d_offsets, offset_bits == 64, B, plan->T, w.d_order[order_slot], stream));
     a.order = w.d_order[order_slot];
   }
-  if (prof_begin) HIP_TRY(hipEventRecord(prof_begin, stream));
   // Tables for both kernels, and a forward long enough not to notice two events (the size from
   // which the bags are ordered): the general kernel runs on the slot's side stream, beside the
   // lean one, forked off behind the scheduler and joined before the forward's stream goes on.
@@ -1380,7 +1344,6 @@ int tbe_forward_impl(
     if (side) HIP_TRY(hipStreamWaitEvent(stream, w.side_join[order_slot], 0));
     else HIP_TRY(launch_lookup(a, index_bits == 64, stream));
   }
-  if (prof_end) HIP_TRY(hipEventRecord(prof_end, stream));
   return 0;
 }
 } // namespace
@@ -1562,31 +1525,10 @@ int fbgemm_amd_tbe_forward_nobag(
   return 0;
 }
 
-int fbgemm_amd_tbe_plan_profile(fbgemm_amd_tbe_plan* plan, int32_t slots) {
-  if (!plan || slots < 0) return fail(FBGEMM_AMD_E_ARG, "bad profile arguments");
+int fbgemm_amd_tbe_plan_reuse_order(fbgemm_amd_tbe_plan* plan, int32_t on) {
+  if (!plan) return fail(FBGEMM_AMD_E_ARG, "plan is null");
   std::lock_guard<std::mutex> lk(plan->mu);
-  for (hipEvent_t e : plan->prof_ev) (void)hipEventDestroy(e);
-  plan->prof_ev.clear();
-  plan->prof_count = 0;
-  for (int i = 0; i < 2 * slots; ++i) {
-    hipEvent_t e;
-    HIP_TRY(hipEventCreate(&e));
-    plan->prof_ev.push_back(e);
-  }
-  return 0;
-}
-
-int fbgemm_amd_tbe_plan_profile_read(fbgemm_amd_tbe_plan* plan, float* ms, int32_t cap, int32_t* n) {
-  if (!plan || !ms || !n || cap < 0) return fail(FBGEMM_AMD_E_ARG, "bad profile arguments");
-  std::lock_guard<std::mutex> lk(plan->mu);
-  const int64_t slots = (int64_t)plan->prof_ev.size() / 2;
-  const int64_t have = std::min<int64_t>(std::min<int64_t>(plan->prof_count, slots), cap);
-  for (int64_t i = 0; i < have; ++i) {
-    HIP_TRY(hipEventSynchronize(plan->prof_ev[2 * i + 1]));
-    HIP_TRY(hipEventElapsedTime(&ms[i], plan->prof_ev[2 * i], plan->prof_ev[2 * i + 1]));
-  }
-  *n = (int32_t)have;
-  plan->prof_count = 0;
+  plan->reuse_order = on != 0;
   return 0;
 }
 

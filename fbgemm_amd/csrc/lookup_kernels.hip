@@ -1,5 +1,5 @@
 // gfx950 kernels around the pooled lookup: the bag scheduler, lengths ->
-// offsets, the status block, pruned_array_lookup, the calibration copy, and
+// offsets, the status block, pruned_array_lookup, and
 // the launchers the C ABI calls. The lookup kernels themselves are in
 // lookup_general.h (any shape) and compiled one instance per translation unit.
 #include "lookup_device.h"
@@ -142,21 +142,7 @@ __global__ __launch_bounds__(256) void pruned_array_lookup_kernel(
   }
 }
 
-// Plain 16-byte-per-lane copy of a known size: the yardstick hardware byte
-// counters are scaled against.
-__global__ __launch_bounds__(256) void calibration_copy_kernel(const uint4* src, uint4* dst, int64_t n16) {
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (int64_t)gridDim.x * blockDim.x)
-    dst[i] = src[i];
-}
-
 // ---- launchers (called from the C ABI) ---------------------------------------
-
-hipError_t launch_calibration_copy(const void* src, void* dst, int64_t bytes, hipStream_t stream) {
-  const int64_t n16 = bytes / 16;
-  if (n16 <= 0) return hipSuccess;
-  hipLaunchKernelGGL(calibration_copy_kernel, dim3(256 * 16), dim3(256), 0, stream, (const uint4*)src, (uint4*)dst, n16);
-  return hipGetLastError();
-}
 
 hipError_t launch_lookup_i64(const LookupArgs& a, unsigned blocks, hipStream_t stream);
 hipError_t launch_lookup_i32(const LookupArgs& a, unsigned blocks, hipStream_t stream);

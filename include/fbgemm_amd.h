@@ -302,16 +302,6 @@ int fbgemm_amd_tbe_forward_nobag(
     int64_t indices_numel, int64_t offsets_numel, int32_t D, int32_t output_ty,
     void* d_output, void* d_status, void* stream);
 
-/* Timing of the lookup kernel alone (without the bag scheduler that runs
- * before it), for benchmarks: after fbgemm_amd_tbe_plan_profile(plan, slots)
- * every forward of the plan records a HIP event on its stream before and
- * after the lookup kernel, into a ring of `slots` pairs (0 switches it off).
- * fbgemm_amd_tbe_plan_profile_read waits for the recorded forwards, writes
- * their durations in milliseconds (at most `cap`, at most `slots`) and
- * restarts the ring. No counterpart in the reference. */
-int fbgemm_amd_tbe_plan_profile(fbgemm_amd_tbe_plan* plan, int32_t slots);
-int fbgemm_amd_tbe_plan_profile_read(fbgemm_amd_tbe_plan* plan, float* ms, int32_t cap, int32_t* n);
-
 /* Rows the plan inferred for table t (what an index is checked against). */
 int64_t fbgemm_amd_tbe_plan_num_rows(const fbgemm_amd_tbe_plan* plan, int32_t t);
 /* Padded row bytes of table t. */
@@ -503,39 +493,6 @@ int fbgemm_amd_rowwise_prune_gather(const void* d_weights, int64_t rows, int64_t
 /* Wait for everything enqueued on `stream` (hipStreamSynchronize), for callers
  * of the asynchronous entry points that hold no HIP headers. */
 int fbgemm_amd_stream_synchronize(void* stream);
-
-/* ---- measurement aid -------------------------------------------------------- *
- * No counterpart in the reference. A plain device-to-device copy of `bytes`
- * (a multiple of 16) by a kernel named calibration_copy_kernel: profiles scale
- * the hardware byte counters of the lookup kernel against what the same
- * counters read for this copy of known size. */
-int fbgemm_amd_calibration_copy(const void* d_src, void* d_dst, int64_t bytes, void* stream);
-
-/* Two more yardsticks (no counterpart in the reference, not on the product path):
- * what this GPU sustains for the access patterns a pooled lookup is made of.
- * _stream_read: every lane reads 16 bytes per load, 8 loads in flight, through
- *   `bytes` of d_src once (kernel stream_read_kernel); d_sink: 8192 dwords.
- * _gather: `n` rows d_rows[i] (int32, each < rows) of a table whose rows are
- *   row_stride bytes apart; lanes_per_row consecutive lanes read 16 bytes each
- *   from byte_offset on (4 = what rows with a 4-byte header in front of their
- *   data give: loads at 4-byte alignment), 8 rows per lane group in flight, as
- *   the lookup kernels do (kernel gather_lines_kernel, `waves` workgroups of one
- *   wave each); d_sink: `waves` dwords. */
-int fbgemm_amd_ceiling_stream_read(const void* d_src, int64_t bytes, void* d_sink, void* stream);
-int fbgemm_amd_ceiling_gather(const void* d_table, int64_t rows, int64_t row_stride, int32_t lanes_per_row,
-                              int32_t byte_offset, const int32_t* d_rows, int64_t n, void* d_sink, int32_t waves,
-                              void* stream);
-
-/* Process-wide switches for A/B measurements and tests (no counterpart in the
- * reference; results are bit-identical under every setting of both).
- * fbgemm_amd_set_lean: 1 = shapes the lean kernel takes go to it (the default,
- * also FBGEMM_AMD_LEAN in the environment at load time), 0 = everything goes
- * through the general kernel, -1 = back to the default.
- * fbgemm_amd_set_narrow_below_waves: launches of fewer waves than this take
- * 4-byte lanes (default 1024, FBGEMM_AMD_NARROW_BELOW_WAVES at load time; -1 =
- * back to the default). */
-int fbgemm_amd_set_lean(int32_t on);
-int fbgemm_amd_set_narrow_below_waves(int32_t waves);
 
 /* ---- row-size arithmetic (host, no GPU) ------------------------------------ *
  * embedding_common.h:189-225. */

@@ -1,6 +1,7 @@
 """CPU-side checks of the boundary: the shared library loads without a GPU and
-exports every entry point include/fbgemm_amd.h declares; the host-only helpers
-agree with the oracle; the Python face refuses CPU tensors instead of
+exports every entry point include/fbgemm_amd.h declares (the benchmark-only
+header include/fbgemm_amd_bench.h likewise, in its two libraries); the host-only
+helpers agree with the oracle; the Python face refuses CPU tensors instead of
 falling back."""
 import ctypes
 import os
@@ -12,8 +13,8 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def declared_functions():
-    text = open(os.path.join(ROOT, "include", "fbgemm_amd.h")).read()
+def declared_functions(header="fbgemm_amd.h"):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(fbgemm_amd_[a-z0-9_]+)\s*\(", text)))
 
@@ -31,6 +32,28 @@ def test_library_exports_every_declared_symbol():
     # and the Python binding table covers the same set
     assert sorted(fbgemm_amd.SYMBOLS) == names
     fbgemm_amd.lib()
+
+
+def test_bench_header_matches_its_two_libraries():
+    """include/fbgemm_amd_bench.h: fbgemm_amd_bench_* come from libfbgemm_amd_bench.so, the
+    switches from the product library; nothing of it is declared in the drop-in header, and the
+    product library exports no yardstick."""
+    from fbgemm_amd import _lib
+    if not os.path.exists(_lib.BENCH_LIB_PATH):
+        from fbgemm_amd import build
+        build.build_bench_library()
+    names = declared_functions("fbgemm_amd_bench.h")
+    yard = [n for n in names if n.startswith("fbgemm_amd_bench_")]
+    switches = [n for n in names if not n.startswith("fbgemm_amd_bench_")]
+    assert sorted(_lib.BENCH_SYMBOLS) == yard and sorted(_lib.BENCH_SWITCHES) == switches
+    bench = ctypes.CDLL(_lib.BENCH_LIB_PATH)
+    main = ctypes.CDLL(_lib.LIB_PATH)
+    for n in yard:
+        assert hasattr(bench, n) and not hasattr(main, n), n
+    for n in switches:
+        assert hasattr(main, n), n
+    assert not set(names) & set(declared_functions())
+    _lib.bench_lib()
 
 
 def test_row_size_helpers_match_oracle(oracle):

@@ -18,7 +18,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 def test_cpp_factories_against_oracle():
     exe = os.path.join(ROOT, "tests", "cpp", "_build", "test_factories")
-    assert os.path.exists(exe), "build it with `python -m fbgemm_amd.build`"
+    assert os.path.exists(exe), "build it with `python tests/cpp/build_cpp_tests.py`"
     proc = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
     print(proc.stdout[-3000:])
     assert proc.returncode == 0 and "PASSED" in proc.stdout
