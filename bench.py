@@ -740,34 +740,6 @@ def sample_tables(p):
     return sorted(set(seen.values()) | {0, p.T // 2, p.T - 1})
 
 
-def ordered(bits16):
-    """16-bit float patterns as integers in value order (so that neighbours differ by one)."""
-    import numpy as np
-    b = bits16.astype(np.int32)
-    return np.where(b & 0x8000, -(b & 0x7fff), b)
-
-
-def within_grade(got, want, out_ty, np):
-    """Tolerance-grade comparison: fp32 within 1e-5 of the larger of |want| and the largest
-    magnitude in the bag's block (a sum that cancels to near zero is held to the size of what
-    was summed); fp16 / bf16 within one unit in the last place, or within that same 1e-5 of
-    the block's magnitude. Returns (ok, worst)."""
-    if out_ty == 0:
-        g, w = got.astype(np.float64), want.astype(np.float64)
-    elif out_ty == 1:
-        g, w = got.view(np.float16).astype(np.float64), want.view(np.float16).astype(np.float64)
-    else:
-        g = (got.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
-        w = (want.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
-    scale = np.maximum(np.abs(w), np.abs(w).max(axis=1, keepdims=True))
-    rel = np.where(np.isfinite(w), np.abs(g - w) / np.maximum(scale, 1e-30), 0.0)
-    if out_ty == 0:
-        return bool((rel <= 1e-5).all()), float(rel.max(initial=0.0))
-    d = np.abs(ordered(got) - ordered(want))
-    d = np.where(rel <= 1e-5, np.minimum(d, 1), d)
-    return bool((d <= 1).all()), int(d.max(initial=0))
-
-
 def parity_gate(p, out, launch, torch, np, accumulate="exact"):
     """One forward, then the sampled tables' blocks of its output against the
     oracle on the same inputs: bit for bit (exact), or to the stated tolerance
@@ -775,8 +747,9 @@ def parity_gate(p, out, launch, torch, np, accumulate="exact"):
     import oracle
     launch()
     torch.cuda.synchronize()
+    from fbgemm_amd import tolerance
     tables = sample_tables(p)
-    worst = 0
+    worst, worst_block, needed, cancels = 0, 0.0, 0, 0
     for t in tables:
         s, e = int(p.host_offsets[t * p.B]), int(p.host_offsets[(t + 1) * p.B])
         elem = 4 if int(p.tys[t]) == 0 else 2 if int(p.tys[t]) == 1 else 1
@@ -791,13 +764,15 @@ def parity_gate(p, out, launch, torch, np, accumulate="exact"):
         if accumulate == "exact":
             same = ok and (got.reshape(-1).view(want.dtype) == want).all()
         else:
-            same, w = within_grade(got.reshape(p.B, -1), want.reshape(p.B, -1), p.output_dtype, np)
-            worst = max(worst, w)
-            same = ok and same
+            r = tolerance.grade(got.reshape(p.B, -1), want.reshape(p.B, -1), p.output_dtype, np)
+            worst, worst_block = max(worst, r["worst"]), max(worst_block, r["worst_block"])
+            needed, cancels = needed + r["needed_block_clause"], cancels + r["cancellations"]
+            same = ok and r["ok"]
         if not same:
             raise AssertionError(f"parity gate: table {t} of {p.name} differs from the oracle; nothing was timed")
     how = "bit for bit" if accumulate == "exact" else (
-        f"to tolerance (worst: {worst} {'units in the last place' if p.output_dtype else 'relative'})")
+        f"to tolerance (worst element-wise: {worst} {'units in the last place' if p.output_dtype else 'relative'}; "
+        f"{needed} of {cancels} cancellations needed the block-relative clause, worst {worst_block:.3g} of the block)")
     print(f"parity gate: tables {tables} of {p.name} match the oracle {how}", file=sys.stderr)
     return tables
 

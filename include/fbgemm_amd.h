@@ -120,10 +120,16 @@ typedef struct fbgemm_amd_spmdm_config {
  *   element, out = acc + sum of the biases: a third fewer vector instructions
  *   per 4-bit element. Same index order, one lane per output column, so results
  *   are deterministic and differ from the reference's by a few fp32 roundings of
- *   the partial sums (tests hold it to 1e-5 of the bag's sum of magnitudes for
- *   fp32 output and to one unit in the last place of fp16 / bf16 output).
+ *   the partial sums (tests hold every element that is not a cancellation to
+ *   1e-5 relative for fp32 output and to one unit in the last place of fp16 /
+ *   bf16 output). A call of few, long bags (fewer than 256 waves, 32 rows per
+ *   bag and more) over such rows is cut into segments whose fp32 partial sums
+ *   are added in order afterwards: still deterministic, another association of
+ *   the same sum.
  * Rows the lean kernel does not take (odd widths, 2-bit, fp32, ...) and fp16 /
- * bf16 / fp32 / fp8 rows are computed the EXACT way in either mode. */
+ * bf16 / fp32 / fp8 rows are computed the EXACT way in either mode, never in
+ * segments: a table-batched plan cuts bags only when every one of its tables
+ * has 4- or 8-bit rows of a lean shape. */
 enum { FBGEMM_AMD_ACC_EXACT = 0, FBGEMM_AMD_ACC_FAST = 1 };
 
 /* Enqueue one pooled lookup. d_weights may be NULL (unweighted).
@@ -145,7 +151,10 @@ int fbgemm_amd_spmdm_launch(
 /* fbgemm_amd_spmdm_launch for callers that cannot allocate device memory (code
  * under HIP graph capture, tight serving loops, harnesses that forbid
  * hipMalloc). It has no counterpart in the reference. Same arguments, same
- * kernels, same results bit for bit; the two pieces of scratch the call above
+ * kernels; the same results bit for bit with FBGEMM_AMD_ACC_EXACT, and with
+ * FBGEMM_AMD_ACC_FAST whenever the call above does not cut the bags into
+ * segments (this entry point never does: the segments' partial sums need
+ * scratch of a size it has no place for). The two pieces of scratch the call above
  * takes from hipMalloc'ed buffers (the prefix sum of the lengths when
  * use_offsets == 0, and the bag order of the scheduler for calls of 2^21
  * lookups and more) live in a static device array of the library instead

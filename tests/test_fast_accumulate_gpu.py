@@ -3,13 +3,13 @@
 In this mode the biases of a bag are summed apart from the scaled elements and
 bags of a launch too small to fill the device are cut into segments whose
 partial sums are added afterwards, so the fp32 roundings are not the
-reference's. The stated bound of the path: fp32 output within 1e-5 relative,
-fp16 / bf16 output within one unit in the last place. "Relative" is taken
-against the larger of |expected| and the largest magnitude in the bag's output
-row: a sum that cancels to nearly zero is held to the size of what was summed
-(for 16-bit outputs too: an element a thousand times smaller than its row may
-be off by more than one of ITS last places and still within 1e-5 of the row).
-Each test prints the worst error it met. The default mode stays bit-exact and
+reference's. The stated bound of the path, element by element: fp32 output
+within 1e-5 relative, fp16 / bf16 output within one unit in the last place.
+Every element that is not a cancellation (|expected| at least 2^-10 of the
+largest magnitude in the bag's block of the output) is held to exactly that;
+an element below it may instead be within 1e-5 of the block's magnitude
+(fbgemm_amd/tolerance.py). Each test prints the worst error it met and how
+many elements needed the second clause. The default mode stays bit-exact and
 is what every other test file checks."""
 import numpy as np
 import pytest
@@ -44,37 +44,29 @@ def cu(a):
     return torch.from_numpy(np.ascontiguousarray(a)).cuda()
 
 
-def ordered(bits16):
-    b = bits16.astype(np.int32)
-    return np.where(b & 0x8000, -(b & 0x7fff), b)
-
-
-def as_float(bits16, out_ty):
-    if out_ty == FP16:
-        return bits16.view(np.float16).astype(np.float64)
-    return (bits16.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+NEEDED_BLOCK_CLAUSE = {"elements": 0, "cancellations": 0, "needed": 0}
 
 
 def check_grade(got, want, out_ty, rows, what):
-    """got / want: fp32 arrays or uint16 bit patterns, reshaped to [rows, -1]. fp32: within 1e-5 of
-    the larger of |want| and the largest magnitude of the bag's row. fp16 / bf16: within one unit
-    in the last place, or (elements that nearly cancel) within that same 1e-5 of the row's
-    magnitude. Returns the worst error: relative (fp32) or units in the last place."""
-    got, want = got.reshape(rows, -1), want.reshape(rows, -1)
-    if out_ty == FP32:
-        g, w = got.astype(np.float64), want.astype(np.float64)
-    else:
-        g, w = as_float(got, out_ty), as_float(want, out_ty)
-    scale = np.maximum(np.abs(w), np.abs(w).max(axis=1, keepdims=True))
-    rel = np.where(np.isfinite(w), np.abs(g - w) / np.maximum(scale, 1e-30), 0.0)
-    if out_ty == FP32:
-        worst = float(rel.max(initial=0.0))
-        assert worst <= 1e-5, f"{what}: relative error {worst:.3g} exceeds 1e-5"
-        return worst
-    d = np.where(rel <= 1e-5, np.minimum(np.abs(ordered(got) - ordered(want)), 1), np.abs(ordered(got) - ordered(want)))
-    worst = int(d.max(initial=0))
-    assert worst <= 1, f"{what}: {worst} units in the last place"
-    return worst
+    """got / want: fp32 arrays or uint16 bit patterns, reshaped to [rows, -1] (one table's block per
+    row). Asserts the bound of fbgemm_amd/tolerance.py and returns the worst element-wise error:
+    relative (fp32) or units in the last place."""
+    from fbgemm_amd import tolerance
+    r = tolerance.grade(got.reshape(rows, -1), want.reshape(rows, -1), out_ty, np)
+    NEEDED_BLOCK_CLAUSE["elements"] += r["elements"]
+    NEEDED_BLOCK_CLAUSE["cancellations"] += r["cancellations"]
+    NEEDED_BLOCK_CLAUSE["needed"] += r["needed_block_clause"]
+    unit = "relative" if out_ty == FP32 else "units in the last place"
+    assert r["ok"], (f"{what}: worst element-wise error {r['worst']:.3g} {unit}; {r['needed_block_clause']} of "
+                     f"{r['cancellations']} cancellations needed the block clause, worst {r['worst_block']:.3g} of the block")
+    return r["worst"]
+
+
+@pytest.fixture(scope="module", autouse=True)
+def report_block_clause():
+    yield
+    print(f"\ntolerance grade: {NEEDED_BLOCK_CLAUSE['needed']} of {NEEDED_BLOCK_CLAUSE['elements']} elements "
+          f"({NEEDED_BLOCK_CLAUSE['cancellations']} cancellations) needed the block-relative clause")
 
 
 def bits_of(t, out_ty):
@@ -178,6 +170,36 @@ def test_table_batched_fast_mode(ops, oracle, B, max_L):
                         c0, c1 = int(D_offsets[t]), int(D_offsets[t + 1])
                         check_grade(np.ascontiguousarray(g[:, c0:c1]), np.ascontiguousarray(want.reshape(B, total_D)[:, c0:c1]), out_ty, B,
                                     f"B={B} L<{max_L} align={row_alignment} w={weighted} pool={pooling} out={out_ty} table={t}")
+
+
+@pytest.mark.parametrize("ty", [FP16, FP32, INT2])
+def test_rows_without_fast_arithmetic_stay_exact_with_long_bags(ops, oracle, ty):
+    """fp16 / fp32 / 2-bit rows are summed the reference's way in either mode. A call of few, long
+    bags over them is not cut into segments either (4- and 8-bit rows of such a call are): the
+    results stay bit-identical, for a single table and for a plan that holds one such table."""
+    rng = np.random.default_rng(77 + ty)
+    nb, rows, D, L = 3, 900, 128, 400
+    table, _ = H.make_table(rng, ty, rows, D, False)
+    idx, off, _ = H.make_bags(rng, rows, nb, L, np.int64, np.int32, fixed_len=L)
+    kern = (ops.generate_embedding_spmdm_nbit_with_strides(2, D, False, False, 16, False, True, -1, -1, False) if ty == INT2 else
+            ops.generate_embedding_spmdm_with_strides(ty, D, False, False, 16, False, True, -1, -1, False))
+    out = torch.empty(nb * D, dtype=torch.float32, device="cuda")
+    assert kern(nb, len(idx), rows, cu(table), cu(idx), cu(off), None, out, accumulate=ops.ACC_FAST)
+    ok, want = oracle.spmdm(ty, D, table, idx, off, scale_bias_last=False, data_size=rows)
+    assert ok
+    H.assert_same_bits(out.cpu().numpy(), want, f"single table ty={ty}, fast mode, long bags")
+    # the same kind of table beside 4-bit ones in a plan: no table of the plan is cut into segments
+    specs = [(500, 128, INT4), (300, D, ty), (400, 256, INT4)]
+    weights, wo, tys, D_offsets, idx, off, _ = tbe_problem(rng, specs, 2, 900, 16, False)
+    T, total_D = len(specs), int(D_offsets[-1])
+    got = ops.int_nbit_split_embedding_codegen_lookup_function(
+        cu(weights), torch.zeros(0, dtype=torch.uint8, device="cuda"), cu(np.zeros(T, np.int32)), cu(wo), cu(tys),
+        cu(D_offsets), total_D, 128, 256, 0, 128, 128, cu(idx), cu(off), 0, None, FP32, row_alignment=16, accumulate=ops.ACC_FAST)
+    rc, want = oracle.tbe_forward(weights, wo, tys, D_offsets, total_D, idx, off, 0, None, FP32, 16)
+    assert rc == 0
+    c0, c1 = int(D_offsets[1]), int(D_offsets[2])
+    H.assert_same_bits(np.ascontiguousarray(got.cpu().numpy()[:, c0:c1]), np.ascontiguousarray(want.reshape(2, total_D)[:, c0:c1]),
+                       f"table of ty={ty} in a fast-mode plan, long bags")
 
 
 def test_rebuilding_rank_records_leaves_the_split_bag_scratch_alone(ops, oracle):
