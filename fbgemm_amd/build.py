@@ -16,7 +16,7 @@ SOURCES = ["lookup_lean_i64_exact.hip", "lookup_lean_i64_fast.hip", "lookup_lean
            "lookup_i64.hip", "lookup_i32.hip", "lookup_i64_general.hip", "lookup_i32_general.hip",
            "lookup_kernels.hip", "index_ops_kernels.hip", "quantize_kernels.hip", "sequence_kernels.hip",
            "prune_kernels.hip", "remap_rank_kernels.hip", "split_bag_kernels.hip", "update_kernels.hip", "c_api.cpp"]
-HEADERS = ["cache_policy.h", "lookup_common.h", "lookup_device.h", "lookup_general.h", "lookup_lean.h", os.path.join("..", "..", "include", "fbgemm_amd.h"),
+HEADERS = ["cache_policy.h", "launchers.h", "lookup_common.h", "lookup_device.h", "lookup_general.h", "lookup_lean.h", os.path.join("..", "..", "include", "fbgemm_amd.h"),
            os.path.join("..", "..", "include", "fbgemm_amd_bench.h")]
 
 # -ffp-contract=off: the kernels spell out every fma; nothing else may be fused,
