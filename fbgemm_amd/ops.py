@@ -277,7 +277,7 @@ def _plan_for(dev_weights, uvm_weights, weights_placements, weights_offsets, wei
     # host copy a plan needs is made once per distinct set of tensors.
     key = (weights_offsets.data_ptr(), weights_tys.data_ptr(), D_offsets.data_ptr(),
            weights_placements.data_ptr(), weights_offsets._version, D_offsets._version,
-           weights_tys._version, D_offsets.numel(), dev_weights.numel(), uvm_weights.numel(),
+           weights_tys._version, weights_placements._version, D_offsets.numel(), dev_weights.numel(), uvm_weights.numel(),
            row_alignment)
     entry = _plans.get(key)
     if entry is None:
@@ -386,8 +386,15 @@ def int_nbit_split_embedding_codegen_lookup_function(
         ro = index_remappings_offsets.to(torch.int64).contiguous()
         # the compact form of order-preserving mappings, made once per array and offsets (and again when either changes)
         key = TbePlan.rank_key(index_remappings, index_remappings_offsets)
-        if getattr(plan, "_rank_key", None) != key and not torch.cuda.is_current_stream_capturing():
-            plan.set_index_remappings(index_remappings, index_remappings_offsets)
+        if getattr(plan, "_rank_key", None) != key:
+            if torch.cuda.is_current_stream_capturing():
+                # building the compact form allocates and synchronizes; and a mapping edited in place keeps its
+                # address, so the forward would take the records made from the old contents into the graph
+                if getattr(plan, "_rank_key", None) is not None:
+                    raise RuntimeError("the pruned-row mappings changed since the plan's compact form of them was made: "
+                                       "run one forward outside the stream capture after changing them")
+            else:
+                plan.set_index_remappings(index_remappings, index_remappings_offsets)
     check(_lib.lib().fbgemm_amd_tbe_forward_pruned(
         plan.handle, _ptr(dev_weights), _ptr(uvm_weights), _ptr(indices.contiguous()),
         _ptr(offsets.contiguous()), _bits(indices), indices.numel(), offsets.numel(), pooling_mode,

@@ -102,3 +102,117 @@ def test_forward_replays_from_a_graph(oracle):
     again = call()
     torch.cuda.synchronize()
     H.assert_same_bits(again.cpu().view(torch.int16).numpy().view(np.uint16), want, "eager after trim")
+
+
+def test_forward_with_both_kernels_replays_from_a_graph(oracle):
+    """A forward large enough to order its bags, over tables for both lookup kernels (4-bit rows of a
+    lean shape, and 2-bit / odd-width rows): the general kernel runs on the plan's side stream beside
+    the lean one (event fork and join). Captured, that is a graph with two branches; every replay is
+    checked against the oracle, with eager forwards of the same plan in between."""
+    assert torch.cuda.is_available()
+    from fbgemm_amd import ops
+    from helpers import INT2
+    from test_tbe_gpu import build_weights
+    rng = np.random.default_rng(77)
+    specs = [(3000, 128, INT4), (500, 32, INT2), (2000, 64, INT4), (700, 40, INT4)]
+    T, B, L = len(specs), 4096, 130  # 2.13 M lookups: the scheduler runs, and with it the side stream
+    weights, wo, _ = build_weights(rng, specs, 16)
+    tys = np.array([s[2] for s in specs], np.uint8)
+    D_offsets = np.concatenate([[0], np.cumsum([s[1] for s in specs])]).astype(np.int32)
+    total_D = int(D_offsets[-1])
+    lens = rng.integers(L - 30, L + 31, size=T * B)
+    lens[-1] += T * B * L - int(lens.sum())
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    n = int(off[-1])
+    assert n >= 1 << 21
+
+    def draw():
+        return np.concatenate([rng.integers(0, specs[t][0], size=int(off[(t + 1) * B] - off[t * B])) for t in range(T)]).astype(np.int64)
+
+    idx = draw()
+    d_idx, d_off = cu(idx), cu(off)
+    meta = (cu(weights), torch.zeros(0, dtype=torch.uint8, device="cuda"), cu(np.zeros(T, np.int32)), cu(wo), cu(tys), cu(D_offsets))
+    st = ops.Status()
+    call = lambda: ops.int_nbit_split_embedding_codegen_lookup_function(
+        *meta, total_D, 32, 128, 0, 0, 0, d_idx, d_off, 0, None, FP16, row_alignment=16, status=st)
+
+    def expect(idx):
+        rc, want = oracle.tbe_forward(weights, wo, tys, D_offsets, total_D, idx, off, 0, None, FP16, 16)
+        assert rc == 0
+        return want
+
+    eager = call()
+    torch.cuda.synchronize()
+    H.assert_same_bits(eager.cpu().view(torch.int16).numpy().view(np.uint16), expect(idx), "eager")
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            captured = call()
+    torch.cuda.synchronize()
+    for replay in range(3):
+        idx = draw()
+        d_idx.copy_(cu(idx))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        H.assert_same_bits(captured.cpu().view(torch.int16).numpy().view(np.uint16), expect(idx), f"replay {replay}")
+        again = call()
+        torch.cuda.synchronize()
+        assert torch.equal(again, captured)
+    assert st.read() == (0, -1)
+
+
+def test_mappings_changed_before_a_capture_are_refused(oracle):
+    """Pruned-row mappings edited in place keep their address: a forward under stream capture cannot
+    rebuild the plan's compact form of them (that allocates and synchronizes) and must not take the
+    old one into the graph. It raises; after one forward outside the capture the capture works."""
+    assert torch.cuda.is_available()
+    from fbgemm_amd import ops
+    from test_tbe_gpu import build_weights
+    rng = np.random.default_rng(5)
+    logical, kept = 400, 250
+    m = np.full(logical, -1, np.int32)
+    m[np.sort(rng.choice(logical, kept, replace=False))] = np.arange(kept, dtype=np.int32)
+    specs = [(kept, 64, INT4)]
+    weights, wo, _ = build_weights(rng, specs, 16)
+    tys, D_offsets = np.array([INT4], np.uint8), np.array([0, 64], np.int32)
+    B, L = 8, 5
+    off = (np.arange(B + 1) * L).astype(np.int64)
+    idx = rng.integers(0, logical, size=B * L).astype(np.int64)
+    d_remap, d_remap_off = cu(m), cu(np.array([0, logical], np.int64))
+    meta = (cu(weights), torch.zeros(0, dtype=torch.uint8, device="cuda"), cu(np.zeros(1, np.int32)), cu(wo), cu(tys), cu(D_offsets))
+    d_idx, d_off = cu(idx), cu(off)
+    call = lambda: ops.int_nbit_split_embedding_codegen_lookup_function(
+        *meta, 64, 0, 64, 0, 0, 0, d_idx, d_off, 0, None, FP16, row_alignment=16,
+        index_remappings=d_remap, index_remappings_offsets=d_remap_off)
+
+    def expect(mapping):
+        dense = oracle.pruned_array_lookup(idx, off, mapping, np.array([0, logical], np.int64))
+        rc, want = oracle.tbe_forward(weights, wo, tys, D_offsets, 64, dense, off, 0, None, FP16, 16)
+        assert rc == 0
+        return want
+
+    H.assert_same_bits(call().cpu().view(torch.int16).numpy().view(np.uint16), expect(m), "first forward")
+    # prune one more row, in place: kept rows behind it move up by one
+    victim = int(np.nonzero(m >= 0)[0][3])
+    m2 = m.copy()
+    m2[victim] = -1
+    m2[m2 > m[victim]] -= 1
+    d_remap.copy_(cu(m2))
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        graph = torch.cuda.CUDAGraph()
+        with pytest.raises(RuntimeError, match="outside the stream capture"):
+            with torch.cuda.graph(graph, stream=side):
+                call()
+    torch.cuda.synchronize()
+    H.assert_same_bits(call().cpu().view(torch.int16).numpy().view(np.uint16), expect(m2), "forward after the change")
+    with torch.cuda.stream(side):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            captured = call()
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    H.assert_same_bits(captured.cpu().view(torch.int16).numpy().view(np.uint16), expect(m2), "replay")

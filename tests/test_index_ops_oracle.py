@@ -217,3 +217,29 @@ def test_library_host_insert_builds_the_oracles_table(idt, hdt):
     rc = _lib.lib().fbgemm_amd_pruned_hashmap_insert_host(
         p(k3), p(k3), p(o3), 8 * k3.itemsize, 2, p(tiny), 8 * tiny.itemsize, p(h3), 1)
     assert rc < 0
+
+
+@pytest.mark.parametrize("idx_dtype,remap_dtype", [(np.int32, np.int32), (np.int64, np.int32), (np.int64, np.int64), (np.int32, np.int64)])
+def test_pruned_array_lookup_is_numpy_indexing(oracle, idx_dtype, remap_dtype):
+    """oracle.pruned_array_lookup against its definition in numpy (embedding_forward_quantized_cpu_template.cpp:605-659):
+    dense[i] = remap[remap_offsets[t] + indices[i]] for the positions of a table that owns a mapping, a copy
+    for a table whose slice of the mapping array is empty (capacity 0: the table is not pruned)."""
+    rng = np.random.default_rng(31)
+    T, B = 5, 7
+    caps = [40, 0, 25, 0, 60]  # tables 1 and 3 are not pruned
+    remap_offsets = np.concatenate([[0], np.cumsum(caps)]).astype(np.int64)
+    remap = np.concatenate([np.where(rng.random(c) < 0.4, -1, rng.integers(0, 1000, size=c)) for c in caps]).astype(remap_dtype)
+    lens = rng.integers(0, 9, size=T * B)
+    offsets = np.concatenate([[0], np.cumsum(lens)]).astype(idx_dtype)
+    indices = np.concatenate([rng.integers(0, caps[t] if caps[t] else 500, size=int(lens[t * B:(t + 1) * B].sum()))
+                              for t in range(T)]).astype(idx_dtype)
+    got = oracle.pruned_array_lookup(indices, offsets, remap, remap_offsets)
+    want = indices.copy()
+    for t in range(T):
+        s, e = int(offsets[t * B]), int(offsets[(t + 1) * B])
+        if caps[t]:
+            want[s:e] = remap[remap_offsets[t] + indices[s:e]].astype(idx_dtype)
+    assert got.dtype == indices.dtype and (got == want).all()
+    # every table unpruned: the identity
+    none = oracle.pruned_array_lookup(indices, offsets, np.zeros(0, remap_dtype), np.zeros(T + 1, np.int64))
+    assert (none == indices).all()
