@@ -183,9 +183,10 @@ def test_mappings_changed_before_a_capture_are_refused(oracle):
     d_remap, d_remap_off = cu(m), cu(np.array([0, logical], np.int64))
     meta = (cu(weights), torch.zeros(0, dtype=torch.uint8, device="cuda"), cu(np.zeros(1, np.int32)), cu(wo), cu(tys), cu(D_offsets))
     d_idx, d_off = cu(idx), cu(off)
+    st = ops.Status()  # read by the test, not by the forward: a forward under capture cannot synchronize
     call = lambda: ops.int_nbit_split_embedding_codegen_lookup_function(
         *meta, 64, 0, 64, 0, 0, 0, d_idx, d_off, 0, None, FP16, row_alignment=16,
-        index_remappings=d_remap, index_remappings_offsets=d_remap_off)
+        index_remappings=d_remap, index_remappings_offsets=d_remap_off, status=st)
 
     def expect(mapping):
         dense = oracle.pruned_array_lookup(idx, off, mapping, np.array([0, logical], np.int64))
@@ -201,12 +202,18 @@ def test_mappings_changed_before_a_capture_are_refused(oracle):
     m2[m2 > m[victim]] -= 1
     d_remap.copy_(cu(m2))
     side = torch.cuda.Stream()
+    refused = None
     with torch.cuda.stream(side):
         graph = torch.cuda.CUDAGraph()
-        with pytest.raises(RuntimeError, match="outside the stream capture"):
-            with torch.cuda.graph(graph, stream=side):
+        with torch.cuda.graph(graph, stream=side):
+            d_off.add_(0)  # something to capture: the refused forward launches nothing
+            try:
                 call()
+            except RuntimeError as e:  # caught inside, so that the capture ends in order
+                refused = str(e)
     torch.cuda.synchronize()
+    assert refused is not None and "outside the stream capture" in refused, refused
+    del graph
     H.assert_same_bits(call().cpu().view(torch.int16).numpy().view(np.uint16), expect(m2), "forward after the change")
     with torch.cuda.stream(side):
         graph = torch.cuda.CUDAGraph()
@@ -216,3 +223,4 @@ def test_mappings_changed_before_a_capture_are_refused(oracle):
     graph.replay()
     torch.cuda.synchronize()
     H.assert_same_bits(captured.cpu().view(torch.int16).numpy().view(np.uint16), expect(m2), "replay")
+    assert st.read() == (0, -1)

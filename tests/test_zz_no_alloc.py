@@ -78,3 +78,55 @@ def test_noalloc_rejects_more_bags_than_its_array_holds():
     p = C.c_void_p(dummy.data_ptr())
     rc = lib.fbgemm_amd_spmdm_launch_noalloc(C.byref(cfg), 65537, 0, 1, p, p, p, None, p, None, p, None)
     assert rc == -1 and b"at most 65536 bags" in lib.fbgemm_amd_last_error()
+
+
+def test_noalloc_allocates_nothing_and_replays_from_a_graph():
+    """What the entry point exists for: after its first call on the device (which asks the runtime
+    for the address of the static array) further calls leave the device's free memory as it is, and
+    a call that uses both pieces of scratch (lengths, and 2^21 lookups for the bag order) can be
+    captured in a HIP graph; every replay gives the bits of the allocating entry point."""
+    import fbgemm_amd
+    from fbgemm_amd._lib import SpmdmConfig
+    lib = fbgemm_amd.lib()
+    rng = np.random.default_rng(9)
+    ty, D, rows, nb, avg = INT4, 128, 150_000, 48_000, 46
+    table, _ = H.make_table(rng, ty, rows, D, True)
+    lens = rng.integers(avg - 4, avg + 5, size=nb).astype(np.int32)
+    n_idx = int(lens.sum())
+    assert n_idx >= 1 << 21
+    cu = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    t_table, t_lens = cu(table), cu(lens)
+    t_idx = cu(rng.integers(0, rows, size=n_idx).astype(np.int64))
+    st = torch.zeros(16, dtype=torch.uint8, device="cuda")
+    cfg = SpmdmConfig(weight_ty=ty, output_ty=FP16, index_bits=64, offset_bits=32, block_size=D, output_stride=-1,
+                      input_stride=-1, normalize_by_lengths=0, is_weight_positional=0, use_offsets=0, scale_bias_last=1)
+    out = torch.full((nb * D,), -7.0, dtype=torch.float16, device="cuda")
+    ref = torch.full((nb * D,), -7.0, dtype=torch.float16, device="cuda")
+    # outside any capture: the first call, which takes the array's device address
+    assert _call(lib, lib.fbgemm_amd_spmdm_launch_noalloc, cfg, nb, n_idx, rows, t_table, t_idx, t_lens, None, out, st) == 0
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    for _ in range(3):
+        assert _call(lib, lib.fbgemm_amd_spmdm_launch_noalloc, cfg, nb, n_idx, rows, t_table, t_idx, t_lens, None, out, st) == 0
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before, "the entry point that allocates nothing changed the device's free memory"
+
+    p = lambda t: C.c_void_p(t.data_ptr())
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+            rc = lib.fbgemm_amd_spmdm_launch_noalloc(C.byref(cfg), nb, n_idx, rows, p(t_table), p(t_idx), p(t_lens), None, p(out),
+                                                     None, p(st), stream)
+            assert rc == 0, lib.fbgemm_amd_last_error().decode()
+    torch.cuda.synchronize()
+    for replay in range(3):
+        t_idx.copy_(cu(rng.integers(0, rows, size=n_idx).astype(np.int64)))
+        out.fill_(-7.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert _call(lib, lib.fbgemm_amd_spmdm_launch, cfg, nb, n_idx, rows, t_table, t_idx, t_lens, None, ref, st) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.int16), ref.view(torch.int16)), f"replay {replay} differs from the allocating entry point"
