@@ -427,12 +427,15 @@ def gather_ceiling(a):
         tb = int((gib << 30) * a.scale)
         rows = tb // 128
         uni = torch.randint(0, rows, (n,), dtype=torch.int32, device="cuda", generator=gen)
-        rec = gather_case("uniform random 128-byte lines (aligned)", tb, 128, 8, 0, uni, modes[0])
-        if gib == max(sizes):
-            headline = rec
+        if a.ceiling_index in ("uniform", "both"):
+            rec = gather_case("uniform random 128-byte lines (aligned)", tb, 128, 8, 0, uni, modes[0])
+            if gib == max(sizes):
+                headline = rec
         if a.ceiling_index in ("zipf", "both"):
-            gather_case("Zipf(1.1) 128-byte lines (aligned)", tb, 128, 8, 0, zipf_rows(rows), modes[0])
-        if gib == max(sizes):
+            rec = gather_case("Zipf(1.1) 128-byte lines (aligned)", tb, 128, 8, 0, zipf_rows(rows), modes[0])
+            if gib == max(sizes) and headline is None:
+                headline = rec
+        if gib == max(sizes) and a.ceiling_index != "zipf":
             gather_case("uniform random 128-byte lines (aligned)", tb, 128, 8, 0, uni, modes[1])
             gather_case("uniform random 128-byte lines (aligned)", tb, 128, 8, 0, uni, modes[2])
         del uni

@@ -25,8 +25,11 @@ echo "pass: kernel trace ($(date +%T))"
 timeout -k 10 900 rocprofv3 --kernel-trace --stats --output-format csv -d $RAW/trace -o t -- $BENCH --steps 20 --warmup 3 > $RAW/trace.log 2>&1 || { echo "trace run failed" | tee -a "$OUT"; tail -5 $RAW/trace.log; exit 1; }
 grep '^{' $RAW/trace.log | tail -1 | cut -c1-3000 >> "$OUT"
 python3 profile_summary.py $RAW/trace | grep -v '^#' >> "$OUT"
-# PROFILE_SHORT=1 keeps the byte counters only (for workloads whose set-up takes minutes)
-if [ -n "$PROFILE_SHORT" ]; then
+# PROFILE_SHORT=1 keeps the byte counters only (for workloads whose set-up takes minutes);
+# PROFILE_PASSES="A B;C" names the passes (counters of a pass separated by blanks, passes by semicolons)
+if [ -n "$PROFILE_PASSES" ]; then
+  IFS=';' read -r -a PASSES <<< "$PROFILE_PASSES"
+elif [ -n "$PROFILE_SHORT" ]; then
   PASSES=("FETCH_SIZE" "WRITE_SIZE" "TCC_HIT_sum TCC_MISS_sum" "GRBM_GUI_ACTIVE")
 else
   PASSES=("FETCH_SIZE" "WRITE_SIZE" "TCC_HIT_sum TCC_MISS_sum" "TCC_EA0_RDREQ_sum"
@@ -41,6 +44,6 @@ for pass in "${PASSES[@]}"; do
   timeout -s KILL 600 rocprofv3 --pmc $pass --output-format csv -d $RAW/pmc_$n -o p -- $BENCH --steps 3 --warmup 1 > $RAW/pmc_$n.log 2>&1 || { echo "pass failed: $pass" >> "$OUT"; tail -3 $RAW/pmc_$n.log >> "$OUT"; exit 1; }
   python3 profile_summary.py $RAW/pmc_$n | grep -v '^#\|^launch' >> "$OUT"
 done
-python3 profile_summary.py $RAW/pmc_GRBM_GUI_ACTIVE | grep '^launch' >> "$OUT"
+[ -d $RAW/pmc_GRBM_GUI_ACTIVE ] && python3 profile_summary.py $RAW/pmc_GRBM_GUI_ACTIVE | grep '^launch' >> "$OUT"
 rm -rf $RAW
 echo "summary written to $OUT"
