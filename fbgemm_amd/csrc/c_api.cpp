@@ -496,11 +496,11 @@ int spmdm_launch_impl(
   }
   plan_lanes(d, (uintptr_t)d_input, out_stride, has_sb, false);
   // few, long bags, and the caller accepts sums in another order: cut every bag into K segments.
-  // Only rows the tolerance-grade arithmetic applies to: every other row type is summed the
-  // reference's way in either mode, and stays so.
+  // 4- and 8-bit rows only: every other row type is summed the reference's way in either mode,
+  // in one piece.
   int K = 1;
   if (!noalloc && cfg->accumulate == FBGEMM_AMD_ACC_FAST && !cfg->is_weight_positional && output_size * 32 <= 0x7fffffffLL &&
-      (ty == ST_INT4 || ty == ST_INT8) && lean_enabled() && lean_shape(d)) {
+      (ty == ST_INT4 || ty == ST_INT8)) {
     const int G16 = bags_per_wave(d.lanes, d.packed);
     K = split_factor((output_size + G16 - 1) / G16, index_size / output_size);
   }
@@ -1070,8 +1070,8 @@ int tbe_forward_impl(
   // (Only when every table has rows the tolerance-grade arithmetic applies to: fp16 / fp32 / 2-bit
   // / odd-shaped tables are summed the reference's way in either mode, and a bag cut into
   // segments is not.)
-  bool all_fast_rows = lean_enabled();
-  for (const TableDesc& d : plan->tables) all_fast_rows = all_fast_rows && (d.ty == ST_INT4 || d.ty == ST_INT8) && lean_shape(d);
+  bool all_fast_rows = true;
+  for (const TableDesc& d : plan->tables) all_fast_rows = all_fast_rows && (d.ty == ST_INT4 || d.ty == ST_INT8);
   if (allow_split && plan->accumulate == FBGEMM_AMD_ACC_FAST && all_fast_rows && (int64_t)B * 32 <= 0x7fffffffLL) {
     int64_t wide_waves = 0;
     for (const TableDesc& d : plan->tables) wide_waves += (B + d.bags - 1) / d.bags;

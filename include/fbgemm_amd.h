@@ -126,10 +126,12 @@ typedef struct fbgemm_amd_spmdm_config {
  *   bag and more) over such rows is cut into segments whose fp32 partial sums
  *   are added in order afterwards: still deterministic, another association of
  *   the same sum.
- * Rows the lean kernel does not take (odd widths, 2-bit, fp32, ...) and fp16 /
- * bf16 / fp32 / fp8 rows are computed the EXACT way in either mode, never in
- * segments: a table-batched plan cuts bags only when every one of its tables
- * has 4- or 8-bit rows of a lean shape. */
+ * Only 4- and 8-bit rows of the regular shapes (whole 16-byte chunks, 32
+ * columns per lane) have the FAST arithmetic; 4- and 8-bit rows of other widths
+ * are summed the EXACT way inside a segment but may still be cut into segments.
+ * 2-bit, fp16 / bf16 / fp32 / fp8 rows are computed the EXACT way in either
+ * mode and never in segments: a table-batched plan cuts bags only when every
+ * one of its tables has 4- or 8-bit rows. */
 enum { FBGEMM_AMD_ACC_EXACT = 0, FBGEMM_AMD_ACC_FAST = 1 };
 
 /* Enqueue one pooled lookup. d_weights may be NULL (unweighted).

@@ -9,7 +9,7 @@ CFG=${1:-3}; OUT=${2:-profile_summary.txt}; shift; shift
 export TMPDIR=/tmp
 RAW=$(mktemp -d /tmp/fbgemm_amd_prof.XXXXXX)
 mkdir -p "$(dirname "$OUT")"
-BENCH="python3 bench.py --config $CFG --no-cpu --no-also --one-mode --no-check --calibration-copy-mib 1024 $*"
+BENCH="python3 bench.py --config $CFG --no-cpu --no-also --one-mode --no-check --clock-warmup-s 0 --calibration-copy-mib 1024 $*"
 {
   echo "# rocprofv3 summary, bench.py --config $CFG $*"
   echo "# commands (each its own run):"
