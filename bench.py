@@ -61,6 +61,10 @@ def parse():
                          "prints it under \"other_accumulate\" (--one-mode skips that)")
     ap.add_argument("--one-mode", "--no-exact", dest="other_mode", action="store_false",
                     help="do not also time the other accumulate mode")
+    ap.add_argument("--int8-output", action="store_true",
+                    help="table-batched configurations: the operator's 8-bit pooled output ([B, total_D + 8 T]: every table's "
+                         "pooled vector quantized row-wise in the lookup's output stage) instead of the configuration's float "
+                         "output; needs --no-check --one-mode (the tests hold that output to the oracles, the gate here does not)")
     ap.add_argument("--no-rank-records", action="store_true",
                     help="config 4 only: read the int32 mapping arrays in the forward instead of the compact "
                          "bitmap-and-rank form of the (order-preserving) mappings")
@@ -127,7 +131,7 @@ def profile_kernel_us(config_id):
     return round(sum(ns) / 1e3, 2) if ns else None
 
 
-def tbe_runner(p, torch, accumulate="exact", rank_records=True):
+def tbe_runner(p, torch, accumulate="exact", rank_records=True, int8_output=False):
     """Returns (launch, out, status, plan) for a TbeProblem: launch() enqueues one forward."""
     from fbgemm_amd import _lib, ops
 
@@ -138,13 +142,15 @@ def tbe_runner(p, torch, accumulate="exact", rank_records=True):
     _lib.check(lib.fbgemm_amd_tbe_plan_set_accumulate(plan.handle, 1 if accumulate == "fast" else 0))
     out_dt = {0: torch.float32, 1: torch.float16, 5: torch.bfloat16}[p.output_dtype]
     out = torch.empty((p.B, p.total_D), dtype=out_dt, device=dev)
+    if int8_output:
+        out = torch.empty((p.B, p.total_D + 8 * p.T), dtype=torch.uint8, device=dev)
     st = ops.Status(dev)
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     args = (plan.handle, C.c_void_p(p.dev_weights.data_ptr()), None, C.c_void_p(p.indices.data_ptr()),
             C.c_void_p(p.offsets.data_ptr()), 64 if p.indices.dtype == torch.int64 else 32, p.indices.numel(),
             p.offsets.numel(), p.pooling_mode,
             None if p.indice_weights is None else C.c_void_p(p.indice_weights.data_ptr()),
-            p.output_dtype, C.c_void_p(out.data_ptr()),
+            ops.INT8 if int8_output else p.output_dtype, C.c_void_p(out.data_ptr()),
             C.c_void_p(p.extra["remap"].data_ptr()) if "remap" in p.extra else None, 32,
             C.c_void_p(p.extra["remap_offsets"].data_ptr()) if "remap" in p.extra else None,
             p.extra["remap_offsets"].numel() if "remap" in p.extra else 0,
@@ -787,7 +793,9 @@ def time_tbe(p, a, torch, np, steps, warmup, graph, accumulate):
     """Parity gate, warm-up, `steps` timed forwards of one table-batched problem.
     Returns the figures of the JSON line that depend on the measurement."""
     from fbgemm_amd import _lib
-    launch, out, st, plan = tbe_runner(p, torch, accumulate, not a.no_rank_records)
+    if a.int8_output:
+        assert not a.check and not a.other_mode, "--int8-output needs --no-check --one-mode"
+    launch, out, st, plan = tbe_runner(p, torch, accumulate, not a.no_rank_records, a.int8_output)
     torch.cuda.synchronize()
     checked = parity_gate(p, out, launch, torch, np, accumulate) if a.check else None
     # The parity gate leaves the device idle for seconds while the host computes the expected
@@ -896,6 +904,8 @@ def main():
         lookups, useful = p.lookups, p.useful_row_bytes()
         other = p.other_bytes()
         name, dtype_out = p.name, {0: "fp32", 1: "fp16", 5: "bf16"}[p.output_dtype]
+        if a.int8_output:
+            dtype_out = "int8 rows with fp32 scale and bias per (bag, table)"
         launches_per_step = 1
         torch.cuda.synchronize()
         build_s = time.time() - t_build

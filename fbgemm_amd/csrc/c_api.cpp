@@ -717,6 +717,10 @@ struct fbgemm_amd_tbe_plan {
     hipStream_t side_stream[ORDER_SLOTS] = {nullptr, nullptr, nullptr, nullptr};
     hipEvent_t side_fork[ORDER_SLOTS] = {nullptr, nullptr, nullptr, nullptr};
     hipEvent_t side_join[ORDER_SLOTS] = {nullptr, nullptr, nullptr, nullptr};
+    // the tables on the general kernel's list (the 8-bit pooled output of the lean kernel's tables
+    // is written by the lookup itself, these go through the quantizer afterwards)
+    int32_t* d_general_tables = nullptr;
+    int32_t n_general_tables = 0;
     bool pinned = false;         // used by a forward under stream capture: a graph may hold its pointers
     uint64_t last_use = 0;
   };
@@ -773,6 +777,9 @@ void free_work(fbgemm_amd_tbe_plan::Work& w) {
     w.side_fork[k] = w.side_join[k] = nullptr;
     w.side_stream[k] = nullptr;
   }
+  if (w.d_general_tables) (void)hipFree(w.d_general_tables);
+  w.d_general_tables = nullptr;
+  w.n_general_tables = 0;
 }
 
 // The per-wave work list of one kernel over the tables `members` (indices into `tables`).
@@ -1012,7 +1019,7 @@ int tbe_forward_impl(
     int64_t indices_numel, int64_t offsets_numel, int32_t pooling_mode,
     const float* d_indice_weights, int32_t output_ty, void* d_output,
     const void* d_index_remappings, int32_t remap_bits, const int64_t* d_index_remappings_offsets,
-    int64_t index_remappings_offsets_numel, void* d_status, void* stream_, bool allow_split) {
+    int64_t index_remappings_offsets_numel, void* d_status, void* stream_, bool allow_split, uint8_t* d_q8_out = nullptr) {
   if (!plan) return fail(FBGEMM_AMD_E_ARG, "plan is null");
   if (d_index_remappings && (!d_index_remappings_offsets || (remap_bits != 32 && remap_bits != 64)))
     return fail(FBGEMM_AMD_E_ARG, "a remap array needs its T+1 offsets and 32- or 64-bit entries");
@@ -1024,26 +1031,18 @@ int tbe_forward_impl(
   if (output_ty == ST_INT8) {
     // The reference's GPU operator quantizes every table's pooled vector row-wise to 8 bits in its
     // output stage ([B, total_D + 8 T]: D_t bytes, fp32 scale, fp32 bias per table;
-    // embedding_forward_quantized_split_nbit_kernel_template.cu:535-566). Here: the fp32 forward into
-    // plan-owned scratch, then one launch that quantizes all (bag, table) segments.
+    // embedding_forward_quantized_split_nbit_kernel_template.cu:535-566). Here: the lean kernel
+    // does the same for its tables (lean_store_q8); the other tables, and forwards whose bags are
+    // cut into segments, go as floats into plan-owned scratch, and one more launch quantizes
+    // their (bag, table) segments.
     if (offsets_numel < 1 || (offsets_numel - 1) % plan->T != 0) return fail(FBGEMM_AMD_E_ARG, "offsets must hold T*B+1 entries");
     const int64_t B = (offsets_numel - 1) / plan->T;
     if (B == 0) return 0;
     if (!d_output) return fail(FBGEMM_AMD_E_ARG, "null data pointer");
-    float* tmp;
-    {
-      std::lock_guard<std::mutex> lk(plan->mu);
-      if (int rc = grow(&plan->pooled_tmp, &plan->pooled_tmp_cap, B * plan->total_D, (hipStream_t)stream_)) return rc;
-      tmp = plan->pooled_tmp;
-    }
-    if (int rc = tbe_forward_impl(plan, d_dev_weights, d_uvm_weights, d_indices, d_offsets, index_bits, offset_bits,
-                                  indices_numel, offsets_numel, pooling_mode, d_indice_weights, ST_FP32, tmp,
-                                  d_index_remappings, remap_bits, d_index_remappings_offsets,
-                                  index_remappings_offsets_numel, d_status, stream_, allow_split))
-      return rc;
-    HIP_TRY(launch_quantize_segments(tmp, B, plan->T, plan->d_D_offsets, (int32_t)plan->total_D, plan->max_D,
-                                     (uint8_t*)d_output, (hipStream_t)stream_));
-    return 0;
+    return tbe_forward_impl(plan, d_dev_weights, d_uvm_weights, d_indices, d_offsets, index_bits, offset_bits,
+                            indices_numel, offsets_numel, pooling_mode, d_indice_weights, ST_FP32, nullptr,
+                            d_index_remappings, remap_bits, d_index_remappings_offsets,
+                            index_remappings_offsets_numel, d_status, stream_, allow_split, (uint8_t*)d_output);
   }
   if (output_ty != ST_FP32 && output_ty != ST_FP16 && output_ty != ST_BF16)
     return fail(FBGEMM_AMD_E_UNSUPPORTED, "output type %d is not supported", output_ty);
@@ -1056,12 +1055,27 @@ int tbe_forward_impl(
   if (B64 == 0) return 0;
   if (B64 > 0x7fffffffLL) return fail(FBGEMM_AMD_E_ARG, "B exceeds 2^31-1");
   const int32_t B = (int32_t)B64;
-  if (!d_offsets || !d_output || (indices_numel > 0 && !d_indices)) return fail(FBGEMM_AMD_E_ARG, "null data pointer");
+  if (!d_offsets || (!d_output && !d_q8_out) || (indices_numel > 0 && !d_indices)) return fail(FBGEMM_AMD_E_ARG, "null data pointer");
   // the lane shapes of the plan assume what every device allocator gives (the
   // reference's kernels load uint4 from the same buffers)
   if ((uintptr_t)d_dev_weights % 16 || (uintptr_t)d_uvm_weights % 16)
     return fail(FBGEMM_AMD_E_ARG, "weights buffers must be 16-byte aligned");
   hipStream_t stream = (hipStream_t)stream_;
+  // 8-bit pooled output: the float scratch [B, total_D] for what the lean kernel does not
+  // quantize itself, made when a forward first needs it (not under a stream capture)
+  auto pooled_scratch = [&](float** out) -> int {
+    std::lock_guard<std::mutex> lk(plan->mu);
+    const int64_t need = (int64_t)B * plan->total_D;
+    if (plan->pooled_tmp_cap < need) {
+      hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+      (void)hipStreamIsCapturing(stream, &cap);
+      if (cap != hipStreamCaptureStatusNone)
+        return fail(FBGEMM_AMD_E_ARG, "the first 8-bit forward of this size allocates float scratch: run it once outside the stream capture");
+    }
+    if (int rc = grow(&plan->pooled_tmp, &plan->pooled_tmp_cap, need, stream)) return rc;
+    *out = plan->pooled_tmp;
+    return 0;
+  };
   if (plan->has_fp8 && plan->fp8_shift == 0)
     return fail(FBGEMM_AMD_E_ARG, "the plan holds FP8 tables: set their exponent bits and bias first (fbgemm_amd_tbe_plan_set_fp8)");
 
@@ -1097,8 +1111,16 @@ int tbe_forward_impl(
                                     FBGEMM_AMD_POOL_SUM, d_indice_weights, ST_FP32, partial, d_index_remappings, remap_bits,
                                     d_index_remappings_offsets, index_remappings_offsets_numel, d_status, stream_, false))
         return rc;
+      if (d_q8_out) {
+        float* tmp = nullptr;
+        if (int rc = pooled_scratch(&tmp)) return rc;
+        d_output = tmp;
+      }
       HIP_TRY(launch_combine_segments(partial, plan->total_D, B, K, plan->T, plan->d_D_offsets, 0, d_offsets, offset_bits == 64,
                                       pooling_mode == FBGEMM_AMD_POOL_MEAN, d_output, output_ty, plan->total_D, stream));
+      if (d_q8_out)
+        HIP_TRY(launch_quantize_segments((const float*)d_output, B, plan->T, plan->d_D_offsets, (int32_t)plan->total_D, plan->max_D,
+                                         d_q8_out, nullptr, 0, stream));
       return 0;
     }
   }
@@ -1160,6 +1182,12 @@ int tbe_forward_impl(
       } undo{&nw};
       if (int rc = build_work_list(tables, lean_members, B, &nw.lean)) return rc;
       if (int rc = build_work_list(tables, general_members, B, &nw.general)) return rc;
+      if (!general_members.empty()) {
+        const std::vector<int32_t> ids(general_members.begin(), general_members.end());
+        HIP_TRY(hipMalloc((void**)&nw.d_general_tables, sizeof(int32_t) * ids.size()));
+        HIP_TRY(hipMemcpy(nw.d_general_tables, ids.data(), sizeof(int32_t) * ids.size(), hipMemcpyHostToDevice));
+        nw.n_general_tables = (int32_t)ids.size();
+      }
       // the bag order: one buffer for this stream, one ahead for the next stream
       for (int k = 0; k < 2; ++k) HIP_TRY(hipMalloc((void**)&nw.d_order[k], sizeof(BagEntry) * (size_t)plan->T * (size_t)B));
       nw.order_stream[0] = stream;
@@ -1238,6 +1266,11 @@ int tbe_forward_impl(
     reuse_order = plan->reuse_order;
   }
 
+  if (d_q8_out && w.general.num_waves > 0) {
+    float* tmp = nullptr;
+    if (int rc = pooled_scratch(&tmp)) return rc;
+    d_output = tmp;
+  }
   LookupArgs a;
   memset(&a, 0, sizeof(a));
   a.tables = variant == 2 ? plan->d_tables_narrow : (variant == 1 ? plan->d_tables_packed : plan->d_tables);
@@ -1289,11 +1322,20 @@ int tbe_forward_impl(
     l.work = w.lean.d_work;
     l.xcd_start = w.lean.d_xcd_start;
     l.num_waves = w.lean.num_waves;
+    if (d_q8_out) { // the 8-bit pooled output of these tables is made here
+      l.out = d_q8_out;
+      l.out_ty = ST_INT8;
+      l.out_stride = (int64_t)plan->total_D + 8 * (int64_t)plan->T;
+      l.out_aligned = (uintptr_t)d_q8_out % 16 == 0;
+    }
     HIP_TRY(launch_lookup_lean(l, index_bits == 64, exact, stream));
   }
   if (w.general.num_waves > 0) {
     if (side) HIP_TRY(hipStreamWaitEvent(stream, w.side_join[order_slot], 0));
     else HIP_TRY(launch_lookup(a, index_bits == 64, stream));
+    if (d_q8_out)
+      HIP_TRY(launch_quantize_segments((const float*)d_output, B, plan->T, plan->d_D_offsets, (int32_t)plan->total_D, plan->max_D,
+                                       d_q8_out, w.lean.num_waves > 0 ? w.d_general_tables : nullptr, w.n_general_tables, stream));
   }
   return 0;
 }

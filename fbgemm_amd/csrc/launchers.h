@@ -49,7 +49,8 @@ hipError_t launch_compressed_indices_remap(const void* indices, bool idx64, cons
                                            int64_t* before, int64_t* partial, int32_t* mapped, Status* status,
                                            hipStream_t stream);
 hipError_t launch_quantize_segments(const float* input, int64_t lines, int32_t T, const int32_t* d_seg_offsets,
-                                    int32_t total_D, int32_t max_D, uint8_t* output, hipStream_t stream);
+                                    int32_t total_D, int32_t max_D, uint8_t* output, const int32_t* d_tables,
+                                    int32_t n_tables, hipStream_t stream);
 hipError_t launch_bounds_check(const int64_t* rows_per_table, int32_t T, void* indices, void* offsets, bool is64,
                                int64_t num_indices, int64_t total_B, int64_t B, const int32_t* B_offsets, int mode,
                                int64_t* warning, int64_t* fixed, int64_t* partial, Status* status, hipStream_t stream);

@@ -145,7 +145,8 @@ struct LookupArgs {
   int64_t num_waves;         // waves with work (longest run when xcd_start is used)
   int32_t B;                 // bags per table
   int32_t T;
-  int32_t out_ty;            // ST_FP32, ST_FP16 or ST_BF16
+  int32_t out_ty;            // ST_FP32, ST_FP16 or ST_BF16; the lean kernel also takes ST_INT8 (lean_store_q8: `out` is bytes,
+                             // out_stride bytes per line, table t's block 8 t bytes behind its column)
   int32_t off64;             // offsets are int64 (else int32)
   int32_t normalize;         // mean pooling: scale by 1/len, len counting skipped rows
   int32_t positional;        // weight of entry i of a bag is sample_weights[i]

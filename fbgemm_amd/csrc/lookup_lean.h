@@ -348,8 +348,145 @@ __device__ __forceinline__ void lean_store_interleaved(const LookupArgs& a, cons
   }
 }
 
-template <bool EXACT, int TY, int C, bool INHDR>
-__device__ __forceinline__ void lean_write(const LookupArgs& a, const TableDesc& d, const LeanLane& L, float (&acc)[C * (TY == ST_INT4 ? 32 : (TY == ST_INT8 ? 16 : 8))], float bsum, uint32_t* lds) {
+// The 8-bit pooled output (output type ST_INT8 of a table-batched forward): the bag's block of
+// the line is the pooled fp32 vector quantized row-wise to 8 bits, D bytes followed by an fp32
+// scale and an fp32 bias, the block of table t starting 8 t bytes behind its float column (the
+// reference operator's output stage, embedding_forward_quantized_split_nbit_kernel_template.cu:
+// 535-560; the arithmetic is the core library's FloatToFused8BitRowwiseQuantizedSBFloat,
+// src/QuantUtils.cc:677-718, which is what the reference's test expects of it and what
+// quantize_rowwise_kernel computes from a float forward):
+//   scale = (max - min) / 255, bias = min, q = lrintf((x - min) * (255 / (max - min + 1e-8))),
+// min and max being the FIRST smallest / largest element of the block, which only shows when
+// the extreme is a zero and zeros of both signs are in the block.
+// `pooled` holds the wave's pooled vectors, D floats per bag slot (lean_store_q8 puts them
+// there). The lanes of a bag take groups of 4 columns in turn, so one store instruction writes
+// 4 * lanes consecutive bytes per bag, and exchange their extremes by lane shuffles (any number
+// of lanes per bag). One copy of this code serves every row type.
+__device__ __forceinline__ void lean_q8_from_lds(const LookupArgs& a, const TableDesc& d, const LeanLane& L, int table,
+                                                 const float* pooled) {
+  const int S = d.lanes, D = d.D;
+  const int base = (int)threadIdx.x - L.sub; // first lane of the bag
+  const float* mine = pooled + (size_t)L.grp * D;
+  const int nq = D >> 2; // whole groups of 4 columns; the D & 3 columns behind them are lane 0's
+  float lo = __builtin_inff(), hi = -__builtin_inff();
+  auto see = [&](float x) {
+    lo = x < lo ? x : lo;
+    hi = hi < x ? x : hi;
+  };
+  for (int q = L.sub; q < nq; q += S) {
+    const float4 v = *reinterpret_cast<const float4*>(mine + 4 * q);
+    see(v.x);
+    see(v.y);
+    see(v.z);
+    see(v.w);
+  }
+  if (L.sub == 0)
+    for (int c = nq * 4; c < D; ++c) see(mine[c]);
+  for (int j = 0; j < S; ++j) {
+    const float ol = __shfl(lo, base + j, 64), oh = __shfl(hi, base + j, 64);
+    lo = ol < lo ? ol : lo;
+    hi = hi < oh ? oh : hi;
+  }
+  float minimum = lo, maximum = hi;
+  if (__builtin_amdgcn_ballot_w64(L.bag_ok && (lo == 0.0f || hi == 0.0f)) != 0ull) {
+    // A zero extreme: every element is on one side of it, so the first of the equal extremes is
+    // the first zero of the block, of either sign (positions compared), and it is the same
+    // element for the minimum and for the maximum when both are zero.
+    constexpr int NONE = 0x7fffffff;
+    int zi = NONE;
+    float zv = 0.0f;
+    auto zero_at = [&](float x, int col) {
+      if (zi == NONE && x == 0.0f) {
+        zi = col;
+        zv = x;
+      }
+    };
+    for (int q = L.sub; q < nq; q += S) {
+      const float4 v = *reinterpret_cast<const float4*>(mine + 4 * q);
+      zero_at(v.x, 4 * q);
+      zero_at(v.y, 4 * q + 1);
+      zero_at(v.z, 4 * q + 2);
+      zero_at(v.w, 4 * q + 3);
+    }
+    if (L.sub == 0)
+      for (int c = nq * 4; c < D; ++c) zero_at(mine[c], c);
+    const int my_zi = zi;
+    const float my_zv = zv;
+    for (int j = 0; j < S; ++j) {
+      const int oi = __shfl(my_zi, base + j, 64);
+      const float ov = __shfl(my_zv, base + j, 64);
+      if (oi < zi) {
+        zi = oi;
+        zv = ov;
+      }
+    }
+    if (lo == 0.0f && zi != NONE) minimum = zv;
+    if (hi == 0.0f && zi != NONE) maximum = zv;
+  }
+  if (!L.bag_ok) return;
+  const float range = maximum - minimum;
+  const float inverse_scale = 255.0f / (range + 1e-8f);
+  auto quant = [&](float x) { return (uint32_t)(int)__builtin_rintf((x - minimum) * inverse_scale) & 0xffu; }; // to nearest, ties to even
+  uint8_t* row = reinterpret_cast<uint8_t*>(a.out) + (int64_t)L.bag * a.out_stride + d.out_col + 8 * (int64_t)table;
+  const bool words = (reinterpret_cast<uintptr_t>(row) & 3) == 0;
+  for (int q = L.sub; q < nq; q += S) {
+    const float4 v = *reinterpret_cast<const float4*>(mine + 4 * q);
+    const uint32_t w = quant(v.x) | (quant(v.y) << 8) | (quant(v.z) << 16) | (quant(v.w) << 24);
+    if (words) {
+      *reinterpret_cast<uint32_t*>(row + 4 * q) = w;
+    } else {
+      for (int k = 0; k < 4; ++k) row[4 * q + k] = (uint8_t)(w >> (8 * k));
+    }
+  }
+  if (L.sub == 0) {
+    for (int c = nq * 4; c < D; ++c) row[c] = (uint8_t)quant(mine[c]);
+    const uint32_t sb[2] = {float_to_bits(range / 255.0f), float_to_bits(minimum)};
+    uint8_t* p = row + D;
+    if ((reinterpret_cast<uintptr_t>(p) & 3) == 0) {
+      reinterpret_cast<uint32_t*>(p)[0] = sb[0];
+      reinterpret_cast<uint32_t*>(p)[1] = sb[1];
+    } else {
+      for (int b = 0; b < 8; ++b) p[b] = (uint8_t)(sb[b >> 2] >> (8 * (b & 3)));
+    }
+  }
+}
+
+// The pooled vectors of the wave into LDS, D floats per bag slot, then lean_q8_from_lds. `lds`
+// must hold the wave's whole output as floats (at most 64 lanes * 32 columns = LEAN_LDS_WORDS)
+// and is free once the last block is pooled.
+template <int TY, int C, bool INHDR>
+__device__ __forceinline__ void lean_store_q8(const LookupArgs& a, const TableDesc& d, const LeanLane& L, int table,
+                                              const float (&acc)[C * (TY == ST_INT4 ? 32 : (TY == ST_INT8 ? 16 : 8))], uint32_t* lds) {
+  constexpr int E = TY == ST_INT4 ? 32 : (TY == ST_INT8 ? 16 : 8);
+  const int S = d.lanes, D = d.D;
+  float* mine = reinterpret_cast<float*>(lds) + (size_t)L.grp * D;
+#pragma unroll
+  for (int c = 0; c < C; ++c) {
+    // first column of the chunk (whole-row chunks start E / 4 columns early: the header)
+    const int col0 = (L.sub + c * S) * E - (INHDR ? E / 4 : 0);
+#pragma unroll
+    for (int e = 0; e < E; e += 4) {
+      const int col = col0 + e;
+      if (!L.bag_ok || L.idle) continue;
+      if (col >= 0 && col + 4 <= D) {
+        *reinterpret_cast<float4*>(mine + col) = make_float4(acc[c * E + e], acc[c * E + e + 1], acc[c * E + e + 2], acc[c * E + e + 3]);
+      } else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+          if (col + k >= 0 && col + k < D) mine[col + k] = acc[c * E + e + k];
+      }
+    }
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  lean_q8_from_lds(a, d, L, table, reinterpret_cast<const float*>(lds));
+}
+
+// VIA_LDS: floating-point output goes through lean_store_interleaved where its shape allows.
+// Q8: the kernel instance that writes the 8-bit pooled output (and nothing else).
+template <bool EXACT, int TY, int C, bool INHDR, bool VIA_LDS, bool Q8>
+__device__ __forceinline__ void lean_write(const LookupArgs& a, const TableDesc& d, const LeanLane& L, int table, float (&acc)[C * (TY == ST_INT4 ? 32 : (TY == ST_INT8 ? 16 : 8))], float bsum, uint32_t* lds) {
   constexpr bool QUANT = TY == ST_INT8 || TY == ST_INT4;
   constexpr int E = TY == ST_INT4 ? 32 : (TY == ST_INT8 ? 16 : 8);
   constexpr int NACC = C * E;
@@ -363,8 +500,12 @@ __device__ __forceinline__ void lean_write(const LookupArgs& a, const TableDesc&
 #pragma unroll
     for (int e = 0; e < NACC; ++e) acc[e] *= inv_len;
   }
+  if constexpr (Q8) {
+    lean_store_q8<TY, C, INHDR>(a, d, L, table, acc, lds);
+    return;
+  }
   // whole 16-byte (8-byte) pieces at aligned places: through LDS, interleaved
-  if (lds && vec_ok) {
+  if (VIA_LDS && vec_ok) {
     if (a.out_ty == ST_FP32) {
       if ((d.D * 4) % 16 == 0) {
         lean_store_interleaved<TY, C, INHDR, 4>(a, d, L, acc, lds);
@@ -418,7 +559,7 @@ __device__ __forceinline__ void lean_write(const LookupArgs& a, const TableDesc&
 // valid row its units are not loaded at all.)
 // Returns false (wave-uniform, nothing written) when a scale is too large for
 // the pre-scaled arithmetic.
-template <typename index_t, bool EXACT, int TY, int C, bool INHDR, int R>
+template <typename index_t, bool EXACT, int TY, int C, bool INHDR, int R, bool Q8>
 __device__ __forceinline__ bool pool_lean(const LookupArgs& a, const TableDesc& d, int table, int first_slot, int lane,
                                           uint32_t* lds) {
   constexpr bool QUANT = TY == ST_INT8 || TY == ST_INT4;
@@ -745,15 +886,15 @@ __device__ __forceinline__ bool pool_lean(const LookupArgs& a, const TableDesc& 
     if (__builtin_amdgcn_ballot_w64(big) != 0ull) return false; // wave-uniform
   }
   lean_report_bad(a, bad_pos);
-  lean_write<EXACT, TY, C, INHDR>(a, d, L, acc, bsum, lds);
+  lean_write<EXACT, TY, C, INHDR, true, Q8>(a, d, L, table, acc, bsum, lds);
   return true;
 }
 
 // The same bags, one row at a time, integers converted to float before the fma:
 // for waves that met a scale the pre-scaled arithmetic cannot take. Every lane
 // walks its bag's entries itself; nothing is staged.
-template <typename index_t, bool EXACT, int TY, int C, bool INHDR>
-__device__ __forceinline__ void pool_lean_slow(const LookupArgs& a, const TableDesc& d, int table, int first_slot, int lane) {
+template <typename index_t, bool EXACT, int TY, int C, bool INHDR, bool Q8>
+__device__ __forceinline__ void pool_lean_slow(const LookupArgs& a, const TableDesc& d, int table, int first_slot, int lane, uint32_t* lds) {
   constexpr int E = TY == ST_INT4 ? 32 : 16;
   const LeanLane L = lean_lane<index_t>(a, d, table, first_slot, lane);
   const int S = d.lanes;
@@ -789,33 +930,33 @@ __device__ __forceinline__ void pool_lean_slow(const LookupArgs& a, const TableD
     }
   }
   lean_report_bad(a, bad_pos);
-  lean_write<EXACT, TY, C, INHDR>(a, d, L, acc, bsum, nullptr);
+  lean_write<EXACT, TY, C, INHDR, false, Q8>(a, d, L, table, acc, bsum, lds);
 }
 
-template <typename index_t, bool EXACT, int TY, int C, bool INHDR>
+template <typename index_t, bool EXACT, int TY, int C, bool INHDR, bool Q8>
 __device__ __forceinline__ void run_lean(const LookupArgs& a, const TableDesc& d, int table, int first_slot, int lane,
                                          uint32_t* lds) {
   bool done;
-  if (d.lanes >= 8) done = pool_lean<index_t, EXACT, TY, C, INHDR, 1>(a, d, table, first_slot, lane, lds);
-  else if (d.lanes >= 4) done = pool_lean<index_t, EXACT, TY, C, INHDR, 2>(a, d, table, first_slot, lane, lds);
-  else done = pool_lean<index_t, EXACT, TY, C, INHDR, 4>(a, d, table, first_slot, lane, lds);
+  if (d.lanes >= 8) done = pool_lean<index_t, EXACT, TY, C, INHDR, 1, Q8>(a, d, table, first_slot, lane, lds);
+  else if (d.lanes >= 4) done = pool_lean<index_t, EXACT, TY, C, INHDR, 2, Q8>(a, d, table, first_slot, lane, lds);
+  else done = pool_lean<index_t, EXACT, TY, C, INHDR, 4, Q8>(a, d, table, first_slot, lane, lds);
   if constexpr (TY == ST_INT4 || TY == ST_INT8) {
-    if (!done) pool_lean_slow<index_t, EXACT, TY, C, INHDR>(a, d, table, first_slot, lane);
+    if (!done) pool_lean_slow<index_t, EXACT, TY, C, INHDR, Q8>(a, d, table, first_slot, lane, lds);
   }
 }
 
 // Row types and the chunks per lane the host picks for lean shapes: 1 (4-bit), 2 (8-bit), 4 (fp16).
-template <typename index_t, bool EXACT>
+template <typename index_t, bool EXACT, bool Q8>
 __device__ __forceinline__ void lean_dispatch(const LookupArgs& a, const TableDesc& d, int table, int first_slot, int lane,
                                               uint32_t* lds) {
   if (d.ty == ST_INT4) {
-    if (d.inline_hdr) run_lean<index_t, EXACT, ST_INT4, 1, true>(a, d, table, first_slot, lane, lds);
-    else run_lean<index_t, EXACT, ST_INT4, 1, false>(a, d, table, first_slot, lane, lds);
+    if (d.inline_hdr) run_lean<index_t, EXACT, ST_INT4, 1, true, Q8>(a, d, table, first_slot, lane, lds);
+    else run_lean<index_t, EXACT, ST_INT4, 1, false, Q8>(a, d, table, first_slot, lane, lds);
   } else if (d.ty == ST_INT8) {
-    if (d.inline_hdr) run_lean<index_t, EXACT, ST_INT8, 2, true>(a, d, table, first_slot, lane, lds);
-    else run_lean<index_t, EXACT, ST_INT8, 2, false>(a, d, table, first_slot, lane, lds);
+    if (d.inline_hdr) run_lean<index_t, EXACT, ST_INT8, 2, true, Q8>(a, d, table, first_slot, lane, lds);
+    else run_lean<index_t, EXACT, ST_INT8, 2, false, Q8>(a, d, table, first_slot, lane, lds);
   } else if (d.ty == ST_FP16) {
-    run_lean<index_t, EXACT, ST_FP16, 4, false>(a, d, table, first_slot, lane, lds);
+    run_lean<index_t, EXACT, ST_FP16, 4, false, Q8>(a, d, table, first_slot, lane, lds);
   }
 }
 
@@ -824,7 +965,7 @@ __device__ __forceinline__ void lean_dispatch(const LookupArgs& a, const TableDe
 #endif
 
 // Same work list and workgroup -> XCD mapping as lookup_kernel.
-template <typename index_t, bool EXACT>
+template <typename index_t, bool EXACT, bool Q8>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(FBGEMM_AMD_LEAN_MIN_WAVES, 8))) void lookup_lean_kernel(const LookupArgs a) {
   // 8 KB: while a bag is pooled, two buffers of staged rows (2 KB) and the multipliers (4 KB); at the end, the wave's output
   __shared__ __attribute__((aligned(16))) uint32_t lds[LEAN_LDS_WORDS + MAX_GROUPS];
@@ -849,12 +990,12 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(FBGEMM_AMD_L
     first_slot = (int)(wave * a.single.bags);
   }
   const TableDesc d = a.tables ? a.tables[table] : a.single;
-  lean_dispatch<index_t, EXACT>(a, d, table, first_slot, lane, lds);
+  lean_dispatch<index_t, EXACT, Q8>(a, d, table, first_slot, lane, lds);
 }
 
-#define FBGEMM_AMD_DEFINE_LEAN_LAUNCH(FN, INDEX_T, EXACT)                                                \
+#define FBGEMM_AMD_DEFINE_LEAN_LAUNCH(FN, INDEX_T, EXACT, Q8)                                            \
   hipError_t FN(const LookupArgs& a, unsigned blocks, hipStream_t stream) {                              \
-    hipLaunchKernelGGL((lookup_lean_kernel<INDEX_T, EXACT>), dim3(blocks), dim3(64), 0, stream, a);      \
+    hipLaunchKernelGGL((lookup_lean_kernel<INDEX_T, EXACT, Q8>), dim3(blocks), dim3(64), 0, stream, a);  \
     return hipGetLastError();                                                                            \
   }
 

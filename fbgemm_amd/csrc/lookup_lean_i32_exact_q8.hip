@@ -1,0 +1,6 @@
+// One instance of the lean pooled-lookup kernel: the one that writes the 8-bit pooled output.
+#include "lookup_lean.h"
+
+namespace fbgemm_amd {
+FBGEMM_AMD_DEFINE_LEAN_LAUNCH(launch_lookup_lean_i32_exact_q8, int32_t, true, true)
+} // namespace fbgemm_amd

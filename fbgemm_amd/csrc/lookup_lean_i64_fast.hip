@@ -2,5 +2,5 @@
 #include "lookup_lean.h"
 
 namespace fbgemm_amd {
-FBGEMM_AMD_DEFINE_LEAN_LAUNCH(launch_lookup_lean_i64_fast, int64_t, false)
+FBGEMM_AMD_DEFINE_LEAN_LAUNCH(launch_lookup_lean_i64_fast, int64_t, false, false)
 } // namespace fbgemm_amd

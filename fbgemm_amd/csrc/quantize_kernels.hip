@@ -117,7 +117,7 @@ template <bool HALF_IN, int BITS>
 __global__ __launch_bounds__(256) void quantize_rowwise_kernel(
     const void* input, int64_t rows, int32_t cols_arg, int32_t sb_float, int32_t layout,
     int64_t out_stride, uint8_t* output, int32_t lpr, const int32_t* seg_offsets, int32_t seg_T, int64_t seg_in_stride,
-    const void* min_max) {
+    const void* min_max, const int32_t* seg_tables) {
   constexpr int bits = BITS;
   const int lane = threadIdx.x & 63;
   const int sub = lane & (lpr - 1);
@@ -132,13 +132,15 @@ __global__ __launch_bounds__(256) void quantize_rowwise_kernel(
   // Segment mode (seg_offsets != null): "row" r is the segment of table t = r % seg_T in
   // line b = r / seg_T of a [lines, seg_in_stride] matrix: columns seg_offsets[t] .. seg_offsets[t+1],
   // quantized to seg_offsets[t] + t * 8 bytes into line b of the output (every segment carries its
-  // own 8 bytes of scale and bias behind its data).
+  // own 8 bytes of scale and bias behind its data). With seg_tables the segments are those of the
+  // seg_T tables it lists (t = seg_tables[r % seg_T]) and the others are left alone.
   int32_t cols = cols_arg;
   const void* in_row;
   uint8_t* out_row;
   if (seg_offsets) {
     const int64_t b = row / seg_T;
-    const int32_t t = (int32_t)(row - b * seg_T);
+    int32_t t = (int32_t)(row - b * seg_T);
+    if (seg_tables) t = seg_tables[t];
     const int32_t c0 = seg_offsets[t];
     cols = seg_offsets[t + 1] - c0;
     in_row = reinterpret_cast<const uint8_t*>(input) + (b * seg_in_stride + c0) * (HALF_IN ? 2 : 4);
@@ -469,7 +471,7 @@ hipError_t launch_quantize_rowwise(const void* input, bool half_in, int64_t rows
   const dim3 grid(stream_blocks(blocks)), block(256);
 #define FBGEMM_AMD_LAUNCH_Q(H, B) \
   hipLaunchKernelGGL((quantize_rowwise_kernel<H, B>), grid, block, 0, stream, input, rows, cols, sb_float, layout, \
-                     out_stride, (uint8_t*)output, lpr, (const int32_t*)nullptr, 0, (int64_t)0, min_max)
+                     out_stride, (uint8_t*)output, lpr, (const int32_t*)nullptr, 0, (int64_t)0, min_max, (const int32_t*)nullptr)
   if (half_in) {
     if (bits == 2) FBGEMM_AMD_LAUNCH_Q(true, 2);
     else if (bits == 4) FBGEMM_AMD_LAUNCH_Q(true, 4);
@@ -485,17 +487,20 @@ hipError_t launch_quantize_rowwise(const void* input, bool half_in, int64_t rows
 
 // Every (line, table) segment of a [lines, total_D] fp32 matrix to 8-bit rows with an fp32
 // (scale, bias) trailer each: line b of the output holds, for t = 0 .. T-1, D_t bytes and 8 bytes.
+// d_tables (or null): the n_tables tables whose segments are quantized; the others are left alone.
 hipError_t launch_quantize_segments(const float* input, int64_t lines, int32_t T, const int32_t* d_seg_offsets,
-                                    int32_t total_D, int32_t max_D, uint8_t* output, hipStream_t stream) {
-  if (lines <= 0 || T <= 0 || max_D <= 0) return hipSuccess;
+                                    int32_t total_D, int32_t max_D, uint8_t* output, const int32_t* d_tables,
+                                    int32_t n_tables, hipStream_t stream) {
+  if (lines <= 0 || T <= 0 || max_D <= 0 || (d_tables && n_tables <= 0)) return hipSuccess;
   const int lpr = lanes_per_row(max_D, RUN);
-  const int64_t rows = lines * T;
+  const int32_t seg_T = d_tables ? n_tables : T;
+  const int64_t rows = lines * seg_T;
   const int64_t rows_per_block = 4 * (64 / lpr);
   const int64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
   const dim3 grid(stream_blocks(blocks)), block(256);
   hipLaunchKernelGGL((quantize_rowwise_kernel<false, 8>), grid, block, 0, stream, (const void*)input, rows, max_D, 1, 0,
-                     (int64_t)total_D + 8 * (int64_t)T, output, lpr, d_seg_offsets, T, (int64_t)total_D,
-                     (const void*)nullptr);
+                     (int64_t)total_D + 8 * (int64_t)T, output, lpr, d_seg_offsets, seg_T, (int64_t)total_D,
+                     (const void*)nullptr, d_tables);
   return hipGetLastError();
 }
 

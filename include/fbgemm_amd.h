@@ -222,8 +222,11 @@ void fbgemm_amd_tbe_plan_destroy(fbgemm_amd_tbe_plan* plan);
  * shape: fbgemm_gpu/fbgemm_gpu/sparse_ops.py:571-577): d_output is uint8
  * [B, total_D + 8 T]; per bag and table, the pooled fp32 vector quantized
  * row-wise to 8 bits as FloatToFused8BitRowwiseQuantized does (D_t bytes, fp32
- * scale, fp32 bias), table t starting at byte D_offsets[t] + 8 t. Two launches
- * more than the float outputs and a plan-owned fp32 [B, total_D] scratch. */
+ * scale, fp32 bias), table t starting at byte D_offsets[t] + 8 t. Tables of
+ * the regular shapes are quantized in the lookup kernel's own output stage, as
+ * in the reference; tables of other shapes (and forwards that cut their bags
+ * into segments) go as floats through a plan-owned fp32 [B, total_D] scratch
+ * and one more launch. */
 int fbgemm_amd_tbe_forward(
     fbgemm_amd_tbe_plan* plan, const void* d_dev_weights, const void* d_uvm_weights,
     const void* d_indices, const void* d_offsets, int32_t index_bits,

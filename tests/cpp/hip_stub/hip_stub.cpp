@@ -184,7 +184,7 @@ hipError_t launch_compressed_indices_remap(const void*, bool, const int32_t*, in
   return LAUNCHED();
 }
 hipError_t launch_quantize_segments(const float* input, int64_t lines, int32_t, const int32_t*, int32_t total_D, int32_t, uint8_t*,
-                                    hipStream_t) {
+                                    const int32_t*, int32_t, hipStream_t) {
   (void)*(volatile const float*)&input[lines * total_D - 1];
   return LAUNCHED();
 }

@@ -517,6 +517,51 @@ def test_pooled_int8_output_is_the_rowwise_quantized_fp32_output(ops, oracle, po
         H.assert_same_bits(f.cpu().numpy(), pooled, "fp32 forward after the 8-bit one")
 
 
+@pytest.mark.parametrize("mixed", [False, True])
+def test_pooled_int8_output_at_a_size_the_lean_kernel_takes(ops, oracle, mixed):
+    """A forward large enough for 16-byte lanes: the lean kernel quantizes its tables' pooled
+    vectors in its own output stage (no float round trip); with `mixed`, tables of other shapes
+    sit between them and go through the float scratch and the quantizer, which must leave the
+    lean tables' blocks alone. Empty bags (an all-zero block: both extremes are zeros), bags
+    whose weights are all -0.0 or 0.0 (zeros of both signs: the FIRST zero decides the sign of
+    the stored bias and scale) and mean pooling are in. Byte for byte against pooled oracle +
+    quantizer oracle."""
+    rng = np.random.default_rng(1350 + mixed)
+    specs = [(500, 64, INT4), (300, 128, INT8), (200, 64, FP16), (400, 256, INT4), (250, 32, INT8), (100, 96, INT4)]
+    if mixed:
+        specs = [specs[0], (300, 40, INT2), specs[1], (60, 8, FP32), specs[2], specs[3], (50, 4, INT8), specs[4], specs[5]]
+    T, B = len(specs), 1500
+    weights, wo, _ = build_weights(rng, specs, 16)
+    lens = rng.integers(0, 12, size=T * B)
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    idx = np.concatenate([rng.integers(0, specs[t][0], size=int(lens[t * B:(t + 1) * B].sum())) for t in range(T)]).astype(np.int64)
+    idx[rng.random(len(idx)) < 0.05] = -1
+    psw = rng.uniform(-1, 1, len(idx)).astype(np.float32)
+    for b in range(0, T * B, 7):  # every seventh bag: weights that are zeros of one sign or of both
+        lo, hi = int(off[b]), int(off[b + 1])
+        psw[lo:hi] = [0.0, -0.0, 0.0][b % 3]
+        if b % 3 == 2 and hi - lo > 1:
+            psw[lo] = -0.0
+    tys = np.array([s[2] for s in specs], np.uint8)
+    D_offsets = np.concatenate([[0], np.cumsum([s[1] for s in specs])]).astype(np.int32)
+    total_D = int(D_offsets[-1])
+    maxd = lambda ty: max([s[1] for s in specs if s[2] == ty], default=0)
+    for pooling, w in ((0, None), (0, psw), (1, None)):
+        got = ops.int_nbit_split_embedding_codegen_lookup_function(
+            cu(weights), torch.zeros(0, dtype=torch.uint8, device="cuda"), cu(np.zeros(T, np.int32)), cu(wo), cu(tys),
+            cu(D_offsets), total_D, maxd(INT2), maxd(INT4), maxd(INT8), maxd(FP16), maxd(FP32), cu(idx), cu(off),
+            pooling, None if w is None else cu(w), INT8, row_alignment=16)
+        assert got.dtype == torch.uint8 and tuple(got.shape) == (B, total_D + 8 * T)
+        got = got.cpu().numpy()
+        rc, pooled = oracle.tbe_forward(weights, wo, tys, D_offsets, total_D, idx, off, pooling, w, FP32, 16)
+        assert rc == 0
+        for t in range(T):
+            D = specs[t][1]
+            want = oracle.quantize_rowwise(np.ascontiguousarray(pooled[:, D_offsets[t]:D_offsets[t + 1]]), 8, True)
+            block = got[:, D_offsets[t] + 8 * t:D_offsets[t] + 8 * t + D + 8]
+            assert (block == want).all(), (mixed, pooling, w is not None, t, np.argwhere(block != want)[:4])
+
+
 @pytest.mark.parametrize("pooling", [0, 2])
 def test_tables_in_both_weights_buffers(ops, oracle, pooling):
     """weights_placements: tables 1 and 3 live in the second buffer (uvm_weights), whose offsets
