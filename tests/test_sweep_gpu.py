@@ -119,3 +119,54 @@ def test_table_batched_sweep(ops, oracle, routes, chunk):
     for seed in range(20_000 + chunk * CHUNK, 20_000 + (chunk + 1) * CHUNK):
         routes(np.random.default_rng(seed + 1_000_000))
         table_batched_case(ops, oracle, seed)
+
+
+def int8_output_case(ops, oracle, seed):
+    """The 8-bit pooled output of a random table-batched forward: every (bag, table) block byte for
+    byte against the pooled oracle followed by the quantizer oracle (the lean kernel's own output
+    stage, the float route through the quantizer, and plans that mix the two)."""
+    rng = np.random.default_rng(seed)
+    T, B = int(rng.integers(1, 9)), int(rng.integers(1, 70))
+    specs = []
+    for _ in range(T):
+        ty = int(rng.choice([INT8, INT4, INT4, INT2, FP16, FP32]))
+        specs.append((int(rng.integers(1, 300)), int(rng.choice(DIMS_BATCHED)), ty))
+    align = int(rng.choice([16, 16, 1, 4]))
+    weights, wo, _ = TB.build_weights(rng, specs, align)
+    max_len = int(rng.choice([3, 10, 45]))
+    lens = rng.integers(0, max_len, size=T * B)
+    dt = rng.choice([np.int32, np.int64])
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(dt)
+    idx = np.concatenate([rng.integers(0, specs[t][0], size=int(lens[t * B:(t + 1) * B].sum())) for t in range(T)]
+                         + [np.zeros(0, np.int64)]).astype(dt)
+    if len(idx):
+        idx[rng.random(len(idx)) < 0.1] = -1
+    pooling = int(rng.integers(0, 2))
+    psw = rng.normal(size=len(idx)).astype(np.float32) if rng.random() < 0.5 else None
+    if psw is not None and len(psw):
+        psw[rng.random(len(psw)) < 0.05] = -0.0  # zeros of both signs among a block's terms
+    tys = np.array([s[2] for s in specs], np.uint8)
+    D_offsets = np.concatenate([[0], np.cumsum([s[1] for s in specs])]).astype(np.int32)
+    total_D = int(D_offsets[-1])
+    maxd = lambda ty: max([s[1] for s in specs if s[2] == ty], default=0)
+    cu = TB.cu
+    got = ops.int_nbit_split_embedding_codegen_lookup_function(
+        cu(weights), torch.zeros(0, dtype=torch.uint8, device="cuda"), cu(np.zeros(T, np.int32)), cu(wo), cu(tys),
+        cu(D_offsets), total_D, maxd(INT2), maxd(INT4), maxd(INT8), maxd(FP16), maxd(FP32), cu(idx), cu(off),
+        pooling, None if psw is None else cu(psw), INT8, row_alignment=align).cpu().numpy()
+    assert got.shape == (B, total_D + 8 * T)
+    rc, pooled = oracle.tbe_forward(weights, wo, tys, D_offsets, total_D, idx, off, pooling, psw, FP32, align)
+    assert rc == 0
+    for t in range(T):
+        D = specs[t][1]
+        want = oracle.quantize_rowwise(np.ascontiguousarray(pooled[:, D_offsets[t]:D_offsets[t + 1]]), 8, True)
+        block = got[:, D_offsets[t] + 8 * t:D_offsets[t] + 8 * t + D + 8]
+        assert (block == want).all(), (f"8-bit output seed {seed}: specs={specs} B={B} align={align} pooling={pooling} "
+                                       f"weighted={psw is not None} table={t}", np.argwhere(block != want)[:4])
+
+
+@pytest.mark.parametrize("chunk", range(4))
+def test_table_batched_int8_output_sweep(ops, oracle, routes, chunk):
+    for seed in range(30_000 + chunk * 150, 30_000 + (chunk + 1) * 150):
+        routes(np.random.default_rng(seed + 1_000_000))
+        int8_output_case(ops, oracle, seed)
