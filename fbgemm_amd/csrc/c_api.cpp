@@ -687,6 +687,13 @@ struct fbgemm_amd_tbe_plan {
   int64_t seg_offsets_cap = 0;
   float* seg_partial = nullptr;   // split bags: the segments' fp32 sums [B*K, total_D]
   int64_t seg_partial_cap = 0;
+  // pooled_tmp and seg_* are shared by all streams that run forwards of the plan. Forwards that use
+  // them are enqueued one at a time (shared_mu), and one on another stream than the last waits on
+  // the device for that one's last use (shared_done, recorded behind it): see SharedScratchUse.
+  std::mutex shared_mu;
+  hipEvent_t shared_done = nullptr;
+  hipStream_t shared_stream = nullptr;
+  bool shared_used = false;
   // the same tables with bags laid end to end where that saves a request per row
   // (see bags_per_wave); empty when no table has such a shape. Used for long bags.
   std::vector<TableDesc> tables_packed;
@@ -972,6 +979,7 @@ void fbgemm_amd_tbe_plan_destroy(fbgemm_amd_tbe_plan* plan) {
   if (plan->pooled_tmp) (void)hipFree(plan->pooled_tmp);
   if (plan->seg_offsets) (void)hipFree(plan->seg_offsets);
   if (plan->seg_partial) (void)hipFree(plan->seg_partial);
+  if (plan->shared_done) (void)hipEventDestroy(plan->shared_done);
   if (plan->d_rank_records) (void)hipFree(plan->d_rank_records);
   if (plan->d_rank_offsets) (void)hipFree(plan->d_rank_offsets);
   if (plan->d_rank_remap_offsets) (void)hipFree(plan->d_rank_remap_offsets);
@@ -1011,6 +1019,42 @@ int fbgemm_amd_tbe_forward(
 } // extern "C"
 
 namespace {
+// A forward's use of the scratch all streams of a plan share (the float scratch of the 8-bit pooled
+// output, the segment offsets and partial sums of split bags). begin(): from here to the end of
+// the scope no other host thread enqueues such a forward of the plan, and if the last one ran on
+// another stream this stream waits, on the device, for the event recorded behind it. The end of
+// the scope records that event behind this forward. Under stream capture nothing is recorded or
+// waited for (a graph cannot wait for work outside it): captured forwards of one plan that use
+// this scratch are the caller's to order.
+struct SharedScratchUse {
+  fbgemm_amd_tbe_plan* plan = nullptr;
+  hipStream_t stream = nullptr;
+  bool record = false;
+  std::unique_lock<std::mutex> host;
+  int begin(fbgemm_amd_tbe_plan* p, hipStream_t s) {
+    if (plan) return 0; // already begun
+    plan = p;
+    stream = s;
+    host = std::unique_lock<std::mutex>(p->shared_mu);
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    (void)hipStreamIsCapturing(s, &cap);
+    if (cap != hipStreamCaptureStatusNone) return 0;
+    if (!p->shared_done) HIP_TRY(hipEventCreateWithFlags(&p->shared_done, hipEventDisableTiming));
+    if (p->shared_used && p->shared_stream != s) HIP_TRY(hipStreamWaitEvent(s, p->shared_done, 0));
+    record = true;
+    return 0;
+  }
+  ~SharedScratchUse() {
+    if (!record) return;
+    if (hipEventRecord(plan->shared_done, stream) == hipSuccess) {
+      plan->shared_stream = stream;
+      plan->shared_used = true;
+    } else {
+      (void)hipGetLastError();
+    }
+  }
+};
+
 // The forward behind fbgemm_amd_tbe_forward[_pruned]. offset_bits: the width of d_offsets (the
 // operator's offsets have the width of its indices; the segment offsets of split bags are int64).
 int tbe_forward_impl(
@@ -1061,6 +1105,7 @@ int tbe_forward_impl(
   if ((uintptr_t)d_dev_weights % 16 || (uintptr_t)d_uvm_weights % 16)
     return fail(FBGEMM_AMD_E_ARG, "weights buffers must be 16-byte aligned");
   hipStream_t stream = (hipStream_t)stream_;
+  SharedScratchUse shared; // begun where the forward turns out to use the plan's shared scratch
   // 8-bit pooled output: the float scratch [B, total_D] for what the lean kernel does not
   // quantize itself, made when a forward first needs it (not under a stream capture)
   auto pooled_scratch = [&](float** out) -> int {
@@ -1091,6 +1136,7 @@ int tbe_forward_impl(
     for (const TableDesc& d : plan->tables) wide_waves += (B + d.bags - 1) / d.bags;
     const int K = split_factor(wide_waves, indices_numel / ((int64_t)plan->T * B));
     if (K > 1) {
+      if (int rc = shared.begin(plan, stream)) return rc;
       hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
       (void)hipStreamIsCapturing(stream, &cap);
       const int64_t vbags = (int64_t)plan->T * B * K;
@@ -1267,6 +1313,7 @@ int tbe_forward_impl(
   }
 
   if (d_q8_out && w.general.num_waves > 0) {
+    if (int rc = shared.begin(plan, stream)) return rc;
     float* tmp = nullptr;
     if (int rc = pooled_scratch(&tmp)) return rc;
     d_output = tmp;

@@ -562,6 +562,59 @@ def test_pooled_int8_output_at_a_size_the_lean_kernel_takes(ops, oracle, mixed):
             assert (block == want).all(), (mixed, pooling, w is not None, t, np.argwhere(block != want)[:4])
 
 
+def test_int8_output_forwards_of_one_plan_on_two_streams(ops, oracle):
+    """Forwards of one plan that go through the plan's float scratch (8-bit output of tables the
+    lean kernel does not take) may be issued on different streams without ordering them: the
+    library makes the later one wait for the earlier one's use of the scratch. Through the C ABI,
+    without a synchronization between the calls: two streams, two sets of indices, alternating,
+    every result against the same forward run alone."""
+    import ctypes as C
+    import fbgemm_amd
+    lib = fbgemm_amd.lib()
+    rng = np.random.default_rng(1360)
+    specs = [(500, 64, INT4), (300, 40, INT2), (60, 8, FP32), (200, 64, FP16), (100, 72, INT8)]
+    T, B = len(specs), 1200
+    weights, wo, _ = build_weights(rng, specs, 16)
+    tys = np.array([s[2] for s in specs], np.uint8)
+    D_offsets = np.concatenate([[0], np.cumsum([s[1] for s in specs])]).astype(np.int32)
+    total_D = int(D_offsets[-1])
+    d_weights = cu(weights)
+    plan = ops.TbePlan(torch.from_numpy(wo), torch.from_numpy(tys), torch.from_numpy(D_offsets),
+                       torch.zeros(T, dtype=torch.int32), d_weights.numel(), 0, 16)
+    inputs = []
+    for _ in range(2):
+        lens = rng.integers(0, 12, size=T * B)
+        off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+        idx = np.concatenate([rng.integers(0, specs[t][0], size=int(lens[t * B:(t + 1) * B].sum())) for t in range(T)]).astype(np.int64)
+        inputs.append((cu(idx), cu(off), torch.zeros((B, total_D + 8 * T), dtype=torch.uint8, device="cuda"), ops.Status("cuda")))
+    p = lambda t: C.c_void_p(t.data_ptr())
+
+    def enqueue(k):
+        idx, off, out, st = inputs[k]
+        rc = lib.fbgemm_amd_tbe_forward(plan.handle, p(d_weights), None, p(idx), p(off), 64, idx.numel(), off.numel(), 0, None,
+                                        INT8, p(out), p(st.buf), C.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert rc == 0, lib.fbgemm_amd_last_error().decode()
+
+    alone = []
+    for k in (0, 1):
+        enqueue(k)
+        torch.cuda.synchronize()
+        alone.append(inputs[k][2].clone())
+    assert not torch.equal(alone[0], alone[1])
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    for rep in range(20):
+        for k in (0, 1):
+            inputs[k][2].zero_()
+        torch.cuda.synchronize()
+        for k in (0, 1, 0, 1):
+            with torch.cuda.stream(streams[k]):
+                enqueue(k)
+        torch.cuda.synchronize()
+        for k in (0, 1):
+            assert torch.equal(inputs[k][2], alone[k]), f"round {rep}: the forward on stream {k} differs from the same forward run alone"
+            assert inputs[k][3].read()[0] == 0
+
+
 @pytest.mark.parametrize("pooling", [0, 2])
 def test_tables_in_both_weights_buffers(ops, oracle, pooling):
     """weights_placements: tables 1 and 3 live in the second buffer (uvm_weights), whose offsets
