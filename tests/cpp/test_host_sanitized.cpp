@@ -137,6 +137,10 @@ void work_list_cache_and_graphs() {
   CHECK(fbgemm_amd_set_lean(-1) == 0);
   CHECK(forward(plan, p, b, 5, big_n, s0, /*INT8 output*/ 2) == 0);
   CHECK(forward(plan, p, b, 40, big_n, s0, 2) == 0); // the scratch of the 8-bit output grows
+  CHECK(forward(plan, p, b, 40, big_n, s1, 2) == 0); // another stream: waits for the event behind the last use
+  hip_stub_set_capturing(s2, true);
+  CHECK(forward(plan, p, b, 40, big_n, s2, 2) == 0); // under capture nothing is recorded or waited for
+  hip_stub_set_capturing(s2, false);
   CHECK(fbgemm_amd_tbe_plan_reuse_order(plan, 1) == 0);
   CHECK(forward(plan, p, b, 5, big_n, s0) == 0);
   CHECK(fbgemm_amd_tbe_plan_reuse_order(plan, 0) == 0);
