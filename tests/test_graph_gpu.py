@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 
 import helpers as H
-from helpers import FP16, INT4, INT8
+from helpers import FP16, FP32, INT4, INT8
 
 torch = pytest.importorskip("torch")
 pytestmark = pytest.mark.gpu
@@ -157,6 +157,71 @@ def test_forward_with_both_kernels_replays_from_a_graph(oracle):
         graph.replay()
         torch.cuda.synchronize()
         H.assert_same_bits(captured.cpu().view(torch.int16).numpy().view(np.uint16), expect(idx), f"replay {replay}")
+        again = call()
+        torch.cuda.synchronize()
+        assert torch.equal(again, captured)
+    assert st.read() == (0, -1)
+
+
+@pytest.mark.parametrize("mixed", [False, True])
+def test_int8_output_forward_replays_from_a_graph(oracle, mixed):
+    """The 8-bit pooled output under capture: the lean kernel's instances that quantize in their
+    output stage, and (mixed) the float route through the plan's scratch and the quantizer beside
+    them, with the side stream's fork and join. Every replay byte for byte against the pooled
+    oracle + quantizer oracle, eager forwards of the same plan in between."""
+    assert torch.cuda.is_available()
+    from fbgemm_amd import ops
+    from helpers import INT2, INT8
+    from test_tbe_gpu import build_weights
+    rng = np.random.default_rng(79 + mixed)
+    specs = [(3000, 128, INT4), (2000, 64, INT4), (900, 64, INT8)] + ([(500, 32, INT2), (700, 40, INT4)] if mixed else [])
+    T, B, L = len(specs), 4096, 180 if not mixed else 110
+    weights, wo, _ = build_weights(rng, specs, 16)
+    tys = np.array([s[2] for s in specs], np.uint8)
+    D_offsets = np.concatenate([[0], np.cumsum([s[1] for s in specs])]).astype(np.int32)
+    total_D = int(D_offsets[-1])
+    lens = rng.integers(L - 30, L + 31, size=T * B)
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    assert int(off[-1]) >= 1 << 21  # the scheduler runs (and, mixed, the side stream)
+
+    def draw():
+        return np.concatenate([rng.integers(0, specs[t][0], size=int(off[(t + 1) * B] - off[t * B])) for t in range(T)]).astype(np.int64)
+
+    idx = draw()
+    d_idx, d_off = cu(idx), cu(off)
+    meta = (cu(weights), torch.zeros(0, dtype=torch.uint8, device="cuda"), cu(np.zeros(T, np.int32)), cu(wo), cu(tys), cu(D_offsets))
+    st = ops.Status()
+    maxd = lambda ty: max([s[1] for s in specs if s[2] == ty], default=0)
+    call = lambda: ops.int_nbit_split_embedding_codegen_lookup_function(
+        *meta, total_D, maxd(INT2), maxd(INT4), maxd(INT8), 0, 0, d_idx, d_off, 0, None, INT8, row_alignment=16, status=st)
+
+    def check(got, idx, what):
+        rc, pooled = oracle.tbe_forward(weights, wo, tys, D_offsets, total_D, idx, off, 0, None, FP32, 16)
+        assert rc == 0
+        got = got.cpu().numpy()
+        for t in range(T):
+            D = specs[t][1]
+            want = oracle.quantize_rowwise(np.ascontiguousarray(pooled[:, D_offsets[t]:D_offsets[t + 1]]), 8, True)
+            block = got[:, D_offsets[t] + 8 * t:D_offsets[t] + 8 * t + D + 8]
+            assert (block == want).all(), (what, t, np.argwhere(block != want)[:4])
+
+    eager = call()  # outside the capture: work lists, side stream, float scratch
+    torch.cuda.synchronize()
+    check(eager, idx, "eager")
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            captured = call()
+    torch.cuda.synchronize()
+    for replay in range(3):
+        idx = draw()
+        d_idx.copy_(cu(idx))
+        captured.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        check(captured, idx, f"replay {replay}")
         again = call()
         torch.cuda.synchronize()
         assert torch.equal(again, captured)
