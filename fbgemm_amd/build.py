@@ -13,6 +13,7 @@ OUT = os.path.join(HERE, "lib", "libfbgemm_amd.so")
 
 # the lookup kernels compile one instance per translation unit (the slowest files first)
 SOURCES = ["lookup_lean_i64_exact.hip", "lookup_lean_i64_fast.hip", "lookup_lean_i32_exact.hip", "lookup_lean_i32_fast.hip",
+           "lookup_lean_i64_exact_w4.hip", "lookup_lean_i64_fast_w4.hip", "lookup_lean_i32_exact_w4.hip", "lookup_lean_i32_fast_w4.hip",
            "lookup_lean_i64_exact_q8.hip", "lookup_lean_i64_fast_q8.hip", "lookup_lean_i32_exact_q8.hip", "lookup_lean_i32_fast_q8.hip",
            "lookup_i64.hip", "lookup_i32.hip", "lookup_i64_general.hip", "lookup_i32_general.hip",
            "lookup_kernels.hip", "index_ops_kernels.hip", "quantize_kernels.hip", "sequence_kernels.hip",

@@ -207,6 +207,14 @@ bool lean_shape(const TableDesc& d) {
   return true;
 }
 
+// Shapes of the lean kernel's four-waves-per-SIMD instance (lookup_lean_wide4_kernel): 4-bit rows,
+// bags of 8 lanes and more (one entry per staging lane), the header fetched by a staging lane.
+// FBGEMM_AMD_WIDE4=0 keeps such launches on the general-purpose lean kernel.
+bool lean_wide4_shape(const TableDesc& d) {
+  static const int enabled = env_int("FBGEMM_AMD_WIDE4", 1);
+  return enabled && lean_shape(d) && d.ty == ST_INT4 && d.lanes >= 8 && !d.inline_hdr;
+}
+
 struct DeviceScratch {
   Status* status = nullptr;
   int64_t* offsets = nullptr; // lengths -> offsets
@@ -601,14 +609,14 @@ int spmdm_launch_impl(
     v.check_total = 0;
     v.out_aligned = 1;
     v.num_waves = (pooled_bags + G - 1) / G;
-    if (lean_enabled() && lean_shape(d)) HIP_TRY(launch_lookup_lean(v, cfg->index_bits == 64, false, stream));
+    if (lean_enabled() && lean_shape(d)) HIP_TRY(launch_lookup_lean(v, cfg->index_bits == 64, false, false, stream));
     else HIP_TRY(launch_lookup(v, cfg->index_bits == 64, stream));
     HIP_TRY(launch_combine_segments(s->seg_partial, D, (int32_t)output_size, K, 1, nullptr, (int32_t)D, a.offsets, a.off64 != 0,
                                     cfg->normalize_by_lengths != 0, d_out, cfg->output_ty, out_stride, stream));
     return 0;
   }
   if (lean_enabled() && !cfg->is_weight_positional && lean_shape(d))
-    HIP_TRY(launch_lookup_lean(a, cfg->index_bits == 64, cfg->accumulate != FBGEMM_AMD_ACC_FAST, stream));
+    HIP_TRY(launch_lookup_lean(a, cfg->index_bits == 64, cfg->accumulate != FBGEMM_AMD_ACC_FAST, false, stream));
   else
     HIP_TRY(launch_lookup(a, cfg->index_bits == 64, stream));
   return 0;
@@ -728,6 +736,11 @@ struct fbgemm_amd_tbe_plan {
     // is written by the lookup itself, these go through the quantizer afterwards)
     int32_t* d_general_tables = nullptr;
     int32_t n_general_tables = 0;
+    bool lean_wide4 = false;     // every table of the lean list has the shape of the four-waves-per-SIMD instance
+    // that instance's redo queue, one per bag-order buffer (made with it): lean.num_waves work items
+    // and two counters that are zero between forwards
+    WaveWork* d_redo[ORDER_SLOTS] = {nullptr, nullptr, nullptr, nullptr};
+    int32_t* d_redo_count[ORDER_SLOTS] = {nullptr, nullptr, nullptr, nullptr};
     bool pinned = false;         // used by a forward under stream capture: a graph may hold its pointers
     uint64_t last_use = 0;
   };
@@ -777,6 +790,10 @@ void free_work(fbgemm_amd_tbe_plan::Work& w) {
   for (int k = 0; k < fbgemm_amd_tbe_plan::ORDER_SLOTS; ++k) {
     if (w.d_order[k]) (void)hipFree(w.d_order[k]);
     w.d_order[k] = nullptr;
+    if (w.d_redo[k]) (void)hipFree(w.d_redo[k]);
+    if (w.d_redo_count[k]) (void)hipFree(w.d_redo_count[k]);
+    w.d_redo[k] = nullptr;
+    w.d_redo_count[k] = nullptr;
     w.order_claimed[k] = false;
     if (w.side_fork[k]) (void)hipEventDestroy(w.side_fork[k]);
     if (w.side_join[k]) (void)hipEventDestroy(w.side_join[k]);
@@ -1026,6 +1043,19 @@ namespace {
 // the scope records that event behind this forward. Under stream capture nothing is recorded or
 // waited for (a graph cannot wait for work outside it): captured forwards of one plan that use
 // this scratch are the caller's to order.
+// Buffer k of a work set's bag orders, with the redo queue of the four-waves-per-SIMD lean
+// instance when the set uses it. Allocates: not under stream capture.
+int make_order_slot(fbgemm_amd_tbe_plan::Work& W, int k, int32_t T, int32_t B) {
+  HIP_TRY(hipMalloc((void**)&W.d_order[k], sizeof(BagEntry) * (size_t)T * (size_t)B));
+  if (W.lean_wide4 && W.lean.num_waves > 0) {
+    HIP_TRY(hipMalloc((void**)&W.d_redo[k], sizeof(WaveWork) * (size_t)W.lean.num_waves));
+    HIP_TRY(hipMalloc((void**)&W.d_redo_count[k], 2 * sizeof(int32_t)));
+    const int32_t zeros[2] = {0, 0};
+    HIP_TRY(hipMemcpy(W.d_redo_count[k], zeros, sizeof(zeros), hipMemcpyHostToDevice));
+  }
+  return 0;
+}
+
 struct SharedScratchUse {
   fbgemm_amd_tbe_plan* plan = nullptr;
   hipStream_t stream = nullptr;
@@ -1226,6 +1256,8 @@ int tbe_forward_impl(
         fbgemm_amd_tbe_plan::Work* w;
         ~Undo() { if (w) free_work(*w); }
       } undo{&nw};
+      nw.lean_wide4 = !lean_members.empty();
+      for (int t : lean_members) nw.lean_wide4 = nw.lean_wide4 && lean_wide4_shape(tables[(size_t)t]);
       if (int rc = build_work_list(tables, lean_members, B, &nw.lean)) return rc;
       if (int rc = build_work_list(tables, general_members, B, &nw.general)) return rc;
       if (!general_members.empty()) {
@@ -1235,7 +1267,8 @@ int tbe_forward_impl(
         nw.n_general_tables = (int32_t)ids.size();
       }
       // the bag order: one buffer for this stream, one ahead for the next stream
-      for (int k = 0; k < 2; ++k) HIP_TRY(hipMalloc((void**)&nw.d_order[k], sizeof(BagEntry) * (size_t)plan->T * (size_t)B));
+      for (int k = 0; k < 2; ++k)
+        if (int rc = make_order_slot(nw, k, plan->T, B)) return rc;
       nw.order_stream[0] = stream;
       nw.order_claimed[0] = true;
       // A caller whose batch size keeps changing would grow this cache without bound. Past
@@ -1270,7 +1303,7 @@ int tbe_forward_impl(
       if (!W.order_claimed[k] && W.d_order[k]) order_slot = k;
     for (int k = 0; k < NS && order_slot < 0 && !capturing; ++k)
       if (!W.d_order[k]) {
-        HIP_TRY(hipMalloc((void**)&W.d_order[k], sizeof(BagEntry) * (size_t)plan->T * (size_t)B));
+        if (int rc = make_order_slot(W, k, plan->T, B)) return rc;
         order_slot = k;
       }
     if (order_slot < 0) order_slot = 0;
@@ -1281,7 +1314,7 @@ int tbe_forward_impl(
       if (!capturing)
         for (int k = 0; k < NS; ++k)
           if (!W.d_order[k]) {
-            HIP_TRY(hipMalloc((void**)&W.d_order[k], sizeof(BagEntry) * (size_t)plan->T * (size_t)B));
+            if (int rc = make_order_slot(W, k, plan->T, B)) return rc;
             break;
           }
     }
@@ -1375,7 +1408,14 @@ int tbe_forward_impl(
       l.out_stride = (int64_t)plan->total_D + 8 * (int64_t)plan->T;
       l.out_aligned = (uintptr_t)d_q8_out % 16 == 0;
     }
-    HIP_TRY(launch_lookup_lean(l, index_bits == 64, exact, stream));
+    // the four-waves-per-SIMD instance: forwards that order their bags (large ones: its second,
+    // usually idle launch does not show there), float output
+    const bool wide4 = w.lean_wide4 && !d_q8_out && a.order && w.d_redo[order_slot] && w.d_redo_count[order_slot];
+    if (wide4) {
+      l.redo = w.d_redo[order_slot];
+      l.redo_count = w.d_redo_count[order_slot];
+    }
+    HIP_TRY(launch_lookup_lean(l, index_bits == 64, exact, wide4, stream));
   }
   if (w.general.num_waves > 0) {
     if (side) HIP_TRY(hipStreamWaitEvent(stream, w.side_join[order_slot], 0));

@@ -9,7 +9,7 @@
 
 namespace fbgemm_amd {
 hipError_t launch_lookup(const LookupArgs& a, bool idx64, hipStream_t stream);
-hipError_t launch_lookup_lean(const LookupArgs& a, bool idx64, bool exact, hipStream_t stream);
+hipError_t launch_lookup_lean(const LookupArgs& a, bool idx64, bool exact, bool wide4, hipStream_t stream);
 hipError_t launch_lengths_to_offsets(const void* lengths, bool is64, int64_t n, int64_t* offsets, hipStream_t stream);
 hipError_t launch_status_clear(Status* st, hipStream_t stream);
 hipError_t launch_bag_order(const void* offsets, bool off64, int32_t B, int32_t T, BagEntry* order, hipStream_t stream);

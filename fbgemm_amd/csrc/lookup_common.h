@@ -155,6 +155,12 @@ struct LookupArgs {
   int32_t out_aligned;       // `out` is 16-byte aligned (vector stores allowed)
   int32_t fp8_shift;         // FP8 rows: 16 + exponent bits (moves the 7 low bits to fp32's exponent/mantissa)
   float fp8_mult;            // FP8 rows: 2^(127 - exponent bias)
+  // lookup_lean_wide4_kernel only: where a wave that meets a scale too large for its arithmetic
+  // leaves its work item (redo[atomicAdd(redo_count, 1)]) for lookup_lean_wide4_redo_kernel, which
+  // pools those items the plain way afterwards. redo_count[1] counts that kernel's workgroups; its
+  // last one sets both counters back to zero.
+  WaveWork* redo;
+  int32_t* redo_count;
   Status* status;
 };
 

@@ -153,20 +153,30 @@ hipError_t launch_lookup_lean_i64_exact(const LookupArgs& a, unsigned blocks, hi
 hipError_t launch_lookup_lean_i32_exact(const LookupArgs& a, unsigned blocks, hipStream_t stream);
 hipError_t launch_lookup_lean_i64_fast(const LookupArgs& a, unsigned blocks, hipStream_t stream);
 hipError_t launch_lookup_lean_i32_fast(const LookupArgs& a, unsigned blocks, hipStream_t stream);
+hipError_t launch_lookup_lean_i64_exact_w4(const LookupArgs& a, unsigned blocks, hipStream_t stream);
+hipError_t launch_lookup_lean_i32_exact_w4(const LookupArgs& a, unsigned blocks, hipStream_t stream);
+hipError_t launch_lookup_lean_i64_fast_w4(const LookupArgs& a, unsigned blocks, hipStream_t stream);
+hipError_t launch_lookup_lean_i32_fast_w4(const LookupArgs& a, unsigned blocks, hipStream_t stream);
 hipError_t launch_lookup_lean_i64_exact_q8(const LookupArgs& a, unsigned blocks, hipStream_t stream);
 hipError_t launch_lookup_lean_i32_exact_q8(const LookupArgs& a, unsigned blocks, hipStream_t stream);
 hipError_t launch_lookup_lean_i64_fast_q8(const LookupArgs& a, unsigned blocks, hipStream_t stream);
 hipError_t launch_lookup_lean_i32_fast_q8(const LookupArgs& a, unsigned blocks, hipStream_t stream);
 
 // The lean kernel (lookup_lean.h) over a work list (or a single table) whose tables all
-// have a lean shape. `exact` selects the reference's sequence of roundings.
-hipError_t launch_lookup_lean(const LookupArgs& a, bool idx64, bool exact, hipStream_t stream) {
+// have a lean shape. `exact` selects the reference's sequence of roundings; `wide4`: every table
+// of the launch has the shape lookup_lean_wide4_kernel takes.
+hipError_t launch_lookup_lean(const LookupArgs& a, bool idx64, bool exact, bool wide4, hipStream_t stream) {
   if (a.num_waves <= 0) return hipSuccess;
   const int64_t blocks = a.xcd_start ? 8 * a.num_waves : a.num_waves;
   if (blocks > 0x7fffffffLL || a.positional) return hipErrorInvalidValue;
   if (a.out_ty == ST_INT8) { // the instances whose output stage quantizes the pooled vectors (lean_store_q8)
     if (exact) return idx64 ? launch_lookup_lean_i64_exact_q8(a, (unsigned)blocks, stream) : launch_lookup_lean_i32_exact_q8(a, (unsigned)blocks, stream);
     return idx64 ? launch_lookup_lean_i64_fast_q8(a, (unsigned)blocks, stream) : launch_lookup_lean_i32_fast_q8(a, (unsigned)blocks, stream);
+  }
+  if (wide4) { // two launches: the kernel, and the one that pools what it has queued
+    if (!a.redo || !a.redo_count) return hipErrorInvalidValue;
+    if (exact) return idx64 ? launch_lookup_lean_i64_exact_w4(a, (unsigned)blocks, stream) : launch_lookup_lean_i32_exact_w4(a, (unsigned)blocks, stream);
+    return idx64 ? launch_lookup_lean_i64_fast_w4(a, (unsigned)blocks, stream) : launch_lookup_lean_i32_fast_w4(a, (unsigned)blocks, stream);
   }
   if (exact) return idx64 ? launch_lookup_lean_i64_exact(a, (unsigned)blocks, stream) : launch_lookup_lean_i32_exact(a, (unsigned)blocks, stream);
   return idx64 ? launch_lookup_lean_i64_fast(a, (unsigned)blocks, stream) : launch_lookup_lean_i32_fast(a, (unsigned)blocks, stream);

@@ -559,7 +559,7 @@ __device__ __forceinline__ void lean_write(const LookupArgs& a, const TableDesc&
 // valid row its units are not loaded at all.)
 // Returns false (wave-uniform, nothing written) when a scale is too large for
 // the pre-scaled arithmetic.
-template <typename index_t, bool EXACT, int TY, int C, bool INHDR, int R, bool Q8>
+template <typename index_t, bool EXACT, int TY, int C, bool INHDR, int R, bool Q8, int UL_CAP = 4, bool HDR_EARLY = false>
 __device__ __forceinline__ bool pool_lean(const LookupArgs& a, const TableDesc& d, int table, int first_slot, int lane,
                                           uint32_t* lds) {
   constexpr bool QUANT = TY == ST_INT8 || TY == ST_INT4;
@@ -570,7 +570,8 @@ __device__ __forceinline__ bool pool_lean(const LookupArgs& a, const TableDesc& 
   // arithmetic (2.71 against 2.76 ms), except where the staging lanes hold 4 entries each and
   // fetch the row headers: their registers and 4-load units together do not fit the 168
   // registers that 3 waves per SIMD leave a lane.
-  constexpr int UL = !QUANT ? 4 : (EXACT || (R == 4 && !INHDR)) ? 2 : 4;
+  constexpr int UL_RULE = !QUANT ? 4 : (EXACT || (R == 4 && !INHDR)) ? 2 : 4;
+  constexpr int UL = UL_RULE < UL_CAP ? UL_RULE : UL_CAP;
   constexpr int HALF = UL / C;                                     // rows per unit
   constexpr int U = LEAN_BLOCK / HALF;                             // units per block
   constexpr int SL = LEAN_BLOCK / R;                               // staging lanes per bag
@@ -678,7 +679,7 @@ __device__ __forceinline__ bool pool_lean(const LookupArgs& a, const TableDesc& 
   // in the bit-exact mode with one entry per staging lane (eight or more lanes per bag) the
   // multipliers are wanted so soon after the short two-row units that the later request cost
   // 2 % where the merged requests saved 1 %.
-  constexpr bool HDRS_WITH_UNITS = !(TY == ST_INT8 && C == 2 && R >= 2) && !(EXACT && R == 1);
+  constexpr bool HDRS_WITH_UNITS = !(TY == ST_INT8 && C == 2 && R >= 2) && !(EXACT && R == 1) && !HDR_EARLY;
   auto issue_hdrs = [&]() {
     if constexpr (QUANT && !INHDR) {
 #pragma unroll
@@ -964,24 +965,21 @@ __device__ __forceinline__ void lean_dispatch(const LookupArgs& a, const TableDe
 #define FBGEMM_AMD_LEAN_MIN_WAVES 3 // waves per SIMD the register allocation must leave room for
 #endif
 
-// Same work list and workgroup -> XCD mapping as lookup_kernel.
-template <typename index_t, bool EXACT, bool Q8>
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(FBGEMM_AMD_LEAN_MIN_WAVES, 8))) void lookup_lean_kernel(const LookupArgs a) {
-  // 8 KB: while a bag is pooled, two buffers of staged rows (2 KB) and the multipliers (4 KB); at the end, the wave's output
-  __shared__ __attribute__((aligned(16))) uint32_t lds[LEAN_LDS_WORDS + MAX_GROUPS];
-  const int lane = threadIdx.x;
+// Same work list and workgroup -> XCD mapping as lookup_kernel. One wave per workgroup.
+// Returns false when the workgroup has no work item.
+__device__ __forceinline__ bool lean_work_item(const LookupArgs& a, int& table, int& first_slot) {
   int64_t wave;
   if (a.xcd_start) {
     const int xb = blockIdx.x & 7;
     const int64_t w = (int64_t)(blockIdx.x >> 3);
     const int64_t lo = a.xcd_start[xb], hi = a.xcd_start[xb + 1];
-    if (w >= hi - lo) return;
+    if (w >= hi - lo) return false;
     wave = lo + w;
   } else {
     wave = (int64_t)blockIdx.x;
-    if (wave >= a.num_waves) return;
+    if (wave >= a.num_waves) return false;
   }
-  int table = 0, first_slot;
+  table = 0;
   if (a.work) {
     const WaveWork ww = a.work[wave];
     table = ww.table;
@@ -989,13 +987,80 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(FBGEMM_AMD_L
   } else {
     first_slot = (int)(wave * a.single.bags);
   }
+  return true;
+}
+
+template <typename index_t, bool EXACT, bool Q8>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(FBGEMM_AMD_LEAN_MIN_WAVES, 8))) void lookup_lean_kernel(const LookupArgs a) {
+  // 8 KB: while a bag is pooled, two buffers of staged rows (2 KB) and the multipliers (4 KB); at the end, the wave's output
+  __shared__ __attribute__((aligned(16))) uint32_t lds[LEAN_LDS_WORDS + MAX_GROUPS];
+  int table, first_slot;
+  if (!lean_work_item(a, table, first_slot)) return;
   const TableDesc d = a.tables ? a.tables[table] : a.single;
-  lean_dispatch<index_t, EXACT, Q8>(a, d, table, first_slot, lane, lds);
+  lean_dispatch<index_t, EXACT, Q8>(a, d, table, first_slot, (int)threadIdx.x, lds);
+}
+
+// The instance for launches in which every table has 4-bit rows in bags of 8 lanes and more with
+// the header fetched by a staging lane (lean_wide4_shape): that one instantiation of pool_lean,
+// with units of 2 loads and the headers asked for at staging time, needs 125 (exact) / 123
+// (tolerance-grade) vector registers, so four waves fit a SIMD where the kernel above, which
+// carries every row type and lane count, fits three. 16 instead of 12 waves per compute unit
+// hide more of each other's waits: the HBM-sized configuration takes 8 % less in the exact mode
+// and 3 % less in the tolerance-grade mode.
+// The rare path (a scale too large for the pre-scaled arithmetic) is not part of this kernel:
+// inlined behind the common path it costs 30 registers more, and any spill makes every wave of
+// the kernel reserve scratch memory. A wave that meets such a scale writes nothing and queues its
+// work item; lookup_lean_wide4_redo_kernel, launched behind this kernel in every forward, pools
+// the queued items with pool_lean_slow (usually none: 256 workgroups that read a zero and leave).
+template <typename index_t, bool EXACT>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 8))) void lookup_lean_wide4_kernel(const LookupArgs a) {
+  __shared__ __attribute__((aligned(16))) uint32_t lds[LEAN_LDS_WORDS + MAX_GROUPS];
+  int table, first_slot;
+  if (!lean_work_item(a, table, first_slot)) return;
+  const TableDesc d = a.tables ? a.tables[table] : a.single;
+  const int lane = (int)threadIdx.x;
+  const bool done = pool_lean<index_t, EXACT, ST_INT4, 1, false, 1, false, 2, true>(a, d, table, first_slot, lane, lds);
+  if (!done && lane == 0) { // wave-uniform verdict; nothing has been written or reported
+    const int k = atomicAdd(a.redo_count, 1);
+    WaveWork ww;
+    ww.table = table;
+    ww.first_bag = first_slot;
+    a.redo[k] = ww;
+  }
+}
+
+constexpr int LEAN_REDO_WORKGROUPS = 256;
+template <typename index_t, bool EXACT>
+__global__ __launch_bounds__(64) void lookup_lean_wide4_redo_kernel(const LookupArgs a) {
+  __shared__ __attribute__((aligned(16))) uint32_t lds[LEAN_LDS_WORDS + MAX_GROUPS];
+  const int lane = (int)threadIdx.x;
+  const int count = __hip_atomic_load(a.redo_count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  // the ticket is taken once the count has arrived (its increment depends on it): whoever draws the
+  // last ticket knows that every workgroup of the launch holds its copy of the count
+  int ticket = 0;
+  if (lane == 0) ticket = atomicAdd(a.redo_count + 1, count >= 0 ? 1 : 2);
+  ticket = __builtin_amdgcn_readfirstlane(ticket);
+  for (int i = (int)blockIdx.x; i < count; i += (int)gridDim.x) {
+    const WaveWork ww = a.redo[i];
+    const TableDesc d = a.tables ? a.tables[ww.table] : a.single;
+    pool_lean_slow<index_t, EXACT, ST_INT4, 1, false, false>(a, d, ww.table, ww.first_bag, lane, lds);
+  }
+  if (ticket == (int)gridDim.x - 1 && lane == 0) { // for the next forward
+    a.redo_count[0] = 0;
+    a.redo_count[1] = 0;
+  }
 }
 
 #define FBGEMM_AMD_DEFINE_LEAN_LAUNCH(FN, INDEX_T, EXACT, Q8)                                            \
   hipError_t FN(const LookupArgs& a, unsigned blocks, hipStream_t stream) {                              \
     hipLaunchKernelGGL((lookup_lean_kernel<INDEX_T, EXACT, Q8>), dim3(blocks), dim3(64), 0, stream, a);  \
+    return hipGetLastError();                                                                            \
+  }
+
+#define FBGEMM_AMD_DEFINE_LEAN_WIDE4_LAUNCH(FN, INDEX_T, EXACT)                                           \
+  hipError_t FN(const LookupArgs& a, unsigned blocks, hipStream_t stream) {                              \
+    hipLaunchKernelGGL((lookup_lean_wide4_kernel<INDEX_T, EXACT>), dim3(blocks), dim3(64), 0, stream, a); \
+    hipLaunchKernelGGL((lookup_lean_wide4_redo_kernel<INDEX_T, EXACT>), dim3(LEAN_REDO_WORKGROUPS), dim3(64), 0, stream, a); \
     return hipGetLastError();                                                                            \
   }
 

@@ -18,7 +18,7 @@ import os
 import sys
 from collections import defaultdict
 
-OURS = ("lookup_lean_kernel", "split_offsets_kernel", "combine_segments_kernel", "gather_lines_lds_kernel", "gather_lines_kernel", "stream_read_kernel", "remap_rank_build", "inplace_update_kernel", "remap_row_idx_kernel", "sequence_lookup_kernel", "row_lookup_kernel", "pruned_array_lookup", "pruned_hashmap_lookup", "lookup_kernel",
+OURS = ("lookup_lean_wide4_redo_kernel", "lookup_lean_wide4_kernel", "lookup_lean_kernel", "split_offsets_kernel", "combine_segments_kernel", "gather_lines_lds_kernel", "gather_lines_kernel", "stream_read_kernel", "remap_rank_build", "inplace_update_kernel", "remap_row_idx_kernel", "sequence_lookup_kernel", "row_lookup_kernel", "pruned_array_lookup", "pruned_hashmap_lookup", "lookup_kernel",
         "calibration_copy_kernel", "float_to_hfp8_kernel", "hfp8_to_float_kernel", "prune_count", "prune_carry", "prune_remap",
         "prune_gather", "remap_count", "remap_move", "remap_offsets",
         "bag_order_kernel", "lengths_to_offsets", "bounds_partial_max", "bounds_carry", "bounds_fix_offsets",

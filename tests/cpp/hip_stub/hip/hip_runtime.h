@@ -52,5 +52,6 @@ void hip_stub_fail_malloc_after(long n);
 long hip_stub_live_allocations(void);
 long hip_stub_total_allocations(void);
 long hip_stub_launches(void);
+long hip_stub_wide4_launches(void); // launches of the lean kernel's four-waves-per-SIMD instance
 // A stream handle that stands for a caller's stream (never dereferenced).
 hipStream_t hip_stub_stream(int id);

@@ -15,7 +15,7 @@ namespace {
 std::mutex g_mu;
 std::set<void*> g_live;
 std::set<hipStream_t> g_capturing;
-std::atomic<long> g_total{0}, g_launches{0}, g_fail_after{-1};
+std::atomic<long> g_total{0}, g_launches{0}, g_fail_after{-1}, g_wide4{0};
 struct Obj { int kind; };
 } // namespace
 
@@ -111,6 +111,7 @@ long hip_stub_live_allocations(void) {
 }
 long hip_stub_total_allocations(void) { return g_total.load(); }
 long hip_stub_launches(void) { return g_launches.load(); }
+long hip_stub_wide4_launches(void) { return g_wide4.load(); }
 hipStream_t hip_stub_stream(int id) {
   static hipStubStream streams[16];
   return &streams[id & 15];
@@ -129,7 +130,15 @@ hipError_t launch_lookup(const LookupArgs& a, bool, hipStream_t) {
   if (a.rank_offsets) (void)*(volatile const int64_t*)&a.rank_offsets[0];
   return LAUNCHED();
 }
-hipError_t launch_lookup_lean(const LookupArgs& a, bool idx64, bool, hipStream_t s) { return launch_lookup(a, idx64, s); }
+hipError_t launch_lookup_lean(const LookupArgs& a, bool idx64, bool, bool wide4, hipStream_t s) {
+  if (wide4) { // the redo queue of that instance must be there, and as long as the work list
+    if (!a.redo || !a.redo_count) return hipErrorInvalidValue;
+    (void)*(volatile const int32_t*)&a.redo_count[1];
+    (void)*(volatile const int32_t*)&a.redo[a.num_waves - 1].first_bag;
+    ++g_wide4;
+  }
+  return launch_lookup(a, idx64, s);
+}
 hipError_t launch_lengths_to_offsets(const void*, bool, int64_t n, int64_t* offsets, hipStream_t) {
   for (int64_t i = 0; i <= n; ++i) offsets[i] = 0; // the whole buffer must be there
   return LAUNCHED();

@@ -276,9 +276,44 @@ void allocation_failures_in_a_first_forward() {
   }
 }
 
+// A plan whose tables all have 4-bit rows in bags of 8 lanes: forwards that order their bags take the
+// lean kernel's four-waves-per-SIMD instance, whose redo queue is made with every bag-order buffer
+// (three streams, allocation failures in between) and freed with the work set.
+void plan_of_wide_4bit_tables() {
+  Problem p;
+  p.T = 3;
+  int64_t off = 0;
+  p.D_offsets.push_back(0);
+  for (int t = 0; t < p.T; ++t) {
+    p.wo.push_back(off);
+    p.tys.push_back(3);
+    p.D_offsets.push_back(p.D_offsets.back() + 256);
+    off += (fbgemm_amd_padded_row_size_in_bytes(256, 3, 16, 4) * 100 + 127) / 128 * 128;
+  }
+  p.bytes = off;
+  // about 19 rows per bag: enough lookups for the bag order, bags too short for the end-to-end lane shapes
+  const int64_t big_n = 1 << 21, B = 36000;
+  Buffers b(p, B, big_n);
+  const long base = hip_stub_live_allocations();
+  for (long k = -1; k < 12; ++k) {
+    fbgemm_amd_tbe_plan* plan = nullptr;
+    CHECK(fbgemm_amd_tbe_plan_create(&plan, p.T, p.wo.data(), p.tys.data(), p.D_offsets.data(), nullptr, p.bytes, 0, 16) == 0);
+    hip_stub_fail_malloc_after(k);
+    (void)forward(plan, p, b, B, big_n, hip_stub_stream(0));
+    hip_stub_fail_malloc_after(-1);
+    for (int s = 0; s < 3; ++s) CHECK(forward(plan, p, b, B, big_n, hip_stub_stream(s)) == 0);
+    CHECK(forward(plan, p, b, B, big_n, hip_stub_stream(1), /*INT8 output*/ 2) == 0);
+    CHECK(forward(plan, p, b, 48, 100, hip_stub_stream(1)) == 0); // a small forward: no bag order, no queue
+    fbgemm_amd_tbe_plan_destroy(plan);
+    CHECK(hip_stub_live_allocations() == base);
+  }
+  CHECK(hip_stub_wide4_launches() >= 13 * 3); // the forwards above did take that instance
+}
+
 } // namespace
 
 int main() {
+  plan_of_wide_4bit_tables();
   plan_create_failures();
   work_list_cache_and_graphs();
   remappings_twice_and_split_bags();

@@ -562,6 +562,47 @@ def test_pooled_int8_output_at_a_size_the_lean_kernel_takes(ops, oracle, mixed):
             assert (block == want).all(), (mixed, pooling, w is not None, t, np.argwhere(block != want)[:4])
 
 
+@pytest.mark.parametrize("accumulate", ["exact", "fast"])
+def test_plan_of_wide_4bit_tables_with_scales_beyond_the_prescaled_range(ops, oracle, accumulate):
+    """A forward that orders its bags over tables that all have 4-bit rows in bags of 8 lanes and
+    more (D = 256 and 1024 at 16-byte row alignment, bags of about 15 rows): the lean kernel's
+    four-waves-per-SIMD instance. That instance does not carry the plain arithmetic: a wave that
+    meets weight x scale beyond 2^100 queues its bags for the kernel behind it. Some bags here have
+    per-sample weights of 2^110, one of them in the last wave of a table; the fp32 output matches
+    the oracle bit for bit in the exact mode and to the bound in the tolerance-grade mode, twice in a row (the queue's counters are set
+    back by every forward)."""
+    rng = np.random.default_rng(1370)
+    specs = [(4000, 256, INT4), (1500, 1024, INT4), (2500, 256, INT4)]
+    T, B = len(specs), 48_000
+    weights, wo, _ = build_weights(rng, specs, 16)
+    lens = rng.poisson(15, size=T * B)
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    assert int(off[-1]) >= 1 << 21
+    tys = np.array([s[2] for s in specs], np.uint8)
+    D_offsets = np.concatenate([[0], np.cumsum([s[1] for s in specs])]).astype(np.int32)
+    total_D = int(D_offsets[-1])
+    for rep in range(2):
+        idx = np.concatenate([rng.integers(0, specs[t][0], size=int(off[(t + 1) * B] - off[t * B])) for t in range(T)]).astype(np.int64)
+        psw = rng.uniform(0, 1, len(idx)).astype(np.float32)
+        huge = list(rng.integers(0, T * B, size=12)) + [B - 1, 2 * B - 1]
+        for b in huge:
+            psw[int(off[b]):int(off[b + 1])] = np.float32(2.0 ** 110)
+        got = ops.int_nbit_split_embedding_codegen_lookup_function(
+            cu(weights), torch.zeros(0, dtype=torch.uint8, device="cuda"), cu(np.zeros(T, np.int32)), cu(wo), cu(tys),
+            cu(D_offsets), total_D, 0, 1024, 0, 0, 0, cu(idx), cu(off), 0, cu(psw), FP32, row_alignment=16,
+            accumulate=ops.ACC_FAST if accumulate == "fast" else ops.ACC_EXACT).cpu().numpy()
+        rc, want = oracle.tbe_forward(weights, wo, tys, D_offsets, total_D, idx, off, 0, psw, FP32, 16)
+        assert rc == 0
+        if accumulate == "exact":
+            H.assert_same_bits(got, want, f"wide 4-bit plan, pass {rep}")
+        else:
+            from fbgemm_amd import tolerance
+            for t in range(T):
+                blk = slice(int(D_offsets[t]), int(D_offsets[t + 1]))
+                r = tolerance.grade(np.ascontiguousarray(got[:, blk]), np.ascontiguousarray(want[:, blk]), FP32, np)
+                assert r["ok"], (t, r)
+
+
 def test_int8_output_forwards_of_one_plan_on_two_streams(ops, oracle):
     """Forwards of one plan that go through the plan's float scratch (8-bit output of tables the
     lean kernel does not take) may be issued on different streams without ordering them: the
