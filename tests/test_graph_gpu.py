@@ -228,6 +228,69 @@ def test_int8_output_forward_replays_from_a_graph(oracle, mixed):
     assert st.read() == (0, -1)
 
 
+def test_wide_4bit_plan_with_its_redo_queue_replays_from_a_graph(oracle):
+    """A plan whose tables all have 4-bit rows in bags of 8 lanes: the lean kernel's four-waves-per-SIMD
+    instance and the kernel behind it that pools what that instance queues (bags with weight x scale
+    beyond the pre-scaled range). The queue's counters are set back by the second kernel itself, so a
+    captured forward replays: every replay draws new indices and moves the huge weights to other bags,
+    and is checked bit for bit against the oracle."""
+    assert torch.cuda.is_available()
+    from fbgemm_amd import ops
+    from test_tbe_gpu import build_weights
+    rng = np.random.default_rng(81)
+    specs = [(3000, 256, INT4), (2000, 256, INT4)]
+    T, B = len(specs), 72_000
+    weights, wo, _ = build_weights(rng, specs, 16)
+    tys = np.array([s[2] for s in specs], np.uint8)
+    D_offsets = np.concatenate([[0], np.cumsum([s[1] for s in specs])]).astype(np.int32)
+    total_D = int(D_offsets[-1])
+    lens = rng.poisson(15, size=T * B)
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    n = int(off[-1])
+    assert (1 << 21) <= n < 20 * T * B  # the bags are ordered; short enough to keep 8 lanes per bag
+
+    def draw():
+        idx = np.concatenate([rng.integers(0, specs[t][0], size=int(off[(t + 1) * B] - off[t * B])) for t in range(T)]).astype(np.int64)
+        w = rng.uniform(0, 1, n).astype(np.float32)
+        for b in rng.integers(0, T * B, size=9):
+            w[int(off[b]):int(off[b + 1])] = np.float32(2.0 ** 108)
+        return idx, w
+
+    idx, w = draw()
+    d_idx, d_off, d_w = cu(idx), cu(off), cu(w)
+    meta = (cu(weights), torch.zeros(0, dtype=torch.uint8, device="cuda"), cu(np.zeros(T, np.int32)), cu(wo), cu(tys), cu(D_offsets))
+    st = ops.Status()
+    call = lambda: ops.int_nbit_split_embedding_codegen_lookup_function(
+        *meta, total_D, 0, 256, 0, 0, 0, d_idx, d_off, 0, d_w, FP32, row_alignment=16, status=st)
+
+    def expect(idx, w):
+        rc, want = oracle.tbe_forward(weights, wo, tys, D_offsets, total_D, idx, off, 0, w, FP32, 16)
+        assert rc == 0
+        return want
+
+    eager = call()
+    torch.cuda.synchronize()
+    H.assert_same_bits(eager.cpu().numpy(), expect(idx, w), "eager")
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            captured = call()
+    torch.cuda.synchronize()
+    for replay in range(3):
+        idx, w = draw()
+        d_idx.copy_(cu(idx))
+        d_w.copy_(cu(w))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        H.assert_same_bits(captured.cpu().numpy(), expect(idx, w), f"replay {replay}")
+        again = call()
+        torch.cuda.synchronize()
+        assert torch.equal(again, captured)
+    assert st.read() == (0, -1)
+
+
 def test_mappings_changed_before_a_capture_are_refused(oracle):
     """Pruned-row mappings edited in place keep their address: a forward under stream capture cannot
     rebuild the plan's compact form of them (that allocates and synchronizes) and must not take the
