@@ -202,6 +202,39 @@ def test_rows_without_fast_arithmetic_stay_exact_with_long_bags(ops, oracle, ty)
                        f"table of ty={ty} in a fast-mode plan, long bags")
 
 
+def test_int8_pooled_output_of_split_bags(ops, oracle):
+    """The 8-bit pooled output of a tolerance-grade forward whose few, long bags are cut into
+    segments: partial sums, the ordered combine into the plan's float scratch, then the quantizer
+    over every (bag, table) block. The pooled floats are within the mode's bound of the oracle's, so
+    every dequantized element is within half a quantization step (plus that bound) of the oracle's
+    pooled value, and scale and bias are those of a vector within the bound."""
+    rng = np.random.default_rng(4242)
+    specs = [(500, 128, INT4), (300, 64, INT8), (700, 256, INT4)]
+    T, B, L = len(specs), 5, 400
+    weights, wo, tys, D_offsets, idx, off, _ = tbe_problem(rng, specs, B, L, 16, False)
+    total_D = int(D_offsets[-1])
+    maxd = lambda ty: max([s[1] for s in specs if s[2] == ty], default=0)
+    got = ops.int_nbit_split_embedding_codegen_lookup_function(
+        cu(weights), torch.zeros(0, dtype=torch.uint8, device="cuda"), cu(np.zeros(T, np.int32)), cu(wo), cu(tys),
+        cu(D_offsets), total_D, 0, maxd(INT4), maxd(INT8), 0, 0, cu(idx), cu(off), 0, None, INT8, row_alignment=16,
+        accumulate=ops.ACC_FAST).cpu().numpy()
+    assert got.shape == (B, total_D + 8 * T)
+    rc, pooled = oracle.tbe_forward(weights, wo, tys, D_offsets, total_D, idx, off, 0, None, FP32, 16)
+    assert rc == 0
+    for t in range(T):
+        D = specs[t][1]
+        block = got[:, D_offsets[t] + 8 * t:D_offsets[t] + 8 * t + D + 8]
+        want = pooled[:, D_offsets[t]:D_offsets[t + 1]].astype(np.float64)
+        scale = np.ascontiguousarray(block[:, D:D + 4]).view(np.float32).astype(np.float64)
+        bias = np.ascontiguousarray(block[:, D + 4:D + 8]).view(np.float32).astype(np.float64)
+        mag = np.abs(want).max(axis=1, keepdims=True)
+        rng_w = want.max(axis=1, keepdims=True) - want.min(axis=1, keepdims=True)
+        assert np.all(np.abs(bias - want.min(axis=1, keepdims=True)) <= 1e-5 * mag), t
+        assert np.all(np.abs(scale * 255.0 - rng_w) <= 4e-5 * mag), t
+        deq = block[:, :D].astype(np.float64) * scale + bias
+        assert np.all(np.abs(deq - want) <= 0.5 * scale + 4e-5 * mag), (t, np.abs(deq - want).max(), scale.max())
+
+
 def test_rebuilding_rank_records_leaves_the_split_bag_scratch_alone(ops, oracle):
     """A plan that has cut long bags into segments (plan-owned scratch) and is then given its
     pruned-row mappings twice: building the compact mappings again replaces only what was made
