@@ -15,10 +15,13 @@
 //  * entries are staged 8 per bag at a time whatever the round size, so a line
 //    of indices or per-sample weights is asked for at most twice instead of
 //    once per round of 2 or 4 rows;
-//  * a block in which every bag of the wave has all 8 rows (the normal case
-//    once bags are ordered by length) runs as straight-line code of its own;
-//    blocks with holes take a second, predicated copy of the code, so neither
-//    pays for the other;
+//  * the rows of a bag arrive through a software pipeline (pool_lean): units of
+//    2 or 4 sixteen-byte loads per lane in two register sets that take turns,
+//    the next block's row numbers staged in a second LDS buffer while the
+//    current block is added up; an entry that adds nothing loads a row the wave
+//    fetches anyway and carries the multiplier (-0, -0, -0), so no load needs a
+//    predicate. Blocks whose units all exist run a copy of the loop without
+//    conditions round the loads;
 //  * EXACT selects the arithmetic: true is the reference's sequence of
 //    roundings, acc = fma(scale, q, acc + bias) per element
 //    (src/RefImplementations.cc:1326-1333,1519-1527), bit-identical to the CPU
@@ -31,6 +34,10 @@
 //    row-at-a-time loop that converts integers to float before the fma. Both
 //    round identically; the slow one only has to be correct.
 //  * what is staged per entry is the row number (32 bits), not its byte offset.
+// Three kinds of kernel are made from this file: lookup_lean_kernel (every shape,
+// float output), its Q8 instances (the 8-bit pooled output quantized in the
+// output stage, lean_store_q8) and lookup_lean_wide4_kernel with its redo kernel
+// (one shape, four waves per SIMD).
 #pragma once
 #include "lookup_device.h"
 
