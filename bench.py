@@ -61,6 +61,10 @@ def parse():
                          "prints it under \"other_accumulate\" (--one-mode skips that)")
     ap.add_argument("--one-mode", "--no-exact", dest="other_mode", action="store_false",
                     help="do not also time the other accumulate mode")
+    ap.add_argument("--wide4", choices=["auto", "on", "off"], default="auto",
+                    help="large forwards whose lean tables all have 4-bit rows in bags of 8 lanes and more (config 5): the lean "
+                         "kernel's four-waves-per-SIMD instance always / never, or (auto, the library's default) whichever of the "
+                         "two kernels the first forwards measure as the faster one")
     ap.add_argument("--int8-output", action="store_true",
                     help="table-batched configurations: the operator's 8-bit pooled output ([B, total_D + 8 T]: every table's "
                          "pooled vector quantized row-wise in the lookup's output stage) instead of the configuration's float "
@@ -803,6 +807,7 @@ def time_tbe(p, a, torch, np, steps, warmup, graph, accumulate):
     from fbgemm_amd import _lib
     if a.int8_output:
         assert not a.check and not a.other_mode, "--int8-output needs --no-check --one-mode"
+    _lib.check(_lib.lib().fbgemm_amd_set_wide4({"auto": -1, "on": 2, "off": 0}[getattr(a, "wide4", "auto")]))
     launch, out, st, plan = tbe_runner(p, torch, accumulate, not a.no_rank_records, a.int8_output)
     torch.cuda.synchronize()
     checked = parity_gate(p, out, launch, torch, np, accumulate) if a.check else None

@@ -73,6 +73,7 @@ SYMBOLS = {
 BENCH_SWITCHES = {
     "fbgemm_amd_set_lean": (C.c_int, [_I32]),
     "fbgemm_amd_set_narrow_below_waves": (C.c_int, [_I32]),
+    "fbgemm_amd_set_wide4": (C.c_int, [_I32]),
     "fbgemm_amd_tbe_plan_reuse_order": (C.c_int, [_P, _I32]),
 }
 # ... and the yardsticks of libfbgemm_amd_bench.so

@@ -209,10 +209,17 @@ bool lean_shape(const TableDesc& d) {
 
 // Shapes of the lean kernel's four-waves-per-SIMD instance (lookup_lean_wide4_kernel): 4-bit rows,
 // bags of 8 lanes and more (one entry per staging lane), the header fetched by a staging lane.
-// FBGEMM_AMD_WIDE4=0 keeps such launches on the general-purpose lean kernel.
 bool lean_wide4_shape(const TableDesc& d) {
-  static const int enabled = env_int("FBGEMM_AMD_WIDE4", 1);
-  return enabled && lean_shape(d) && d.ty == ST_INT4 && d.lanes >= 8 && !d.inline_hdr;
+  return lean_shape(d) && d.ty == ST_INT4 && d.lanes >= 8 && !d.inline_hdr;
+}
+// When forwards that could take that instance do: 0 never, 2 always, 1 (default) whichever of
+// the two kernels the first forwards of a work set measure as the faster one (FBGEMM_AMD_WIDE4 at
+// load time; fbgemm_amd_set_wide4 for tests and benchmarks).
+int g_wide4_override = -1;
+int wide4_mode() {
+  static const int dflt = env_int("FBGEMM_AMD_WIDE4", 1);
+  const int m = g_wide4_override >= 0 ? g_wide4_override : dflt;
+  return m < 0 ? 0 : (m > 2 ? 2 : m);
 }
 
 struct DeviceScratch {
@@ -631,6 +638,11 @@ int fbgemm_amd_set_narrow_below_waves(int32_t waves) {
   return 0;
 }
 
+int fbgemm_amd_set_wide4(int32_t mode) {
+  g_wide4_override = mode < 0 ? -1 : (mode > 2 ? 2 : mode);
+  return 0;
+}
+
 int fbgemm_amd_set_lean(int32_t on) {
   g_lean_override = on < 0 ? -1 : (on != 0);
   return 0;
@@ -741,6 +753,18 @@ struct fbgemm_amd_tbe_plan {
     // and two counters that are zero between forwards
     WaveWork* d_redo[ORDER_SLOTS] = {nullptr, nullptr, nullptr, nullptr};
     int32_t* d_redo_count[ORDER_SLOTS] = {nullptr, nullptr, nullptr, nullptr};
+    // Which of the two lean kernels the set's forwards take when both can (wide4_mode() == 1):
+    // the first forwards outside a capture run them in turn between two events and wait for the
+    // second one (eight forwards of a new batch size that synchronize, like the first one, which
+    // allocates); the first sample of each kernel is dropped, and after three more of each the
+    // faster one stays (a tie goes to the general-purpose kernel, which is one launch less). Both
+    // compute the same bits.
+    int w4_decided = -1;            // -1: still measuring; 0 / 1: the general-purpose kernel / the four-wave instance
+    int w4_seen[2] = {0, 0};        // measurements started, per kernel
+    int w4_samples[2] = {0, 0};     // measurements kept
+    float w4_ms[2] = {0.0f, 0.0f};  // their sum
+    bool w4_busy = false;           // a forward is measuring (one at a time: the two events are the set's)
+    hipEvent_t w4_ev[2] = {nullptr, nullptr};
     bool pinned = false;         // used by a forward under stream capture: a graph may hold its pointers
     uint64_t last_use = 0;
   };
@@ -800,6 +824,10 @@ void free_work(fbgemm_amd_tbe_plan::Work& w) {
     if (w.side_stream[k]) (void)hipStreamDestroy(w.side_stream[k]);
     w.side_fork[k] = w.side_join[k] = nullptr;
     w.side_stream[k] = nullptr;
+  }
+  for (int k = 0; k < 2; ++k) {
+    if (w.w4_ev[k]) (void)hipEventDestroy(w.w4_ev[k]);
+    w.w4_ev[k] = nullptr;
   }
   if (w.d_general_tables) (void)hipFree(w.d_general_tables);
   w.d_general_tables = nullptr;
@@ -1216,6 +1244,8 @@ int tbe_forward_impl(
   const RankRecord* rank_records = nullptr;
   const int64_t* rank_offsets = nullptr;
   bool reuse_order = false;
+  bool use_w4 = false;  // the lean tables take the four-waves-per-SIMD instance
+  int measure_w4 = -1;  // >= 0: this forward times its lean kernel (0 / 1: which one) for the work set's choice
   {
     std::lock_guard<std::mutex> lk(plan->mu);
     // the lane shapes depend on B and (through the average bag length) on the number of indices:
@@ -1258,6 +1288,8 @@ int tbe_forward_impl(
       } undo{&nw};
       nw.lean_wide4 = !lean_members.empty();
       for (int t : lean_members) nw.lean_wide4 = nw.lean_wide4 && lean_wide4_shape(tables[(size_t)t]);
+      if (nw.lean_wide4)
+        for (int k = 0; k < 2; ++k) HIP_TRY(hipEventCreateWithFlags(&nw.w4_ev[k], hipEventDefault));
       if (int rc = build_work_list(tables, lean_members, B, &nw.lean)) return rc;
       if (int rc = build_work_list(tables, general_members, B, &nw.general)) return rc;
       if (!general_members.empty()) {
@@ -1335,6 +1367,21 @@ int tbe_forward_impl(
         (void)hipGetLastError();
       }
     }
+    // the lean kernel of this forward, where there is a choice
+    if (W.lean_wide4 && !d_q8_out && W.d_redo[order_slot] && W.d_redo_count[order_slot] && sort_bags_default() &&
+        indices_numel >= (int64_t)SORT_MIN_LOOKUPS) {
+      const int mode = wide4_mode();
+      if (mode == 2) {
+        use_w4 = true;
+      } else if (mode == 1 && W.w4_decided >= 0) {
+        use_w4 = W.w4_decided == 1;
+      } else if (mode == 1 && !capturing && W.w4_ev[0] && W.w4_ev[1] && !W.w4_busy) {
+        measure_w4 = W.w4_seen[0] <= W.w4_seen[1] ? 0 : 1;
+        W.w4_seen[measure_w4] += 1;
+        W.w4_busy = true;
+        use_w4 = measure_w4 == 1;
+      }
+    }
     w = W;
     exact = plan->accumulate != FBGEMM_AMD_ACC_FAST;
     if (d_index_remappings && plan->d_rank_records && plan->rank_source == d_index_remappings && plan->rank_bits == remap_bits) {
@@ -1345,6 +1392,32 @@ int tbe_forward_impl(
     reuse_order = plan->reuse_order;
   }
 
+  // a forward that times its lean kernel: when it leaves it waits for the second event, adds the
+  // sample to the set's statistics, decides when there are enough, and gives the turn back
+  struct Measuring {
+    fbgemm_amd_tbe_plan* plan;
+    fbgemm_amd_tbe_plan::WorkKey key;
+    hipEvent_t start, stop;
+    int which;
+    bool recorded = false;
+    ~Measuring() {
+      if (which < 0) return;
+      float ms = 0.0f;
+      const bool have = recorded && hipEventSynchronize(stop) == hipSuccess && hipEventElapsedTime(&ms, start, stop) == hipSuccess && ms > 0.0f;
+      if (!have) (void)hipGetLastError();
+      std::lock_guard<std::mutex> lk(plan->mu);
+      auto it = plan->work.find(key);
+      if (it == plan->work.end() || it->second.w4_ev[1] != stop) return; // the set has been dropped meanwhile
+      fbgemm_amd_tbe_plan::Work& W = it->second;
+      W.w4_busy = false;
+      if (have && W.w4_seen[which] > 1) { // the first sample of each kernel is not kept
+        W.w4_ms[which] += ms;
+        W.w4_samples[which] += 1;
+      }
+      if (W.w4_decided < 0 && W.w4_samples[0] >= 3 && W.w4_samples[1] >= 3)
+        W.w4_decided = W.w4_ms[1] / (float)W.w4_samples[1] < 0.99f * W.w4_ms[0] / (float)W.w4_samples[0] ? 1 : 0;
+    }
+  } measuring{plan, fbgemm_amd_tbe_plan::WorkKey{B, variant, lean ? 1 : 0}, w.w4_ev[0], w.w4_ev[1], measure_w4};
   if (d_q8_out && w.general.num_waves > 0) {
     if (int rc = shared.begin(plan, stream)) return rc;
     float* tmp = nullptr;
@@ -1410,12 +1483,15 @@ int tbe_forward_impl(
     }
     // the four-waves-per-SIMD instance: forwards that order their bags (large ones: its second,
     // usually idle launch does not show there), float output
-    const bool wide4 = w.lean_wide4 && !d_q8_out && a.order && w.d_redo[order_slot] && w.d_redo_count[order_slot];
+    const bool wide4 = use_w4 && a.order;
     if (wide4) {
       l.redo = w.d_redo[order_slot];
       l.redo_count = w.d_redo_count[order_slot];
     }
-    HIP_TRY(launch_lookup_lean(l, index_bits == 64, exact, wide4, stream));
+    if (measure_w4 >= 0) (void)hipEventRecord(w.w4_ev[0], stream);
+    const hipError_t launched = launch_lookup_lean(l, index_bits == 64, exact, wide4, stream);
+    if (measure_w4 >= 0 && launched == hipSuccess && hipEventRecord(w.w4_ev[1], stream) == hipSuccess) measuring.recorded = true;
+    HIP_TRY(launched);
   }
   if (w.general.num_waves > 0) {
     if (side) HIP_TRY(hipStreamWaitEvent(stream, w.side_join[order_slot], 0));

@@ -51,9 +51,15 @@ int fbgemm_amd_bench_gather(const void* d_table, int64_t rows, int64_t row_strid
  * through the general kernel, -1 = back to the default.
  * fbgemm_amd_set_narrow_below_waves: launches of fewer waves than this take
  * 4-byte lanes (default 1024, FBGEMM_AMD_NARROW_BELOW_WAVES at load time; -1 =
- * back to the default). */
+ * back to the default).
+ * fbgemm_amd_set_wide4: which lean kernel large forwards take whose lean tables
+ * all have 4-bit rows in bags of 8 lanes and more: 0 = the general-purpose one,
+ * 2 = the four-waves-per-SIMD instance, 1 = whichever the first forwards of a
+ * batch size measure as the faster (the default, FBGEMM_AMD_WIDE4 at load
+ * time), -1 = back to the default. */
 int fbgemm_amd_set_lean(int32_t on);
 int fbgemm_amd_set_narrow_below_waves(int32_t waves);
+int fbgemm_amd_set_wide4(int32_t mode);
 
 /* Timing of the lookup kernels alone: while `on` is 1, forwards of the plan skip
  * the bag scheduler and take the bag order the last forward on the same stream

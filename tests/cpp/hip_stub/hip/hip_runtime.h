@@ -21,7 +21,7 @@ typedef struct hipStubStream* hipStream_t;
 typedef struct hipStubEvent* hipEvent_t;
 enum hipMemcpyKind { hipMemcpyHostToHost = 0, hipMemcpyHostToDevice = 1, hipMemcpyDeviceToHost = 2, hipMemcpyDeviceToDevice = 3 };
 enum hipStreamCaptureStatus { hipStreamCaptureStatusNone = 0, hipStreamCaptureStatusActive = 1 };
-enum : unsigned { hipStreamNonBlocking = 1, hipEventDisableTiming = 2 };
+enum : unsigned { hipStreamNonBlocking = 1, hipEventDisableTiming = 2, hipEventDefault = 0 };
 
 hipError_t hipMalloc(void** p, size_t bytes);
 hipError_t hipFree(void* p);
@@ -40,6 +40,8 @@ hipError_t hipStreamWaitEvent(hipStream_t stream, hipEvent_t event, unsigned fla
 hipError_t hipEventCreateWithFlags(hipEvent_t* event, unsigned flags);
 hipError_t hipEventDestroy(hipEvent_t event);
 hipError_t hipEventRecord(hipEvent_t event, hipStream_t stream);
+hipError_t hipEventSynchronize(hipEvent_t event);
+hipError_t hipEventElapsedTime(float* ms, hipEvent_t start, hipEvent_t stop);
 hipError_t hipGetSymbolAddressStub(void** p, const void* symbol);
 #define hipGetSymbolAddress(p, sym) hipGetSymbolAddressStub((p), (const void*)(sym))
 
@@ -53,5 +55,8 @@ long hip_stub_live_allocations(void);
 long hip_stub_total_allocations(void);
 long hip_stub_launches(void);
 long hip_stub_wide4_launches(void); // launches of the lean kernel's four-waves-per-SIMD instance
+// what hipEventElapsedTime reports from now on: `general_ms` for a measurement of a forward whose last lean launch was
+// the general-purpose kernel, `wide4_ms` for one of the four-wave instance
+void hip_stub_set_elapsed_ms(float general_ms, float wide4_ms);
 // A stream handle that stands for a caller's stream (never dereferenced).
 hipStream_t hip_stub_stream(int id);

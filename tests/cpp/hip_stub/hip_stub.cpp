@@ -16,6 +16,8 @@ std::mutex g_mu;
 std::set<void*> g_live;
 std::set<hipStream_t> g_capturing;
 std::atomic<long> g_total{0}, g_launches{0}, g_fail_after{-1}, g_wide4{0};
+std::atomic<int> g_last_lean_wide4{0};
+std::atomic<float> g_elapsed_general{1.0f}, g_elapsed_wide4{1.0f};
 struct Obj { int kind; };
 } // namespace
 
@@ -94,6 +96,18 @@ hipError_t hipEventRecord(hipEvent_t event, hipStream_t) {
   event->id++; // touches the event: a destroyed one is the sanitizer's to report
   return hipSuccess;
 }
+hipError_t hipEventSynchronize(hipEvent_t event) {
+  if (!event) return hipErrorInvalidValue;
+  (void)event->id;
+  return hipSuccess;
+}
+hipError_t hipEventElapsedTime(float* ms, hipEvent_t start, hipEvent_t stop) {
+  if (!start || !stop) return hipErrorInvalidValue;
+  (void)start->id;
+  (void)stop->id;
+  *ms = g_last_lean_wide4.load() ? g_elapsed_wide4.load() : g_elapsed_general.load();
+  return hipSuccess;
+}
 hipError_t hipGetSymbolAddressStub(void** p, const void* symbol) {
   *p = const_cast<void*>(symbol);
   return hipSuccess;
@@ -112,6 +126,10 @@ long hip_stub_live_allocations(void) {
 long hip_stub_total_allocations(void) { return g_total.load(); }
 long hip_stub_launches(void) { return g_launches.load(); }
 long hip_stub_wide4_launches(void) { return g_wide4.load(); }
+void hip_stub_set_elapsed_ms(float general_ms, float wide4_ms) {
+  g_elapsed_general = general_ms;
+  g_elapsed_wide4 = wide4_ms;
+}
 hipStream_t hip_stub_stream(int id) {
   static hipStubStream streams[16];
   return &streams[id & 15];
@@ -137,6 +155,7 @@ hipError_t launch_lookup_lean(const LookupArgs& a, bool idx64, bool, bool wide4,
     (void)*(volatile const int32_t*)&a.redo[a.num_waves - 1].first_bag;
     ++g_wide4;
   }
+  g_last_lean_wide4 = wide4 ? 1 : 0;
   return launch_lookup(a, idx64, s);
 }
 hipError_t launch_lengths_to_offsets(const void*, bool, int64_t n, int64_t* offsets, hipStream_t) {

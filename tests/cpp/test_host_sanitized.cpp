@@ -295,6 +295,7 @@ void plan_of_wide_4bit_tables() {
   const int64_t big_n = 1 << 21, B = 36000;
   Buffers b(p, B, big_n);
   const long base = hip_stub_live_allocations();
+  CHECK(fbgemm_amd_set_wide4(2) == 0); // always that instance
   for (long k = -1; k < 12; ++k) {
     fbgemm_amd_tbe_plan* plan = nullptr;
     CHECK(fbgemm_amd_tbe_plan_create(&plan, p.T, p.wo.data(), p.tys.data(), p.D_offsets.data(), nullptr, p.bytes, 0, 16) == 0);
@@ -308,6 +309,26 @@ void plan_of_wide_4bit_tables() {
     CHECK(hip_stub_live_allocations() == base);
   }
   CHECK(hip_stub_wide4_launches() >= 13 * 3); // the forwards above did take that instance
+  // The default: the first forwards of a batch size time the two kernels in turn (waiting for the second event),
+  // then the faster one stays. Under capture nothing is measured.
+  CHECK(fbgemm_amd_set_wide4(-1) == 0);
+  for (int faster = 0; faster < 2; ++faster) {
+    hip_stub_set_elapsed_ms(1.0f, faster ? 0.5f : 0.995f); // the four-wave instance has to win by 1 %
+    fbgemm_amd_tbe_plan* plan = nullptr;
+    CHECK(fbgemm_amd_tbe_plan_create(&plan, p.T, p.wo.data(), p.tys.data(), p.D_offsets.data(), nullptr, p.bytes, 0, 16) == 0);
+    CHECK(forward(plan, p, b, B, big_n, hip_stub_stream(0)) == 0);
+    hip_stub_set_capturing(hip_stub_stream(1), true);
+    const long before_capture = hip_stub_wide4_launches();
+    CHECK(forward(plan, p, b, B, big_n, hip_stub_stream(1)) == 0); // undecided and capturing: the general-purpose kernel
+    CHECK(hip_stub_wide4_launches() == before_capture);
+    hip_stub_set_capturing(hip_stub_stream(1), false);
+    for (int i = 0; i < 24; ++i) CHECK(forward(plan, p, b, B, big_n, hip_stub_stream(i % 3)) == 0);
+    const long settled = hip_stub_wide4_launches();
+    for (int i = 0; i < 6; ++i) CHECK(forward(plan, p, b, B, big_n, hip_stub_stream(i % 3)) == 0);
+    CHECK(hip_stub_wide4_launches() - settled == (faster ? 6 : 0));
+    fbgemm_amd_tbe_plan_destroy(plan);
+    CHECK(hip_stub_live_allocations() == base);
+  }
 }
 
 } // namespace

@@ -228,15 +228,19 @@ def test_int8_output_forward_replays_from_a_graph(oracle, mixed):
     assert st.read() == (0, -1)
 
 
-def test_wide_4bit_plan_with_its_redo_queue_replays_from_a_graph(oracle):
+def test_wide_4bit_plan_with_its_redo_queue_replays_from_a_graph(oracle, request):
     """A plan whose tables all have 4-bit rows in bags of 8 lanes: the lean kernel's four-waves-per-SIMD
     instance and the kernel behind it that pools what that instance queues (bags with weight x scale
     beyond the pre-scaled range). The queue's counters are set back by the second kernel itself, so a
     captured forward replays: every replay draws new indices and moves the huge weights to other bags,
     and is checked bit for bit against the oracle."""
     assert torch.cuda.is_available()
+    import fbgemm_amd
     from fbgemm_amd import ops
     from test_tbe_gpu import build_weights
+    lib = fbgemm_amd.lib()
+    lib.fbgemm_amd_set_wide4(2)  # that instance, not whichever the first forwards find faster
+    request.addfinalizer(lambda: lib.fbgemm_amd_set_wide4(-1))
     rng = np.random.default_rng(81)
     specs = [(3000, 256, INT4), (2000, 256, INT4)]
     T, B = len(specs), 72_000

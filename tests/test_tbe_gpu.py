@@ -563,7 +563,7 @@ def test_pooled_int8_output_at_a_size_the_lean_kernel_takes(ops, oracle, mixed):
 
 
 @pytest.mark.parametrize("accumulate", ["exact", "fast"])
-def test_plan_of_wide_4bit_tables_with_scales_beyond_the_prescaled_range(ops, oracle, accumulate):
+def test_plan_of_wide_4bit_tables_with_scales_beyond_the_prescaled_range(ops, oracle, accumulate, request):
     """A forward that orders its bags over tables that all have 4-bit rows in bags of 8 lanes and
     more (D = 256 and 1024 at 16-byte row alignment, bags of about 15 rows): the lean kernel's
     four-waves-per-SIMD instance. That instance does not carry the plain arithmetic: a wave that
@@ -571,6 +571,8 @@ def test_plan_of_wide_4bit_tables_with_scales_beyond_the_prescaled_range(ops, or
     per-sample weights of 2^110, one of them in the last wave of a table; the fp32 output matches
     the oracle bit for bit in the exact mode and to the bound in the tolerance-grade mode, twice in a row (the queue's counters are set
     back by every forward)."""
+    import fbgemm_amd
+    lib = fbgemm_amd.lib()
     rng = np.random.default_rng(1370)
     specs = [(4000, 256, INT4), (1500, 1024, INT4), (2500, 256, INT4)]
     T, B = len(specs), 48_000
@@ -581,6 +583,8 @@ def test_plan_of_wide_4bit_tables_with_scales_beyond_the_prescaled_range(ops, or
     tys = np.array([s[2] for s in specs], np.uint8)
     D_offsets = np.concatenate([[0], np.cumsum([s[1] for s in specs])]).astype(np.int32)
     total_D = int(D_offsets[-1])
+    lib.fbgemm_amd_set_wide4(2)  # that instance, not whichever the first forwards find faster
+    request.addfinalizer(lambda: lib.fbgemm_amd_set_wide4(-1))
     for rep in range(2):
         idx = np.concatenate([rng.integers(0, specs[t][0], size=int(off[(t + 1) * B] - off[t * B])) for t in range(T)]).astype(np.int64)
         psw = rng.uniform(0, 1, len(idx)).astype(np.float32)
@@ -601,6 +605,31 @@ def test_plan_of_wide_4bit_tables_with_scales_beyond_the_prescaled_range(ops, or
                 blk = slice(int(D_offsets[t]), int(D_offsets[t + 1]))
                 r = tolerance.grade(np.ascontiguousarray(got[:, blk]), np.ascontiguousarray(want[:, blk]), FP32, np)
                 assert r["ok"], (t, r)
+
+
+def test_wide_4bit_plan_settles_on_one_of_its_two_lean_kernels(ops, oracle):
+    """By default the first forwards of such a plan (per batch size) run the general-purpose lean
+    kernel and the four-waves-per-SIMD instance in turn, timed by events, and then stay with the
+    faster one. Both compute the same bits: twenty forwards of the same inputs, each equal to the
+    oracle's result, whatever kernel it took."""
+    rng = np.random.default_rng(1371)
+    specs = [(4000, 256, INT4), (2500, 256, INT4)]
+    T, B = len(specs), 72_000
+    weights, wo, _ = build_weights(rng, specs, 16)
+    lens = rng.poisson(15, size=T * B)
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    assert (1 << 21) <= int(off[-1]) < 20 * T * B
+    idx = np.concatenate([rng.integers(0, specs[t][0], size=int(off[(t + 1) * B] - off[t * B])) for t in range(T)]).astype(np.int64)
+    tys = np.array([s[2] for s in specs], np.uint8)
+    D_offsets = np.concatenate([[0], np.cumsum([s[1] for s in specs])]).astype(np.int32)
+    total_D = int(D_offsets[-1])
+    args = (cu(weights), torch.zeros(0, dtype=torch.uint8, device="cuda"), cu(np.zeros(T, np.int32)), cu(wo), cu(tys),
+            cu(D_offsets), total_D, 0, 256, 0, 0, 0, cu(idx), cu(off), 0, None, FP16)
+    rc, want = oracle.tbe_forward(weights, wo, tys, D_offsets, total_D, idx, off, 0, None, FP16, 16)
+    assert rc == 0
+    for k in range(20):
+        got = ops.int_nbit_split_embedding_codegen_lookup_function(*args, row_alignment=16)
+        H.assert_same_bits(got.cpu().view(torch.int16).numpy().view(np.uint16), want, f"forward {k}")
 
 
 def test_int8_output_forwards_of_one_plan_on_two_streams(ops, oracle):
