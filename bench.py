@@ -134,13 +134,18 @@ def profile_kernel_us(config_id):
     path = os.path.join(ROOT, "profiles", f"lookup_kernel_config{config_id}.txt")
     if not os.path.exists(path):
         return None
-    vals = dict(re.findall(r"stats\s+(\w+)(?:<\w+>)?: calls=\d+ avg_ns=([0-9.e+]+)", open(path).read()))
-    lean = [float(vals[k]) for k in LOOKUP_KERNELS[:-1] if k in vals]
-    general = float(vals.get("lookup_kernel", 0.0))
+    rows = re.findall(r"stats\s+(\w+)(?:<\w+>)?: calls=(\d+) avg_ns=([0-9.e+]+)", open(path).read())
+    calls = {k: int(c) for k, c, _ in rows}
+    total = {k: int(c) * float(v) for k, c, v in rows}
+    # every forward launches one of the two lean kernels (the trace holds both while the plan is still
+    # choosing between them); the redo kernel goes with the four-wave instance
+    forwards = calls.get("lookup_lean_kernel", 0) + calls.get("lookup_lean_wide4_kernel", 0)
+    lean = sum(total.get(k, 0.0) for k in LOOKUP_KERNELS[:-1]) / forwards if forwards else 0.0
+    general = total.get("lookup_kernel", 0.0) / calls["lookup_kernel"] if calls.get("lookup_kernel") else 0.0
     if not lean and not general:
         return None
     # with kernels of both kinds the general one runs beside the lean one (side stream): the longer of the two
-    return round(max(sum(lean), general) / 1e3, 2)
+    return round(max(lean, general) / 1e3, 2)
 
 
 def tbe_runner(p, torch, accumulate="exact", rank_records=True, int8_output=False):
