@@ -374,7 +374,9 @@ __device__ __forceinline__ void lean_q8_from_lds(const LookupArgs& a, const Tabl
   const int S = d.lanes, D = d.D;
   const int base = (int)threadIdx.x - L.sub; // first lane of the bag
   const float* mine = pooled + (size_t)L.grp * D;
-  const int nq = D >> 2; // whole groups of 4 columns; the D & 3 columns behind them are lane 0's
+  // whole groups of 4 columns, read as 16 bytes (every bag's floats start at a multiple of 16 bytes
+  // when D is a multiple of 4; otherwise all columns are lane 0's, one by one)
+  const int nq = (D & 3) == 0 ? D >> 2 : 0;
   float lo = __builtin_inff(), hi = -__builtin_inff();
   auto see = [&](float x) {
     lo = x < lo ? x : lo;
@@ -475,7 +477,7 @@ __device__ __forceinline__ void lean_store_q8(const LookupArgs& a, const TableDe
     for (int e = 0; e < E; e += 4) {
       const int col = col0 + e;
       if (!L.bag_ok || L.idle) continue;
-      if (col >= 0 && col + 4 <= D) {
+      if (col >= 0 && col + 4 <= D && (D & 3) == 0) {
         *reinterpret_cast<float4*>(mine + col) = make_float4(acc[c * E + e], acc[c * E + e + 1], acc[c * E + e + 2], acc[c * E + e + 3]);
       } else {
 #pragma unroll

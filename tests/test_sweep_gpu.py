@@ -130,7 +130,10 @@ def int8_output_case(ops, oracle, seed):
     specs = []
     for _ in range(T):
         ty = int(rng.choice([INT8, INT4, INT4, INT2, FP16, FP32]))
-        specs.append((int(rng.integers(1, 300)), int(rng.choice(DIMS_BATCHED)), ty))
+        D = int(rng.choice(DIMS_BATCHED))
+        if ty in (INT8, INT4, FP16) and rng.random() < 0.25:
+            D = int(rng.choice([2, 6, 10, 14, 18, 26, 30, 38, 50, 70]))  # widths that are not a multiple of 4
+        specs.append((int(rng.integers(1, 300)), D, ty))
     align = int(rng.choice([16, 16, 1, 4]))
     weights, wo, _ = TB.build_weights(rng, specs, align)
     max_len = int(rng.choice([3, 10, 45]))
