@@ -174,7 +174,7 @@ hipError_t launch_lookup_lean(const LookupArgs& a, bool idx64, bool exact, bool 
     return idx64 ? launch_lookup_lean_i64_fast_q8(a, (unsigned)blocks, stream) : launch_lookup_lean_i32_fast_q8(a, (unsigned)blocks, stream);
   }
   if (wide4) { // two launches: the kernel, and the one that pools what it has queued
-    if (!a.redo || !a.redo_count) return hipErrorInvalidValue;
+    if (!a.redo || !a.redo_count || !a.tables) return hipErrorInvalidValue;
     if (exact) return idx64 ? launch_lookup_lean_i64_exact_w4(a, (unsigned)blocks, stream) : launch_lookup_lean_i32_exact_w4(a, (unsigned)blocks, stream);
     return idx64 ? launch_lookup_lean_i64_fast_w4(a, (unsigned)blocks, stream) : launch_lookup_lean_i32_fast_w4(a, (unsigned)blocks, stream);
   }

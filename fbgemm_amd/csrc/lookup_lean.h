@@ -1009,13 +1009,16 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(FBGEMM_AMD_L
   lean_dispatch<index_t, EXACT, Q8>(a, d, table, first_slot, (int)threadIdx.x, lds);
 }
 
-// The instance for launches in which every table has 4-bit rows in bags of 8 lanes and more with
-// the header fetched by a staging lane (lean_wide4_shape): that one instantiation of pool_lean,
-// with units of 2 loads and the headers asked for at staging time, needs 125 (exact) / 123
-// (tolerance-grade) vector registers, so four waves fit a SIMD where the kernel above, which
-// carries every row type and lane count, fits three. 16 instead of 12 waves per compute unit
-// hide more of each other's waits: the HBM-sized configuration takes 8 % less in the exact mode
-// and 3 % less in the tolerance-grade mode.
+// The instance for table-batched launches in which every table has 4-bit rows in bags of 8 lanes
+// and more with the header fetched by a staging lane (lean_wide4_shape): that one instantiation
+// of pool_lean (in the exact mode with units of 2 loads and the headers asked for at staging
+// time, as in the kernel above; in the tolerance-grade mode with units of 4 and the headers next
+// to their rows) needs 114 / 127 vector registers, so four waves fit a SIMD where the kernel
+// above, which carries every row type and lane count, fits three. 16 instead of 12 waves per
+// compute unit hide more of each other's waits: the HBM-sized configuration takes 14 % less in
+// the exact mode and 8 % less in the tolerance-grade mode. (The table's descriptor is read from
+// the device array only: the choice between that and the single-table descriptor of the
+// launch arguments alone costs the registers that make the difference between 127 and a spill.)
 // The rare path (a scale too large for the pre-scaled arithmetic) is not part of this kernel:
 // inlined behind the common path it costs 30 registers more, and any spill makes every wave of
 // the kernel reserve scratch memory. A wave that meets such a scale writes nothing and queues its
@@ -1026,9 +1029,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 8))) void
   __shared__ __attribute__((aligned(16))) uint32_t lds[LEAN_LDS_WORDS + MAX_GROUPS];
   int table, first_slot;
   if (!lean_work_item(a, table, first_slot)) return;
-  const TableDesc d = a.tables ? a.tables[table] : a.single;
+  const TableDesc d = a.tables[table]; // table-batched launches only
   const int lane = (int)threadIdx.x;
-  const bool done = pool_lean<index_t, EXACT, ST_INT4, 1, false, 1, false, 2, true>(a, d, table, first_slot, lane, lds);
+  const bool done = pool_lean<index_t, EXACT, ST_INT4, 1, false, 1, false, EXACT ? 2 : 4, EXACT>(a, d, table, first_slot, lane, lds);
   if (!done && lane == 0) { // wave-uniform verdict; nothing has been written or reported
     const int k = atomicAdd(a.redo_count, 1);
     WaveWork ww;
